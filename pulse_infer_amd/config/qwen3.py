@@ -1,0 +1,245 @@
+"""Qwen3 dense decoder configuration, read from config.json's own keys.
+
+Required keys are the ones the reference requires
+(reference: src/model/qwen3/config.cpp:250-325); optional sampling defaults
+come from generation_config.json (reference: src/model/qwen3/config.cpp:333-365).
+Keys the reference never reads (``attention_bias``, ``hidden_act``,
+``rope_scaling``) are read here only to refuse values this engine has no
+formula for.  The sliding-window keys choose a window per layer.
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional
+
+from .base import ConfigError, JsonReader, read_json_file, require_positive, resolve_model_dir
+from ..models.spec import LayerSpec, ModelSpec, PartSpec, RunSpec
+
+ARCHITECTURE = "Qwen3ForCausalLM"
+
+
+@dataclass
+class Qwen3Config:
+    vocab_size: int
+    hidden_size: int
+    intermediate_size: int
+    num_hidden_layers: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    head_dim: int
+    max_position_embeddings: int
+    rms_norm_eps: float
+    rope_theta: float
+    tie_word_embeddings: bool = False
+    torch_dtype: str = "bfloat16"
+    eos_token_ids: List[int] = field(default_factory=list)
+    use_sliding_window: bool = False
+    sliding_window: Optional[int] = None
+    max_window_layers: Optional[int] = None
+    layer_types: Optional[List[str]] = None
+    # sampling defaults (generation_config.json)
+    temperature: float = 0.0
+    top_k: int = 0
+    top_p: float = 0.0
+    architecture: str = ARCHITECTURE
+
+    # ------------------------------------------------------------------ reading
+    @classmethod
+    def from_dict(cls, data: Dict[str, Any], origin: str = "<dict>",
+                  generation: Optional[Dict[str, Any]] = None,
+                  generation_origin: str = "<dict>") -> "Qwen3Config":
+        r = JsonReader(data, origin)
+        num_heads = r.integer("num_attention_heads")
+        hidden = r.integer("hidden_size")
+        rope_theta = cls._read_rope_theta(r)
+        dtype = r.string("torch_dtype", None)
+        if dtype is None:
+            dtype = r.string("dtype", "bfloat16")
+        cfg = cls(
+            vocab_size=r.integer("vocab_size"),
+            hidden_size=hidden,
+            intermediate_size=r.integer("intermediate_size"),
+            num_hidden_layers=r.integer("num_hidden_layers"),
+            num_attention_heads=num_heads,
+            num_key_value_heads=r.integer("num_key_value_heads", num_heads),
+            head_dim=r.integer("head_dim", hidden // num_heads if num_heads > 0 else 0),
+            max_position_embeddings=r.integer("max_position_embeddings"),
+            rms_norm_eps=r.number("rms_norm_eps"),
+            rope_theta=rope_theta,
+            tie_word_embeddings=r.boolean("tie_word_embeddings", False),
+            torch_dtype=dtype,
+            eos_token_ids=r.int_or_int_list("eos_token_id"),
+            use_sliding_window=r.boolean("use_sliding_window", False),
+            sliding_window=r.integer("sliding_window", None),
+            max_window_layers=r.integer("max_window_layers", None),
+            layer_types=r.string_list("layer_types"),
+        )
+        # values this engine has no formula for
+        if r.boolean("attention_bias", False):
+            raise ConfigError(f"'attention_bias': true is not supported (in '{origin}')")
+        act = r.string("hidden_act", "silu")
+        if act != "silu":
+            raise ConfigError(f"'hidden_act': '{act}' is not supported, only 'silu' (in '{origin}')")
+        scaling = r.raw("rope_scaling")
+        if scaling is not None and not (isinstance(scaling, dict) and scaling.get("rope_type", scaling.get("type")) == "default"):
+            raise ConfigError(f"'rope_scaling' other than null is not supported (in '{origin}')")
+
+        if generation is not None:
+            g = JsonReader(generation, generation_origin)
+            eos = g.int_or_int_list("eos_token_id")
+            if eos:
+                cfg.eos_token_ids = eos
+            cfg.temperature = g.number("temperature", cfg.temperature)
+            cfg.top_k = g.integer("top_k", cfg.top_k)
+            cfg.top_p = g.number("top_p", cfg.top_p)
+        cfg.validate(origin)
+        return cfg
+
+    @staticmethod
+    def _read_rope_theta(r: JsonReader) -> float:
+        if r.has("rope_theta"):
+            return r.number("rope_theta")
+        params = r.raw("rope_parameters")
+        if isinstance(params, dict) and isinstance(params.get("rope_theta"), (int, float)):
+            kind = params.get("rope_type", "default")
+            if kind != "default":
+                raise ConfigError(f"rope_type '{kind}' is not supported (in '{r.origin}')")
+            return float(params["rope_theta"])
+        return r.number("rope_theta")  # raises the named error
+
+    @classmethod
+    def load(cls, path: str) -> "Qwen3Config":
+        model_dir = resolve_model_dir(path)
+        config_path = os.path.join(model_dir, "config.json")
+        data = read_json_file(config_path)
+        gen_path = os.path.join(model_dir, "generation_config.json")
+        generation = read_json_file(gen_path) if os.path.exists(gen_path) else None
+        return cls.from_dict(data, config_path, generation, gen_path)
+
+    # --------------------------------------------------------------- validation
+    def validate(self, origin: str = "<config>") -> None:
+        """Reference checks (src/model/qwen3/config.cpp:209-227) plus the ones the kernels need."""
+        require_positive(
+            origin,
+            vocab_size=self.vocab_size, hidden_size=self.hidden_size,
+            intermediate_size=self.intermediate_size, num_hidden_layers=self.num_hidden_layers,
+            num_attention_heads=self.num_attention_heads, num_key_value_heads=self.num_key_value_heads,
+            head_dim=self.head_dim, max_position_embeddings=self.max_position_embeddings,
+        )
+        if self.num_attention_heads % self.num_key_value_heads != 0:
+            raise ConfigError(
+                f"num_attention_heads({self.num_attention_heads}) is not divisible by "
+                f"num_key_value_heads({self.num_key_value_heads}) in '{origin}'")
+        if self.head_dim % 2 != 0:
+            raise ConfigError(f"head_dim({self.head_dim}) must be even for rotary pairs in '{origin}'")
+        if not self.rms_norm_eps >= 0.0:
+            raise ConfigError(f"rms_norm_eps({self.rms_norm_eps}) must not be negative in '{origin}'")
+        if not self.rope_theta > 0.0:
+            raise ConfigError(f"rope_theta({self.rope_theta}) must be positive in '{origin}'")
+        if self.torch_dtype not in ("bfloat16", "float32", "float16"):
+            raise ConfigError(f"torch_dtype '{self.torch_dtype}' is not supported in '{origin}'")
+        if self.use_sliding_window:
+            if self.sliding_window is None or self.sliding_window <= 0:
+                raise ConfigError(f"use_sliding_window needs a positive 'sliding_window' in '{origin}'")
+        if self.layer_types is not None:
+            if len(self.layer_types) != self.num_hidden_layers:
+                raise ConfigError(
+                    f"layer_types has {len(self.layer_types)} entries for {self.num_hidden_layers} layers in '{origin}'")
+            for kind in self.layer_types:
+                if kind not in ("full_attention", "sliding_attention"):
+                    raise ConfigError(f"layer type '{kind}' is not supported in '{origin}'")
+            if "sliding_attention" in self.layer_types and (self.sliding_window is None or self.sliding_window <= 0):
+                raise ConfigError(f"sliding_attention layers need a positive 'sliding_window' in '{origin}'")
+
+    # ------------------------------------------------------------------ writing
+    def to_dict(self) -> Dict[str, Any]:
+        out: Dict[str, Any] = {
+            "architectures": [self.architecture],
+            "model_type": "qwen3",
+            "vocab_size": self.vocab_size,
+            "hidden_size": self.hidden_size,
+            "intermediate_size": self.intermediate_size,
+            "num_hidden_layers": self.num_hidden_layers,
+            "num_attention_heads": self.num_attention_heads,
+            "num_key_value_heads": self.num_key_value_heads,
+            "head_dim": self.head_dim,
+            "max_position_embeddings": self.max_position_embeddings,
+            "rms_norm_eps": self.rms_norm_eps,
+            "rope_theta": self.rope_theta,
+            "rope_scaling": None,
+            "tie_word_embeddings": self.tie_word_embeddings,
+            "torch_dtype": self.torch_dtype,
+            "hidden_act": "silu",
+            "attention_bias": False,
+            "use_sliding_window": self.use_sliding_window,
+            "sliding_window": self.sliding_window,
+            "max_window_layers": self.max_window_layers,
+        }
+        if self.layer_types is not None:
+            out["layer_types"] = list(self.layer_types)
+        if self.eos_token_ids:
+            out["eos_token_id"] = self.eos_token_ids[0] if len(self.eos_token_ids) == 1 else list(self.eos_token_ids)
+        return out
+
+    # --------------------------------------------------------- layers from keys
+    def layer_window(self, layer: int) -> Optional[int]:
+        """The attention window of one layer, or None for all keys.
+
+        ``layer_types`` decides where given; else, with ``use_sliding_window``,
+        the first ``max_window_layers`` layers see all keys and the rest a window.
+        """
+        if self.layer_types is not None:
+            return self.sliding_window if self.layer_types[layer] == "sliding_attention" else None
+        if not self.use_sliding_window:
+            return None
+        first_windowed = self.max_window_layers if self.max_window_layers is not None else 0
+        return self.sliding_window if layer >= first_windowed else None
+
+    def model_spec(self) -> ModelSpec:
+        """The decoder as data (reference order of operations: src/model/qwen3/model.cpp:750-926)."""
+        norm = PartSpec("rmsnorm", {"size": self.hidden_size, "eps": self.rms_norm_eps})
+        rope = PartSpec("rope", {
+            "theta": self.rope_theta, "rotary_dim": self.head_dim, "head_dim": self.head_dim,
+            "pairing": "interleaved",
+        })
+        layers = []
+        for i in range(self.num_hidden_layers):
+            mixer = PartSpec("attention", {
+                "hidden_size": self.hidden_size,
+                "num_heads": self.num_attention_heads,
+                "num_kv_heads": self.num_key_value_heads,
+                "head_dim": self.head_dim,
+                "qk_norm": True,
+                "qk_norm_eps": self.rms_norm_eps,
+                "scale": float(self.head_dim) ** -0.5,
+                "window": self.layer_window(i),
+                "position": "rope",
+                "prefix": "self_attn",
+            })
+            ffn = PartSpec("gated_mlp", {
+                "hidden_size": self.hidden_size,
+                "intermediate_size": self.intermediate_size,
+                "activation": "silu",
+                "prefix": "mlp",
+            })
+            block = PartSpec("prenorm", {"mixer_norm": "input_layernorm", "ffn_norm": "post_attention_layernorm"})
+            layers.append(LayerSpec(prefix=f"model.layers.{i}", mixer=mixer, ffn=ffn, norm=norm, block=block))
+        spec = ModelSpec(
+            architecture=self.architecture,
+            vocab_size=self.vocab_size,
+            hidden_size=self.hidden_size,
+            max_positions=self.max_position_embeddings,
+            embedding=PartSpec("embedding", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size,
+                                             "name": "model.embed_tokens.weight"}),
+            layers=layers,
+            order=[RunSpec(layer=i) for i in range(self.num_hidden_layers)],
+            final_norm=norm,
+            final_norm_prefix="model.norm",
+            head=PartSpec("lm_head", {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size,
+                                      "name": "lm_head.weight", "tied": self.tie_word_embeddings,
+                                      "tied_to": "model.embed_tokens.weight"}),
+            positions={"rope": rope},
+        )
+        spec.validate()
+        return spec

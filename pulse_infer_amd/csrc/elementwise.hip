@@ -1,0 +1,202 @@
+// Row-wise kernels around the matrix products: embedding gather, residual add
+// fused with RMSNorm (optionally on gathered rows), SwiGLU, and the rotation
+// table of the position encoding.  All arithmetic is float32 (the rotation
+// angle float64); storage types are template arguments.
+#include "common.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+// ---------------------------------------------------------------- error text
+static thread_local char g_error[512] = "";
+
+extern "C" const char* pulse_last_error() { return g_error; }
+
+void pulse_set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+// ------------------------------------------------------------------ embedding
+// out[t, :] = table[ids[t], :] widened to float32 (the residual stream).
+// Ids are checked on the host; a bad id here still reads nothing out of range
+// and raises *bad_id so that the caller can fail.
+// (reference: src/ops/kernels/cuda/embedding_kernel.cu:7-28 leaves zeros silently)
+template <typename TW>
+__global__ void embed_gather_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
+                                    float* __restrict__ out, int hidden, int vocab, int* bad_id) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    float* dst = out + static_cast<int64_t>(t) * hidden;
+    if (id < 0 || id >= vocab) {
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = 0.f;
+        if (threadIdx.x == 0) *bad_id = 1;
+        return;
+    }
+    const TW* src = table + static_cast<int64_t>(id) * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32<TW>(src[i]);
+}
+
+extern "C" int pulse_embed_gather(const int* ids, const void* table, int table_dtype, float* out,
+                                  int tokens, int hidden, int vocab, int* bad_id, hipStream_t stream) {
+    PULSE_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embed_gather: bad sizes T=%d H=%d V=%d", tokens, hidden, vocab);
+    PULSE_REQUIRE(pulse_dtype_ok(table_dtype), "embed_gather: bad dtype tag %d", table_dtype);
+    PULSE_REQUIRE(ids && table && out && bad_id, "embed_gather: null pointer");
+    if (tokens == 0) return 0;
+    PULSE_DISPATCH_DTYPE(table_dtype, TW,
+        hipLaunchKernelGGL(embed_gather_kernel<TW>, dim3(tokens), dim3(256), 0, stream, ids,
+                           static_cast<const TW*>(table), out, hidden, vocab, bad_id));
+    PULSE_LAUNCH_CHECK("embed_gather");
+    return 0;
+}
+
+// --------------------------------------------------- residual add + RMSNorm
+// For output row r (input row s = rows ? rows[r] : r):
+//   v = h[s] + delta[s]            (delta optional)
+//   h[s] = v                       (only when write_back)
+//   y[r] = v * (1 / sqrt(mean(v^2) + eps)) * w      one rounding at the end
+// (formula: src/ops/kernels/cuda/rmsnorm_kernel.cu:97-157; the reference adds the
+// residual in a separate kernel, src/ops/kernels/cuda/add_kernel.cu:73-92)
+template <typename TD, typename TW, typename TY>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                   const int* __restrict__ rows, const TW* __restrict__ w,
+                                   TY* __restrict__ y, int hidden, float eps, int write_back) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x;
+    const int64_t s = rows ? rows[r] : r;
+    float* hrow = h + s * hidden;
+    const TD* drow = delta ? delta + s * hidden : nullptr;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v = hrow[i];
+        if (drow) v += to_f32<TD>(drow[i]);
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(hidden) + eps);
+    TY* yrow = y + static_cast<int64_t>(r) * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        float v = hrow[i];
+        if (drow) v += to_f32<TD>(drow[i]);
+        if (write_back) hrow[i] = v;
+        yrow[i] = from_f32<TY>(v * inv * to_f32<TW>(w[i]));
+    }
+}
+
+extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, const int* rows,
+                                 const void* w, int w_dtype, void* y, int y_dtype, int out_rows,
+                                 int hidden, float eps, int write_back, hipStream_t stream) {
+    PULSE_REQUIRE(out_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d H=%d", out_rows, hidden);
+    PULSE_REQUIRE(pulse_dtype_ok(delta_dtype) && pulse_dtype_ok(w_dtype) && pulse_dtype_ok(y_dtype),
+                  "add_rmsnorm: bad dtype tag");
+    PULSE_REQUIRE(h && w && y, "add_rmsnorm: null pointer");
+    PULSE_REQUIRE(!(rows && write_back), "add_rmsnorm: write_back with gathered rows is not supported");
+    if (out_rows == 0) return 0;
+    PULSE_DISPATCH_DTYPE(delta_dtype, TD, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(y_dtype, TY,
+        hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, TY>), dim3(out_rows), dim3(256), 0, stream, h,
+                           static_cast<const TD*>(delta), rows, static_cast<const TW*>(w),
+                           static_cast<TY*>(y), hidden, eps, write_back))));
+    PULSE_LAUNCH_CHECK("add_rmsnorm");
+    return 0;
+}
+
+// -------------------------------------------------------------- residual add
+// h += delta (used where no norm follows).
+template <typename TD>
+__global__ void residual_add_kernel(float* __restrict__ h, const TD* __restrict__ delta, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) h[i] += to_f32<TD>(delta[i]);
+}
+
+extern "C" int pulse_residual_add(float* h, const void* delta, int delta_dtype, int64_t n, hipStream_t stream) {
+    PULSE_REQUIRE(n >= 0 && pulse_dtype_ok(delta_dtype) && h && delta, "residual_add: bad arguments");
+    if (n == 0) return 0;
+    const int64_t blocks = (n + 255) / 256;
+    PULSE_REQUIRE(blocks < (1ll << 31), "residual_add: too many elements (%lld)", static_cast<long long>(n));
+    PULSE_DISPATCH_DTYPE(delta_dtype, TD,
+        hipLaunchKernelGGL(residual_add_kernel<TD>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, h,
+                           static_cast<const TD*>(delta), n));
+    PULSE_LAUNCH_CHECK("residual_add");
+    return 0;
+}
+
+// --------------------------------------------------------------------- SwiGLU
+// gu is [T, 2*I]: gate in columns [0, I), up in [I, 2I).  out[t, i] = silu(g) * u,
+// silu(x) = x / (1 + exp(-x)), product in float32, one rounding.
+// (reference: src/ops/kernels/cuda/silu_kernel.cu:82-97 then mul_kernel.cu:39-46, two roundings)
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int64_t total) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int64_t t = idx / inter;
+    const int i = static_cast<int>(idx - t * inter);
+    const T* row = gu + t * 2 * inter;
+    const float g = to_f32<T>(row[i]);
+    const float u = to_f32<T>(row[inter + i]);
+    const float s = g / (1.0f + expf(-g));
+    out[idx] = from_f32<T>(s * u);
+}
+
+extern "C" int pulse_swiglu(const void* gu, void* out, int dtype, int tokens, int inter, hipStream_t stream) {
+    PULSE_REQUIRE(tokens >= 0 && inter > 0 && pulse_dtype_ok(dtype) && gu && out, "swiglu: bad arguments");
+    const int64_t total = static_cast<int64_t>(tokens) * inter;
+    if (total == 0) return 0;
+    const int64_t blocks = (total + 255) / 256;
+    PULSE_REQUIRE(blocks < (1ll << 31), "swiglu: too many elements");
+    PULSE_DISPATCH_DTYPE(dtype, T,
+        hipLaunchKernelGGL(swiglu_kernel<T>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
+                           static_cast<const T*>(gu), static_cast<T*>(out), inter, total));
+    PULSE_LAUNCH_CHECK("swiglu");
+    return 0;
+}
+
+// ------------------------------------------------------------- rotation table
+// cos_out/sin_out [T, half]: angle = position * inv_freq[i], the product and the
+// functions in float64, then rounded to float32 once.  inv_freq[i] = theta^(-2i/rotary_dim)
+// comes from the host in float64.
+// (reference angle: src/ops/kernels/cuda/rope_kernel.cu:119-123, float32 throughout)
+__global__ void rope_table_kernel(const int* __restrict__ positions, const double* __restrict__ inv_freq,
+                                  float* __restrict__ cos_out, float* __restrict__ sin_out, int half, int64_t total) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int64_t t = idx / half;
+    const int i = static_cast<int>(idx - t * half);
+    const double angle = static_cast<double>(positions[t]) * inv_freq[i];
+    double s, c;
+    sincos(angle, &s, &c);
+    cos_out[idx] = static_cast<float>(c);
+    sin_out[idx] = static_cast<float>(s);
+}
+
+extern "C" int pulse_rope_table(const int* positions, const double* inv_freq, float* cos_out, float* sin_out,
+                                int tokens, int half, hipStream_t stream) {
+    PULSE_REQUIRE(tokens >= 0 && half > 0 && positions && inv_freq && cos_out && sin_out, "rope_table: bad arguments");
+    const int64_t total = static_cast<int64_t>(tokens) * half;
+    if (total == 0) return 0;
+    const int64_t blocks = (total + 255) / 256;
+    hipLaunchKernelGGL(rope_table_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, positions,
+                       inv_freq, cos_out, sin_out, half, total);
+    PULSE_LAUNCH_CHECK("rope_table");
+    return 0;
+}
+
+// ------------------------------------------------------------- row gather
+// out[r, :] = in[rows[r], :] for float32 rows (used to pick the wanted rows of the residual).
+__global__ void gather_rows_kernel(const float* __restrict__ in, const int* __restrict__ rows,
+                                   float* __restrict__ out, int hidden) {
+    const int r = blockIdx.x;
+    const float* src = in + static_cast<int64_t>(rows[r]) * hidden;
+    float* dst = out + static_cast<int64_t>(r) * hidden;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = src[i];
+}
+
+extern "C" int pulse_gather_rows(const float* in, const int* rows, float* out, int out_rows, int hidden,
+                                 hipStream_t stream) {
+    PULSE_REQUIRE(out_rows >= 0 && hidden > 0 && in && rows && out, "gather_rows: bad arguments");
+    if (out_rows == 0) return 0;
+    hipLaunchKernelGGL(gather_rows_kernel, dim3(out_rows), dim3(256), 0, stream, in, rows, out, hidden);
+    PULSE_LAUNCH_CHECK("gather_rows");
+    return 0;
+}

@@ -1,0 +1,177 @@
+"""The step function.
+
+``ModelRunner.step(entries)`` takes a batch of (request, its next tokens, the
+places whose logits are wanted): portions of prompts beside single decoded
+tokens, cut anywhere.  It runs only those tokens, as one batch, against the
+cache that earlier steps left, and returns float32 logits for the wanted places
+in the order of the entries and of ``want``.  Pages must have been reserved
+before (``reserve``); the step itself allocates no page.
+
+(reference: Qwen3Model::forward_batched, src/model/qwen3/model.cpp:1179-1374,
+which takes flat tokens/positions/seq_ids, grows pages inside the forward and
+returns logits for every token.)
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager, PagedKVSpec, StateSpec
+from ..models.causal_lm import CausalLM
+from ..parts.base import EntryMeta, PagedCacheView, StateView, StepContext
+
+
+class StepError(ValueError):
+    """The batch handed to ``step`` breaks one of its preconditions."""
+
+
+@dataclass
+class StepEntry:
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=list)  # indices into ``tokens``
+
+
+class _Staging:
+    """Pinned host buffers for a step's integer metadata, used in turn."""
+
+    def __init__(self, device: torch.device, depth: int = 2):
+        self.device = device
+        self.host: List[Optional[torch.Tensor]] = [None] * depth
+        self.events: List[Optional[torch.cuda.Event]] = [None] * depth
+        self.turn = 0
+
+    def upload(self, data: np.ndarray) -> torch.Tensor:
+        i = self.turn
+        self.turn = (self.turn + 1) % len(self.host)
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        n = int(data.size)
+        if self.host[i] is None or self.host[i].numel() < n:
+            self.host[i] = torch.empty(max(n, 4096), dtype=torch.int32, pin_memory=True)
+        self.host[i][:n].numpy()[:] = data
+        dev = torch.empty(n, dtype=torch.int32, device=self.device)
+        dev.copy_(self.host[i][:n], non_blocking=True)
+        if self.events[i] is None:
+            self.events[i] = torch.cuda.Event()
+        self.events[i].record()
+        return dev
+
+
+class ModelRunner:
+    def __init__(self, model: CausalLM, page_size: int, num_pages: int, max_requests: int = 64):
+        self.model = model
+        self.device = model.device
+        self.cache = CacheManager(model.run_cache_specs(), page_size, num_pages, max_requests)
+        self.cache.allocate_storage(self.device, model.act_dtype)
+        self.views: List[Any] = []
+        order = model.spec.order
+        for index, run in enumerate(order):
+            source = run.cache_of if run.cache_of is not None else index
+            spec = self.cache.run_specs[source]
+            if isinstance(spec, PagedKVSpec):
+                g, i = self.cache.run_group[source]
+                group = self.cache.groups[g]
+                self.views.append(PagedCacheView(group=g, keys=group.keys[i], values=group.values[i],
+                                                 page_size=group.page_size, writable=run.cache_of is None))
+            elif isinstance(spec, StateSpec):
+                self.views.append(StateView(self.cache.state[source]))
+            else:
+                self.views.append(None)
+        self._staging = _Staging(self.device)
+        self.max_positions = model.spec.max_positions
+        self.steps = 0
+        self.tokens_run = 0
+
+    # ----------------------------------------------------------------- requests
+    def add_request(self, request: Hashable) -> int:
+        return self.cache.add_request(request)
+
+    def free_request(self, request: Hashable) -> None:
+        self.cache.free_request(request)
+
+    def reserve(self, request: Hashable, length: int) -> None:
+        self.cache.reserve(request, length)
+
+    # --------------------------------------------------------------------- step
+    def _check(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        seen = set()
+        vocab = self.model.vocab_size
+        for e in entries:
+            if e.request in seen:
+                raise StepError(f"request {e.request!r} appears twice in one step")
+            seen.add(e.request)
+            if not self.cache.has_request(e.request):
+                raise StepError(f"request {e.request!r} is not live (add_request first)")
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.request!r} brings no tokens")
+            start = self.cache.computed(e.request)
+            if start + n > self.max_positions:
+                raise StepError(f"request {e.request!r} would reach position {start + n - 1}, the model allows "
+                                f"{self.max_positions} positions")
+            if self.cache.reserved(e.request) < start + n:
+                raise StepError(f"request {e.request!r}: pages are reserved for {self.cache.reserved(e.request)} "
+                                f"tokens, the step needs {start + n}")
+            for tok in e.tokens:
+                if not 0 <= int(tok) < vocab:
+                    raise StepError(f"request {e.request!r}: token id {tok} is outside the vocabulary of {vocab}")
+            for w in e.want:
+                if not 0 <= int(w) < n:
+                    raise StepError(f"request {e.request!r}: wanted place {w} is outside its {n} tokens")
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        self._check(entries)
+        cache = self.cache
+        metas: List[EntryMeta] = []
+        row = 0
+        for e in entries:
+            metas.append(EntryMeta(e.request, cache.slot_of(e.request), cache.computed(e.request), len(e.tokens), row))
+            row += len(e.tokens)
+        total, batch = row, len(metas)
+        want_rows = [m.first_row + int(w) for e, m in zip(entries, metas) for w in e.want]
+        widths = []
+        for g in cache.groups:
+            widths.append(max(1, max(g.pages_for(m.start + m.count) for m in metas)))
+
+        # one flat int32 array: [ids | positions | token_entry | start | count | first_row | slot | want | tables...]
+        sizes = [total, total, total, batch, batch, batch + 1, batch, len(want_rows)] + [batch * w for w in widths]
+        offsets = np.concatenate([[0], np.cumsum(sizes)])
+        flat = np.zeros(int(offsets[-1]), dtype=np.int32)
+        ids, pos, tok_entry = (flat[offsets[i]:offsets[i + 1]] for i in range(3))
+        for i, (e, m) in enumerate(zip(entries, metas)):
+            sl = slice(m.first_row, m.first_row + m.count)
+            ids[sl] = np.asarray(e.tokens, dtype=np.int32)
+            pos[sl] = np.arange(m.start, m.start + m.count, dtype=np.int32)
+            tok_entry[sl] = i
+        flat[offsets[3]:offsets[4]] = [m.start for m in metas]
+        flat[offsets[4]:offsets[5]] = [m.count for m in metas]
+        flat[offsets[5]:offsets[6]] = [m.first_row for m in metas] + [total]
+        flat[offsets[6]:offsets[7]] = [m.slot for m in metas]
+        flat[offsets[7]:offsets[8]] = want_rows
+        for gi, (g, w) in enumerate(zip(cache.groups, widths)):
+            table = np.full((batch, w), -1, dtype=np.int32)
+            for i, m in enumerate(metas):
+                pages = cache.table(gi, m.request)[:w]
+                table[i, :len(pages)] = pages
+            flat[offsets[8 + gi]:offsets[9 + gi]] = table.reshape(-1)
+
+        dev = self._staging.upload(flat)
+        part = [dev[offsets[i]:offsets[i + 1]] for i in range(len(sizes))]
+        ctx = StepContext(
+            num_tokens=total, entries=metas, token_ids=part[0], positions=part[1], token_entry=part[2],
+            entry_start=part[3], entry_count=part[4], entry_first_row=part[5], entry_slot=part[6],
+            block_tables={gi: part[8 + gi].view(batch, w) for gi, w in enumerate(widths)},
+            want_rows=part[7], num_wanted=len(want_rows), workspace=self.model.workspace,
+            max_count=max(m.count for m in metas), max_context=max(m.start + m.count for m in metas))
+        logits = self.model.forward(ctx, self.views)
+        for m in metas:
+            cache.advance(m.request, m.start + m.count)
+        self.steps += 1
+        self.tokens_run += total
+        return logits

@@ -1,0 +1,258 @@
+"""Python faces of the HIP entry points.
+
+Each function checks on the host that devices, storage types, shapes and
+strides are what its kernel assumes, then launches on torch's current stream.
+Tensors are passed as raw device pointers; nothing here allocates unless a
+result tensor is asked for, and nothing falls back to another implementation.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .library import KernelError, call
+
+_TAG = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _tag(t: torch.Tensor, what: str) -> int:
+    try:
+        return _TAG[t.dtype]
+    except KeyError:
+        raise KernelError(f"{what}: storage type {t.dtype} is not supported (float32 or bfloat16)") from None
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def _i32(v: int) -> ctypes.c_int:
+    return ctypes.c_int(int(v))
+
+
+def _i64(v: int) -> ctypes.c_int64:
+    return ctypes.c_int64(int(v))
+
+
+def _f32(v: float) -> ctypes.c_float:
+    return ctypes.c_float(float(v))
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelError(msg)
+
+
+def _gpu(what: str, *tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError(f"{what}: every tensor must live on the GPU, got one on {t.device}")
+
+
+def _int_vec(what: str, t: torch.Tensor, n: Optional[int] = None) -> None:
+    _need(t.dtype == torch.int32 and t.is_contiguous(), f"{what} must be a contiguous int32 tensor")
+    if n is not None:
+        _need(t.numel() >= n, f"{what} holds {t.numel()} entries, {n} are needed")
+
+
+# ---------------------------------------------------------------------------
+def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, bad_id: torch.Tensor) -> None:
+    """out[t] = float32(table[ids[t]]); ``bad_id`` (int32[1]) is raised for an id outside the table."""
+    _gpu("embed_gather", ids, table, out, bad_id)
+    tokens = ids.numel()
+    vocab, hidden = table.shape
+    _int_vec("embed_gather: ids", ids)
+    _need(table.is_contiguous() and out.is_contiguous(), "embed_gather: table and out must be contiguous")
+    _need(out.dtype == torch.float32 and tuple(out.shape) == (tokens, hidden),
+          f"embed_gather: out must be float32 [{tokens}, {hidden}], got {out.dtype} {tuple(out.shape)}")
+    _need(bad_id.dtype == torch.int32 and bad_id.numel() >= 1, "embed_gather: bad_id must be int32[1]")
+    call("pulse_embed_gather", _ptr(ids), _ptr(table), _i32(_tag(table, "embed_gather")), _ptr(out),
+         _i32(tokens), _i32(hidden), _i32(vocab), _ptr(bad_id), _stream())
+
+
+def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: Optional[torch.Tensor] = None, write_back: bool = True) -> None:
+    """out[r] = rmsnorm(h[s] + delta[s]) * weight, s = rows[r] or r; with write_back h[s] keeps the sum."""
+    _gpu("add_rmsnorm", h, delta, weight, out, rows)
+    _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "add_rmsnorm: h must be contiguous float32 [T, H]")
+    hidden = h.shape[1]
+    n_out = rows.numel() if rows is not None else h.shape[0]
+    if rows is not None:
+        _int_vec("add_rmsnorm: rows", rows)
+        write_back = False
+    if delta is not None:
+        _need(delta.shape == h.shape and delta.is_contiguous(), "add_rmsnorm: delta must match h")
+    _need(weight.numel() == hidden and weight.is_contiguous(), f"add_rmsnorm: weight must hold {hidden} values")
+    _need(out.is_contiguous() and tuple(out.shape) == (n_out, hidden),
+          f"add_rmsnorm: out must be [{n_out}, {hidden}], got {tuple(out.shape)}")
+    call("pulse_add_rmsnorm", _ptr(h), _ptr(delta), _i32(_tag(delta, "add_rmsnorm") if delta is not None else 0),
+         _ptr(rows), _ptr(weight), _i32(_tag(weight, "add_rmsnorm")), _ptr(out), _i32(_tag(out, "add_rmsnorm")),
+         _i32(n_out), _i32(hidden), _f32(eps), _i32(1 if (write_back and delta is not None) else 0), _stream())
+
+
+def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
+    _gpu("residual_add", h, delta)
+    _need(h.dtype == torch.float32 and h.is_contiguous() and delta.is_contiguous() and h.shape == delta.shape,
+          "residual_add: h must be contiguous float32 and delta of the same shape")
+    call("pulse_residual_add", _ptr(h), _ptr(delta), _i32(_tag(delta, "residual_add")), _i64(h.numel()), _stream())
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+    _gpu("swiglu", gate_up, out)
+    tokens, two_i = gate_up.shape
+    _need(two_i % 2 == 0 and tuple(out.shape) == (tokens, two_i // 2), "swiglu: out must be [T, I] for gate_up [T, 2I]")
+    _need(gate_up.is_contiguous() and out.is_contiguous() and gate_up.dtype == out.dtype,
+          "swiglu: contiguous tensors of one storage type are needed")
+    call("pulse_swiglu", _ptr(gate_up), _ptr(out), _i32(_tag(out, "swiglu")), _i32(tokens), _i32(two_i // 2), _stream())
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos_out: torch.Tensor, sin_out: torch.Tensor) -> None:
+    """cos/sin of position * inv_freq, computed in float64 and stored as float32 [T, half]."""
+    _gpu("rope_table", positions, inv_freq, cos_out, sin_out)
+    tokens, half = positions.numel(), inv_freq.numel()
+    _int_vec("rope_table: positions", positions)
+    _need(inv_freq.dtype == torch.float64 and inv_freq.is_contiguous(), "rope_table: inv_freq must be float64")
+    for t in (cos_out, sin_out):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (tokens, half),
+              f"rope_table: tables must be float32 [{tokens}, {half}]")
+    call("pulse_rope_table", _ptr(positions), _ptr(inv_freq), _ptr(cos_out), _ptr(sin_out), _i32(tokens), _i32(half),
+         _stream())
+
+
+def gather_rows(src: torch.Tensor, rows: torch.Tensor, out: torch.Tensor) -> None:
+    _gpu("gather_rows", src, rows, out)
+    _int_vec("gather_rows: rows", rows)
+    _need(src.dtype == torch.float32 and out.dtype == torch.float32 and src.is_contiguous() and out.is_contiguous()
+          and out.shape[0] == rows.numel() and out.shape[1] == src.shape[1], "gather_rows: bad tensors")
+    call("pulse_gather_rows", _ptr(src), _ptr(rows), _ptr(out), _i32(rows.numel()), _i32(src.shape[1]), _stream())
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """out[M, N] = a[M, K] @ w[N, K]^T with float32 fused multiply-adds in a fixed order."""
+    _gpu("gemm_f32", a, w, out)
+    _need(a.dim() == 2 and w.dim() == 2 and out.dim() == 2, "gemm_f32: matrices are needed")
+    m, k = a.shape
+    n, k2 = w.shape
+    _need(k == k2, f"gemm_f32: inner sizes differ: a is [{m}, {k}], w is [{n}, {k2}]")
+    _need(tuple(out.shape) == (m, n), f"gemm_f32: out must be [{m}, {n}], got {tuple(out.shape)}")
+    _need(a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, "gemm_f32: rows must be contiguous")
+    call("pulse_gemm_f32", _ptr(a), _i32(_tag(a, "gemm_f32")), _ptr(w), _i32(_tag(w, "gemm_f32")), _ptr(out),
+         _i32(_tag(out, "gemm_f32")), _i32(m), _i32(n), _i32(k), _i64(a.stride(0) if m > 1 else k),
+         _i64(w.stride(0) if n > 1 else k), _i64(out.stride(0) if m > 1 else n), _stream())
+
+
+def _check_cache(what: str, kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, d: int):
+    _need(kcache.dim() == 4 and vcache.dim() == 4, f"{what}: caches must be [pages, kv_heads, ., .]")
+    pages, h, page_size, dd = kcache.shape
+    _need(h == nkv and dd == d, f"{what}: key cache is {tuple(kcache.shape)}, expected [P, {nkv}, page, {d}]")
+    _need(tuple(vcache.shape) == (pages, nkv, d, page_size),
+          f"{what}: value cache is {tuple(vcache.shape)}, expected {(pages, nkv, d, page_size)}")
+    _need(kcache.is_contiguous() and vcache.is_contiguous() and kcache.dtype == vcache.dtype,
+          f"{what}: caches must be contiguous and of one storage type")
+    return pages, page_size
+
+
+def qk_rope_kv(qkv: torch.Tensor, nq: int, nkv: int, d: int, q_weight: Optional[torch.Tensor],
+               k_weight: Optional[torch.Tensor], eps: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+               rotary_dim: int, pairing: int, kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor],
+               positions: torch.Tensor, token_entry: torch.Tensor, block_table: Optional[torch.Tensor],
+               write_kv: bool = True) -> None:
+    """Per-head norm and rotation of q (in place) and k, and the page write of k and v."""
+    _gpu("qk_rope_kv", qkv, q_weight, k_weight, cos, sin, kcache, vcache, positions, token_entry, block_table)
+    tokens = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1, "qk_rope_kv: qkv must be [T, columns] with contiguous rows")
+    cols = (nq + 2 * nkv) * d if write_kv else nq * d
+    _need(qkv.shape[1] >= cols, f"qk_rope_kv: qkv has {qkv.shape[1]} columns, {cols} are needed")
+    _int_vec("qk_rope_kv: positions", positions, tokens)
+    _int_vec("qk_rope_kv: token_entry", token_entry, tokens)
+    w_tag = 0
+    if q_weight is not None:
+        _need(k_weight is not None and q_weight.numel() == d and k_weight.numel() == d
+              and q_weight.dtype == k_weight.dtype and q_weight.is_contiguous() and k_weight.is_contiguous(),
+              f"qk_rope_kv: the two norm weights must hold {d} values of one storage type")
+        w_tag = _tag(q_weight, "qk_rope_kv")
+    if cos is not None:
+        half = rotary_dim // 2
+        for t in (cos, sin):
+            _need(t is not None and t.dtype == torch.float32 and t.is_contiguous() and t.shape[0] >= tokens
+                  and t.shape[1] == half, f"qk_rope_kv: cos/sin must be float32 [T, {half}]")
+    pages = page_size = width = 0
+    c_tag = 0
+    if write_kv:
+        _need(kcache is not None and vcache is not None and block_table is not None, "qk_rope_kv: the cache is missing")
+        pages, page_size = _check_cache("qk_rope_kv", kcache, vcache, nkv, d)
+        _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+              "qk_rope_kv: block_table must be contiguous int32 [entries, width]")
+        width = block_table.shape[1]
+        c_tag = _tag(kcache, "qk_rope_kv")
+    call("pulse_qk_rope_kv", _ptr(qkv), _i32(_tag(qkv, "qk_rope_kv")), _i64(qkv.stride(0)), _ptr(q_weight),
+         _ptr(k_weight), _i32(w_tag), _f32(eps), _ptr(cos), _ptr(sin), _i32(rotary_dim if cos is not None else 0),
+         _i32(pairing), _ptr(kcache if write_kv else None), _ptr(vcache if write_kv else None), _i32(c_tag),
+         _ptr(positions), _ptr(token_entry), _ptr(block_table if write_kv else None), _i32(width), _i32(tokens),
+         _i32(nq), _i32(nkv), _i32(d), _i32(page_size), _i32(pages), _i32(1 if write_kv else 0), _stream())
+
+
+def attn_generic(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
+                 vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
+                 scale: float, window: int = 0) -> None:
+    """Paged causal attention, one wavefront per (token, head), float32 arithmetic.
+
+    ``q`` is [T, >= nq*d] (rows may be strided, e.g. the front of a fused qkv buffer); ``out`` is [T, nq*d].
+    """
+    _gpu("attn_generic", q, out, kcache, vcache, positions, token_entry, block_table)
+    tokens = q.shape[0]
+    _need(q.dim() == 2 and out.dim() == 2 and q.stride(1) == 1 and out.stride(1) == 1 and q.dtype == out.dtype,
+          "attn_generic: q and out must be matrices of one storage type with contiguous rows")
+    _need(q.shape[1] >= nq * d and out.shape[1] >= nq * d and out.shape[0] == tokens, "attn_generic: q/out too narrow")
+    pages, page_size = _check_cache("attn_generic", kcache, vcache, nkv, d)
+    _int_vec("attn_generic: positions", positions, tokens)
+    _int_vec("attn_generic: token_entry", token_entry, tokens)
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+          "attn_generic: block_table must be contiguous int32 [entries, width]")
+    call("pulse_attn_generic", _ptr(q), _i64(q.stride(0)), _ptr(out), _i64(out.stride(0)), _i32(_tag(q, "attn_generic")),
+         _ptr(kcache), _ptr(vcache), _i32(_tag(kcache, "attn_generic")), _ptr(positions), _ptr(token_entry),
+         _ptr(block_table), _i32(block_table.shape[1]), _i32(tokens), _i32(nq), _i32(nkv), _i32(d), _i32(page_size),
+         _i32(pages), _f32(scale), _i32(window), _stream())
+
+
+def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.Tensor] = None,
+           top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
+           uniform: Optional[torch.Tensor] = None, penalty: Optional[torch.Tensor] = None,
+           seen_row: Optional[torch.Tensor] = None, seen_masks: Optional[torch.Tensor] = None,
+           banned: Optional[torch.Tensor] = None) -> None:
+    """out[r] = next token of row r (largest logit when temperature is absent or <= 0)."""
+    _gpu("sample", logits, out, temperature, top_k, top_p, uniform, penalty, seen_row, seen_masks, banned)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1, "sample: logits must be float32 [R, V]")
+    rows, vocab = logits.shape
+    _int_vec("sample: out", out, rows)
+    for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                        ("top_p", top_p, torch.float32), ("uniform", uniform, torch.float32),
+                        ("penalty", penalty, torch.float32), ("seen_row", seen_row, torch.int32)):
+        if t is not None:
+            _need(t.dtype == dt and t.is_contiguous() and t.numel() >= rows, f"sample: {name} must be {dt}[{rows}]")
+    words = 0
+    for name, t in (("seen_masks", seen_masks), ("banned", banned)):
+        if t is not None:
+            _need(t.dtype == torch.int32 and t.is_contiguous(), f"sample: {name} must be contiguous int32 words")
+            w = t.shape[-1]
+            _need(words in (0, w), "sample: masks differ in width")
+            words = w
+    call("pulse_sample", _ptr(logits), _i32(rows), _i32(vocab), _i64(logits.stride(0) if rows > 1 else vocab),
+         _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform), _ptr(penalty), _ptr(seen_row), _ptr(seen_masks),
+         _ptr(banned), _i32(words), _ptr(out), _stream())
+
+
+def mark_seen(masks: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, vocab: int) -> None:
+    _gpu("mark_seen", masks, rows, tokens)
+    _need(masks.dtype == torch.int32 and masks.dim() == 2 and masks.is_contiguous(), "mark_seen: masks must be int32 [slots, words]")
+    _int_vec("mark_seen: rows", rows)
+    _int_vec("mark_seen: tokens", tokens, rows.numel())
+    call("pulse_mark_seen", _ptr(masks), _i32(masks.shape[1]), _ptr(rows), _ptr(tokens), _i32(rows.numel()),
+         _i32(vocab), _stream())

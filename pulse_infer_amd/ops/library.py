@@ -1,0 +1,59 @@
+"""Loading the compiled HIP kernels.
+
+There is no fallback: when the library cannot be loaded or built, every op
+raises ``KernelLibraryError``.  A library that matches the current sources is
+loaded as it is; otherwise it is compiled first (seconds, with progress lines).
+"""
+from __future__ import annotations
+
+import ctypes
+import threading
+from typing import Optional
+
+from ..csrc import build as _build
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+class KernelError(RuntimeError):
+    """An entry point refused its arguments or a launch failed."""
+
+
+_lock = threading.Lock()
+_lib: Optional[ctypes.CDLL] = None
+_lib_path: Optional[str] = None
+
+
+def library_path() -> Optional[str]:
+    return _lib_path
+
+
+def load() -> ctypes.CDLL:
+    global _lib, _lib_path
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        try:
+            path = _build.existing_library() or _build.build()
+            lib = ctypes.CDLL(path)
+        except Exception as exc:  # noqa: BLE001 - one loud error, whatever went wrong
+            raise KernelLibraryError(
+                f"the HIP kernel library of pulse_infer_amd is not available: {exc}. "
+                "Build it with `python -m pulse_infer_amd.csrc.build` (needs hipcc).") from exc
+        lib.pulse_last_error.restype = ctypes.c_char_p
+        _lib, _lib_path = lib, path
+        return lib
+
+
+def call(name: str, *args) -> None:
+    """Call an entry point; a non-zero return becomes a ``KernelError`` with the library's message."""
+    lib = load()
+    fn = getattr(lib, name)
+    fn.restype = ctypes.c_int
+    code = fn(*args)
+    if code != 0:
+        raise KernelError(f"{name}: {lib.pulse_last_error().decode(errors='replace')}")

@@ -1,0 +1,97 @@
+"""Causal attention over a paged cache, with grouped key/value heads, optional
+per-head RMSNorm of q and k, an optional window and a pluggable position encoding.
+
+Order of operations per token (reference: src/model/qwen3/model.cpp:784-876):
+q, k, v = x Wq^T, x Wk^T, x Wv^T; q, k <- RMSNorm over head_dim (one weight for
+all heads); q, k <- rotation at the token's position; k, v written to the
+cache; o = softmax(q K^T * scale) V over keys lo..position of the same request;
+output = o Wo^T.  Query head h reads kv head h // (num_heads // num_kv_heads).
+A window w gives lo = max(0, position - w + 1); without one lo = 0.
+
+The three projections are one product with the row-stacked weight (a layout
+choice); norm, rotation and the cache write are one kernel; the attention
+kernel is chosen by size and storage type.
+"""
+from __future__ import annotations
+
+from typing import Any, Dict, Optional
+
+import torch
+
+from ..cache.manager import PagedKVSpec
+from ..ops import kernels
+from ..weights.store import TensorSpec
+from .base import MIXERS, BuildContext, PagedCacheView, Part, StepContext
+from .linear import Linear
+
+
+@MIXERS.register("attention")
+class PagedAttention(Part):
+    @classmethod
+    def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
+        hidden, nq, nkv, d = (params[k] for k in ("hidden_size", "num_heads", "num_kv_heads", "head_dim"))
+        specs = {
+            "q_proj.weight": TensorSpec((nq * d, hidden), fan_in=hidden),
+            "k_proj.weight": TensorSpec((nkv * d, hidden), fan_in=hidden),
+            "v_proj.weight": TensorSpec((nkv * d, hidden), fan_in=hidden),
+            "o_proj.weight": TensorSpec((hidden, nq * d), fan_in=nq * d),
+        }
+        if params.get("qk_norm", False):
+            specs["q_norm.weight"] = TensorSpec((d,), kind="norm")
+            specs["k_norm.weight"] = TensorSpec((d,), kind="norm")
+        return specs
+
+    def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
+        self.hidden = int(params["hidden_size"])
+        self.nq = int(params["num_heads"])
+        self.nkv = int(params["num_kv_heads"])
+        self.d = int(params["head_dim"])
+        if self.nq % self.nkv:
+            raise ValueError(f"{self.nq} query heads are not a multiple of {self.nkv} key/value heads")
+        self.scale = float(params["scale"])
+        self.window = params.get("window")
+        if self.window is not None and int(self.window) <= 0:
+            raise ValueError(f"an attention window must be positive, got {self.window}")
+        self.qk_norm = bool(params.get("qk_norm", False))
+        self.eps = float(params.get("qk_norm_eps", 0.0))
+        self.position = params.get("position")
+        self.encodings = build.positions
+        if self.position is not None and self.position not in self.encodings:
+            raise KeyError(f"attention refers to position encoding '{self.position}', the model defines "
+                           f"{sorted(self.encodings)}")
+        load = build.loader
+        self.qkv = Linear(load.get_concat([f"{prefix}.q_proj.weight", f"{prefix}.k_proj.weight",
+                                           f"{prefix}.v_proj.weight"]), build.mode)
+        self.o = Linear(load.get(f"{prefix}.o_proj.weight"), build.mode)
+        self.q_w = load.get(f"{prefix}.q_norm.weight") if self.qk_norm else None
+        self.k_w = load.get(f"{prefix}.k_norm.weight") if self.qk_norm else None
+        self.act_dtype = build.act_dtype
+        self.options = build.options
+
+    def cache_spec(self) -> PagedKVSpec:
+        return PagedKVSpec(self.nkv, self.d, int(self.window) if self.window is not None else None)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: PagedCacheView) -> torch.Tensor:
+        tokens = x.shape[0]
+        ws = ctx.workspace
+        write = cache.writable
+        q_cols = self.nq * self.d
+        cols = (self.nq + 2 * self.nkv) * self.d if write else q_cols
+        qkv = ws.buffer("attention.qkv", tokens, cols, self.act_dtype)
+        self.qkv.forward(x, qkv, rows=None if write else q_cols)
+        tables = ctx.position_product(self.position, self.encodings) if self.position is not None else None
+        table = ctx.block_tables[cache.group]
+        kernels.qk_rope_kv(
+            qkv, self.nq, self.nkv, self.d, self.q_w, self.k_w, self.eps,
+            tables.cos if tables is not None else None, tables.sin if tables is not None else None,
+            tables.rotary_dim if tables is not None else 0, tables.pairing if tables is not None else 0,
+            cache.keys, cache.values, ctx.positions, ctx.token_entry, table, write_kv=write)
+        attn = ws.buffer("attention.out", tokens, q_cols, self.act_dtype)
+        self.attend(qkv, attn, ctx, cache, table)
+        out = ws.buffer("attention.proj", tokens, self.hidden, self.act_dtype)
+        return self.o.forward(attn, out)
+
+    def attend(self, q: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: PagedCacheView,
+               table: torch.Tensor) -> None:
+        kernels.attn_generic(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
+                             ctx.token_entry, table, self.scale, int(self.window) if self.window is not None else 0)

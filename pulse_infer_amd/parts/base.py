@@ -1,0 +1,188 @@
+"""What a part is, and the registries that parts are chosen from.
+
+A model is put together from five kinds of part, each registered under a name
+and built from a ``PartSpec`` (its kind and its parameters):
+
+* **mixer** — mixes information along the sequence (attention here).
+  ``cache_spec()`` says what it keeps between steps; ``forward(x, ctx, cache)``
+  maps the normed input ``[T, H]`` to the update of the residual ``[T, H]``.
+* **feed-forward** — ``forward(x, ctx)``, token by token.
+* **norm** — ``apply(h, delta, out, rows)``: normalise ``h + delta`` (float32
+  residual), optionally only gathered rows.
+* **position encoding** — ``prepare(ctx)`` once per step gives whatever its
+  mixers consume (rotation tables here).
+* **block** — the arrangement of the above around the residual stream.
+
+Every part states the tensors it loads with ``weight_specs(params)`` (names
+relative to its prefix), so the loader can check a checkpoint, and the random
+initialiser can create one, before anything is built.  No part knows which
+model it is in; sizes and constants arrive as parameters.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Tuple
+
+import torch
+
+from ..weights.store import TensorSpec, WeightLoader
+
+
+class Registry:
+    """Name -> class, one per kind of part."""
+
+    def __init__(self, what: str):
+        self.what = what
+        self._items: Dict[str, Any] = {}
+
+    def register(self, name: str, replace: bool = False) -> Callable[[Any], Any]:
+        def deco(cls: Any) -> Any:
+            if name in self._items and not replace:
+                raise ValueError(f"{self.what} '{name}' is already registered")
+            self._items[name] = cls
+            cls.kind = name
+            return cls
+        return deco
+
+    def unregister(self, name: str) -> None:
+        self._items.pop(name, None)
+
+    def get(self, name: str) -> Any:
+        try:
+            return self._items[name]
+        except KeyError:
+            raise KeyError(f"unknown {self.what} '{name}'; registered: {', '.join(sorted(self._items)) or '<none>'}") from None
+
+    def names(self) -> List[str]:
+        return sorted(self._items)
+
+
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+NORMS = Registry("norm")
+POSITIONS = Registry("position encoding")
+BLOCKS = Registry("block")
+
+
+class Workspace:
+    """Named device buffers that grow to the largest size asked for and are reused by every step."""
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self._flat: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+
+    def buffer(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
+        need = max(1, rows * cols)
+        key = (name, dtype)
+        flat = self._flat.get(key)
+        if flat is None or flat.numel() < need:
+            flat = torch.empty(need, dtype=dtype, device=self.device)
+            self._flat[key] = flat
+        return flat[: rows * cols].view(rows, cols)
+
+
+@dataclass
+class BuildContext:
+    """What a part gets when it is built."""
+
+    loader: WeightLoader
+    mode: str                    # "bfloat16" or "float32": how the run computes
+    device: torch.device
+    act_dtype: torch.dtype       # storage type of activations between kernels
+    workspace: Workspace
+    positions: Dict[str, Any] = field(default_factory=dict)  # name -> position encoding instance
+    options: Dict[str, Any] = field(default_factory=dict)
+
+
+@dataclass
+class EntryMeta:
+    """One request's share of a step (host side)."""
+
+    request: Any
+    slot: int
+    start: int      # position of its first token in this step = tokens already in the cache
+    count: int      # tokens in this step
+    first_row: int  # where they start among the step's tokens
+
+
+@dataclass
+class PagedCacheView:
+    """The pages of one run of a paged group."""
+
+    group: int
+    keys: torch.Tensor     # [pages, kv_heads, page_size, head_dim]
+    values: torch.Tensor   # [pages, kv_heads, head_dim, page_size]
+    page_size: int
+    writable: bool = True  # False: the run reads a cache that another run writes
+
+
+@dataclass
+class StateView:
+    """The per-request state of one run: row ``slot`` belongs to the request in that slot."""
+
+    state: torch.Tensor    # [slots, *shape]
+
+
+@dataclass
+class StepContext:
+    """Everything a part may need to know about the step being run."""
+
+    num_tokens: int
+    entries: List[EntryMeta]
+    token_ids: torch.Tensor      # int32 [T]
+    positions: torch.Tensor      # int32 [T]
+    token_entry: torch.Tensor    # int32 [T] index into entries
+    entry_start: torch.Tensor    # int32 [B]
+    entry_count: torch.Tensor    # int32 [B]
+    entry_first_row: torch.Tensor  # int32 [B + 1] (prefix sums of counts)
+    entry_slot: torch.Tensor     # int32 [B]
+    block_tables: Dict[int, torch.Tensor]  # group -> int32 [B, width]
+    want_rows: torch.Tensor      # int32 [R] rows whose logits are wanted
+    num_wanted: int
+    workspace: Workspace
+    max_count: int = 1           # most tokens of one entry
+    max_context: int = 1         # longest context (start + count) of an entry
+    extras: Dict[str, Any] = field(default_factory=dict)  # per-step products of position encodings etc.
+
+    def position_product(self, name: str, encodings: Dict[str, Any]) -> Any:
+        """What position encoding ``name`` prepared for this step (prepared on first use)."""
+        key = f"position:{name}"
+        if key not in self.extras:
+            self.extras[key] = encodings[name].prepare(self)
+        return self.extras[key]
+
+
+class ResidualStream:
+    """The float32 residual ``h`` and the update that has not been added to it yet.
+
+    Adding is deferred so that it happens inside the next norm's kernel.
+    """
+
+    def __init__(self, h: torch.Tensor):
+        self.h = h
+        self.pending: Optional[torch.Tensor] = None
+
+    def normed(self, norm: Any, out: torch.Tensor) -> torch.Tensor:
+        norm.apply(self.h, self.pending, out)
+        self.pending = None
+        return out
+
+    def push(self, delta: torch.Tensor) -> None:
+        if self.pending is not None:
+            from ..ops import kernels
+            kernels.residual_add(self.h, self.pending)
+        self.pending = delta
+
+
+class Part:
+    """Base of all parts: declares the tensors it loads."""
+
+    kind = "?"
+
+    @classmethod
+    def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
+        return {}
+
+
+def joined(prefix: str, name: str) -> str:
+    return f"{prefix}.{name}" if prefix else name

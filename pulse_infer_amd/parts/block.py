@@ -1,0 +1,53 @@
+"""Arrangements of mixer, feed-forward and norms around the residual stream.
+
+``prenorm``: h <- h + mixer(norm_a(h)); h <- h + ffn(norm_b(h))
+(reference: src/model/qwen3/model.cpp:779-923).  The additions are deferred into
+the next norm's kernel through ``ResidualStream``.
+"""
+from __future__ import annotations
+
+from typing import Any, Dict, Optional
+
+from ..models.spec import LayerSpec
+from ..weights.store import TensorSpec
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BuildContext, Part, ResidualStream, StepContext, joined
+
+
+@BLOCKS.register("prenorm")
+class PreNormBlock(Part):
+    @classmethod
+    def layer_weight_specs(cls, layer: LayerSpec) -> Dict[str, TensorSpec]:
+        """All tensors of one layer, by full name."""
+        p = layer.block.params
+        out: Dict[str, TensorSpec] = {}
+        norm_cls = NORMS.get(layer.norm.kind)
+        for which in ("mixer_norm", "ffn_norm"):
+            for name, spec in norm_cls.weight_specs(layer.norm.params).items():
+                out[joined(joined(layer.prefix, p[which]), name)] = spec
+        for part, registry in ((layer.mixer, MIXERS), (layer.ffn, FEED_FORWARDS)):
+            sub = joined(layer.prefix, part.params.get("prefix", ""))
+            for name, spec in registry.get(part.kind).weight_specs(part.params).items():
+                out[joined(sub, name)] = spec
+        return out
+
+    def __init__(self, layer: LayerSpec, build: BuildContext):
+        p = layer.block.params
+        norm_cls = NORMS.get(layer.norm.kind)
+        self.mixer_norm = norm_cls(layer.norm.params, joined(layer.prefix, p["mixer_norm"]), build)
+        self.ffn_norm = norm_cls(layer.norm.params, joined(layer.prefix, p["ffn_norm"]), build)
+        self.mixer = MIXERS.get(layer.mixer.kind)(layer.mixer.params,
+                                                  joined(layer.prefix, layer.mixer.params.get("prefix", "")), build)
+        self.ffn = FEED_FORWARDS.get(layer.ffn.kind)(layer.ffn.params,
+                                                     joined(layer.prefix, layer.ffn.params.get("prefix", "")), build)
+        self.hidden = int(layer.norm.params["size"])
+        self.act_dtype = build.act_dtype
+
+    def cache_spec(self) -> Optional[Any]:
+        return self.mixer.cache_spec()
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Any) -> None:
+        x = ctx.workspace.buffer("block.normed", ctx.num_tokens, self.hidden, self.act_dtype)
+        stream.normed(self.mixer_norm, x)
+        stream.push(self.mixer.forward(x, ctx, cache))
+        stream.normed(self.ffn_norm, x)
+        stream.push(self.ffn.forward(x, ctx))

@@ -1,0 +1,56 @@
+"""Token embedding and output head.
+
+Embedding: row gather into the float32 residual (reference: src/layer/embedding.cpp:132-153).
+Head: logits = n W^T in float32, for the wanted rows only; W is ``lm_head.weight`` when the
+checkpoint holds it, else the embedding table when the configuration ties them
+(reference: src/model/qwen3/model.cpp:1009-1021, :1322-1371).
+"""
+from __future__ import annotations
+
+from typing import Any, Dict
+
+import torch
+
+from ..ops import kernels
+from ..weights.store import TensorSpec
+from .base import BuildContext, Part
+from .linear import Linear
+
+
+class TokenEmbedding(Part):
+    @classmethod
+    def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
+        return {params["name"]: TensorSpec((params["vocab_size"], params["hidden_size"]), kind="embedding",
+                                           fan_in=params["hidden_size"])}
+
+    def __init__(self, params: Dict[str, Any], build: BuildContext):
+        self.vocab = int(params["vocab_size"])
+        self.hidden = int(params["hidden_size"])
+        self.table = build.loader.get(params["name"])
+        self.bad_id = torch.zeros(1, dtype=torch.int32, device=build.device)
+
+    def forward(self, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        kernels.embed_gather(ids, self.table, out, self.bad_id)
+        return out
+
+
+class OutputHead(Part):
+    @classmethod
+    def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
+        # with tied embeddings the head's own tensor may be absent; if present it is used
+        return {params["name"]: TensorSpec((params["vocab_size"], params["hidden_size"]), fan_in=params["hidden_size"],
+                                           optional=bool(params.get("tied", False)))}
+
+    def __init__(self, params: Dict[str, Any], build: BuildContext, embedding: TokenEmbedding):
+        self.vocab = int(params["vocab_size"])
+        if build.loader.has(params["name"]):
+            weight = build.loader.get(params["name"])
+        elif params.get("tied", False):
+            weight = embedding.table
+        else:
+            raise KeyError(f"'{params['name']}' is missing and the configuration does not tie it to the embedding")
+        self.linear = Linear(weight, build.mode)
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """out: float32 [R, vocab]."""
+        return self.linear.forward(x, out)

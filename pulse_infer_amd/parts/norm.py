@@ -1,0 +1,29 @@
+"""RMSNorm: y = x / sqrt(mean(x^2) + eps) * w, float32 inside, one rounding
+(reference: src/ops/kernels/cuda/rmsnorm_kernel.cu:97-157; layer: src/layer/rmsnorm.cpp:9-157)."""
+from __future__ import annotations
+
+from typing import Any, Dict, Optional
+
+import torch
+
+from ..ops import kernels
+from ..weights.store import TensorSpec
+from .base import NORMS, BuildContext, Part
+
+
+@NORMS.register("rmsnorm")
+class RMSNorm(Part):
+    @classmethod
+    def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
+        return {"weight": TensorSpec((params["size"],), kind="norm")}
+
+    def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
+        self.size = int(params["size"])
+        self.eps = float(params["eps"])
+        self.weight = build.loader.get(f"{prefix}.weight")
+
+    def apply(self, h: torch.Tensor, delta: Optional[torch.Tensor], out: torch.Tensor,
+              rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """out = norm(h + delta) * w; h keeps the sum unless rows are gathered."""
+        kernels.add_rmsnorm(h, delta, self.weight, self.eps, out, rows=rows)
+        return out
