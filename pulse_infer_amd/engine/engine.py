@@ -1,0 +1,189 @@
+"""The serving loop: scheduler -> step function -> sampler -> scheduler.
+
+``ContinuousBatchEngine`` keeps the reference engine's interface
+(reference: include/pulse/scheduler/continuous_batch_engine.hpp:14-35,
+src/scheduler/continuous_batch_engine.cpp:66-305) with token ids in place of
+text: ``add_request``, ``run_until_complete``, ``get_result``, ``get_request``,
+``get_stats``.  ``LLM`` is the Python entry point on top of it.
+"""
+from __future__ import annotations
+
+import sys
+import time
+from typing import Any, Dict, List, Optional, Sequence
+
+import torch
+
+from ..models.factory import build_model, load_model
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler
+from .request import InferenceRequest
+from .runner import ModelRunner, StepEntry
+from .scheduler import ContinuousBatchScheduler, ScheduledBatch, Stats
+
+DEFAULT_MAX_SEQUENCES = 32  # reference: src/scheduler/continuous_batch_engine.cpp:73
+
+
+class ContinuousBatchEngine:
+    def __init__(self, model: Any, max_batch_size: int, chunk_size: int, *, page_size: int = 16,
+                 num_pages: int = 1024, max_sequences: int = DEFAULT_MAX_SEQUENCES,
+                 max_num_batched_tokens: Optional[int] = None, eos_token_ids: Sequence[int] = (),
+                 banned_tokens: Optional[Sequence[int]] = None, seed: int = 0):
+        self.model = model
+        slots = max(max_sequences, max_batch_size)
+        self.runner = ModelRunner(model, page_size=page_size, num_pages=num_pages, max_requests=slots)
+        self.scheduler = ContinuousBatchScheduler(
+            max_batch_size, max_sequences, chunk_size, max_num_batched_tokens, cache=self.runner.cache,
+            max_positions=model.spec.max_positions)
+        self.sampler = Sampler(model.vocab_size, slots, model.device, banned_tokens)
+        self.eos_token_ids = list(eos_token_ids)
+        self.seed = int(seed)
+        self.last_batch: Optional[ScheduledBatch] = None
+
+    # ------------------------------------------------------------------ intake
+    def add_request(self, prompt_tokens: Sequence[int], max_new_tokens: int,
+                    sampling: Optional[SamplingParams] = None) -> int:
+        vocab = self.model.vocab_size
+        for tok in prompt_tokens:
+            if not 0 <= int(tok) < vocab:
+                raise ValueError(f"prompt token id {tok} is outside the vocabulary of {vocab}")
+        return self.scheduler.add_request(prompt_tokens, max_new_tokens, sampling)
+
+    # -------------------------------------------------------------------- loop
+    def step(self) -> ScheduledBatch:
+        """One scheduling decision, one model step, one sampling call."""
+        batch = self.scheduler.schedule_next_batch()
+        self.last_batch = batch
+        if batch.empty():
+            return batch
+        cache = self.runner.cache
+        for request in batch.admitted:
+            self.sampler.start_request(cache.slot_of(request.request_id), request.sampling,
+                                       request.prompt_tokens + request.generated_tokens)
+        entries = [StepEntry(p.request.request_id, p.tokens, [len(p.tokens) - 1] if p.samples else [])
+                   for p in batch.portions]
+        logits = self.runner.step(entries)
+        self.scheduler.tokens_computed += batch.num_tokens()
+        finished: List[int] = []
+        sampled = [p for p in batch.portions if p.samples]
+        for p in batch.portions:
+            p.request.add_computed_tokens(len(p.tokens))
+        live = []
+        for row, p in enumerate(sampled):
+            if not p.request.can_generate_more:  # nothing more to generate (max_new_tokens == 0)
+                p.request.finish("length")
+                finished.append(p.request.request_id)
+            else:
+                live.append((row, p.request))
+        if live:
+            rows = logits if len(live) == logits.shape[0] else logits[[r for r, _ in live]]
+            requests = [q for _, q in live]
+            tokens = self.sampler.sample(
+                rows, [q.sampling for q in requests], [cache.slot_of(q.request_id) for q in requests],
+                [q.num_generated for q in requests], [self.seed + q.request_id for q in requests])
+            noted_slots, noted_tokens = [], []
+            for q, tok in zip(requests, tokens):
+                if q.sampling.presence_penalty > 0.0 and tok >= 0:
+                    noted_slots.append(cache.slot_of(q.request_id))
+                    noted_tokens.append(tok)
+                if not q.add_sampled_token(tok, self.eos_token_ids):
+                    finished.append(q.request_id)
+            self.sampler.note_tokens(noted_slots, noted_tokens)
+        self.scheduler.update_after_step(finished)
+        return batch
+
+    def run_until_complete(self, print_progress: bool = False) -> None:
+        step = 0
+        while self.scheduler.has_work():
+            if print_progress and step % 10 == 0:
+                s = self.scheduler.get_stats()
+                print(f"Continuous batch step {step} running={s.num_running} waiting={s.num_waiting} "
+                      f"finished={s.num_finished}", file=sys.stderr, flush=True)
+            if self.step().empty():
+                break
+            step += 1
+        if print_progress:
+            s = self.scheduler.get_stats()
+            print(f"Continuous batch complete steps={step} total_requests={s.total_requests}", file=sys.stderr,
+                  flush=True)
+
+    # ----------------------------------------------------------------- results
+    def get_result(self, request_id: int) -> List[int]:
+        """The generated ids of a finished request, cut before the first end-of-sequence id
+        (reference: src/scheduler/continuous_batch_engine.cpp:114-130); empty while it still runs."""
+        request = self.scheduler.get_request(request_id)
+        if request is None or not request.is_finished:
+            return []
+        out: List[int] = []
+        for tok in request.generated_tokens:
+            if not request.sampling.ignore_eos and tok in self.eos_token_ids:
+                break
+            out.append(tok)
+        return out
+
+    def get_request(self, request_id: int) -> Optional[InferenceRequest]:
+        return self.scheduler.get_request(request_id)
+
+    def get_stats(self) -> Stats:
+        return self.scheduler.get_stats()
+
+
+class LLM:
+    """Python entry point: a model folder in, generated token ids out."""
+
+    def __init__(self, model: Any, config: Any = None, *, max_batch_size: int = 8, chunk_size: int = 256,
+                 page_size: int = 16, num_pages: Optional[int] = None, max_sequences: int = DEFAULT_MAX_SEQUENCES,
+                 max_num_batched_tokens: Optional[int] = None, seed: int = 0):
+        self.model = model
+        self.config = config
+        if num_pages is None:
+            # room for max_sequences contexts of up to 4096 tokens, bounded by the model's positions
+            per_request = min(model.spec.max_positions, 4096)
+            num_pages = max(64, max_sequences * ((per_request + page_size - 1) // page_size))
+        eos = list(getattr(config, "eos_token_ids", []) or [])
+        self.engine = ContinuousBatchEngine(
+            model, max_batch_size, chunk_size, page_size=page_size, num_pages=num_pages, max_sequences=max_sequences,
+            max_num_batched_tokens=max_num_batched_tokens, eos_token_ids=eos, seed=seed)
+
+    @classmethod
+    def from_pretrained(cls, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0", **engine_options):
+        config, model = load_model(model_dir, mode=dtype, device=device)
+        return cls(model, config, **engine_options)
+
+    @classmethod
+    def from_config_random(cls, config: Any, seed: int = 0, init: Any = "fan_in", dtype: str = "bfloat16",
+                           device: str = "cuda:0", **engine_options):
+        """Random weights made on the GPU, without a file (for sizes not worth writing to disk)."""
+        from ..models.causal_lm import expected_tensors
+        from ..weights.random_init import RandomSource
+
+        source = RandomSource(expected_tensors(config.model_spec()), seed, init, torch.bfloat16, device=device)
+        model = build_model(config, source, mode=dtype, device=device)
+        return cls(model, config, **engine_options)
+
+    def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 32, temperature: float = 0.0,
+                 top_k: int = 0, top_p: float = 0.0, presence_penalty: float = 0.0, seed: Optional[int] = None,
+                 ignore_eos: bool = False, sampling: Optional[Sequence[SamplingParams]] = None) -> List[List[int]]:
+        ids = []
+        for i, prompt in enumerate(prompts):
+            params = sampling[i] if sampling is not None else SamplingParams(
+                temperature=temperature, top_k=top_k, top_p=top_p, presence_penalty=presence_penalty,
+                seed=None if seed is None else seed + i, ignore_eos=ignore_eos)
+            ids.append(self.engine.add_request(prompt, max_new_tokens, params))
+        self.engine.run_until_complete()
+        return [self.engine.get_result(i) for i in ids]
+
+    def step_raw(self, entries: Sequence[Dict[str, Any]], end: Sequence[Any] = ()) -> torch.Tensor:
+        """Run one step of given tokens: entries are {"id", "tokens", "want"}; float32 logits [wanted, vocab]."""
+        runner = self.engine.runner
+        batch = []
+        for item in entries:
+            rid = ("raw", item["id"])
+            if not runner.cache.has_request(rid):
+                runner.add_request(rid)
+            runner.reserve(rid, runner.cache.computed(rid) + len(item["tokens"]))
+            batch.append(StepEntry(rid, list(item["tokens"]), list(item.get("want", []))))
+        logits = runner.step(batch)
+        for rid in end:
+            runner.free_request(("raw", rid))
+        return logits

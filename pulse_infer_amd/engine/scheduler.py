@@ -1,0 +1,271 @@
+"""Continuous batching with chunked prefill under a token budget.
+
+The queues and the first-come-first-served admission are the reference's
+(reference: include/pulse/scheduler/continuous_batch_scheduler.hpp:27-147):
+every step takes all running requests, then admits waiting ones while the batch
+has room (``max_batch_size`` requests) and fewer than ``max_sequences`` run.
+What the reference leaves out is decided here:
+
+* **token budget** — a step computes at most ``max_num_batched_tokens`` tokens:
+  decoding requests come first with one token each, what is left goes to
+  prefilling requests in order of arrival, each at most ``chunk_size`` tokens,
+  cut anywhere.
+* **pages** — every portion is reserved in the cache before the step; a request
+  is admitted only if its first portion fits.  When a running request cannot
+  get the page it needs, the most recently admitted running request is
+  preempted: its pages and slot are given back, it returns to the front of the
+  waiting queue and is later computed again from its first token (prompt and
+  generated tokens alike), which reproduces what it had.  A prefill portion is
+  shortened rather than preempting anyone.  A request that could never fit the
+  pool or the model's positions is refused at ``add_request``.
+  (The reference aborts the whole run when pages run out,
+  src/runtime/block_manager.cpp:44-46, src/scheduler/continuous_batch_engine.cpp:98-101.)
+"""
+from __future__ import annotations
+
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, List, Optional, Sequence
+
+from ..cache.manager import CacheManager
+from ..sampling.params import SamplingParams
+from .request import InferenceRequest, RequestState
+
+
+class SchedulerError(RuntimeError):
+    pass
+
+
+@dataclass
+class ScheduledPortion:
+    request: InferenceRequest
+    tokens: List[int]
+    start: int
+    samples: bool  # the portion ends the request's pending input: its last row is sampled from
+
+
+@dataclass
+class ScheduledBatch:
+    portions: List[ScheduledPortion] = field(default_factory=list)
+    preempted: List[InferenceRequest] = field(default_factory=list)
+    admitted: List[InferenceRequest] = field(default_factory=list)
+
+    @property
+    def requests(self) -> List[InferenceRequest]:
+        return [p.request for p in self.portions]
+
+    def batch_size(self) -> int:
+        return len(self.portions)
+
+    def num_tokens(self) -> int:
+        return sum(len(p.tokens) for p in self.portions)
+
+    def empty(self) -> bool:
+        return not self.portions
+
+
+@dataclass
+class Stats:
+    num_running: int = 0
+    num_waiting: int = 0
+    num_finished: int = 0
+    total_requests: int = 0
+    num_steps: int = 0
+    num_preemptions: int = 0
+    tokens_computed: int = 0
+    tokens_generated: int = 0
+    pages_high_water: int = 0
+
+
+class ContinuousBatchScheduler:
+    def __init__(self, max_batch_size: int, max_sequences: int, chunk_size: int = 256,
+                 max_num_batched_tokens: Optional[int] = None, cache: Optional[CacheManager] = None,
+                 max_positions: Optional[int] = None):
+        if max_batch_size <= 0 or max_sequences <= 0 or chunk_size <= 0:
+            raise ValueError("max_batch_size, max_sequences and chunk_size must be positive")
+        self.max_batch_size = int(max_batch_size)
+        self.max_sequences = int(max_sequences)
+        self.chunk_size = int(chunk_size)
+        self.max_num_batched_tokens = int(max_num_batched_tokens) if max_num_batched_tokens else \
+            self.max_batch_size * self.chunk_size
+        if self.max_num_batched_tokens <= 0:
+            raise ValueError("max_num_batched_tokens must be positive")
+        self.cache = cache
+        self.max_positions = max_positions
+        self.next_request_id = 0
+        self.waiting: Deque[InferenceRequest] = deque()
+        self.running: List[InferenceRequest] = []
+        self.request_map: Dict[int, InferenceRequest] = {}
+        self.num_steps = 0
+        self.num_preemptions = 0
+        self.tokens_computed = 0
+
+    # ------------------------------------------------------------------ intake
+    def add_request(self, prompt_tokens: Sequence[int], max_new_tokens: int,
+                    sampling: Optional[SamplingParams] = None) -> int:
+        request = InferenceRequest(self.next_request_id, prompt_tokens, max_new_tokens, sampling)
+        # the last sampled token is never fed back, so a request holds at most prompt + max_new - 1 tokens
+        longest = request.prompt_len + max(0, request.max_new_tokens - 1)
+        if self.max_positions is not None and longest > self.max_positions:
+            raise SchedulerError(f"request needs {longest} positions, the model allows {self.max_positions}")
+        if self.cache is not None:
+            for g, need in zip(self.cache.groups, self.cache.pages_needed_new(longest)):
+                if g.spec.window is None and need > g.pool.num_pages:
+                    raise SchedulerError(f"request needs {need} cache pages of {g.page_size} tokens, "
+                                         f"the pool has {g.pool.num_pages}")
+        self.next_request_id += 1
+        self.waiting.append(request)
+        self.request_map[request.request_id] = request
+        return request.request_id
+
+    # --------------------------------------------------------------- decisions
+    def _fits(self, request: InferenceRequest, length: int) -> bool:
+        return self.cache is None or self.cache.can_reserve(
+            request.request_id if self.cache.has_request(request.request_id) else None, length)
+
+    def _reserve(self, request: InferenceRequest, length: int) -> None:
+        if self.cache is not None:
+            self.cache.reserve(request.request_id, length)
+
+    def _largest_fitting(self, request: InferenceRequest, want: int) -> int:
+        """The longest portion <= want whose pages are free right now."""
+        if self.cache is None:
+            return want
+        base = request.num_computed_tokens
+        lo, hi = 0, want
+        while lo < hi:  # can_reserve is monotone in the length
+            mid = (lo + hi + 1) // 2
+            if self._fits(request, base + mid):
+                lo = mid
+            else:
+                hi = mid - 1
+        return lo
+
+    def _preempt(self, victim: InferenceRequest, batch: ScheduledBatch) -> None:
+        self.running.remove(victim)
+        if self.cache is not None and self.cache.has_request(victim.request_id):
+            self.cache.free_request(victim.request_id)
+        victim.preempt()
+        self.waiting.appendleft(victim)
+        batch.preempted.append(victim)
+        batch.portions = [p for p in batch.portions if p.request is not victim]
+        self.num_preemptions += 1
+
+    def schedule_next_batch(self) -> ScheduledBatch:
+        batch = ScheduledBatch()
+        budget = self.max_num_batched_tokens
+
+        # 1. running requests that decode: one token each, preempting the newest when pages run out
+        for request in list(self.running):
+            if request not in self.running:  # preempted a moment ago
+                continue
+            if request.num_pending_tokens != 1 or request.is_prefill:
+                continue
+            if budget <= 0 or batch.batch_size() >= self.max_batch_size:
+                break
+            need = request.num_computed_tokens + 1
+            gives_way = False
+            while not self._fits(request, need):
+                victim = self.running[-1]
+                if victim is request:
+                    if len(self.running) == 1:
+                        raise SchedulerError(f"request {request.request_id} cannot get a cache page although "
+                                             "nothing else is running; the pool is too small for it")
+                    gives_way = True  # it is the newest itself
+                    break
+                self._preempt(victim, batch)
+            if gives_way:
+                self._preempt(request, batch)
+                continue
+            self._reserve(request, need)
+            batch.portions.append(ScheduledPortion(request, request.get_next_chunk_tokens(1),
+                                                   request.num_computed_tokens, True))
+            budget -= 1
+
+        # 2. running requests with more than one pending token (prefill, or recomputation after preemption)
+        for request in list(self.running):
+            if request.num_pending_tokens < 1 or (request.num_pending_tokens == 1 and not request.is_prefill):
+                continue
+            if budget <= 0 or batch.batch_size() >= self.max_batch_size:
+                break
+            if any(p.request is request for p in batch.portions):
+                continue
+            want = min(self.chunk_size, request.num_pending_tokens, budget)
+            count = self._largest_fitting(request, want)
+            if count <= 0:
+                continue
+            self._reserve(request, request.num_computed_tokens + count)
+            batch.portions.append(ScheduledPortion(request, request.get_next_chunk_tokens(count),
+                                                   request.num_computed_tokens,
+                                                   count == request.num_pending_tokens))
+            budget -= count
+
+        # 3. admit waiting requests, first come first served
+        while (self.waiting and budget > 0 and batch.batch_size() < self.max_batch_size
+               and len(self.running) < self.max_sequences):
+            request = self.waiting[0]
+            if self.cache is not None and self.cache.slots.num_free == 0:
+                break
+            want = min(self.chunk_size, request.num_pending_tokens, budget)
+            count = self._largest_fitting(request, want)
+            # admit only with room for the whole first portion (or all that the budget allows)
+            if count < want:
+                break
+            self.waiting.popleft()
+            if self.cache is not None:
+                self.cache.add_request(request.request_id)
+            request.start_running()
+            self.running.append(request)
+            batch.admitted.append(request)
+            self._reserve(request, request.num_computed_tokens + count)
+            batch.portions.append(ScheduledPortion(request, request.get_next_chunk_tokens(count),
+                                                   request.num_computed_tokens,
+                                                   count == request.num_pending_tokens))
+            budget -= count
+
+        if batch.empty() and (self.running or self.waiting):
+            raise SchedulerError("nothing can be scheduled although requests remain: the cache pool cannot hold "
+                                 "the first portion of the next request")
+        return batch
+
+    def update_after_step(self, finished_ids: Sequence[int]) -> None:
+        """Take finished requests out of the running list and give their cache back
+        (reference: continuous_batch_scheduler.hpp:75-89)."""
+        self.num_steps += 1
+        for request_id in finished_ids:
+            request = self.request_map.get(request_id)
+            if request is None or request not in self.running:
+                continue
+            if not request.is_finished:
+                request.finish()
+            self.running.remove(request)
+            if self.cache is not None and self.cache.has_request(request_id):
+                self.cache.free_request(request_id)
+
+    # ----------------------------------------------------------------- queries
+    def get_request(self, request_id: int) -> Optional[InferenceRequest]:
+        return self.request_map.get(request_id)
+
+    def has_work(self) -> bool:
+        return bool(self.running) or bool(self.waiting)
+
+    def num_running(self) -> int:
+        return len(self.running)
+
+    def num_active_sequences(self) -> int:
+        return len(self.running)
+
+    def num_waiting(self) -> int:
+        return len(self.waiting)
+
+    def set_chunk_size(self, chunk_size: int) -> None:
+        self.chunk_size = int(chunk_size)
+
+    def get_stats(self) -> Stats:
+        finished = [r for r in self.request_map.values() if r.is_finished]
+        return Stats(
+            num_running=len(self.running), num_waiting=len(self.waiting), num_finished=len(finished),
+            total_requests=len(self.request_map), num_steps=self.num_steps, num_preemptions=self.num_preemptions,
+            tokens_computed=self.tokens_computed,
+            tokens_generated=sum(r.num_generated for r in self.request_map.values()),
+            pages_high_water=max((g.pool.high_water for g in self.cache.groups), default=0) if self.cache else 0)

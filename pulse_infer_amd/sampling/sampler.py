@@ -1,0 +1,77 @@
+"""Choosing next tokens for a batch of logits rows on the GPU.
+
+One kernel call serves all rows; each row carries its own options.  The "seen"
+sets of the presence penalty live in the per-request slots (one bit per
+vocabulary entry), are cleared when a slot is taken and updated as tokens
+arrive.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import torch
+
+from ..ops import kernels
+from .params import SamplingParams, uniform_for
+
+
+class Sampler:
+    def __init__(self, vocab_size: int, num_slots: int, device: torch.device,
+                 banned_tokens: Optional[Sequence[int]] = None):
+        self.vocab = int(vocab_size)
+        self.device = torch.device(device)
+        self.words = (self.vocab + 31) // 32
+        self.num_slots = int(num_slots)
+        self.seen: Optional[torch.Tensor] = None  # [slots, words], made when a request first needs it
+        self.banned: Optional[torch.Tensor] = None
+        if banned_tokens:
+            host = torch.zeros(self.words, dtype=torch.int64)
+            for tok in banned_tokens:
+                if 0 <= tok < self.vocab:
+                    host[tok >> 5] |= 1 << (tok & 31)
+            # keep the bit patterns when narrowing to int32
+            host = torch.where(host >= 2 ** 31, host - 2 ** 32, host)
+            self.banned = host.to(torch.int32).to(self.device)
+
+    # -------------------------------------------------------------- seen sets
+    def start_request(self, slot: int, params: SamplingParams, tokens: Sequence[int]) -> None:
+        """A request took ``slot``: clear its seen set and mark the tokens it starts with."""
+        if params.presence_penalty > 0.0:
+            if self.seen is None:
+                self.seen = torch.zeros((self.num_slots, self.words), dtype=torch.int32, device=self.device)
+            self.seen[slot].zero_()
+            self.note_tokens([slot] * len(tokens), list(tokens))
+
+    def note_tokens(self, slots: Sequence[int], tokens: Sequence[int]) -> None:
+        if self.seen is None or not slots:
+            return
+        rows = torch.tensor(list(slots), dtype=torch.int32, device=self.device)
+        toks = torch.tensor(list(tokens), dtype=torch.int32, device=self.device)
+        kernels.mark_seen(self.seen, rows, toks, self.vocab)
+
+    # ---------------------------------------------------------------- sampling
+    def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], slots: Sequence[int],
+               counters: Sequence[int], default_seeds: Sequence[int]) -> List[int]:
+        """One token per row.  ``counters[r]`` is how many tokens row r's request has drawn before."""
+        rows = logits.shape[0]
+        if rows == 0:
+            return []
+        out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        if all(p.greedy and p.presence_penalty == 0.0 for p in params) and self.banned is None:
+            kernels.sample(logits, out)
+            return out.tolist()
+        temperature = torch.tensor([p.temperature for p in params], dtype=torch.float32, device=self.device)
+        top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32, device=self.device)
+        top_p = torch.tensor([p.top_p for p in params], dtype=torch.float32, device=self.device)
+        uniform = torch.tensor(
+            [uniform_for(p.seed if p.seed is not None else d, c) for p, c, d in zip(params, counters, default_seeds)],
+            dtype=torch.float32, device=self.device)
+        penalty = seen_row = None
+        if self.seen is not None and any(p.presence_penalty > 0.0 for p in params):
+            penalty = torch.tensor([p.presence_penalty for p in params], dtype=torch.float32, device=self.device)
+            seen_row = torch.tensor([s if p.presence_penalty > 0.0 else -1 for p, s in zip(params, slots)],
+                                    dtype=torch.int32, device=self.device)
+        kernels.sample(logits, out, temperature=temperature, top_k=top_k, top_p=top_p, uniform=uniform,
+                       penalty=penalty, seen_row=seen_row, seen_masks=self.seen if penalty is not None else None,
+                       banned=self.banned)
+        return out.tolist()
