@@ -146,7 +146,8 @@ class PlainQwen3:
         k = rms_norm(k, w[p + "self_attn.k_norm.weight"], eps)
         q = rope(q, positions, c["rope_theta"], d, self.pairing)
         k = rope(k, positions, c["rope_theta"], d, self.pairing)
-        o = causal_attention(q, k, v, 1.0 / math.sqrt(d), self.layer_window(index), positions)  # scale: paged_attention.cu:108
+        # keys are indexed by their place in the sequence; positions only enter through the rotation
+        o = causal_attention(q, k, v, 1.0 / math.sqrt(d), self.layer_window(index))  # scale: paged_attention.cu:108
         h = h + linear(o.reshape(t, nq * d), w[p + "self_attn.o_proj.weight"])               # model.cpp:875-886
         m = rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)                       # model.cpp:888
         h = h + gated_mlp(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],

@@ -1,0 +1,141 @@
+"""Configuration and registry (CPU)."""
+import json
+import os
+
+import pytest
+
+from conftest import TINY_A, TINY_B, TINY_W
+from pulse_infer_amd.config import (ConfigError, Qwen3Config, config_from_dict, load_config, lookup_architecture,
+                                    register_architecture, registered_architectures, unregister_architecture)
+
+REQUIRED = ["head_dim", "hidden_size", "intermediate_size", "max_position_embeddings", "num_attention_heads",
+            "num_hidden_layers", "rms_norm_eps", "rope_theta", "vocab_size"]
+
+
+def test_reads_every_size_from_the_keys():
+    a, b = Qwen3Config.from_dict(TINY_A), Qwen3Config.from_dict(TINY_B)
+    for key in REQUIRED + ["num_key_value_heads", "tie_word_embeddings"]:
+        assert getattr(a, key) == TINY_A[key] and getattr(b, key) == TINY_B[key]
+        assert getattr(a, key) != getattr(b, key), f"the tiny configurations should differ in {key}"
+
+
+@pytest.mark.parametrize("key", [k for k in REQUIRED if k != "head_dim"])
+def test_missing_required_key_is_named(key):
+    data = dict(TINY_A)
+    del data[key]
+    with pytest.raises(ConfigError, match=f"'{key}'"):
+        Qwen3Config.from_dict(data, "cfg.json")
+
+
+def test_wrong_type_is_named():
+    with pytest.raises(ConfigError, match="'hidden_size'"):
+        Qwen3Config.from_dict(dict(TINY_A, hidden_size="64"))
+    with pytest.raises(ConfigError, match="'tie_word_embeddings'"):
+        Qwen3Config.from_dict(dict(TINY_A, tie_word_embeddings=1))
+
+
+def test_head_dim_is_free_of_hidden_size():
+    cfg = Qwen3Config.from_dict(TINY_B)
+    assert cfg.num_attention_heads * cfg.head_dim != cfg.hidden_size
+
+
+def test_validation():
+    with pytest.raises(ConfigError, match="not divisible"):
+        Qwen3Config.from_dict(dict(TINY_A, num_attention_heads=5))
+    with pytest.raises(ConfigError, match="Invalid model dimensions"):
+        Qwen3Config.from_dict(dict(TINY_A, vocab_size=0))
+    with pytest.raises(ConfigError, match="even"):
+        Qwen3Config.from_dict(dict(TINY_A, head_dim=15))
+    for key, value in (("attention_bias", True), ("hidden_act", "gelu"), ("rope_scaling", {"rope_type": "yarn"})):
+        with pytest.raises(ConfigError, match=key):
+            Qwen3Config.from_dict(dict(TINY_A, **{key: value}))
+    with pytest.raises(ConfigError, match="sliding_window"):
+        Qwen3Config.from_dict(dict(TINY_A, use_sliding_window=True))
+
+
+def test_eos_int_or_list_and_generation_override(tmp_path):
+    assert Qwen3Config.from_dict(dict(TINY_A, eos_token_id=7)).eos_token_ids == [7]
+    assert Qwen3Config.from_dict(dict(TINY_A, eos_token_id=[7, 9])).eos_token_ids == [7, 9]
+    assert Qwen3Config.from_dict(TINY_A).eos_token_ids == []
+    with pytest.raises(ConfigError, match="eos_token_id"):
+        Qwen3Config.from_dict(dict(TINY_A, eos_token_id="x"))
+    (tmp_path / "config.json").write_text(json.dumps(dict(TINY_A, eos_token_id=3)))
+    (tmp_path / "generation_config.json").write_text(json.dumps(
+        {"eos_token_id": [5, 6], "temperature": 0.6, "top_k": 20, "top_p": 0.95}))
+    cfg = load_config(str(tmp_path))
+    assert cfg.eos_token_ids == [5, 6] and cfg.top_k == 20
+    assert abs(cfg.temperature - 0.6) < 1e-12 and abs(cfg.top_p - 0.95) < 1e-12
+    # a file path stands for its folder
+    assert load_config(str(tmp_path / "config.json")).eos_token_ids == [5, 6]
+
+
+def test_qwen3_0_6b_values(tmp_path):
+    """The values the reference's config demo asserts (demo/qwen3_config_demo.cpp:73-86), as a fixture written here."""
+    (tmp_path / "config.json").write_text(json.dumps(dict(
+        architectures=["Qwen3ForCausalLM"], hidden_size=1024, intermediate_size=3072, num_hidden_layers=28,
+        num_attention_heads=16, num_key_value_heads=8, head_dim=128, max_position_embeddings=40960,
+        vocab_size=151936, rms_norm_eps=1e-6, rope_theta=1000000, tie_word_embeddings=True,
+        torch_dtype="bfloat16", eos_token_id=151645, max_window_layers=28, sliding_window=None,
+        use_sliding_window=False, rope_scaling=None)))
+    (tmp_path / "generation_config.json").write_text(json.dumps(
+        {"eos_token_id": [151645, 151643], "temperature": 0.6, "top_k": 20, "top_p": 0.95}))
+    cfg = load_config(str(tmp_path))
+    assert (cfg.hidden_size, cfg.intermediate_size, cfg.num_hidden_layers) == (1024, 3072, 28)
+    assert (cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim) == (16, 8, 128)
+    assert (cfg.max_position_embeddings, cfg.vocab_size, cfg.torch_dtype) == (40960, 151936, "bfloat16")
+    assert cfg.eos_token_ids == [151645, 151643] and cfg.top_k == 20
+    assert all(cfg.layer_window(i) is None for i in range(28))
+
+
+def test_windows_per_layer():
+    cfg = Qwen3Config.from_dict(TINY_W)
+    assert [cfg.layer_window(i) for i in range(4)] == [None, None, 24, 24]
+    spec = cfg.model_spec()
+    assert [l.mixer.params["window"] for l in spec.layers] == [None, None, 24, 24]
+    typed = Qwen3Config.from_dict(dict(TINY_W, layer_types=["sliding_attention", "full_attention"] * 2))
+    assert [typed.layer_window(i) for i in range(4)] == [24, None, 24, None]
+    with pytest.raises(ConfigError, match="layer_types"):
+        Qwen3Config.from_dict(dict(TINY_W, layer_types=["full_attention"]))
+
+
+def test_model_spec_carries_no_size_of_its_own():
+    for data in (TINY_A, TINY_B):
+        cfg = Qwen3Config.from_dict(data)
+        spec = cfg.model_spec()
+        assert len(spec.layers) == data["num_hidden_layers"] and len(spec.order) == len(spec.layers)
+        m = spec.layers[0].mixer.params
+        assert (m["num_heads"], m["num_kv_heads"], m["head_dim"]) == (
+            data["num_attention_heads"], data["num_key_value_heads"], data["head_dim"])
+        assert m["scale"] == data["head_dim"] ** -0.5 and m["qk_norm_eps"] == data["rms_norm_eps"]
+        assert spec.positions["rope"].params["theta"] == data["rope_theta"]
+        assert spec.layers[0].ffn.params["intermediate_size"] == data["intermediate_size"]
+        assert spec.head.params["tied"] == data["tie_word_embeddings"]
+
+
+def test_round_trip_through_to_dict():
+    cfg = Qwen3Config.from_dict(dict(TINY_W, eos_token_id=[1, 2]))
+    again = Qwen3Config.from_dict(cfg.to_dict())
+    assert again == cfg
+
+
+def test_registry(tmp_path):
+    assert "Qwen3ForCausalLM" in registered_architectures()
+    assert lookup_architecture("Qwen3ForCausalLM").config_class is Qwen3Config
+    with pytest.raises(ConfigError, match="unknown architecture 'NopeForCausalLM'.*Qwen3ForCausalLM"):
+        config_from_dict(dict(TINY_A, architectures=["NopeForCausalLM"]))
+    with pytest.raises(ConfigError, match="architectures"):
+        config_from_dict({k: v for k, v in TINY_A.items() if k != "architectures"})
+    with pytest.raises(ValueError, match="already registered"):
+        register_architecture("Qwen3ForCausalLM", Qwen3Config)
+
+    class Other(Qwen3Config):
+        pass
+
+    register_architecture("OtherForCausalLM", Other)
+    try:
+        (tmp_path / "config.json").write_text(json.dumps(dict(TINY_A, architectures=["OtherForCausalLM"])))
+        assert isinstance(load_config(str(tmp_path)), Other)
+    finally:
+        unregister_architecture("OtherForCausalLM")
+    with pytest.raises(ConfigError, match="does not exist"):
+        load_config(str(tmp_path / "nowhere"))

@@ -1,0 +1,167 @@
+"""The scheduler's decisions (CPU): the reference's two cases, the token budget, decode first,
+shortened portions, preemption when pages run out, refusal of what can never fit."""
+import pytest
+
+from pulse_infer_amd.cache import CacheManager, PagedKVSpec
+from pulse_infer_amd.engine.request import InferenceRequest, RequestState
+from pulse_infer_amd.engine.scheduler import ContinuousBatchScheduler, SchedulerError
+from pulse_infer_amd.sampling.params import SamplingParams
+
+
+def test_request_chunk_state_machine():
+    """reference: tests/scheduler/test_continuous_batch_scheduler.cpp:10-38"""
+    r = InferenceRequest(0, [11, 12, 13], max_new_tokens=2)
+    assert r.state == RequestState.WAITING and r.is_prefill
+    assert r.get_next_chunk_tokens(2) == [11, 12] and r.get_next_chunk_positions(2) == [0, 1]
+    r.start_running()
+    r.add_computed_tokens(2)
+    assert r.get_next_chunk_tokens(2) == [13] and r.get_next_chunk_positions(2) == [2]
+    r.add_computed_tokens(1)
+    assert not r.is_prefill and not r.has_pending_input and r.get_next_chunk_size(2) == 0
+    assert r.add_sampled_token(21, [99]) is True
+    assert r.has_pending_input and r.get_next_chunk_tokens(2) == [21] and r.get_next_chunk_positions(2) == [3]
+    r.add_computed_tokens(1)
+    assert r.add_sampled_token(99, [99]) is False
+    assert r.is_finished and r.generated_tokens == [21, 99] and r.finish_reason == "eos"
+    with pytest.raises(RuntimeError):
+        r.add_computed_tokens(1)
+    with pytest.raises(ValueError):
+        InferenceRequest(1, [1], 5).add_computed_tokens(2)
+
+
+def test_max_new_tokens_and_ignore_eos():
+    r = InferenceRequest(0, [1], 2, SamplingParams(ignore_eos=True))
+    assert r.add_sampled_token(9, [9]) is True
+    assert r.add_sampled_token(9, [9]) is False and r.finish_reason == "length"
+    q = InferenceRequest(1, [1], 5)
+    assert q.add_sampled_token(-1, []) is False and q.finish_reason == "no_token"
+
+
+def _finish_step(s, batch, finished=()):
+    for p in batch.portions:
+        p.request.add_computed_tokens(len(p.tokens))
+    s.update_after_step(list(finished))
+
+
+def test_a_finished_request_frees_a_batch_slot():
+    """reference: tests/scheduler/test_continuous_batch_scheduler.cpp:40-66"""
+    s = ContinuousBatchScheduler(max_batch_size=2, max_sequences=32, chunk_size=4)
+    ids = [s.add_request([1, 2, 3], 4) for _ in range(3)]
+    b1 = s.schedule_next_batch()
+    assert [r.request_id for r in b1.requests] == ids[:2]
+    _finish_step(s, b1, finished=[ids[0]])
+    for r in b1.requests[1:]:
+        r.add_sampled_token(5, [])
+    b2 = s.schedule_next_batch()
+    assert [r.request_id for r in b2.requests] == ids[1:]
+    st = s.get_stats()
+    assert (st.num_running, st.num_waiting, st.num_finished, st.total_requests) == (2, 0, 1, 3)
+
+
+def _cache(pages, page_size=4, slots=8):
+    return CacheManager([PagedKVSpec(1, 8)], page_size=page_size, num_pages=pages, max_requests=slots)
+
+
+def test_token_budget_decode_first_and_portions_cut_anywhere():
+    c = _cache(64)
+    s = ContinuousBatchScheduler(8, 8, chunk_size=16, max_num_batched_tokens=10, cache=c, max_positions=256)
+    a = s.add_request(list(range(7)), 8)
+    b1 = s.schedule_next_batch()
+    assert [(p.request.request_id, len(p.tokens), p.samples) for p in b1.portions] == [(a, 7, True)]
+    _finish_step(s, b1)
+    s.get_request(a).add_sampled_token(3, [])
+    b = s.add_request(list(range(30)), 4)
+    d = s.add_request(list(range(5)), 4)
+    b2 = s.schedule_next_batch()
+    # the decoding request first with one token, the rest of the budget (9) to the next prompt, nothing for the third
+    assert [(p.request.request_id, len(p.tokens), p.start, p.samples) for p in b2.portions] == [(a, 1, 7, True), (b, 9, 0, False)]
+    assert b2.num_tokens() == 10
+    _finish_step(s, b2)
+    s.get_request(a).add_sampled_token(3, [])
+    b3 = s.schedule_next_batch()
+    assert [(p.request.request_id, len(p.tokens), p.start) for p in b3.portions] == [(a, 1, 8), (b, 9, 9)]
+    _finish_step(s, b3)
+    s.get_request(a).add_sampled_token(3, [])
+    b4 = s.schedule_next_batch()
+    assert [(p.request.request_id, len(p.tokens), p.start) for p in b4.portions] == [(a, 1, 9), (b, 9, 18)]
+    _finish_step(s, b4)
+    s.get_request(a).add_sampled_token(3, [])
+    b5 = s.schedule_next_batch()
+    # b's last 3 prompt tokens end its prompt (sampled), and the third request gets what is left of the budget
+    assert [(p.request.request_id, len(p.tokens), p.samples) for p in b5.portions] == [(a, 1, True), (b, 3, True), (d, 5, True)]
+    c.check()
+
+
+def test_admission_waits_for_pages_and_shortens_running_prefill():
+    c = _cache(pages=4)            # 16 tokens
+    s = ContinuousBatchScheduler(4, 4, chunk_size=8, cache=c, max_positions=64)
+    a = s.add_request(list(range(12)), 2)
+    b = s.add_request(list(range(6)), 2)
+    b1 = s.schedule_next_batch()
+    # a takes 8 tokens (2 pages); b's 6 tokens need 2 pages: they fit
+    assert [(p.request.request_id, len(p.tokens)) for p in b1.portions] == [(a, 8), (b, 6)]
+    _finish_step(s, b1)
+    s.get_request(b).add_sampled_token(1, [])
+    e = s.add_request(list(range(3)), 2)
+    b2 = s.schedule_next_batch()
+    # no page is free: b decodes inside its page; a's next portion is not possible; e is not admitted
+    assert [(p.request.request_id, len(p.tokens)) for p in b2.portions] == [(b, 1)]
+    assert s.num_waiting() == 1 and not b2.preempted
+    _finish_step(s, b2)
+    s.get_request(b).add_sampled_token(1, [])     # second token: b is finished (max_new_tokens = 2)
+    s.update_after_step([b])
+    b3 = s.schedule_next_batch()
+    assert [(p.request.request_id, len(p.tokens)) for p in b3.portions] == [(a, 4), (e, 3)]
+    c.check()
+
+
+def test_preemption_of_the_newest_when_a_decode_needs_a_page():
+    c = _cache(pages=4)
+    s = ContinuousBatchScheduler(4, 4, chunk_size=8, cache=c, max_positions=64)
+    a = s.add_request(list(range(8)), 5)
+    b = s.add_request(list(range(8)), 5)
+    b1 = s.schedule_next_batch()
+    assert len(b1.portions) == 2 and c.free_pages() == [0]
+    _finish_step(s, b1)
+    for rid in (a, b):
+        s.get_request(rid).add_sampled_token(7, [])
+    b2 = s.schedule_next_batch()
+    # a needs a fifth page: b, admitted last, is preempted and waits at the front
+    assert [r.request_id for r in b2.preempted] == [b]
+    assert [(p.request.request_id, len(p.tokens)) for p in b2.portions] == [(a, 1)]
+    rb = s.get_request(b)
+    assert rb.state == RequestState.PREEMPTED and rb.num_computed_tokens == 0 and rb.generated_tokens == [7]
+    assert s.waiting[0] is rb and s.get_stats().num_preemptions == 1
+    c.check()
+    _finish_step(s, b2, finished=[a])
+    b3 = s.schedule_next_batch()
+    # b runs again from its first token: prompt and the token it had generated, then sampling goes on
+    assert [(p.request.request_id, p.tokens, p.samples) for p in b3.portions] == [(b, list(range(8)), False)]
+    _finish_step(s, b3)
+    b4 = s.schedule_next_batch()
+    assert [(p.tokens, p.start, p.samples) for p in b4.portions] == [([7], 8, True)]
+    c.check()
+
+
+def test_what_can_never_fit_is_refused():
+    c = _cache(pages=2)
+    s = ContinuousBatchScheduler(2, 2, chunk_size=8, cache=c, max_positions=16)
+    with pytest.raises(SchedulerError, match="positions"):
+        s.add_request(list(range(10)), 8)
+    with pytest.raises(SchedulerError, match="cache pages"):
+        s.add_request(list(range(8)), 2)           # 9 tokens = 3 pages of 4
+    ok = s.add_request(list(range(7)), 2)          # 8 tokens = 2 pages
+    assert s.get_request(ok) is not None
+    with pytest.raises(ValueError):
+        s.add_request([], 2)
+
+
+def test_a_lone_request_that_outgrows_the_pool_is_an_error_not_a_hang():
+    c = _cache(pages=2)
+    s = ContinuousBatchScheduler(2, 2, chunk_size=8, cache=None, max_positions=64)
+    a = s.add_request(list(range(8)), 5)
+    s.cache = c                                    # past the admission check, to reach the running-time decision
+    _finish_step(s, s.schedule_next_batch())
+    s.get_request(a).add_sampled_token(1, [])
+    with pytest.raises(SchedulerError, match="too small"):
+        s.schedule_next_batch()
