@@ -1,0 +1,352 @@
+"""Each HIP kernel alone against its plain float64 formula, at sizes other than the tiny models':
+widths and vocabularies that are no power of two, head sizes in steps of 16, odd head groupings,
+several page sizes, both storage types."""
+import math
+
+import pytest
+import torch
+
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+F64 = torch.float64
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=torch.float32) * scale
+
+
+def tol(dtype):
+    return dict(atol=2e-5, rtol=2e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+def as_stored(x, dtype):
+    """Round to the storage type and give both the device tensor and its exact float64 value."""
+    dev = x.to(dtype).to(DEV)
+    return dev, dev.cpu().to(F64)
+
+
+@pytest.fixture(scope="module")
+def k():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from pulse_infer_amd.ops import kernels, library
+    library.load()
+    return kernels
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed_gather(k, dtype):
+    table, ref = as_stored(rnd(37, 70), dtype)
+    ids = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32, device=DEV)
+    out = torch.full((5, 70), 7.0, device=DEV)
+    bad = torch.zeros(1, dtype=torch.int32, device=DEV)
+    k.embed_gather(ids, table, out, bad)
+    assert torch.equal(out.cpu().to(F64), ref[ids.cpu().long()]) and bad.item() == 0
+    k.embed_gather(torch.tensor([3, 37, -1], dtype=torch.int32, device=DEV), table, out[:3], bad)
+    assert bad.item() == 1 and torch.equal(out[1].cpu(), torch.zeros(70))   # refused loudly, nothing read out of range
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hidden", [48, 1000, 4100])
+def test_add_rmsnorm(k, dtype, hidden):
+    rows, eps = 9, 3e-5
+    h = rnd(rows, hidden, seed=1).to(DEV)
+    delta, dref = as_stored(rnd(rows, hidden, seed=2), dtype)
+    w, wref = as_stored(1 + 0.1 * rnd(hidden, seed=3), dtype)
+    want_sum = h.cpu().to(F64) + dref
+    out = torch.empty(rows, hidden, dtype=dtype, device=DEV)
+    hh = h.clone()
+    k.add_rmsnorm(hh, delta, w, eps, out)
+    assert torch.allclose(out.cpu().to(F64), P.rms_norm(want_sum, wref, eps), **tol(dtype))
+    assert torch.allclose(hh.cpu().to(F64), want_sum, atol=1e-6)            # the residual keeps the sum, in float32
+    # without delta nothing is written back; gathered rows leave h alone
+    hh = h.clone()
+    k.add_rmsnorm(hh, None, w, eps, out)
+    assert torch.equal(hh, h)
+    assert torch.allclose(out.cpu().to(F64), P.rms_norm(h.cpu().to(F64), wref, eps), **tol(dtype))
+    pick = torch.tensor([8, 0, 3], dtype=torch.int32, device=DEV)
+    out3 = torch.empty(3, hidden, dtype=dtype, device=DEV)
+    k.add_rmsnorm(hh, delta, w, eps, out3, rows=pick)
+    assert torch.equal(hh, h)
+    assert torch.allclose(out3.cpu().to(F64), P.rms_norm(want_sum[[8, 0, 3]], wref, eps), **tol(dtype))
+
+
+def test_residual_add_and_gather_rows(k):
+    h = rnd(5, 33).to(DEV)
+    d, dref = as_stored(rnd(5, 33, seed=1), torch.bfloat16)
+    want = h.cpu().to(F64) + dref
+    k.residual_add(h, d)
+    assert torch.allclose(h.cpu().to(F64), want, atol=1e-6)
+    out = torch.empty(2, 33, device=DEV)
+    k.gather_rows(h, torch.tensor([4, 1], dtype=torch.int32, device=DEV), out)
+    assert torch.equal(out, h[[4, 1]])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu(k, dtype):
+    gu, ref = as_stored(rnd(7, 2 * 77, seed=4, scale=3.0), dtype)
+    out = torch.empty(7, 77, dtype=dtype, device=DEV)
+    k.swiglu(gu, out)
+    assert torch.allclose(out.cpu().to(F64), P.silu(ref[:, :77]) * ref[:, 77:], **tol(dtype))
+
+
+@pytest.mark.parametrize("shape", [(1, 7, 5), (3, 70, 33), (65, 129, 100), (130, 64, 257)])
+@pytest.mark.parametrize("types", [(torch.float32, torch.float32, torch.float32),
+                                   (torch.bfloat16, torch.bfloat16, torch.float32),
+                                   (torch.float32, torch.bfloat16, torch.bfloat16)])
+def test_gemm_f32(k, shape, types):
+    m, n, kk = shape
+    a, aref = as_stored(rnd(m, kk, seed=5), types[0])
+    w, wref = as_stored(rnd(n, kk, seed=6), types[1])
+    out = torch.empty(m, n, dtype=types[2], device=DEV)
+    k.gemm_f32(a, w, out)
+    assert torch.allclose(out.cpu().to(F64), aref @ wref.T, **(tol(types[2]) if types[2] == torch.bfloat16
+                                                               else dict(atol=1e-4, rtol=1e-5)))
+
+
+def test_gemm_f32_rows_do_not_depend_on_the_batch(k):
+    a = rnd(40, 300, seed=7).to(DEV)
+    w = rnd(90, 300, seed=8).to(DEV)
+    full = torch.empty(40, 90, device=DEV)
+    k.gemm_f32(a, w, full)
+    one = torch.empty(1, 90, device=DEV)
+    k.gemm_f32(a[17:18], w, one)
+    assert torch.equal(one[0], full[17])                                   # same sums in the same order
+
+
+def test_rope_table(k):
+    theta, rot = 1e6, 48
+    pos = torch.tensor([0, 1, 2, 1000, 40959], dtype=torch.int32, device=DEV)
+    inv = torch.pow(torch.tensor(theta, dtype=F64), -torch.arange(rot // 2, dtype=F64) * 2 / rot).to(DEV)
+    cos = torch.empty(5, rot // 2, device=DEV)
+    sin = torch.empty_like(cos)
+    k.rope_table(pos, inv, cos, sin)
+    angle = pos.cpu().to(F64)[:, None] / theta ** (torch.arange(0, rot, 2, dtype=F64) / rot)
+    assert torch.allclose(cos.cpu().to(F64), torch.cos(angle), atol=1e-7)
+    assert torch.allclose(sin.cpu().to(F64), torch.sin(angle), atol=1e-7)
+
+
+def _cache(pages, nkv, bs, d, dtype):
+    return (torch.zeros(pages, nkv, bs, d, dtype=dtype, device=DEV),
+            torch.zeros(pages, nkv, d, bs, dtype=dtype, device=DEV))
+
+
+def _tables(k, positions, theta, rot):
+    inv = torch.pow(torch.tensor(theta, dtype=F64), -torch.arange(rot // 2, dtype=F64) * 2 / rot).to(DEV)
+    cos = torch.empty(len(positions), rot // 2, device=DEV)
+    sin = torch.empty_like(cos)
+    k.rope_table(torch.tensor(positions, dtype=torch.int32, device=DEV), inv, cos, sin)
+    return cos, sin
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", [
+    dict(nq=5, nkv=5, d=16, rot=16, pairing="interleaved", norm=True, bs=4),
+    dict(nq=6, nkv=2, d=48, rot=48, pairing="interleaved", norm=True, bs=16),
+    dict(nq=4, nkv=1, d=80, rot=32, pairing="interleaved", norm=True, bs=8),    # partial rotation, tail untouched
+    dict(nq=3, nkv=3, d=160, rot=160, pairing="half", norm=False, bs=16),       # other pairing, no norm, > 128 channels
+    dict(nq=2, nkv=1, d=32, rot=0, pairing="interleaved", norm=True, bs=2),     # no position encoding at all
+])
+def test_qk_rope_kv(k, dtype, case):
+    nq, nkv, d, rot, bs = case["nq"], case["nkv"], case["d"], case["rot"], case["bs"]
+    eps, theta = 2e-5, 7e4
+    # two requests in one step: 5 tokens from position 6 (crossing a page edge for small pages) and 1 token at 0
+    positions = [6, 7, 8, 9, 10, 0]
+    entry = [0, 0, 0, 0, 0, 1]
+    width = 10 // bs + 1
+    pages_a = list(range(3, 3 + width))
+    table = torch.full((2, width), -1, dtype=torch.int32)
+    table[0] = torch.tensor(pages_a, dtype=torch.int32)
+    table[1, 0] = 1
+    kc, vc = _cache(3 + width + 1, nkv, bs, d, dtype)
+    qkv, ref = as_stored(rnd(6, (nq + 2 * nkv) * d + 8, seed=9), dtype)      # 8 spare columns: rows are strided
+    qw, qwref = as_stored(1 + 0.1 * rnd(d, seed=10), dtype)
+    kw, kwref = as_stored(1 + 0.1 * rnd(d, seed=11), dtype)
+    cos, sin = _tables(k, positions, theta, rot) if rot else (None, None)
+    k.qk_rope_kv(qkv, nq, nkv, d, qw if case["norm"] else None, kw if case["norm"] else None, eps, cos, sin, rot,
+                 0 if case["pairing"] == "interleaved" else 1, kc, vc,
+                 torch.tensor(positions, dtype=torch.int32, device=DEV), torch.tensor(entry, dtype=torch.int32, device=DEV),
+                 table.to(DEV))
+    q = ref[:, :nq * d].reshape(6, nq, d)
+    kk = ref[:, nq * d:(nq + nkv) * d].reshape(6, nkv, d)
+    vv = ref[:, (nq + nkv) * d:(nq + 2 * nkv) * d].reshape(6, nkv, d)
+    if case["norm"]:
+        q, kk = P.rms_norm(q, qwref, eps), P.rms_norm(kk, kwref, eps)
+    if rot:
+        q = P.rope(q, positions, theta, rot, case["pairing"])
+        kk = P.rope(kk, positions, theta, rot, case["pairing"])
+    got = qkv.cpu().to(F64)
+    assert torch.allclose(got[:, :nq * d].reshape(6, nq, d), q, **tol(dtype))
+    assert torch.equal(got[:, nq * d:], ref[:, nq * d:])                    # k, v and the spare columns stay as they were
+    kcpu, vcpu = kc.cpu().to(F64), vc.cpu().to(F64)
+    touched = torch.zeros(kc.shape[0], bs, dtype=torch.bool)
+    for t, (p, e) in enumerate(zip(positions, entry)):
+        page, slot = int(table[e, p // bs]), p % bs
+        touched[page, slot] = True
+        assert torch.allclose(kcpu[page, :, slot, :], kk[t], **tol(dtype))
+        assert torch.equal(vcpu[page, :, :, slot], vv[t])                   # values are copied as they are
+    assert torch.all(kcpu[~touched.unsqueeze(1).expand(-1, nkv, -1)] == 0)  # nothing else was written
+
+
+def _fill_cache(kc, vc, keys, vals, table_row, bs):
+    """Put keys/vals [S, nkv, d] of one request into its pages."""
+    for j in range(keys.shape[0]):
+        page, slot = table_row[j // bs], j % bs
+        kc[page, :, slot, :] = keys[j]
+        vc[page, :, :, slot] = vals[j]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", [
+    dict(nq=4, nkv=2, d=16, bs=4, window=0),
+    dict(nq=6, nkv=1, d=32, bs=16, window=0),
+    dict(nq=3, nkv=3, d=48, bs=8, window=7),
+    dict(nq=8, nkv=2, d=128, bs=16, window=0),
+    dict(nq=2, nkv=1, d=208, bs=32, window=40),
+])
+def test_attn_generic(k, dtype, case):
+    nq, nkv, d, bs, window = case["nq"], case["nkv"], case["d"], case["bs"], case["window"]
+    lens = [70, 131]                        # contexts of two requests; crossing the 64-key tile and page edges
+    pages = [[126 - 2 * i for i in range((lens[0] + bs - 1) // bs)],       # descending even pages
+             [2 * i + 1 for i in range((lens[1] + bs - 1) // bs)]]         # ascending odd pages
+    width = max(len(p) for p in pages)
+    kc, vc = _cache(128, nkv, bs, d, dtype)
+    refs = []
+    for r, n in enumerate(lens):
+        ks, kref = as_stored(rnd(n, nkv, d, seed=20 + r), dtype)
+        vs, vref = as_stored(rnd(n, nkv, d, seed=30 + r), dtype)
+        _fill_cache(kc, vc, ks, vs, pages[r], bs)
+        refs.append((kref, vref))
+    table = torch.full((2, width), -1, dtype=torch.int32)
+    for r, p in enumerate(pages):
+        table[r, :len(p)] = torch.tensor(p, dtype=torch.int32)
+    # request 0: its last 9 tokens as a portion; request 1: a single decoded token; and an early token of request 1
+    positions = list(range(lens[0] - 9, lens[0])) + [lens[1] - 1]
+    entry = [0] * 9 + [1]
+    q, qref = as_stored(rnd(len(positions), nq * d + 16, seed=40), dtype)
+    out = torch.zeros(len(positions), nq * d, dtype=dtype, device=DEV)
+    scale = 0.37
+    k.attn_generic(q, out, nq, nkv, d, kc, vc, torch.tensor(positions, dtype=torch.int32, device=DEV),
+                   torch.tensor(entry, dtype=torch.int32, device=DEV), table.to(DEV), scale, window)
+    got = out.cpu().to(F64).reshape(-1, nq, d)
+    for t, (p, e) in enumerate(zip(positions, entry)):
+        kref, vref = refs[e]
+        want = P.causal_attention(qref[t:t + 1, :nq * d].reshape(1, nq, d), kref[:p + 1], vref[:p + 1], scale,
+                                  window or None, [p])
+        assert torch.allclose(got[t], want[0], **tol(dtype)), (t, p, e)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attn_generic_one_far_key_and_the_window_edge(k, dtype):
+    """Random keys would hide a key that is skipped or read from the wrong page: make one score stand out."""
+    nq, nkv, d, bs, n = 2, 1, 32, 16, 600
+    pages = list(range(n // bs + 1))
+    table = torch.tensor([pages], dtype=torch.int32, device=DEV)
+    for target, window, seen in ((3, 0, True), (n - 100, 100, True), (n - 101, 100, False), (bs * 7, 0, True),
+                                 (bs * 7 - 1, 0, True), (n - 1, 1, True)):
+        kc, vc = _cache(len(pages), nkv, bs, d, dtype)
+        keys = rnd(n, nkv, d, seed=50, scale=0.1)
+        vals = rnd(n, nkv, d, seed=51)
+        keys[target] = 0
+        keys[target, 0, 0] = 30.0
+        ks, kref = as_stored(keys, dtype)
+        vs, vref = as_stored(vals, dtype)
+        _fill_cache(kc, vc, ks, vs, pages, bs)
+        qv = rnd(1, nq * d, seed=52, scale=0.1)
+        qv[0, 0] = 30.0
+        qv[0, d] = 30.0
+        q, qref = as_stored(qv, dtype)
+        out = torch.zeros(1, nq * d, dtype=dtype, device=DEV)
+        k.attn_generic(q, out, nq, nkv, d, kc, vc, torch.tensor([n - 1], dtype=torch.int32, device=DEV),
+                       torch.tensor([0], dtype=torch.int32, device=DEV), table, 1.0, window)
+        got = out.cpu().to(F64).reshape(nq, d)
+        close = torch.allclose(got, vref[target].expand(nq, d), atol=1e-2)
+        assert close == seen, (target, window)
+        want = P.causal_attention(qref.reshape(1, nq, d), kref, vref, 1.0, window or None, [n - 1])
+        assert torch.allclose(got, want[0], **tol(dtype)), (target, window)
+
+
+def test_argmax_takes_the_lowest_index_among_equals(k):
+    logits = rnd(5, 1009, seed=60).to(DEV)
+    logits[0, 17] = logits[0, 800] = 50.0
+    logits[1, 1008] = 60.0
+    logits[2, 0] = 60.0
+    logits[3] = 1.25
+    logits[4, 5] = float("nan")
+    out = torch.empty(5, dtype=torch.int32, device=DEV)
+    k.sample(logits, out)
+    want = [17, 1008, 0, 0, int(torch.argmax(torch.nan_to_num(logits[4].cpu(), nan=-1e30)))]
+    assert out.tolist() == want
+
+
+def test_temperature_sampling_follows_the_softmax(k):
+    vocab, rows = 700, 4000
+    base = torch.full((vocab,), -30.0)
+    base[[5, 123, 400, 699]] = torch.tensor([1.0, 2.0, 0.5, 1.5])
+    logits = base.repeat(rows, 1).to(DEV)
+    temperature = torch.full((rows,), 0.8, device=DEV)
+    uniform = torch.rand(rows, generator=torch.Generator().manual_seed(1)).to(DEV)
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    k.sample(logits, out, temperature=temperature, uniform=uniform)
+    counts = torch.bincount(out.cpu().long(), minlength=vocab).double() / rows
+    want = torch.softmax(base.double() / 0.8, dim=0)
+    assert torch.allclose(counts, want, atol=0.03)
+    # the same uniform number gives the same token, whatever else is in the batch
+    again = torch.empty(1, dtype=torch.int32, device=DEV)
+    k.sample(logits[7:8], again, temperature=temperature[7:8], uniform=uniform[7:8])
+    assert again.item() == out[7].item()
+
+
+def test_top_k_top_p_penalty_and_banned(k):
+    vocab, rows = 333, 3000
+    base = torch.linspace(-3, 3, vocab)[torch.randperm(vocab, generator=torch.Generator().manual_seed(2))]
+    logits = base.repeat(rows, 1).to(DEV)
+    uniform = torch.rand(rows, generator=torch.Generator().manual_seed(3)).to(DEV)
+    temperature = torch.ones(rows, device=DEV)
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    # top-k: only the k largest ever appear, with renormalised softmax frequencies
+    k.sample(logits, out, temperature=temperature, uniform=uniform,
+             top_k=torch.full((rows,), 5, dtype=torch.int32, device=DEV))
+    top5 = torch.topk(base, 5).indices
+    assert set(out.tolist()) <= set(top5.tolist())
+    freq = torch.bincount(out.cpu().long(), minlength=vocab).double()[top5] / rows
+    assert torch.allclose(freq, torch.softmax(base[top5].double(), 0), atol=0.03)
+    # top-p: the shortest prefix of the sorted distribution whose mass reaches p
+    probs = torch.softmax(base.double(), 0)
+    order = torch.argsort(probs, descending=True)
+    keep = order[: int((torch.cumsum(probs[order], 0) < 0.3).sum()) + 1]
+    k.sample(logits, out, temperature=temperature, uniform=uniform, top_p=torch.full((rows,), 0.3, device=DEV))
+    assert set(out.tolist()) == set(keep.tolist())
+    # presence penalty: a seen token loses `penalty` before the choice; banned ids never appear
+    words = (vocab + 31) // 32
+    seen = torch.zeros(2, words, dtype=torch.int32, device=DEV)
+    best = int(torch.argmax(base))
+    second = int(torch.topk(base, 2).indices[1])
+    k.mark_seen(seen, torch.tensor([1, 1], dtype=torch.int32, device=DEV),
+                torch.tensor([best, 7], dtype=torch.int32, device=DEV), vocab)
+    greedy = torch.empty(2, dtype=torch.int32, device=DEV)
+    k.sample(logits[:2], greedy, penalty=torch.tensor([1.5, 1.5], device=DEV),
+             seen_row=torch.tensor([0, 1], dtype=torch.int32, device=DEV), seen_masks=seen)
+    assert greedy.tolist() == [best, second]
+    banned = torch.zeros(words, dtype=torch.int32)
+    banned[best >> 5] = 1 << (best & 31) if (best & 31) < 31 else -(1 << 31)
+    k.sample(logits[:1], greedy[:1], banned=banned.to(DEV))
+    assert greedy[0].item() == second
+
+
+def test_kernels_refuse_what_they_cannot_do(k):
+    from pulse_infer_amd.ops import KernelError
+    with pytest.raises(KernelError, match="GPU"):
+        k.swiglu(torch.zeros(2, 4), torch.zeros(2, 2))
+    with pytest.raises(KernelError, match="storage type"):
+        k.swiglu(torch.zeros(2, 4, dtype=torch.float16, device=DEV), torch.zeros(2, 2, dtype=torch.float16, device=DEV))
+    with pytest.raises(KernelError, match="inner sizes"):
+        k.gemm_f32(torch.zeros(2, 4, device=DEV), torch.zeros(3, 5, device=DEV), torch.zeros(2, 3, device=DEV))
+    kc, vc = _cache(2, 1, 4, 1024, torch.float32)
+    with pytest.raises(KernelError, match="head_dim"):
+        k.attn_generic(torch.zeros(1, 1024, device=DEV), torch.zeros(1, 1024, device=DEV), 1, 1, 1024, kc, vc,
+                       torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
+                       torch.zeros(1, 1, dtype=torch.int32, device=DEV), 1.0)

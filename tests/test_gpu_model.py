@@ -1,0 +1,218 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16: each request alone and whole;
+most of it in one step and the last 32 tokens one by one; in portions of changing size down to two
+tokens; and mixed, up to four live requests, portions of some beside decoded tokens of others, with so
+few pages that they are used again.  Tolerances are fixed here once and are not to be widened."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT, TINY, token_ids
+
+pytestmark = pytest.mark.gpu
+
+# max |engine - plain| relative to the largest |logit| of the sequence
+TOL = {"float32": 3e-5, "bfloat16": 3e-2}
+# two ways of cutting the same request, same dtype: only the order of float32 sums differs
+SPLIT_TOL = {"float32": 1e-5, "bfloat16": 2e-2}
+
+
+def close(got, want, dtype, what, tol=TOL):
+    got, want = got.double().cpu(), want.double().cpu()
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    scale = max(1.0, float(want.abs().max()))
+    err = float((got - want).abs().max())
+    assert err <= tol[dtype] * scale, f"{what}: max error {err:.3e} exceeds {tol[dtype] * scale:.3e}"
+
+
+@pytest.fixture(scope="module")
+def engines(model_folders):
+    """(name, dtype) -> ModelRunner with a deliberately small pool."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+
+    made = {}
+
+    def get(name, dtype, tokens=256):
+        key = (name, dtype)
+        if key not in made:
+            _, model = load_model(model_folders[name], mode=dtype)
+            page = TINY[name][1]
+            made[key] = ModelRunner(model, page_size=page, num_pages=tokens // page, max_requests=4)
+        return made[key]
+
+    return get
+
+
+def run_alone(runner, ids, cuts, rid="r"):
+    """Feed ids in portions of the given sizes, wanting every position; returns [len(ids), vocab]."""
+    from pulse_infer_amd.engine.runner import StepEntry
+
+    assert sum(cuts) == len(ids)
+    runner.add_request(rid)
+    outs, p = [], 0
+    for n in cuts:
+        runner.reserve(rid, p + n)
+        outs.append(runner.step([StepEntry(rid, ids[p:p + n], list(range(n)))]))
+        p += n
+    runner.free_request(rid)
+    runner.cache.check()
+    return torch.cat(outs)
+
+
+LENGTH = {"A": 100, "B": 150, "W": 170}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "W"])
+def test_whole_tail_and_portions(engines, plain_logits, name, dtype):
+    cfg = TINY[name][0]
+    ids = token_ids(cfg["vocab_size"], LENGTH[name], seed=3)
+    want = plain_logits(name, ids)
+    runner = engines(name, dtype)
+    whole = run_alone(runner, ids, [len(ids)])
+    close(whole, want, dtype, f"{name} whole")
+    tail = run_alone(runner, ids, [len(ids) - 32] + [1] * 32)
+    close(tail, want, dtype, f"{name} last 32 one by one")
+    close(tail, whole, dtype, f"{name} tail against whole", SPLIT_TOL)
+    cuts, left, sizes = [], len(ids), [7, 2, 16, 3, 2, 33, 5, 2, 64, 11, 2]
+    while left:
+        n = min(sizes[len(cuts) % len(sizes)], left)
+        if left - n == 1:          # keep every portion at two tokens or more
+            n += 1
+        cuts.append(n)
+        left -= n
+    portions = run_alone(runner, ids, cuts)
+    close(portions, want, dtype, f"{name} portions {cuts}")
+    close(portions, whole, dtype, f"{name} portions against whole", SPLIT_TOL)
+    first = run_alone(runner, ids[:3], [1, 1, 1])                    # the first tokens of a sequence
+    close(first, want[:3], dtype, f"{name} first tokens")
+
+
+def mixed_trace(vocab, seed):
+    """Six requests, at most four live, over a pool that holds 256 tokens: pages of finished requests are
+    used again by later ones.  Steps mix prompt portions of some with single tokens of others."""
+    rng = np.random.RandomState(seed)
+    lengths = {"a": 60, "b": 45, "c": 64, "d": 30, "e": 50, "f": 58}
+    ids = {k: token_ids(vocab, n, seed=seed * 10 + i) for i, (k, n) in enumerate(lengths.items())}
+    fed = {k: 0 for k in lengths}
+    waiting, live, steps = list(lengths), [], []
+    while waiting or live:
+        held = sum((fed[k] + 63) // 64 * 64 for k in live)
+        while waiting and len(live) < 4 and held + (lengths[waiting[0]] + 63) // 64 * 64 <= 256:
+            k = waiting.pop(0)
+            live.append(k)
+            held += (lengths[k] + 63) // 64 * 64
+        entries, end = [], []
+        for k in list(live):
+            if rng.rand() < 0.2 and len(live) > 1:
+                continue                                             # a request may sit a step out
+            left = lengths[k] - fed[k]
+            if fed[k] >= lengths[k] - 12:
+                n = 1                                                # its last tokens come one by one
+            else:
+                n = int(min(left - 12, rng.choice([2, 3, 5, 8, 13, 21])))
+                n = max(n, 1)
+            entries.append({"id": k, "tokens": ids[k][fed[k]:fed[k] + n], "want": list(range(n))})
+            fed[k] += n
+            if fed[k] == lengths[k]:
+                end.append(k)
+                live.remove(k)
+        if entries:
+            steps.append({"step": len(steps), "entries": entries, "end": end})
+    return ids, steps
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "W"])
+def test_mixed_batches_with_page_reuse(engines, plain_logits, name, dtype):
+    from pulse_infer_amd.engine.runner import StepEntry
+
+    cfg = TINY[name][0]
+    ids, steps = mixed_trace(cfg["vocab_size"], seed=5)
+    runner = engines(name, dtype)
+    got = {k: [] for k in ids}
+    pages_seen = {}
+    most_live = 0
+    for step in steps:
+        entries = []
+        for e in step["entries"]:
+            if not runner.cache.has_request(e["id"]):
+                runner.add_request(e["id"])
+            runner.reserve(e["id"], runner.cache.computed(e["id"]) + len(e["tokens"]))
+            entries.append(StepEntry(e["id"], e["tokens"], e["want"]))
+            pages_seen.setdefault(e["id"], set()).update(p for p in runner.cache.table(0, e["id"]) if p >= 0)
+        most_live = max(most_live, len(runner.cache.requests))
+        logits = runner.step(entries)
+        row = 0
+        for e in step["entries"]:
+            got[e["id"]].append(logits[row:row + len(e["want"])])
+            row += len(e["want"])
+        for k in step["end"]:
+            runner.free_request(k)
+        runner.cache.check()
+    assert most_live == 4 and any(len(s["entries"]) >= 3 for s in steps)
+    assert any(len(e["tokens"]) > 1 for s in steps for e in s["entries"]) and \
+        any(len(e["tokens"]) == 1 and len(s["entries"]) > 1 for s in steps for e in s["entries"])
+    names = list(ids)
+    assert any(pages_seen[a] & pages_seen[b] for i, a in enumerate(names) for b in names[i + 1:]), "no page was used again"
+    for k, parts in got.items():
+        close(torch.cat(parts), plain_logits(name, ids[k]), dtype, f"{name} mixed request {k}")
+
+
+def test_step_refuses_what_it_cannot_run(engines):
+    from pulse_infer_amd.engine.runner import StepEntry, StepError
+
+    runner = engines("A", "float32")
+    with pytest.raises(StepError, match="at least one entry"):
+        runner.step([])
+    with pytest.raises(StepError, match="not live"):
+        runner.step([StepEntry("nobody", [1], [0])])
+    runner.add_request("x")
+    try:
+        with pytest.raises(StepError, match="reserved"):
+            runner.step([StepEntry("x", [1, 2], [0])])
+        runner.reserve("x", 2)
+        with pytest.raises(StepError, match="outside the vocabulary"):
+            runner.step([StepEntry("x", [1, 256], [0])])
+        with pytest.raises(StepError, match="wanted place"):
+            runner.step([StepEntry("x", [1, 2], [2])])
+        with pytest.raises(StepError, match="twice"):
+            runner.step([StepEntry("x", [1], []), StepEntry("x", [2], [])])
+        with pytest.raises(StepError, match="no tokens"):
+            runner.step([StepEntry("x", [], [])])
+        assert runner.step([StepEntry("x", [1, 2], [])]).shape == (0, 256)      # nothing wanted: nothing returned
+        assert runner.cache.computed("x") == 2
+    finally:
+        runner.free_request("x")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(model_folders, plain_logits, tmp_path, dtype):
+    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and `done <step>` lines out."""
+    name = "B"
+    cfg = TINY[name][0]
+    ids, steps = mixed_trace(cfg["vocab_size"], seed=7)
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_folders[name], "--dtype", dtype,
+         "--out", str(out), "--max-tokens", "256"],
+        input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {s['step']}" for s in steps]
+    got = {k: [] for k in ids}
+    for s in steps:
+        data = np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(-1, cfg["vocab_size"])
+        assert data.shape[0] == sum(len(e["want"]) for e in s["entries"])
+        row = 0
+        for e in s["entries"]:
+            got[e["id"]].append(torch.from_numpy(data[row:row + len(e["want"])].copy()))
+            row += len(e["want"])
+    for k, parts in got.items():
+        close(torch.cat(parts), plain_logits(name, ids[k]), dtype, f"trace_run request {k}")
