@@ -77,7 +77,7 @@ def main(argv: Optional[List[str]] = None) -> int:
                    num_pages=args.num_pages, max_num_batched_tokens=args.max_tokens, seed=args.seed)
     if args.random_weights:
         init = args.init if args.init == "fan_in" else float(args.init)
-        llm = LLM.from_config_random(config, seed=args.seed, init=init, dtype=dtype, device=args.device, **options)
+        llm = LLM.from_config_random(config, weights_seed=args.seed, init=init, dtype=dtype, device=args.device, **options)
     else:
         llm = LLM.from_pretrained(model_dir, dtype=dtype, device=args.device, **options)
 

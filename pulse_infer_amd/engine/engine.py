@@ -151,13 +151,13 @@ class LLM:
         return cls(model, config, **engine_options)
 
     @classmethod
-    def from_config_random(cls, config: Any, seed: int = 0, init: Any = "fan_in", dtype: str = "bfloat16",
+    def from_config_random(cls, config: Any, weights_seed: int = 0, init: Any = "fan_in", dtype: str = "bfloat16",
                            device: str = "cuda:0", **engine_options):
         """Random weights made on the GPU, without a file (for sizes not worth writing to disk)."""
         from ..models.causal_lm import expected_tensors
         from ..weights.random_init import RandomSource
 
-        source = RandomSource(expected_tensors(config.model_spec()), seed, init, torch.bfloat16, device=device)
+        source = RandomSource(expected_tensors(config.model_spec()), weights_seed, init, torch.bfloat16, device=device)
         model = build_model(config, source, mode=dtype, device=device)
         return cls(model, config, **engine_options)
 

@@ -1,0 +1,155 @@
+"""Generation through the entry points: greedy against the plain implementation, long decoding,
+continuous batching with portions, preemption when pages run out, seeded sampling, the command line."""
+import json
+
+import pytest
+import torch
+
+from conftest import TINY, token_ids
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+
+
+def make_llm(folder, dtype="float32", **options):
+    from pulse_infer_amd import LLM
+    return LLM.from_pretrained(folder, dtype=dtype, **options)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "W"])
+def test_greedy_generation_matches_the_plain_implementation(gpu, model_folders, plain_models, name):
+    cfg, page = TINY[name]
+    prompts = [token_ids(cfg["vocab_size"], n, seed=20 + n) for n in (5, 11, 17)]
+    llm = make_llm(model_folders[name], "float32", max_batch_size=3, chunk_size=8, page_size=page, num_pages=64)
+    got = llm.generate(prompts, max_new_tokens=8, ignore_eos=True)
+    for prompt, out in zip(prompts, got):
+        assert out == plain_models[name].greedy(prompt, 8)
+    llm.engine.runner.cache.check()
+    assert not llm.engine.runner.cache.requests                       # everything was given back
+    # bfloat16: the same tokens wherever the plain top-two margin is clear of bfloat16's error
+    llm16 = make_llm(model_folders[name], "bfloat16", max_batch_size=3, chunk_size=8, page_size=page, num_pages=64)
+    for prompt, out in zip(prompts, llm16.generate(prompts, max_new_tokens=8, ignore_eos=True)):
+        ids = list(prompt)
+        for tok in out:
+            row = plain_models[name].logits(ids)[-1]
+            top = torch.topk(row, 2)
+            if float(top.values[0] - top.values[1]) > 0.25:
+                assert tok == int(top.indices[0])
+            ids.append(tok)                                           # follow the engine's own path
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_token_by_token(gpu, model_folders, plain_logits, dtype):
+    """240 positions one token at a time (W has windows that pass many pages meanwhile)."""
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from test_gpu_model import close
+
+    for name in ("B", "W"):
+        cfg, page = TINY[name]
+        ids = token_ids(cfg["vocab_size"], 240, seed=33)
+        _, model = load_model(model_folders[name], mode=dtype)
+        runner = ModelRunner(model, page_size=page, num_pages=256 // page, max_requests=2)
+        runner.add_request("r")
+        rows = []
+        for i, tok in enumerate(ids):
+            runner.reserve("r", i + 1)
+            rows.append(runner.step([StepEntry("r", [tok], [0])]))
+        if name == "W":
+            held = [p for p in runner.cache.table(1, "r") if p >= 0]
+            assert len(held) <= cfg["sliding_window"] // page + 2      # the window's pages only
+        runner.free_request("r")
+        close(torch.cat(rows), plain_logits(name, ids), dtype, f"{name} long decoding")
+
+
+def test_continuous_batching_gives_what_each_request_gives_alone(gpu, model_folders):
+    cfg, page = TINY["B"]
+    prompts = [token_ids(cfg["vocab_size"], n, seed=40 + n) for n in (1, 9, 33, 70)]
+    alone = []
+    for p in prompts:
+        alone.append(make_llm(model_folders["B"], max_batch_size=1, chunk_size=256, page_size=page,
+                              num_pages=32).generate([p], max_new_tokens=12, ignore_eos=True)[0])
+    llm = make_llm(model_folders["B"], max_batch_size=4, chunk_size=16, page_size=page, num_pages=32,
+                   max_num_batched_tokens=24)
+    assert llm.generate(prompts, max_new_tokens=12, ignore_eos=True) == alone
+    stats = llm.engine.get_stats()
+    assert stats.num_finished == 4 and stats.tokens_generated == 48 and stats.num_preemptions == 0
+
+
+def test_preemption_reproduces_the_outputs(gpu, model_folders):
+    cfg, page = TINY["A"]                                              # pages of 4 tokens
+    prompts = [token_ids(cfg["vocab_size"], n, seed=50 + n) for n in (14, 15, 13)]
+    roomy = make_llm(model_folders["A"], max_batch_size=3, chunk_size=8, page_size=page, num_pages=64)
+    want = roomy.generate(prompts, max_new_tokens=20, ignore_eos=True)
+    tight = make_llm(model_folders["A"], max_batch_size=3, chunk_size=8, page_size=page, num_pages=17)
+    got = tight.generate(prompts, max_new_tokens=20, ignore_eos=True)
+    stats = tight.engine.get_stats()
+    assert stats.num_preemptions > 0, "the pool was meant to run out"
+    assert got == want
+    tight.engine.runner.cache.check()
+    assert tight.engine.runner.cache.free_pages() == [17]
+
+
+def test_eos_and_max_new_tokens(gpu, model_folders, plain_models):
+    cfg, page = TINY["A"]
+    prompt = token_ids(cfg["vocab_size"], 9, seed=61)
+    path = plain_models["A"].greedy(prompt, 6)
+    from pulse_infer_amd.engine.engine import ContinuousBatchEngine
+    from pulse_infer_amd.models.factory import load_model
+    _, model = load_model(model_folders["A"], mode="float32")
+    engine = ContinuousBatchEngine(model, 2, 8, page_size=page, num_pages=32, eos_token_ids=[path[3]])
+    rid = engine.add_request(prompt, 6)
+    assert engine.get_result(rid) == []                               # nothing while it runs
+    engine.run_until_complete()
+    first_eos = path.index(path[3])
+    assert engine.get_request(rid).generated_tokens == path[:first_eos + 1]   # the end-of-sequence id is kept ...
+    assert engine.get_result(rid) == path[:first_eos]                         # ... and cut from the result
+    assert engine.get_request(rid).finish_reason == "eos"
+    with pytest.raises(ValueError, match="vocabulary"):
+        engine.add_request([cfg["vocab_size"]], 2)
+
+
+def test_seeded_sampling_does_not_depend_on_the_batch(gpu, model_folders):
+    from pulse_infer_amd import SamplingParams
+    cfg, page = TINY["B"]
+    prompts = [token_ids(cfg["vocab_size"], n, seed=70 + n) for n in (4, 21, 9)]
+    params = [SamplingParams(temperature=0.8, seed=100 + i, ignore_eos=True) for i in range(3)]
+    together = make_llm(model_folders["B"], max_batch_size=3, chunk_size=16, page_size=page, num_pages=32).generate(
+        prompts, max_new_tokens=12, sampling=params)
+    for i in (2, 0):
+        alone = make_llm(model_folders["B"], max_batch_size=1, chunk_size=5, page_size=page, num_pages=32).generate(
+            [prompts[i]], max_new_tokens=12, sampling=[params[i]])[0]
+        assert alone == together[i]
+    other = make_llm(model_folders["B"], max_batch_size=3, chunk_size=16, page_size=page, num_pages=32).generate(
+        prompts, max_new_tokens=12, sampling=[SamplingParams(temperature=0.8, seed=900 + i, ignore_eos=True) for i in range(3)])
+    assert other != together                                          # another seed, another path
+    # temperature near zero is greedy; top_k = 1 is greedy whatever the temperature
+    greedy = make_llm(model_folders["B"], page_size=page, num_pages=32).generate(prompts, max_new_tokens=6, ignore_eos=True)
+    topk1 = make_llm(model_folders["B"], page_size=page, num_pages=32).generate(
+        prompts, max_new_tokens=6, sampling=[SamplingParams(temperature=1.3, top_k=1, seed=5, ignore_eos=True)] * 3)
+    assert topk1 == greedy
+    # with a presence penalty large enough no token is generated twice
+    fresh = make_llm(model_folders["B"], page_size=page, num_pages=32).generate(
+        [prompts[1]], max_new_tokens=30, sampling=[SamplingParams(presence_penalty=1000.0, ignore_eos=True)])[0]
+    assert len(set(fresh)) == 30 and not set(fresh) & set(prompts[1])
+
+
+def test_command_line(gpu, model_folders, plain_models, capsys):
+    from pulse_infer_amd import cli
+    cfg, page = TINY["A"]
+    prompt = token_ids(cfg["vocab_size"], 7, seed=81)
+    code = cli.main([model_folders["A"], "--dtype", "f32", "--prompt-ids", ",".join(map(str, prompt)),
+                     "--max-new-tokens", "5", "--page-size", str(page), "--num-pages", "32", "--ignore-eos", "--stats"])
+    lines = capsys.readouterr().out.strip().splitlines()
+    assert code == 0 and json.loads(lines[0])["output_ids"] == plain_models["A"].greedy(prompt, 5)
+    assert lines[1].startswith("Generated 5 tokens in ") and "tokens/s" in lines[1]
+    assert json.loads(lines[2])["tokens_generated"] == 5
+    code = cli.main(["--model", model_folders["A"], "--random-weights", "--seed", "3", "--prompt-len", "6",
+                     "--max-new-tokens", "4", "--temperature", "0.7", "--top-k", "20", "--top-p", "0.95",
+                     "--sample-seed", "1", "--num-pages", "32"])
+    assert code == 0 and len(json.loads(capsys.readouterr().out.splitlines()[0])["output_ids"]) == 4

@@ -1,0 +1,310 @@
+"""Each part alone against its plain formula, models whose order names a layer twice or shares a cache,
+and a toy mixer with state of its own that is registered, built and stepped from here without a change
+to the framework's files."""
+import math
+
+import pytest
+import torch
+
+from conftest import token_ids
+from plain import qwen3_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F64 = torch.float64
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    return (torch.randn(*shape, generator=torch.Generator().manual_seed(seed)) * scale).to(torch.bfloat16)
+
+
+def build_ctx(tensors, mode, positions=None):
+    from pulse_infer_amd.parts.base import BuildContext, Workspace
+    from pulse_infer_amd.weights import DictSource, TensorSpec, WeightLoader
+    expected = {n: TensorSpec(tuple(t.shape)) for n, t in tensors.items()}
+    loader = WeightLoader(DictSource(tensors), expected, mode, DEV)
+    act = torch.float32 if mode == "float32" else torch.bfloat16
+    return BuildContext(loader=loader, mode=mode, device=torch.device(DEV), act_dtype=act,
+                        workspace=Workspace(torch.device(DEV)), positions=positions or {})
+
+
+def step_ctx(build, positions, entry, tables, counts=None):
+    from pulse_infer_amd.parts.base import EntryMeta, StepContext
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    n_entries = max(entry) + 1
+    starts = [min(p for p, e in zip(positions, entry) if e == i) for i in range(n_entries)]
+    counts = [entry.count(i) for i in range(n_entries)]
+    first = [entry.index(i) for i in range(n_entries)]
+    metas = [EntryMeta(i, i, starts[i], counts[i], first[i]) for i in range(n_entries)]
+    return StepContext(num_tokens=len(positions), entries=metas, token_ids=i32([0] * len(positions)),
+                       positions=i32(positions), token_entry=i32(entry), entry_start=i32(starts),
+                       entry_count=i32(counts), entry_first_row=i32(first + [len(positions)]),
+                       entry_slot=i32(list(range(n_entries))), block_tables={0: i32(tables)},
+                       want_rows=i32([]), num_wanted=0, workspace=build.workspace,
+                       max_count=max(counts), max_context=max(positions) + 1)
+
+
+TOL = {"float32": dict(atol=3e-5, rtol=3e-5), "bfloat16": dict(atol=3e-2, rtol=3e-2)}
+
+
+@pytest.mark.parametrize("mode", ["float32", "bfloat16"])
+def test_norm_part(gpu, mode):
+    from pulse_infer_amd.parts.base import NORMS
+    w = (1 + 0.1 * rnd(70, seed=1).float()).to(torch.bfloat16)
+    build = build_ctx({"n.weight": w}, mode)
+    norm = NORMS.get("rmsnorm")({"size": 70, "eps": 1e-4}, "n", build)
+    h = torch.randn(5, 70, generator=torch.Generator().manual_seed(2)).to(DEV)
+    out = torch.empty(5, 70, dtype=build.act_dtype, device=DEV)
+    norm.apply(h, None, out)
+    assert torch.allclose(out.cpu().to(F64), P.rms_norm(h.cpu().to(F64), w.to(F64), 1e-4), **TOL[mode])
+
+
+@pytest.mark.parametrize("mode", ["float32", "bfloat16"])
+def test_feed_forward_part(gpu, mode):
+    from pulse_infer_amd.parts.base import FEED_FORWARDS
+    hidden, inter = 72, 200
+    ws = {"m.gate_proj.weight": rnd(inter, hidden, seed=3, scale=hidden ** -0.5),
+          "m.up_proj.weight": rnd(inter, hidden, seed=4, scale=hidden ** -0.5),
+          "m.down_proj.weight": rnd(hidden, inter, seed=5, scale=inter ** -0.5)}
+    build = build_ctx(ws, mode)
+    mlp = FEED_FORWARDS.get("gated_mlp")({"hidden_size": hidden, "intermediate_size": inter, "activation": "silu"}, "m", build)
+    x = rnd(9, hidden, seed=6).to(build.act_dtype).to(DEV)
+    ctx = step_ctx(build, list(range(9)), [0] * 9, [[0]])
+    out = mlp.forward(x, ctx)
+    want = P.gated_mlp(x.cpu().to(F64), *(ws[f"m.{n}_proj.weight"].to(F64) for n in ("gate", "up", "down")))
+    assert torch.allclose(out.cpu().to(F64), want, **TOL[mode])
+    with pytest.raises(ValueError, match="activation"):
+        FEED_FORWARDS.get("gated_mlp")({"hidden_size": hidden, "intermediate_size": inter, "activation": "relu"}, "m", build)
+
+
+@pytest.mark.parametrize("mode", ["float32", "bfloat16"])
+@pytest.mark.parametrize("variant", ["qwen", "half_partial_window", "no_position_no_norm"])
+def test_attention_part(gpu, mode, variant):
+    """The mixer alone over a cache it fills in two steps (a portion, then another portion and a single token
+    of a second request), against plain attention on the whole sequences."""
+    from pulse_infer_amd.parts.base import MIXERS, POSITIONS, PagedCacheView
+    hidden, nq, nkv, d, bs = 40, 6, 3, 16, 4
+    opts = {"qwen": dict(qk_norm=True, window=None, position="rope", rot=16, pairing="interleaved"),
+            "half_partial_window": dict(qk_norm=True, window=5, position="rope", rot=8, pairing="half"),
+            "no_position_no_norm": dict(qk_norm=False, window=None, position=None, rot=0, pairing="interleaved")}[variant]
+    ws = {"a.q_proj.weight": rnd(nq * d, hidden, seed=7, scale=hidden ** -0.5),
+          "a.k_proj.weight": rnd(nkv * d, hidden, seed=8, scale=hidden ** -0.5),
+          "a.v_proj.weight": rnd(nkv * d, hidden, seed=9, scale=hidden ** -0.5),
+          "a.o_proj.weight": rnd(hidden, nq * d, seed=10, scale=(nq * d) ** -0.5)}
+    if opts["qk_norm"]:
+        ws["a.q_norm.weight"] = (1 + 0.1 * rnd(d, seed=11).float()).to(torch.bfloat16)
+        ws["a.k_norm.weight"] = (1 + 0.1 * rnd(d, seed=12).float()).to(torch.bfloat16)
+    build = build_ctx(ws, mode)
+    theta, eps, scale = 3e3, 1e-5, 0.29
+    if opts["position"]:
+        build.positions["rope"] = POSITIONS.get("rope")(
+            {"theta": theta, "rotary_dim": opts["rot"], "head_dim": d, "pairing": opts["pairing"]}, build)
+    params = {"hidden_size": hidden, "num_heads": nq, "num_kv_heads": nkv, "head_dim": d, "qk_norm": opts["qk_norm"],
+              "qk_norm_eps": eps, "scale": scale, "window": opts["window"], "position": opts["position"]}
+    attn = MIXERS.get("attention")(params, "a", build)
+    spec = attn.cache_spec()
+    assert (spec.num_kv_heads, spec.head_dim, spec.window) == (nkv, d, opts["window"])
+    cache = PagedCacheView(0, torch.zeros(8, nkv, bs, d, dtype=build.act_dtype, device=DEV),
+                           torch.zeros(8, nkv, d, bs, dtype=build.act_dtype, device=DEV), bs)
+    xa, xb = rnd(11, hidden, seed=13), rnd(1, hidden, seed=14)
+    tables = [[5, 2, 7], [3, -1, -1]]
+    dev = lambda t: t.to(build.act_dtype).to(DEV)
+    out1 = attn.forward(dev(xa[:6]), step_ctx(build, list(range(6)), [0] * 6, tables[:1]), cache).clone()
+    out2 = attn.forward(dev(torch.cat([xa[6:], xb])), step_ctx(build, list(range(6, 11)) + [0], [0] * 5 + [1], tables), cache)
+    got = torch.cat([out1, out2]).cpu().to(F64)
+
+    def plain(x):
+        t = x.shape[0]
+        x = x.to(F64)
+        q = P.linear(x, ws["a.q_proj.weight"].to(F64)).view(t, nq, d)
+        k = P.linear(x, ws["a.k_proj.weight"].to(F64)).view(t, nkv, d)
+        v = P.linear(x, ws["a.v_proj.weight"].to(F64)).view(t, nkv, d)
+        if opts["qk_norm"]:
+            q, k = P.rms_norm(q, ws["a.q_norm.weight"].to(F64), eps), P.rms_norm(k, ws["a.k_norm.weight"].to(F64), eps)
+        if opts["position"]:
+            q, k = (P.rope(z, list(range(t)), theta, opts["rot"], opts["pairing"]) for z in (q, k))
+        o = P.causal_attention(q, k, v, scale, opts["window"])
+        return P.linear(o.reshape(t, nq * d), ws["a.o_proj.weight"].to(F64))
+
+    want = torch.cat([plain(xa), plain(xb)])
+    assert torch.allclose(got, want, **TOL[mode])
+
+
+# ----------------------------------------------------------------- toy parts
+def register_toys():
+    """A mixer with state of its own (a decayed running sum per request), a position encoding that adds
+    nothing, and an architecture that uses them beside ordinary attention layers."""
+    from pulse_infer_amd.cache import StateSpec
+    from pulse_infer_amd.config import Qwen3Config, register_architecture
+    from pulse_infer_amd.models.spec import LayerSpec, ModelSpec, PartSpec, RunSpec
+    from pulse_infer_amd.parts.base import MIXERS, Part
+    from pulse_infer_amd.weights import TensorSpec
+
+    @MIXERS.register("toy_running_sum", replace=True)
+    class RunningSum(Part):
+        """state <- decay * state + x_t, output_t = state W^T; the state lives in the request's slot."""
+
+        @classmethod
+        def weight_specs(cls, params):
+            return {"mix.weight": TensorSpec((params["hidden_size"], params["hidden_size"]), fan_in=params["hidden_size"])}
+
+        def __init__(self, params, prefix, build):
+            self.hidden, self.decay = params["hidden_size"], params["decay"]
+            self.weight = build.loader.get(f"{prefix}.mix.weight").float()
+            self.act = build.act_dtype
+
+        def cache_spec(self):
+            return StateSpec((self.hidden,), "float32")
+
+        def forward(self, x, ctx, cache):
+            out = torch.empty(x.shape[0], self.hidden, dtype=torch.float32, device=x.device)
+            for e in ctx.entries:
+                state = cache.state[e.slot]
+                if e.start == 0:
+                    state.zero_()                 # a request (re)starts: its slot may hold an older request's state
+                for row in range(e.first_row, e.first_row + e.count):
+                    state.mul_(self.decay).add_(x[row].float())
+                    out[row] = state @ self.weight.t()
+            return out.to(self.act)
+
+    class ToyConfig(Qwen3Config):
+        def model_spec(self):
+            base = super().model_spec()
+            layers = []
+            for i, layer in enumerate(base.layers):
+                if i % 2 == 1:
+                    mixer = PartSpec("toy_running_sum", {"hidden_size": self.hidden_size, "decay": 0.5, "prefix": "toy"})
+                    layer = LayerSpec(layer.prefix, mixer, layer.ffn, layer.norm, layer.block)
+                layers.append(layer)
+            base.layers = layers
+            base.architecture = "ToyForCausalLM"
+            return base
+
+    register_architecture("ToyForCausalLM", ToyConfig, replace=True)
+    return ToyConfig
+
+
+def plain_toy_logits(plain, ids, decay):
+    """The toy model with plain functions: odd layers use the running sum in place of attention."""
+    c, w = plain.c, plain.w
+    h = P.embedding(w["model.embed_tokens.weight"], ids)
+    pos = list(range(len(ids)))
+    for i in range(c["num_hidden_layers"]):
+        if i % 2 == 0:
+            h = plain.layer(h, i, pos)
+            continue
+        p = f"model.layers.{i}."
+        a = P.rms_norm(h, w[p + "input_layernorm.weight"], c["rms_norm_eps"])
+        state, rows = torch.zeros(h.shape[1], dtype=F64), []
+        for t in range(len(ids)):
+            state = decay * state + a[t]
+            rows.append(state @ w[p + "toy.mix.weight"].T)
+        h = h + torch.stack(rows)
+        m = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], c["rms_norm_eps"])
+        h = h + P.gated_mlp(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return P.linear(P.rms_norm(h, w["model.norm.weight"], c["rms_norm_eps"]), w["lm_head.weight"])
+
+
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped(gpu, tmp_path):
+    from conftest import TINY_B
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.weights import write_model_folder
+    from pulse_infer_amd.config import unregister_architecture
+    from pulse_infer_amd.parts.base import MIXERS
+    from test_gpu_model import close
+
+    toy_config = register_toys()
+    try:
+        cfg = toy_config.from_dict(dict(TINY_B, architectures=["ToyForCausalLM"], num_hidden_layers=4))
+        cfg.architecture = "ToyForCausalLM"
+        folder = write_model_folder(cfg, str(tmp_path / "toy"), seed=21)
+        plain = P.PlainQwen3.from_folder(folder)
+        _, model = load_model(folder, mode="float32")
+        assert type(model.blocks[1].mixer).__name__ == "RunningSum"
+        runner = ModelRunner(model, page_size=16, num_pages=16, max_requests=2)
+        assert len(runner.cache.groups) == 1 and sorted(runner.cache.state_runs) == [1, 3]
+        ids = {k: token_ids(cfg.vocab_size, n, seed=60 + n) for k, n in (("a", 40), ("b", 23), ("c", 31))}
+        got = {k: [] for k in ids}
+        # a and b interleaved (portions beside single tokens); c afterwards in b's slot, whose state must not leak
+        plan = [[("a", 7), ("b", 2)], [("a", 1), ("b", 9)], [("b", 1)], [("a", 20), ("b", 11)], [("a", 12)],
+                [("c", 5)], [("c", 26)]]
+        fed = {k: 0 for k in ids}
+        for step in plan:
+            entries = []
+            for k, n in step:
+                if not runner.cache.has_request(k):
+                    runner.add_request(k)
+                runner.reserve(k, fed[k] + n)
+                entries.append(StepEntry(k, ids[k][fed[k]:fed[k] + n], list(range(n))))
+                fed[k] += n
+            logits = runner.step(entries)
+            row = 0
+            for k, n in step:
+                got[k].append(logits[row:row + n])
+                row += n
+            for k, _ in step:
+                if fed[k] == len(ids[k]) and runner.cache.has_request(k):
+                    runner.free_request(k)
+        for k in ids:
+            close(torch.cat(got[k]), plain_toy_logits(plain, ids[k], 0.5), "float32", f"toy request {k}")
+    finally:
+        unregister_architecture("ToyForCausalLM")
+        MIXERS.unregister("toy_running_sum")
+
+
+def test_order_may_name_a_layer_twice_and_share_a_cache(gpu, tmp_path):
+    """Run order [0, 1, 0(shares nothing), 2 reading run 1's cache]: weights of layer 0 are used twice with a
+    cache each; the last run computes only queries and attends to what run 1 wrote."""
+    from conftest import TINY_A
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.causal_lm import CausalLM
+    from pulse_infer_amd.models.spec import RunSpec
+    from pulse_infer_amd.weights import SafetensorsSource, write_model_folder
+    from test_gpu_model import close
+
+    cfg = Qwen3Config.from_dict(dict(TINY_A, num_hidden_layers=3))
+    folder = write_model_folder(cfg, str(tmp_path / "m"), seed=31)
+    spec = cfg.model_spec()
+    spec.order = [RunSpec(0), RunSpec(1), RunSpec(0), RunSpec(2, cache_of=1)]
+    model = CausalLM(spec, SafetensorsSource(folder), mode="float32")
+    runner = ModelRunner(model, page_size=4, num_pages=32, max_requests=2)
+    assert len(runner.cache.groups[0].runs) == 3          # three runs own pages, the fourth borrows
+    ids = token_ids(cfg.vocab_size, 30, seed=9)
+    runner.add_request("r")
+    outs, fed = [], 0
+    for n in (11, 1, 1, 17):
+        runner.reserve("r", fed + n)
+        outs.append(runner.step([StepEntry("r", ids[fed:fed + n], list(range(n)))]))
+        fed += n
+
+    plain = P.PlainQwen3.from_folder(folder)
+    c, w = plain.c, plain.w
+    pos = list(range(30))
+    h = P.embedding(w["model.embed_tokens.weight"], ids)
+    h = plain.layer(h, 0, pos)
+    # layer 1, keeping its rotated keys and its values for the sharing run
+    nq, nkv, d, eps = c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"], c["rms_norm_eps"]
+    a = P.rms_norm(h, w["model.layers.1.input_layernorm.weight"], eps)
+    k1 = P.rope(P.rms_norm(P.linear(a, w["model.layers.1.self_attn.k_proj.weight"]).view(30, nkv, d),
+                           w["model.layers.1.self_attn.k_norm.weight"], eps), pos, c["rope_theta"])
+    v1 = P.linear(a, w["model.layers.1.self_attn.v_proj.weight"]).view(30, nkv, d)
+    h = plain.layer(h, 1, pos)
+    h = plain.layer(h, 0, pos)
+    p = "model.layers.2."
+    a = P.rms_norm(h, w[p + "input_layernorm.weight"], eps)
+    q = P.rope(P.rms_norm(P.linear(a, w[p + "self_attn.q_proj.weight"]).view(30, nq, d), w[p + "self_attn.q_norm.weight"], eps),
+               pos, c["rope_theta"])
+    o = P.causal_attention(q, k1, v1, d ** -0.5)
+    h = h + P.linear(o.reshape(30, nq * d), w[p + "self_attn.o_proj.weight"])
+    m = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)
+    h = h + P.gated_mlp(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    want = P.linear(P.rms_norm(h, w["model.norm.weight"], eps), w["model.embed_tokens.weight"])
+    close(torch.cat(outs), want, "float32", "shared order")
