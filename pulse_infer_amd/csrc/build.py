@@ -17,7 +17,7 @@ import tempfile
 import threading
 import time
 from concurrent.futures import ThreadPoolExecutor
-from typing import List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ARCH = "gfx950"
@@ -29,6 +29,9 @@ COMMON_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
 ]
+
+
+VARIANT_DIR = os.path.join(HERE, "variants")
 
 
 def sources() -> List[str]:
@@ -144,6 +147,77 @@ def build(force: bool = False, verbose: bool = True) -> str:
         os.replace(tmp, lib)
         with open(stamp, "w") as fh:
             fh.write(source_hash())
+    finally:
+        done.set()
+    if verbose:
+        _log(f"built {lib} in {time.time() - t0:.0f} s")
+    return lib
+
+
+# ------------------------------------------------------------------ variants
+# A variant is one source of csrc/variants compiled with its own -D definitions into a library of
+# its own, e.g. the matrix-core attention for one head size.  Only what a model needs is compiled.
+def variant_name(source: str, defines: Dict[str, int]) -> str:
+    tail = "_".join(f"{k.lower()}{v}" for k, v in sorted(defines.items()))
+    return f"libpulse_{source}_{tail}.so" if tail else f"libpulse_{source}.so"
+
+
+def variant_hash(source: str, defines: Dict[str, int]) -> str:
+    h = hashlib.sha256()
+    h.update(" ".join(COMMON_FLAGS).encode())
+    h.update(repr(sorted(defines.items())).encode())
+    for path in [os.path.join(VARIANT_DIR, source + ".hip")] + [os.path.join(HERE, f) for f in headers()]:
+        with open(path, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def existing_variant(source: str, defines: Dict[str, int]) -> Optional[str]:
+    want, name = variant_hash(source, defines), variant_name(source, defines)
+    for d in build_dirs():
+        lib, stamp = os.path.join(d, name), os.path.join(d, name + ".stamp")
+        try:
+            if os.path.exists(lib) and open(stamp).read().strip() == want:
+                return lib
+        except OSError:
+            continue
+    return None
+
+
+def build_variant(source: str, defines: Dict[str, int], force: bool = False, verbose: bool = True) -> str:
+    if not force:
+        lib = existing_variant(source, defines)
+        if lib:
+            return lib
+    hipcc = find_hipcc()
+    out_dir = next((d for d in build_dirs() if _writable(d)), None)
+    if out_dir is None:
+        raise RuntimeError(f"no writable build folder among {build_dirs()}")
+    name = variant_name(source, defines)
+    lib, stamp = os.path.join(out_dir, name), os.path.join(out_dir, name + ".stamp")
+    if os.path.exists(stamp):
+        os.remove(stamp)
+    t0 = time.time()
+    if verbose:
+        _log(f"compiling {source}.hip {defines} for {ARCH}")
+    done = threading.Event()
+
+    def ticker() -> None:
+        while not done.wait(10.0):
+            _log(f"still compiling {name} ... {time.time() - t0:.0f} s")
+
+    if verbose:
+        threading.Thread(target=ticker, daemon=True).start()
+    try:
+        tmp = lib + f".tmp{os.getpid()}"
+        cmd = [hipcc, *COMMON_FLAGS, "-shared", *[f"-D{k}={v}" for k, v in sorted(defines.items())],
+               os.path.join(VARIANT_DIR, source + ".hip"), os.path.join(HERE, "error_text.hip"), "-o", tmp]
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {source}.hip {defines}:\n{proc.stderr[-4000:]}")
+        os.replace(tmp, lib)
+        with open(stamp, "w") as fh:
+            fh.write(variant_hash(source, defines))
     finally:
         done.set()
     if verbose:

@@ -4,20 +4,6 @@
 // angle float64); storage types are template arguments.
 #include "common.h"
 
-#include <cstdarg>
-#include <cstdio>
-
-// ---------------------------------------------------------------- error text
-static thread_local char g_error[512] = "";
-
-extern "C" const char* pulse_last_error() { return g_error; }
-
-void pulse_set_error(const char* fmt, ...) {
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(g_error, sizeof(g_error), fmt, ap);
-    va_end(ap);
-}
 
 // ------------------------------------------------------------------ embedding
 // out[t, :] = table[ids[t], :] widened to float32 (the residual stream).

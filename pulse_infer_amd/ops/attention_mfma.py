@@ -1,0 +1,80 @@
+"""The matrix-core attention kernel (bfloat16), one compiled library per head size."""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from .kernels import _check_cache, _f32, _gpu, _i32, _i64, _int_vec, _need, _ptr, _stream
+from .library import call_in, load_variant
+
+MAX_HEAD_DIM = 224
+BLOCK_KEYS = 32
+
+
+def supported(head_dim: int, page_size: int, dtype: torch.dtype, cache_dtype: torch.dtype) -> bool:
+    """Sizes the kernel takes; anything else goes to the generic kernel."""
+    return (dtype == torch.bfloat16 and cache_dtype == torch.bfloat16 and head_dim % 16 == 0
+            and 16 <= head_dim <= MAX_HEAD_DIM and page_size % 16 == 0)
+
+
+def tokens_per_item(group: int) -> int:
+    """How many consecutive tokens of a request share one work item (16 columns / heads per kv head)."""
+    gp = 1
+    while gp < group and gp < 16:
+        gp *= 2
+    return 16 // gp
+
+
+def build_items(entries: Sequence, tokens_per: int) -> List[int]:
+    """Flat [first row, token count] pairs covering every entry of a step."""
+    flat: List[int] = []
+    for e in entries:
+        for b in range(0, e.count, tokens_per):
+            flat.extend((e.first_row + b, min(tokens_per, e.count - b)))
+    return flat
+
+
+def choose_splits(num_items: int, nkv: int, group: int, max_context: int, target_groups: int = 1024) -> Tuple[int, int]:
+    """(split_size, n_splits): enough workgroups to fill the chip, whole contexts when there are plenty already."""
+    groups = num_items * nkv * ((group + 15) // 16)
+    whole = (max_context + BLOCK_KEYS - 1) // BLOCK_KEYS * BLOCK_KEYS
+    if groups * 2 > target_groups:
+        return whole, 1
+    want = (target_groups + groups - 1) // groups
+    size = (max_context + want - 1) // want
+    size = max(128, (size + BLOCK_KEYS - 1) // BLOCK_KEYS * BLOCK_KEYS)
+    if size >= whole:
+        return whole, 1
+    return size, (max_context + size - 1) // size
+
+
+def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
+              vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
+              items: torch.Tensor, scale: float, window: int, split_size: int, n_splits: int, max_context: int,
+              part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor]) -> None:
+    _gpu("attn_mfma", q, out, kcache, vcache, positions, token_entry, block_table, items, part_o, part_ml)
+    tokens = q.shape[0]
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.stride(1) == 1 and out.stride(1) == 1,
+          "attn_mfma: q and out must be bfloat16 matrices with contiguous rows")
+    _need(q.shape[1] >= nq * d and out.shape[1] >= nq * d and out.shape[0] == tokens, "attn_mfma: q/out too narrow")
+    pages, page_size = _check_cache("attn_mfma", kcache, vcache, nkv, d)
+    _need(supported(d, page_size, q.dtype, kcache.dtype), f"attn_mfma: head size {d} / page size {page_size} / "
+          f"{kcache.dtype} is not supported by the matrix-core kernel")
+    _int_vec("attn_mfma: positions", positions, tokens)
+    _int_vec("attn_mfma: token_entry", token_entry, tokens)
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+          "attn_mfma: block_table must be contiguous int32 [entries, width]")
+    _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() % 2 == 0, "attn_mfma: items must be int32 pairs")
+    n_items = items.numel() // 2
+    if n_splits > 1:
+        need = tokens * nq * n_splits
+        _need(part_o is not None and part_ml is not None and part_o.dtype == torch.float32
+              and part_ml.dtype == torch.float32 and part_o.numel() >= need * d and part_ml.numel() >= need * 2,
+              "attn_mfma: scratch for the split results is too small")
+    lib = load_variant("attn_mfma", {"PULSE_HEAD_DIM": d})
+    call_in(lib, "pulse_attn_mfma", _ptr(q), _i64(q.stride(0)), _ptr(out), _i64(out.stride(0)), _ptr(kcache),
+            _ptr(vcache), _ptr(positions), _ptr(token_entry), _ptr(block_table), _i32(block_table.shape[1]),
+            _ptr(items), _i32(n_items), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages), _f32(scale),
+            _i32(window), _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml), _stream())

@@ -49,6 +49,37 @@ def load() -> ctypes.CDLL:
         return lib
 
 
+_variants: dict = {}
+
+
+def load_variant(source: str, defines: dict) -> ctypes.CDLL:
+    """A library compiled from csrc/variants/<source>.hip with the given -D definitions (built on first use)."""
+    key = (source, tuple(sorted(defines.items())))
+    lib = _variants.get(key)
+    if lib is not None:
+        return lib
+    with _lock:
+        lib = _variants.get(key)
+        if lib is not None:
+            return lib
+        try:
+            path = _build.existing_variant(source, defines) or _build.build_variant(source, defines)
+            lib = ctypes.CDLL(path)
+        except Exception as exc:  # noqa: BLE001
+            raise KernelLibraryError(f"the HIP kernel variant {source} {defines} is not available: {exc}") from exc
+        lib.pulse_last_error.restype = ctypes.c_char_p
+        _variants[key] = lib
+        return lib
+
+
+def call_in(lib: ctypes.CDLL, name: str, *args) -> None:
+    fn = getattr(lib, name)
+    fn.restype = ctypes.c_int
+    code = fn(*args)
+    if code != 0:
+        raise KernelError(f"{name}: {lib.pulse_last_error().decode(errors='replace')}")
+
+
 def call(name: str, *args) -> None:
     """Call an entry point; a non-zero return becomes a ``KernelError`` with the library's message."""
     lib = load()

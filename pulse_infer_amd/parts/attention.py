@@ -19,7 +19,7 @@ from typing import Any, Dict, Optional
 import torch
 
 from ..cache.manager import PagedKVSpec
-from ..ops import kernels
+from ..ops import attention_mfma, kernels
 from ..weights.store import TensorSpec
 from .base import MIXERS, BuildContext, PagedCacheView, Part, StepContext
 from .linear import Linear
@@ -93,5 +93,26 @@ class PagedAttention(Part):
 
     def attend(self, q: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: PagedCacheView,
                table: torch.Tensor) -> None:
-        kernels.attn_generic(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
-                             ctx.token_entry, table, self.scale, int(self.window) if self.window is not None else 0)
+        window = int(self.window) if self.window is not None else 0
+        use_mfma = (self.options.get("attention", "auto") != "generic"
+                    and attention_mfma.supported(self.d, cache.page_size, q.dtype, cache.keys.dtype))
+        if not use_mfma:
+            kernels.attn_generic(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
+                                 ctx.token_entry, table, self.scale, window)
+            return
+        group = self.nq // self.nkv
+        per = attention_mfma.tokens_per_item(group)
+        key = f"attention.items:{per}"
+        if key not in ctx.extras:  # the same list serves every layer of the step with this grouping
+            flat = attention_mfma.build_items(ctx.entries, per)
+            ctx.extras[key] = torch.tensor(flat, dtype=torch.int32, device=q.device)
+        items = ctx.extras[key]
+        split_size, n_splits = attention_mfma.choose_splits(items.numel() // 2, self.nkv, group, ctx.max_context)
+        part_o = part_ml = None
+        if n_splits > 1:
+            rows = ctx.num_tokens * self.nq * n_splits
+            part_o = ctx.workspace.buffer("attention.part_o", rows, self.d, torch.float32)
+            part_ml = ctx.workspace.buffer("attention.part_ml", rows, 2, torch.float32)
+        attention_mfma.attn_mfma(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
+                                 ctx.token_entry, table, items, self.scale, window, split_size, n_splits,
+                                 ctx.max_context, part_o, part_ml)

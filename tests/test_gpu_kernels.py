@@ -350,3 +350,85 @@ def test_kernels_refuse_what_they_cannot_do(k):
         k.attn_generic(torch.zeros(1, 1024, device=DEV), torch.zeros(1, 1024, device=DEV), 1, 1, 1024, kc, vc,
                        torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
                        torch.zeros(1, 1, dtype=torch.int32, device=DEV), 1.0)
+
+
+# ------------------------------------------------------- matrix-core attention
+def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0):
+    """Requests with contexts `lens`; request 0 brings its last `portion` tokens, the others one token each."""
+    from pulse_infer_amd.ops import attention_mfma as M
+    dtype = torch.bfloat16
+    pages_per = [(n + bs - 1) // bs for n in lens]
+    total = sum(pages_per) + 3
+    perm = torch.randperm(total, generator=torch.Generator().manual_seed(seed)).tolist()
+    kc, vc = _cache(total, nkv, bs, d, dtype)
+    kc.normal_()                      # stale data everywhere, as in pages that are used again
+    vc.normal_()
+    width = max(pages_per)
+    table = torch.full((len(lens), width), -1, dtype=torch.int32)
+    refs, start = [], 0
+    for r, n in enumerate(lens):
+        pages = perm[start:start + pages_per[r]]
+        start += pages_per[r]
+        table[r, :len(pages)] = torch.tensor(pages, dtype=torch.int32)
+        ks, kref = as_stored(rnd(n, nkv, d, seed=100 + 7 * r + seed), dtype)
+        vs, vref = as_stored(rnd(n, nkv, d, seed=200 + 7 * r + seed), dtype)
+        _fill_cache(kc, vc, ks, vs, pages, bs)
+        refs.append((kref, vref))
+    positions = list(range(lens[0] - portion, lens[0])) + [n - 1 for n in lens[1:]]
+    entry = [0] * portion + list(range(1, len(lens)))
+
+    class E:  # what build_items needs of an entry
+        def __init__(self, first_row, count):
+            self.first_row, self.count = first_row, count
+    entries = [E(0, portion)] + [E(portion + i, 1) for i in range(len(lens) - 1)]
+    group = nq // nkv
+    items = torch.tensor(M.build_items(entries, M.tokens_per_item(group)), dtype=torch.int32, device=DEV)
+    q, qref = as_stored(rnd(len(positions), (nq + 2 * nkv) * d, seed=300 + seed), dtype)
+    out = torch.zeros(len(positions), nq * d, dtype=dtype, device=DEV)
+    max_ctx = max(lens)
+    if split is None:
+        split_size, n_splits = M.choose_splits(items.numel() // 2, nkv, group, max_ctx)
+    else:
+        split_size, n_splits = split, (max_ctx + split - 1) // split
+    rows = len(positions) * nq * n_splits
+    part_o = torch.full((rows, d), float("nan"), device=DEV)
+    part_ml = torch.full((rows, 2), float("nan"), device=DEV)
+    scale = d ** -0.5
+    M.attn_mfma(q, out, nq, nkv, d, kc, vc, torch.tensor(positions, dtype=torch.int32, device=DEV),
+                torch.tensor(entry, dtype=torch.int32, device=DEV), table.to(DEV), items, scale, window, split_size,
+                n_splits, max_ctx, part_o, part_ml)
+    got = out.cpu().to(F64).reshape(-1, nq, d)
+    for t, (p, e) in enumerate(zip(positions, entry)):
+        kref, vref = refs[e]
+        want = P.causal_attention(qref[t:t + 1, :nq * d].reshape(1, nq, d), kref[:p + 1], vref[:p + 1], scale,
+                                  window or None, [p])
+        assert torch.allclose(got[t], want[0], atol=2e-2, rtol=2e-2), (t, p, e, float((got[t] - want[0]).abs().max()))
+
+
+@pytest.mark.parametrize("case", [
+    dict(nq=4, nkv=2, d=16, bs=16, window=0, lens=[70, 131, 33], portion=9),
+    dict(nq=6, nkv=1, d=32, bs=16, window=0, lens=[150, 1, 64, 65], portion=70),      # 6 heads: 8 columns a token
+    dict(nq=6, nkv=3, d=48, bs=32, window=24, lens=[170, 90, 24, 25], portion=40),     # window, head size 48
+    dict(nq=32, nkv=8, d=128, bs=16, window=0, lens=[300, 513, 512, 31], portion=37),
+    dict(nq=3, nkv=3, d=80, bs=16, window=0, lens=[97, 40], portion=1),                # no grouping: 16 tokens an item
+    dict(nq=40, nkv=2, d=64, bs=64, window=0, lens=[200, 77], portion=5),              # 20 heads a kv head: two chunks
+    dict(nq=16, nkv=1, d=224, bs=16, window=100, lens=[260, 130], portion=18),
+])
+@pytest.mark.parametrize("split", [None, 32, 128])
+def test_attn_mfma(k, case, split):
+    _mfma_case(k, split=split, **case)
+
+
+def test_attn_mfma_refuses_other_sizes(k):
+    from pulse_infer_amd.ops import KernelError
+    from pulse_infer_amd.ops import attention_mfma as M
+    assert not M.supported(40, 16, torch.bfloat16, torch.bfloat16)       # head size no multiple of 16
+    assert not M.supported(64, 8, torch.bfloat16, torch.bfloat16)        # pages shorter than a key tile
+    assert not M.supported(64, 16, torch.float32, torch.float32)         # the 32-bit path has its own kernel
+    assert not M.supported(256, 16, torch.bfloat16, torch.bfloat16)
+    kc, vc = _cache(2, 1, 8, 64, torch.bfloat16)
+    z = torch.zeros(1, dtype=torch.int32, device=DEV)
+    with pytest.raises(KernelError, match="not supported"):
+        M.attn_mfma(torch.zeros(1, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(1, 64, dtype=torch.bfloat16, device=DEV),
+                    1, 1, 64, kc, vc, z, z, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+                    torch.tensor([0, 1], dtype=torch.int32, device=DEV), 1.0, 0, 32, 1, 1, None, None)

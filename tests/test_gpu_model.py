@@ -39,11 +39,11 @@ def engines(model_folders):
 
     made = {}
 
-    def get(name, dtype, tokens=256):
-        key = (name, dtype)
+    def get(name, dtype, page=None, tokens=256):
+        page = page or TINY[name][1]
+        key = (name, dtype, page)
         if key not in made:
             _, model = load_model(model_folders[name], mode=dtype)
-            page = TINY[name][1]
             made[key] = ModelRunner(model, page_size=page, num_pages=tokens // page, max_requests=4)
         return made[key]
 
@@ -67,15 +67,18 @@ def run_alone(runner, ids, cuts, rid="r"):
 
 
 LENGTH = {"A": 100, "B": 150, "W": 170}
+# (configuration, page size): each configuration's own small page and pages of 16 and more, which in bfloat16
+# take the matrix-core attention kernel
+CASES = [("A", 4), ("A", 16), ("B", 16), ("B", 64), ("W", 8), ("W", 16)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "W"])
-def test_whole_tail_and_portions(engines, plain_logits, name, dtype):
+@pytest.mark.parametrize("name,page", CASES)
+def test_whole_tail_and_portions(engines, plain_logits, name, page, dtype):
     cfg = TINY[name][0]
     ids = token_ids(cfg["vocab_size"], LENGTH[name], seed=3)
     want = plain_logits(name, ids)
-    runner = engines(name, dtype)
+    runner = engines(name, dtype, page)
     whole = run_alone(runner, ids, [len(ids)])
     close(whole, want, dtype, f"{name} whole")
     tail = run_alone(runner, ids, [len(ids) - 32] + [1] * 32)
@@ -130,13 +133,13 @@ def mixed_trace(vocab, seed):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "W"])
-def test_mixed_batches_with_page_reuse(engines, plain_logits, name, dtype):
+@pytest.mark.parametrize("name,page", CASES)
+def test_mixed_batches_with_page_reuse(engines, plain_logits, name, page, dtype):
     from pulse_infer_amd.engine.runner import StepEntry
 
     cfg = TINY[name][0]
     ids, steps = mixed_trace(cfg["vocab_size"], seed=5)
-    runner = engines(name, dtype)
+    runner = engines(name, dtype, page)
     got = {k: [] for k in ids}
     pages_seen = {}
     most_live = 0
