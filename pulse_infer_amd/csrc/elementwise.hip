@@ -71,6 +71,67 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
     }
 }
 
+// The same for rows of up to 256 * 4 * RMS_CHUNKS values with hidden % 4 == 0: one pass, the row held in
+// registers, 16-byte accesses.  Few rows (decoding) are bound by latency, and this halves the dependent loads.
+constexpr int RMS_CHUNKS = 8;
+
+template <typename T> struct Vec4;
+template <> struct Vec4<float> { typedef float4 type; };
+template <> struct Vec4<bf16_t> { typedef ushort4 type; };
+
+__device__ __forceinline__ float4 widen4(float4 v) { return v; }
+__device__ __forceinline__ float4 widen4(ushort4 v) {
+    return make_float4(bf16_to_f32(v.x), bf16_to_f32(v.y), bf16_to_f32(v.z), bf16_to_f32(v.w));
+}
+template <typename T> __device__ __forceinline__ typename Vec4<T>::type narrow4(float4 v);
+template <> __device__ __forceinline__ float4 narrow4<float>(float4 v) { return v; }
+template <> __device__ __forceinline__ ushort4 narrow4<bf16_t>(float4 v) {
+    return make_ushort4(f32_to_bf16(v.x), f32_to_bf16(v.y), f32_to_bf16(v.z), f32_to_bf16(v.w));
+}
+
+template <typename TD, typename TW, typename TY>
+__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                              const int* __restrict__ rows, const TW* __restrict__ w,
+                                                              TY* __restrict__ y, int hidden, float eps, int write_back) {
+    __shared__ float scratch[16];
+    typedef typename Vec4<TD>::type VD;
+    typedef typename Vec4<TW>::type VW;
+    typedef typename Vec4<TY>::type VY;
+    const int r = blockIdx.x;
+    const int64_t s = rows ? rows[r] : r;
+    const int nvec = hidden / 4;
+    float4* hrow = reinterpret_cast<float4*>(h + s * hidden);
+    const VD* drow = delta ? reinterpret_cast<const VD*>(delta + s * hidden) : nullptr;
+    float4 v[RMS_CHUNKS];
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < RMS_CHUNKS; ++c) {
+        const int i = threadIdx.x + c * 256;
+        if (i < nvec) {
+            v[c] = hrow[i];
+            if (drow) {
+                const float4 d = widen4(drow[i]);
+                v[c].x += d.x; v[c].y += d.y; v[c].z += d.z; v[c].w += d.w;
+            }
+            ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(hidden) + eps);
+    VY* yrow = reinterpret_cast<VY*>(y + static_cast<int64_t>(r) * hidden);
+    const VW* wv = reinterpret_cast<const VW*>(w);
+#pragma unroll
+    for (int c = 0; c < RMS_CHUNKS; ++c) {
+        const int i = threadIdx.x + c * 256;
+        if (i < nvec) {
+            if (write_back) hrow[i] = v[c];
+            const float4 ww = widen4(wv[i]);
+            yrow[i] = narrow4<TY>(make_float4(v[c].x * inv * ww.x, v[c].y * inv * ww.y, v[c].z * inv * ww.z,
+                                              v[c].w * inv * ww.w));
+        }
+    }
+}
+
 extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, const int* rows,
                                  const void* w, int w_dtype, void* y, int y_dtype, int out_rows,
                                  int hidden, float eps, int write_back, hipStream_t stream) {
@@ -80,10 +141,19 @@ extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, c
     PULSE_REQUIRE(h && w && y, "add_rmsnorm: null pointer");
     PULSE_REQUIRE(!(rows && write_back), "add_rmsnorm: write_back with gathered rows is not supported");
     if (out_rows == 0) return 0;
-    PULSE_DISPATCH_DTYPE(delta_dtype, TD, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(y_dtype, TY,
-        hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, TY>), dim3(out_rows), dim3(256), 0, stream, h,
-                           static_cast<const TD*>(delta), rows, static_cast<const TW*>(w),
-                           static_cast<TY*>(y), hidden, eps, write_back))));
+    const bool aligned = (reinterpret_cast<uintptr_t>(h) % 16 == 0) && (reinterpret_cast<uintptr_t>(y) % 16 == 0) &&
+                         (reinterpret_cast<uintptr_t>(w) % 16 == 0) && (reinterpret_cast<uintptr_t>(delta) % 16 == 0);
+    if (hidden % 4 == 0 && hidden <= 256 * 4 * RMS_CHUNKS && aligned) {
+        PULSE_DISPATCH_DTYPE(delta_dtype, TD, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(y_dtype, TY,
+            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY>), dim3(out_rows), dim3(256), 0, stream, h,
+                               static_cast<const TD*>(delta), rows, static_cast<const TW*>(w),
+                               static_cast<TY*>(y), hidden, eps, write_back))));
+    } else {
+        PULSE_DISPATCH_DTYPE(delta_dtype, TD, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(y_dtype, TY,
+            hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, TY>), dim3(out_rows), dim3(256), 0, stream, h,
+                               static_cast<const TD*>(delta), rows, static_cast<const TW*>(w),
+                               static_cast<TY*>(y), hidden, eps, write_back))));
+    }
     PULSE_LAUNCH_CHECK("add_rmsnorm");
     return 0;
 }
@@ -109,31 +179,35 @@ extern "C" int pulse_residual_add(float* h, const void* delta, int delta_dtype, 
 }
 
 // --------------------------------------------------------------------- SwiGLU
-// gu is [T, 2*I]: gate in columns [0, I), up in [I, 2I).  out[t, i] = silu(g) * u,
-// silu(x) = x / (1 + exp(-x)), product in float32, one rounding.
+// gu is [T, 2*I].  slab == 0: gate in columns [0, I), up in [I, 2I).  slab > 0: gate and up alternate in
+// slabs of `slab` columns (gate slab, up slab, ...), the layout of a slab-interleaved weight.
+// out[t, i] = silu(g) * u, silu(x) = x / (1 + exp(-x)), product in float32, one rounding.
 // (reference: src/ops/kernels/cuda/silu_kernel.cu:82-97 then mul_kernel.cu:39-46, two roundings)
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int64_t total) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int slab, int64_t total) {
     const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int64_t t = idx / inter;
     const int i = static_cast<int>(idx - t * inter);
     const T* row = gu + t * 2 * inter;
-    const float g = to_f32<T>(row[i]);
-    const float u = to_f32<T>(row[inter + i]);
+    const int gi = slab > 0 ? (i / slab) * 2 * slab + i % slab : i;
+    const int ui = slab > 0 ? gi + slab : inter + i;
+    const float g = to_f32<T>(row[gi]);
+    const float u = to_f32<T>(row[ui]);
     const float s = g / (1.0f + expf(-g));
     out[idx] = from_f32<T>(s * u);
 }
 
-extern "C" int pulse_swiglu(const void* gu, void* out, int dtype, int tokens, int inter, hipStream_t stream) {
+extern "C" int pulse_swiglu(const void* gu, void* out, int dtype, int tokens, int inter, int slab, hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && inter > 0 && pulse_dtype_ok(dtype) && gu && out, "swiglu: bad arguments");
+    PULSE_REQUIRE(slab >= 0 && (slab == 0 || inter % slab == 0), "swiglu: %d columns do not divide into slabs of %d", inter, slab);
     const int64_t total = static_cast<int64_t>(tokens) * inter;
     if (total == 0) return 0;
     const int64_t blocks = (total + 255) / 256;
     PULSE_REQUIRE(blocks < (1ll << 31), "swiglu: too many elements");
     PULSE_DISPATCH_DTYPE(dtype, T,
         hipLaunchKernelGGL(swiglu_kernel<T>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
-                           static_cast<const T*>(gu), static_cast<T*>(out), inter, total));
+                           static_cast<const T*>(gu), static_cast<T*>(out), inter, slab, total));
     PULSE_LAUNCH_CHECK("swiglu");
     return 0;
 }

@@ -272,29 +272,37 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_mfma_kernel(MfmaArgs a
     }
 }
 
-// out[row, head, :] = sum_z w_z o_z / sum_z w_z l_z with w_z = exp2(m_z - max m), over the splits that hold keys of the row.
-__global__ __launch_bounds__(64) void attn_mfma_reduce_kernel(const float* __restrict__ part_o,
-                                                              const float* __restrict__ part_ml,
-                                                              const int* __restrict__ positions, bf16_t* __restrict__ out,
-                                                              int64_t o_stride, int nq, int n_splits, int split_size) {
+// out[row, head, :] = sum_z w_z o_z / sum_z w_z l_z with w_z = exp2(m_z - max m), over the splits that hold keys of
+// the row.  One workgroup per (row, head); the splits' (m, l) pairs go through LDS so that the loads overlap.
+constexpr int MAX_SPLITS = 1024;
+
+__global__ __launch_bounds__(128) void attn_mfma_reduce_kernel(const float* __restrict__ part_o,
+                                                               const float* __restrict__ part_ml,
+                                                               const int* __restrict__ positions, bf16_t* __restrict__ out,
+                                                               int64_t o_stride, int nq, int n_splits, int split_size) {
+    __shared__ float s_w[MAX_SPLITS];
+    __shared__ float s_l[MAX_SPLITS];
     const int64_t row = blockIdx.x;
     const int head = blockIdx.y;
     const int valid = min(n_splits, positions[row] / split_size + 1);
     const int64_t base = (row * nq + head) * n_splits;
-    float mm = -INFINITY;
-    for (int z = 0; z < valid; ++z) mm = fmaxf(mm, part_ml[2 * (base + z)]);
-    float ll = 0.f;
-    for (int z = 0; z < valid; ++z) {
-        const float mz = part_ml[2 * (base + z)];
-        ll += (mz == -INFINITY ? 0.f : exp2f(mz - mm)) * part_ml[2 * (base + z) + 1];
+    for (int z = threadIdx.x; z < valid; z += blockDim.x) {
+        s_w[z] = part_ml[2 * (base + z)];
+        s_l[z] = part_ml[2 * (base + z) + 1];
     }
+    __syncthreads();
+    float mm = -INFINITY;
+    for (int z = 0; z < valid; ++z) mm = fmaxf(mm, s_w[z]);
+    float ll = 0.f;
+    for (int z = 0; z < valid; ++z) ll += (s_w[z] == -INFINITY ? 0.f : exp2f(s_w[z] - mm)) * s_l[z];
     const float inv = ll > 0.f ? 1.0f / ll : 0.f;
     bf16_t* dst = out + row * o_stride + static_cast<int64_t>(head) * D;
-    for (int ch = threadIdx.x; ch < D; ch += 64) {
+    for (int ch = threadIdx.x; ch < D; ch += blockDim.x) {
         float v = 0.f;
+#pragma unroll 4
         for (int z = 0; z < valid; ++z) {
-            const float mz = part_ml[2 * (base + z)];
-            if (mz != -INFINITY) v += exp2f(mz - mm) * part_o[(base + z) * D + ch];
+            const float wz = s_w[z] == -INFINITY ? 0.f : exp2f(s_w[z] - mm);
+            v += wz * part_o[(base + z) * D + ch];
         }
         dst[ch] = f32_to_bf16(v * inv);
     }
@@ -323,6 +331,7 @@ extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64
     PULSE_REQUIRE(static_cast<int64_t>(n_splits) * split_size >= max_context,
                   "attn_mfma: %d splits of %d keys do not cover a context of %d", n_splits, split_size, max_context);
     PULSE_REQUIRE(n_splits == 1 || (part_o && part_ml), "attn_mfma: scratch is missing");
+    PULSE_REQUIRE(n_splits <= MAX_SPLITS, "attn_mfma: at most %d splits, got %d", MAX_SPLITS, n_splits);
     PULSE_REQUIRE(n_splits < 65536 && static_cast<int64_t>(nkv) * ((nq / nkv + 15) / 16) < 65536, "attn_mfma: grid too large");
     PULSE_REQUIRE(q && out && kcache && vcache && positions && token_entry && block_table && items, "attn_mfma: null pointer");
     if (tokens == 0 || n_items == 0) return 0;
@@ -343,7 +352,7 @@ extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64
                        stream, a);
     PULSE_LAUNCH_CHECK("attn_mfma");
     if (n_splits > 1) {
-        hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(tokens, nq), dim3(64), 0, stream, part_o, part_ml, positions,
+        hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(tokens, nq), dim3(128), 0, stream, part_o, part_ml, positions,
                            a.out, o_stride, nq, n_splits, split_size);
         PULSE_LAUNCH_CHECK("attn_mfma_reduce");
     }

@@ -103,14 +103,15 @@ def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
     call("pulse_residual_add", _ptr(h), _ptr(delta), _i32(_tag(delta, "residual_add")), _i64(h.numel()), _stream())
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, slab: int = 0) -> None:
+    """out[t, i] = silu(gate) * up; gate_up holds [gate | up] halves (slab 0) or alternating slabs of ``slab`` columns."""
     _gpu("swiglu", gate_up, out)
     tokens, two_i = gate_up.shape
     _need(two_i % 2 == 0 and tuple(out.shape) == (tokens, two_i // 2), "swiglu: out must be [T, I] for gate_up [T, 2I]")
     _need(gate_up.is_contiguous() and out.is_contiguous() and gate_up.dtype == out.dtype,
           "swiglu: contiguous tensors of one storage type are needed")
-    call("pulse_swiglu", _ptr(gate_up), _ptr(out), _i32(_tag(out, "swiglu")), _i32(tokens), _i32(two_i // 2), _stream())
+    call("pulse_swiglu", _ptr(gate_up), _ptr(out), _i32(_tag(out, "swiglu")), _i32(tokens), _i32(two_i // 2),
+         _i32(slab), _stream())
 
 
 def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, cos_out: torch.Tensor, sin_out: torch.Tensor) -> None:
@@ -146,6 +147,47 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     call("pulse_gemm_f32", _ptr(a), _i32(_tag(a, "gemm_f32")), _ptr(w), _i32(_tag(w, "gemm_f32")), _ptr(out),
          _i32(_tag(out, "gemm_f32")), _i32(m), _i32(n), _i32(k), _i64(a.stride(0) if m > 1 else k),
          _i64(w.stride(0) if n > 1 else k), _i64(out.stride(0) if m > 1 else n), _stream())
+
+
+SKINNY_MAX_ROWS = 64
+SKINNY_SWIGLU_MAX_ROWS = 32
+_OUT_MODES = {"store": None, "add": 2}
+
+
+def gemm_skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the few-rows matrix-core product takes these operands."""
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and w.dim() == 2
+            and a.shape[0] <= SKINNY_MAX_ROWS and a.shape[1] % 8 == 0 and a.stride(1) == 1 and w.stride(1) == 1
+            and (a.shape[0] <= 1 or a.stride(0) % 8 == 0) and (w.shape[0] <= 1 or w.stride(0) % 8 == 0)
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool = False, swiglu: bool = False) -> None:
+    """out = a @ w^T for at most 64 rows of bfloat16, float32 accumulation on the matrix cores.
+
+    ``out`` bfloat16 or float32 is stored; with ``add`` (float32 only) the product is added to it.  With
+    ``swiglu`` the weight holds gate and up rows in alternating slabs of 16 and out is silu(gate) * up.
+    """
+    _gpu("gemm_skinny", a, w, out)
+    _need(gemm_skinny_ok(a, w), "gemm_skinny: needs bfloat16 operands with at most 64 rows, K a multiple of 8, "
+          "contiguous 16-byte aligned rows")
+    m, k = a.shape
+    n, k2 = w.shape
+    _need(k == k2, f"gemm_skinny: inner sizes differ: a is [{m}, {k}], w is [{n}, {k2}]")
+    cols = n // 2 if swiglu else n
+    _need(tuple(out.shape) == (m, cols) and out.stride(1) == 1, f"gemm_skinny: out must be [{m}, {cols}]")
+    if add:
+        _need(out.dtype == torch.float32 and not swiglu, "gemm_skinny: adding needs a float32 target")
+        mode = 2
+    else:
+        mode = 0 if out.dtype == torch.bfloat16 else 1
+        _need(out.dtype in (torch.bfloat16, torch.float32), "gemm_skinny: out must be bfloat16 or float32")
+    if swiglu:
+        _need(m <= SKINNY_SWIGLU_MAX_ROWS and n % 32 == 0 and out.dtype == torch.bfloat16,
+              "gemm_skinny: the SwiGLU epilogue needs at most 32 rows, N a multiple of 32 and bfloat16 output")
+    call("pulse_gemm_skinny", _ptr(a), _i64(a.stride(0) if m > 1 else k), _ptr(w), _i64(w.stride(0) if n > 1 else k),
+         _ptr(out), _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode),
+         _i32(1 if swiglu else 0), _stream())
 
 
 def _check_cache(what: str, kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, d: int):

@@ -71,7 +71,10 @@ class PagedAttention(Part):
     def cache_spec(self) -> PagedKVSpec:
         return PagedKVSpec(self.nkv, self.d, int(self.window) if self.window is not None else None)
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, cache: PagedCacheView) -> torch.Tensor:
+    accepts_residual = True
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: PagedCacheView,
+                residual: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         tokens = x.shape[0]
         ws = ctx.workspace
         write = cache.writable
@@ -89,6 +92,8 @@ class PagedAttention(Part):
         attn = ws.buffer("attention.out", tokens, q_cols, self.act_dtype)
         self.attend(qkv, attn, ctx, cache, table)
         out = ws.buffer("attention.proj", tokens, self.hidden, self.act_dtype)
+        if residual is not None:
+            return self.o.add_into(attn, residual, out)
         return self.o.forward(attn, out)
 
     def attend(self, q: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: PagedCacheView,

@@ -167,7 +167,10 @@ class ResidualStream:
         self.pending = None
         return out
 
-    def push(self, delta: torch.Tensor) -> None:
+    def push(self, delta: Optional[torch.Tensor]) -> None:
+        """Hand over an update; None means the part has already added it to ``h``."""
+        if delta is None:
+            return
         if self.pending is not None:
             from ..ops import kernels
             kernels.residual_add(self.h, self.pending)

@@ -48,6 +48,13 @@ class PreNormBlock(Part):
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: Any) -> None:
         x = ctx.workspace.buffer("block.normed", ctx.num_tokens, self.hidden, self.act_dtype)
         stream.normed(self.mixer_norm, x)
-        stream.push(self.mixer.forward(x, ctx, cache))
+        # a part that says so may add its result into the residual itself and return None
+        if getattr(self.mixer, "accepts_residual", False):
+            stream.push(self.mixer.forward(x, ctx, cache, residual=stream.h))
+        else:
+            stream.push(self.mixer.forward(x, ctx, cache))
         stream.normed(self.ffn_norm, x)
-        stream.push(self.ffn.forward(x, ctx))
+        if getattr(self.ffn, "accepts_residual", False):
+            stream.push(self.ffn.forward(x, ctx, residual=stream.h))
+        else:
+            stream.push(self.ffn.forward(x, ctx))

@@ -1,10 +1,14 @@
 """y = x W^T for a weight stored [out, in] (reference: src/layer/linear.cpp:213).
 
-In the bfloat16 run the product is the vendor library's (torch.matmul, i.e.
-hipBLASLt/rocBLAS, float32 accumulation), as the reference uses cuBLAS
-(src/ops/kernels/cuda/matmul_kernel.cu:132-154).  In the float32 run, for a
-weight kept in 32-bit, and wherever float32 results are asked of bfloat16
-operands, the product is this package's own fused-multiply-add kernel.
+Three products stand behind it:
+
+* few rows (decoding, short portions) of bfloat16: this package's weight-streaming
+  matrix-core kernel, which can also add into the float32 residual or apply SwiGLU;
+* many rows of bfloat16: the vendor library's product (torch.matmul, i.e.
+  hipBLASLt/rocBLAS, float32 accumulation), as the reference uses cuBLAS
+  (src/ops/kernels/cuda/matmul_kernel.cu:132-154);
+* the float32 run, and any weight kept in 32-bit: this package's own
+  fused-multiply-add kernel, with no reduced-precision mode anywhere.
 """
 from __future__ import annotations
 
@@ -25,10 +29,26 @@ class Linear:
         self.library = mode == "bfloat16" and weight.dtype == torch.bfloat16
 
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[int] = None) -> torch.Tensor:
-        """``out`` [M, out_features] receives the product; its storage type chooses the path."""
+        """``out`` [M, out_features] receives the product; its storage type is bfloat16 or float32."""
         w = self.weight if rows is None else self.weight[:rows]
-        if self.library and out.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
-            torch.matmul(x, w.t(), out=out)
-        else:
-            kernels.gemm_f32(x, w, out)
+        if self.library and x.dtype == torch.bfloat16:
+            if kernels.gemm_skinny_ok(x, w):
+                kernels.gemm_skinny(x, w, out)
+                return out
+            if out.dtype == torch.bfloat16:
+                torch.matmul(x, w.t(), out=out)
+                return out
+            if w.shape[1] % 8 == 0:  # float32 results of many rows: the few-rows kernel, 64 rows at a time
+                for r0 in range(0, x.shape[0], kernels.SKINNY_MAX_ROWS):
+                    kernels.gemm_skinny(x[r0:r0 + kernels.SKINNY_MAX_ROWS], w, out[r0:r0 + kernels.SKINNY_MAX_ROWS])
+                return out
+        kernels.gemm_f32(x, w, out)
         return out
+
+    def add_into(self, x: torch.Tensor, residual: torch.Tensor, scratch: torch.Tensor) -> Optional[torch.Tensor]:
+        """residual += x W^T where the kernel can do that itself (returns None); otherwise the product is
+        written to ``scratch`` and returned for the caller to add."""
+        if self.library and x.dtype == torch.bfloat16 and kernels.gemm_skinny_ok(x, self.weight):
+            kernels.gemm_skinny(x, self.weight, residual, add=True)
+            return None
+        return self.forward(x, scratch)

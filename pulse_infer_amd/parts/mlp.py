@@ -4,7 +4,7 @@ gate and up are one product with the row-stacked weight; activation and product 
 kernel in float32 with one rounding."""
 from __future__ import annotations
 
-from typing import Any, Dict
+from typing import Any, Dict, Optional
 
 import torch
 
@@ -12,6 +12,9 @@ from ..ops import kernels
 from ..weights.store import TensorSpec
 from .base import FEED_FORWARDS, BuildContext, Part, StepContext
 from .linear import Linear
+
+
+SLAB = 16  # rows of a weight slab of the few-rows product
 
 
 @FEED_FORWARDS.register("gated_mlp")
@@ -32,16 +35,33 @@ class GatedMLP(Part):
         if activation != "silu":
             raise ValueError(f"gated_mlp has no kernel for activation '{activation}' (only 'silu')")
         load = build.loader
-        self.gate_up = Linear(load.get_concat([f"{prefix}.gate_proj.weight", f"{prefix}.up_proj.weight"]), build.mode)
+        gate, up = load.get(f"{prefix}.gate_proj.weight"), load.get(f"{prefix}.up_proj.weight")
+        # gate and up rows alternate in slabs of 16 where the sizes allow it, so that one workgroup of the
+        # few-rows product holds a gate slab and its up slab and can apply SwiGLU itself (a layout choice)
+        self.slab = SLAB if (build.mode == "bfloat16" and gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16
+                             and self.inter % SLAB == 0) else 0
+        if self.slab:
+            stacked = torch.stack([gate.view(-1, SLAB, self.hidden), up.view(-1, SLAB, self.hidden)], dim=1)
+            self.gate_up = Linear(stacked.reshape(2 * self.inter, self.hidden).contiguous(), build.mode)
+        else:
+            self.gate_up = Linear(load.get_concat([f"{prefix}.gate_proj.weight", f"{prefix}.up_proj.weight"]), build.mode)
+        del gate, up
         self.down = Linear(load.get(f"{prefix}.down_proj.weight"), build.mode)
         self.act_dtype = build.act_dtype
 
-    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+    accepts_residual = True
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, residual: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         tokens = x.shape[0]
         ws = ctx.workspace
-        gu = ws.buffer("mlp.gate_up", tokens, 2 * self.inter, self.act_dtype)
-        self.gate_up.forward(x, gu)
         z = ws.buffer("mlp.act", tokens, self.inter, self.act_dtype)
-        kernels.swiglu(gu, z)
+        if (self.slab and tokens <= kernels.SKINNY_SWIGLU_MAX_ROWS and kernels.gemm_skinny_ok(x, self.gate_up.weight)):
+            kernels.gemm_skinny(x, self.gate_up.weight, z, swiglu=True)
+        else:
+            gu = ws.buffer("mlp.gate_up", tokens, 2 * self.inter, self.act_dtype)
+            self.gate_up.forward(x, gu)
+            kernels.swiglu(gu, z, slab=self.slab)
         out = ws.buffer("mlp.out", tokens, self.hidden, self.act_dtype)
+        if residual is not None:
+            return self.down.add_into(z, residual, out)
         return self.down.forward(z, out)

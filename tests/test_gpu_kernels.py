@@ -432,3 +432,62 @@ def test_attn_mfma_refuses_other_sizes(k):
         M.attn_mfma(torch.zeros(1, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(1, 64, dtype=torch.bfloat16, device=DEV),
                     1, 1, 64, kc, vc, z, z, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
                     torch.tensor([0, 1], dtype=torch.int32, device=DEV), 1.0, 0, 32, 1, 1, None, None)
+
+
+# ------------------------------------------------------------ few-rows product
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("n,kk", [(48, 64), (509, 96), (4096 + 16, 200), (96, 4096)])
+def test_gemm_skinny(k, m, n, kk):
+    a, aref = as_stored(rnd(m, kk, seed=70), torch.bfloat16)
+    w, wref = as_stored(rnd(n, kk, seed=71), torch.bfloat16)
+    want = aref @ wref.T
+    out32 = torch.empty(m, n, device=DEV)
+    k.gemm_skinny(a, w, out32)
+    assert torch.allclose(out32.cpu().to(F64), want, atol=2e-3 * math.sqrt(kk), rtol=1e-5)   # float32 sums of exact products
+    out16 = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+    k.gemm_skinny(a, w, out16)
+    assert torch.equal(out16, out32.to(torch.bfloat16))                # the same sums, rounded once
+    base = rnd(m, n, seed=72).to(DEV)
+    acc = base.clone()
+    k.gemm_skinny(a, w, acc, add=True)
+    assert torch.allclose(acc, base + out32, atol=1e-6, rtol=1e-6)
+    again = torch.empty(m, n, device=DEV)
+    k.gemm_skinny(a, w, again)
+    assert torch.equal(again, out32)                                   # the same from run to run
+    if m > 1:                                                          # strided rows (a view into a wider buffer)
+        wide = torch.zeros(m, kk + 24, dtype=torch.bfloat16, device=DEV)
+        wide[:, :kk] = a
+        k.gemm_skinny(wide[:, :kk], w, again)
+        assert torch.equal(again, out32)
+
+
+@pytest.mark.parametrize("m", [1, 8, 20, 32])
+@pytest.mark.parametrize("inter,kk", [(32, 64), (224, 96), (176, 80), (12288 // 8, 256)])
+def test_gemm_skinny_swiglu(k, m, inter, kk):
+    a, aref = as_stored(rnd(m, kk, seed=73), torch.bfloat16)
+    gate, gref = as_stored(rnd(inter, kk, seed=74, scale=kk ** -0.5), torch.bfloat16)
+    up, uref = as_stored(rnd(inter, kk, seed=75, scale=kk ** -0.5), torch.bfloat16)
+    mixed = torch.stack([gate.view(-1, 16, kk), up.view(-1, 16, kk)], dim=1).reshape(2 * inter, kk).contiguous()
+    out = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    k.gemm_skinny(a, mixed, out, swiglu=True)
+    want = P.silu(aref @ gref.T) * (aref @ uref.T)
+    assert torch.allclose(out.cpu().to(F64), want, atol=1e-2, rtol=1e-2)
+    # the unfused way over the same interleaved layout gives the same, up to the rounding of gate and up
+    gu = torch.empty(m, 2 * inter, dtype=torch.bfloat16, device=DEV)
+    k.gemm_skinny(a, mixed, gu)
+    z = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    k.swiglu(gu, z, slab=16)
+    assert torch.allclose(z.cpu().to(F64), want, atol=2e-2, rtol=2e-2)
+
+
+def test_gemm_skinny_refuses(k):
+    from pulse_infer_amd.ops import KernelError
+    a = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
+    assert not k.gemm_skinny_ok(a, w) and k.gemm_skinny_ok(a[:64], w)
+    assert not k.gemm_skinny_ok(a[:4, :60], w[:, :60])                 # K no multiple of 8
+    assert not k.gemm_skinny_ok(a[:4].float(), w)
+    with pytest.raises(KernelError, match="at most 64 rows"):
+        k.gemm_skinny(a, w, torch.zeros(65, 32, device=DEV))
+    with pytest.raises(KernelError, match="float32 target"):
+        k.gemm_skinny(a[:4], w, torch.zeros(4, 32, dtype=torch.bfloat16, device=DEV), add=True)
