@@ -198,11 +198,49 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
     out[idx] = from_f32<T>(s * u);
 }
 
+// Eight outputs a thread with 16-byte accesses, for bfloat16 rows whose sizes allow it.
+__global__ void swiglu_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int inter, int slab,
+                                     int64_t total8) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total8) return;
+    const int per_row = inter / 8;
+    const int64_t t = idx / per_row;
+    const int i = static_cast<int>(idx - t * per_row) * 8;
+    const bf16_t* row = gu + t * 2 * inter;
+    const int gi = slab > 0 ? (i / slab) * 2 * slab + i % slab : i;
+    const int ui = slab > 0 ? gi + slab : inter + i;
+    const uint4 g4 = *reinterpret_cast<const uint4*>(row + gi);
+    const uint4 u4 = *reinterpret_cast<const uint4*>(row + ui);
+    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w};
+    const uint32_t uw[4] = {u4.x, u4.y, u4.z, u4.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+        const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+        const float z0 = g0 / (1.0f + expf(-g0)) * u0;
+        const float z1 = g1 / (1.0f + expf(-g1)) * u1;
+        ow[j] = static_cast<uint32_t>(f32_to_bf16(z0)) | (static_cast<uint32_t>(f32_to_bf16(z1)) << 16);
+    }
+    *reinterpret_cast<uint4*>(out + t * inter + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 extern "C" int pulse_swiglu(const void* gu, void* out, int dtype, int tokens, int inter, int slab, hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && inter > 0 && pulse_dtype_ok(dtype) && gu && out, "swiglu: bad arguments");
     PULSE_REQUIRE(slab >= 0 && (slab == 0 || inter % slab == 0), "swiglu: %d columns do not divide into slabs of %d", inter, slab);
     const int64_t total = static_cast<int64_t>(tokens) * inter;
     if (total == 0) return 0;
+    const bool wide = dtype == PULSE_BF16 && inter % 8 == 0 && (slab == 0 || slab % 8 == 0) &&
+                      reinterpret_cast<uintptr_t>(gu) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    if (wide) {
+        const int64_t total8 = total / 8;
+        const int64_t blocks = (total8 + 255) / 256;
+        PULSE_REQUIRE(blocks < (1ll << 31), "swiglu: too many elements");
+        hipLaunchKernelGGL(swiglu_bf16x8_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream,
+                           static_cast<const bf16_t*>(gu), static_cast<bf16_t*>(out), inter, slab, total8);
+        PULSE_LAUNCH_CHECK("swiglu");
+        return 0;
+    }
     const int64_t blocks = (total + 255) / 256;
     PULSE_REQUIRE(blocks < (1ll << 31), "swiglu: too many elements");
     PULSE_DISPATCH_DTYPE(dtype, T,

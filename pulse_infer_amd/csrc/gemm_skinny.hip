@@ -19,6 +19,7 @@
 namespace {
 
 constexpr int KWAVES = 8;
+constexpr int UNROLL = 8;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -75,22 +76,33 @@ __global__ __launch_bounds__(KWAVES* PULSE_WAVE) void gemm_skinny_kernel(const b
         xrow[mt] = X + static_cast<int64_t>(xok[mt] ? m : 0) * ldx;
     }
 
-#pragma unroll 4
-    for (int ks = step_begin; ks < step_end; ++ks) {
-        const int k = ks * 32 + kg * 8;
-        const bool kok = k < K;
-        bf16x8 xb[MT], wa[SLABS];
+    // UNROLL k-steps at a time: all their loads are issued before the first product waits for one
+    for (int ks = step_begin; ks < step_end; ks += UNROLL) {
+        bf16x8 xb[UNROLL][MT], wa[UNROLL][SLABS];
 #pragma unroll
-        for (int s = 0; s < SLABS; ++s)
-            wa[s] = (wok[s] && kok) ? *reinterpret_cast<const bf16x8*>(wrow[s] + k) : zeros8();
+        for (int u = 0; u < UNROLL; ++u) {
+            const int k = (ks + u) * 32 + kg * 8;
+            const bool kok = (ks + u < step_end) && k < K;
+            const int kc = kok ? k : 0;  // always a valid address; what lies beyond K is zeroed below
+            // rows beyond N or M read row 0: their products only reach outputs that are never stored
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-            xb[mt] = (xok[mt] && kok) ? *reinterpret_cast<const bf16x8*>(xrow[mt] + k) : zeros8();
+            for (int s = 0; s < SLABS; ++s) {
+                wa[u][s] = *reinterpret_cast<const bf16x8*>(wrow[s] + kc);
+                if (!kok) wa[u][s] = zeros8();
+            }
 #pragma unroll
-        for (int s = 0; s < SLABS; ++s)
+            for (int mt = 0; mt < MT; ++mt) {
+                xb[u][mt] = *reinterpret_cast<const bf16x8*>(xrow[mt] + kc);
+                if (!kok) xb[u][mt] = zeros8();
+            }
+        }
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-                acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[s], xb[mt], acc[s][mt], 0, 0, 0);
+        for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+            for (int s = 0; s < SLABS; ++s)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[u][s], xb[u][mt], acc[s][mt], 0, 0, 0);
     }
 
 #pragma unroll

@@ -202,7 +202,86 @@ __global__ void mark_seen_kernel(uint32_t* __restrict__ masks, int mask_words, c
     atomicOr(masks + static_cast<int64_t>(rows[i]) * mask_words + (tok >> 5), 1u << (tok & 31));
 }
 
+// Greedy choice in two stages so that a few rows of a large vocabulary use the whole chip:
+// each workgroup scans one chunk of a row, then one workgroup per row merges the chunk winners.
+constexpr int ARGMAX_THREADS = 256;
+
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_chunks_kernel(const float* __restrict__ logits, int vocab,
+                                                                       int64_t row_stride, int chunk,
+                                                                       float* __restrict__ part_val,
+                                                                       int* __restrict__ part_idx) {
+    __shared__ float sv[ARGMAX_THREADS / PULSE_WAVE];
+    __shared__ int si[ARGMAX_THREADS / PULSE_WAVE];
+    const int r = blockIdx.y;
+    const int begin = blockIdx.x * chunk;
+    const int end = min(vocab, begin + chunk);
+    const float* row = logits + r * row_stride;
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int i = begin + threadIdx.x; i < end; i += ARGMAX_THREADS) {
+        const float x = row[i];
+        if (x > best) { best = x; best_i = i; }   // NaN never wins; ascending i keeps the lowest index among equals
+    }
+    const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off, PULSE_WAVE);
+        const int oi = __shfl_xor(best_i, off, PULSE_WAVE);
+        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    if (lane == 0) { sv[wave] = best; si[wave] = best_i; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < ARGMAX_THREADS / PULSE_WAVE; ++w)
+            if (sv[w] > best || (sv[w] == best && si[w] < best_i)) { best = sv[w]; best_i = si[w]; }
+        part_val[r * gridDim.x + blockIdx.x] = best;
+        part_idx[r * gridDim.x + blockIdx.x] = best_i;
+    }
+}
+
+__global__ __launch_bounds__(PULSE_WAVE) void argmax_merge_kernel(const float* __restrict__ part_val,
+                                                                  const int* __restrict__ part_idx, int chunks,
+                                                                  int* __restrict__ out) {
+    const int r = blockIdx.x;
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int c = threadIdx.x; c < chunks; c += PULSE_WAVE) {
+        const float v = part_val[r * chunks + c];
+        const int i = part_idx[r * chunks + c];
+        if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+    }
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off, PULSE_WAVE);
+        const int oi = __shfl_xor(best_i, off, PULSE_WAVE);
+        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    if (threadIdx.x == 0) out[r] = best_i == 0x7fffffff ? -1 : best_i;
+}
+
 }  // namespace
+
+// out[r] = index of the largest logit of row r, the lowest index among equals, -1 if none is a number.
+// part_val / part_idx: scratch of rows * pulse_argmax_chunks(vocab) entries each.
+extern "C" int pulse_argmax_chunks(int vocab) {
+    const int chunk = 2048;
+    return (vocab + chunk - 1) / chunk;
+}
+
+extern "C" int pulse_argmax(const float* logits, int rows, int vocab, int64_t row_stride, float* part_val,
+                            int* part_idx, int* out, hipStream_t stream) {
+    PULSE_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "argmax: bad sizes rows=%d V=%d", rows, vocab);
+    PULSE_REQUIRE(rows < 65536, "argmax: at most 65535 rows");
+    PULSE_REQUIRE(logits && part_val && part_idx && out, "argmax: null pointer");
+    if (rows == 0) return 0;
+    const int chunks = pulse_argmax_chunks(vocab);
+    hipLaunchKernelGGL(argmax_chunks_kernel, dim3(chunks, rows), dim3(ARGMAX_THREADS), 0, stream, logits, vocab,
+                       row_stride, 2048, part_val, part_idx);
+    PULSE_LAUNCH_CHECK("argmax_chunks");
+    hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(PULSE_WAVE), 0, stream, part_val, part_idx, chunks, out);
+    PULSE_LAUNCH_CHECK("argmax_merge");
+    return 0;
+}
 
 // out[r] = chosen token of row r, or -1 when no token is allowed.
 // temperature/top_k/top_p/penalty/seen_row/banned may be null (greedy, off, off, none, none, none).

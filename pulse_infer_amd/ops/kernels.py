@@ -149,7 +149,8 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
          _i64(w.stride(0) if n > 1 else k), _i64(out.stride(0) if m > 1 else n), _stream())
 
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 64           # what the kernel takes
+SKINNY_FAST_ROWS = 16          # up to here it beats the vendor library on every layer shape
 SKINNY_SWIGLU_MAX_ROWS = 32
 _OUT_MODES = {"store": None, "add": 2}
 
@@ -289,6 +290,24 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.
     call("pulse_sample", _ptr(logits), _i32(rows), _i32(vocab), _i64(logits.stride(0) if rows > 1 else vocab),
          _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform), _ptr(penalty), _ptr(seen_row), _ptr(seen_masks),
          _ptr(banned), _i32(words), _ptr(out), _stream())
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor, part_val: torch.Tensor, part_idx: torch.Tensor) -> None:
+    """out[r] = index of the largest logit of row r, lowest index among equals (two-stage, for few rows of a wide vocabulary)."""
+    _gpu("argmax", logits, out, part_val, part_idx)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1, "argmax: logits must be float32 [R, V]")
+    rows, vocab = logits.shape
+    chunks = argmax_chunks(vocab)
+    _int_vec("argmax: out", out, rows)
+    _need(part_val.dtype == torch.float32 and part_val.numel() >= rows * chunks and part_val.is_contiguous()
+          and part_idx.dtype == torch.int32 and part_idx.numel() >= rows * chunks and part_idx.is_contiguous(),
+          f"argmax: scratch must hold {rows * chunks} entries")
+    call("pulse_argmax", _ptr(logits), _i32(rows), _i32(vocab), _i64(logits.stride(0) if rows > 1 else vocab),
+         _ptr(part_val), _ptr(part_idx), _ptr(out), _stream())
+
+
+def argmax_chunks(vocab: int) -> int:
+    return (vocab + 2047) // 2048
 
 
 def mark_seen(masks: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor, vocab: int) -> None:

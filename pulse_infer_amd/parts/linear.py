@@ -32,7 +32,8 @@ class Linear:
         """``out`` [M, out_features] receives the product; its storage type is bfloat16 or float32."""
         w = self.weight if rows is None else self.weight[:rows]
         if self.library and x.dtype == torch.bfloat16:
-            if kernels.gemm_skinny_ok(x, w):
+            few = x.shape[0] <= kernels.SKINNY_FAST_ROWS or out.dtype != torch.bfloat16
+            if few and kernels.gemm_skinny_ok(x, w):
                 kernels.gemm_skinny(x, w, out)
                 return out
             if out.dtype == torch.bfloat16:
@@ -48,7 +49,8 @@ class Linear:
     def add_into(self, x: torch.Tensor, residual: torch.Tensor, scratch: torch.Tensor) -> Optional[torch.Tensor]:
         """residual += x W^T where the kernel can do that itself (returns None); otherwise the product is
         written to ``scratch`` and returned for the caller to add."""
-        if self.library and x.dtype == torch.bfloat16 and kernels.gemm_skinny_ok(x, self.weight):
+        if (self.library and x.dtype == torch.bfloat16 and x.shape[0] <= kernels.SKINNY_FAST_ROWS
+                and kernels.gemm_skinny_ok(x, self.weight)):
             kernels.gemm_skinny(x, self.weight, residual, add=True)
             return None
         return self.forward(x, scratch)

@@ -55,7 +55,7 @@ class GatedMLP(Part):
         tokens = x.shape[0]
         ws = ctx.workspace
         z = ws.buffer("mlp.act", tokens, self.inter, self.act_dtype)
-        if (self.slab and tokens <= kernels.SKINNY_SWIGLU_MAX_ROWS and kernels.gemm_skinny_ok(x, self.gate_up.weight)):
+        if (self.slab and tokens <= kernels.SKINNY_FAST_ROWS and kernels.gemm_skinny_ok(x, self.gate_up.weight)):
             kernels.gemm_skinny(x, self.gate_up.weight, z, swiglu=True)
         else:
             gu = ws.buffer("mlp.gate_up", tokens, 2 * self.inter, self.act_dtype)

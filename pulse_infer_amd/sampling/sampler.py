@@ -24,6 +24,8 @@ class Sampler:
         self.num_slots = int(num_slots)
         self.seen: Optional[torch.Tensor] = None  # [slots, words], made when a request first needs it
         self.banned: Optional[torch.Tensor] = None
+        self._part_val: Optional[torch.Tensor] = None
+        self._part_idx: Optional[torch.Tensor] = None
         if banned_tokens:
             host = torch.zeros(self.words, dtype=torch.int64)
             for tok in banned_tokens:
@@ -58,7 +60,11 @@ class Sampler:
             return []
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
         if all(p.greedy and p.presence_penalty == 0.0 for p in params) and self.banned is None:
-            kernels.sample(logits, out)
+            need = rows * kernels.argmax_chunks(logits.shape[1])
+            if self._part_val is None or self._part_val.numel() < need:
+                self._part_val = torch.empty(need, dtype=torch.float32, device=self.device)
+                self._part_idx = torch.empty(need, dtype=torch.int32, device=self.device)
+            kernels.argmax(logits, out, self._part_val, self._part_idx)
             return out.tolist()
         temperature = torch.tensor([p.temperature for p in params], dtype=torch.float32, device=self.device)
         top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32, device=self.device)

@@ -491,3 +491,20 @@ def test_gemm_skinny_refuses(k):
         k.gemm_skinny(a, w, torch.zeros(65, 32, device=DEV))
     with pytest.raises(KernelError, match="float32 target"):
         k.gemm_skinny(a[:4], w, torch.zeros(4, 32, dtype=torch.bfloat16, device=DEV), add=True)
+
+
+def test_two_stage_argmax(k):
+    for rows, vocab in ((1, 5), (3, 2048), (8, 151936), (5, 4097)):
+        logits = rnd(rows, vocab, seed=80 + rows).to(DEV)
+        logits[0, vocab - 1] = logits[0, 0] = 99.0                       # equal maxima far apart: the lowest index wins
+        if rows > 1:
+            logits[1, vocab // 2] = float("nan")
+        chunks = k.argmax_chunks(vocab)
+        out = torch.empty(rows, dtype=torch.int32, device=DEV)
+        k.argmax(logits, out, torch.empty(rows * chunks, device=DEV), torch.empty(rows * chunks, dtype=torch.int32, device=DEV))
+        want = torch.argmax(torch.nan_to_num(logits.cpu(), nan=-1e30), dim=1).tolist()
+        want[0] = 0
+        assert out.tolist() == want
+        single = torch.empty(rows, dtype=torch.int32, device=DEV)
+        k.sample(logits, single)
+        assert single.tolist() == want
