@@ -61,8 +61,34 @@ class _Staging:
         return dev
 
 
+@dataclass
+class _Captured:
+    """A recorded decode step: its integer buffers, the graph, and where the logits appear."""
+
+    host: torch.Tensor
+    host_np: np.ndarray
+    dev: torch.Tensor
+    offsets: np.ndarray
+    widths: List[int]
+    graph: Any = None
+    logits: Any = None
+    workspace: Any = None
+    context: Any = None   # kept alive: the graph reads tensors that the context's parts created (work lists, tables)
+    event: Any = None
+
+    def wait(self) -> None:
+        if self.event is not None:
+            self.event.synchronize()   # the last copy out of the pinned buffer has finished
+
+    def mark(self) -> None:
+        if self.event is None:
+            self.event = torch.cuda.Event()
+        self.event.record()
+
+
 class ModelRunner:
-    def __init__(self, model: CausalLM, page_size: int, num_pages: int, max_requests: int = 64):
+    def __init__(self, model: CausalLM, page_size: int, num_pages: int, max_requests: int = 64,
+                 use_graphs: bool = True):
         self.model = model
         self.device = model.device
         self.cache = CacheManager(model.run_cache_specs(), page_size, num_pages, max_requests)
@@ -82,6 +108,8 @@ class ModelRunner:
             else:
                 self.views.append(None)
         self._staging = _Staging(self.device)
+        self.use_graphs = bool(use_graphs) and model.options.get("decode_graph", True)
+        self._graphs: dict = {}
         self.max_positions = model.spec.max_positions
         self.steps = 0
         self.tokens_run = 0
@@ -125,24 +153,16 @@ class ModelRunner:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {e.request!r}: wanted place {w} is outside its {n} tokens")
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        self._check(entries)
-        cache = self.cache
-        metas: List[EntryMeta] = []
-        row = 0
-        for e in entries:
-            metas.append(EntryMeta(e.request, cache.slot_of(e.request), cache.computed(e.request), len(e.tokens), row))
-            row += len(e.tokens)
-        total, batch = row, len(metas)
-        want_rows = [m.first_row + int(w) for e, m in zip(entries, metas) for w in e.want]
-        widths = []
-        for g in cache.groups:
-            widths.append(max(1, max(g.pages_for(m.start + m.count) for m in metas)))
+    def _layout(self, total: int, batch: int, wanted: int, widths: Sequence[int]) -> np.ndarray:
+        """Offsets of the step's integer arrays in one flat buffer:
+        [ids | positions | token_entry | start | count | first_row | slot | want | tables...]"""
+        sizes = [total, total, total, batch, batch, batch + 1, batch, wanted] + [batch * w for w in widths]
+        return np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
 
-        # one flat int32 array: [ids | positions | token_entry | start | count | first_row | slot | want | tables...]
-        sizes = [total, total, total, batch, batch, batch + 1, batch, len(want_rows)] + [batch * w for w in widths]
-        offsets = np.concatenate([[0], np.cumsum(sizes)])
-        flat = np.zeros(int(offsets[-1]), dtype=np.int32)
+    def _fill(self, flat: np.ndarray, offsets: np.ndarray, entries: Sequence[StepEntry], metas: List[EntryMeta],
+              want_rows: List[int], widths: Sequence[int]) -> None:
+        cache = self.cache
+        total, batch = metas[-1].first_row + metas[-1].count, len(metas)
         ids, pos, tok_entry = (flat[offsets[i]:offsets[i + 1]] for i in range(3))
         for i, (e, m) in enumerate(zip(entries, metas)):
             sl = slice(m.first_row, m.first_row + m.count)
@@ -154,24 +174,104 @@ class ModelRunner:
         flat[offsets[5]:offsets[6]] = [m.first_row for m in metas] + [total]
         flat[offsets[6]:offsets[7]] = [m.slot for m in metas]
         flat[offsets[7]:offsets[8]] = want_rows
-        for gi, (g, w) in enumerate(zip(cache.groups, widths)):
+        for gi, w in enumerate(widths):
             table = np.full((batch, w), -1, dtype=np.int32)
             for i, m in enumerate(metas):
                 pages = cache.table(gi, m.request)[:w]
                 table[i, :len(pages)] = pages
             flat[offsets[8 + gi]:offsets[9 + gi]] = table.reshape(-1)
 
-        dev = self._staging.upload(flat)
-        part = [dev[offsets[i]:offsets[i + 1]] for i in range(len(sizes))]
-        ctx = StepContext(
+    def _context(self, dev: torch.Tensor, offsets: np.ndarray, metas: List[EntryMeta], wanted: int,
+                 widths: Sequence[int], workspace, max_context: int) -> StepContext:
+        total, batch = metas[-1].first_row + metas[-1].count, len(metas)
+        part = [dev[offsets[i]:offsets[i + 1]] for i in range(len(offsets) - 1)]
+        return StepContext(
             num_tokens=total, entries=metas, token_ids=part[0], positions=part[1], token_entry=part[2],
             entry_start=part[3], entry_count=part[4], entry_first_row=part[5], entry_slot=part[6],
             block_tables={gi: part[8 + gi].view(batch, w) for gi, w in enumerate(widths)},
-            want_rows=part[7], num_wanted=len(want_rows), workspace=self.model.workspace,
-            max_count=max(m.count for m in metas), max_context=max(m.start + m.count for m in metas))
-        logits = self.model.forward(ctx, self.views)
+            want_rows=part[7], num_wanted=wanted, workspace=workspace,
+            max_count=max(m.count for m in metas), max_context=max_context)
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        self._check(entries)
+        cache = self.cache
+        metas: List[EntryMeta] = []
+        row = 0
+        for e in entries:
+            metas.append(EntryMeta(e.request, cache.slot_of(e.request), cache.computed(e.request), len(e.tokens), row))
+            row += len(e.tokens)
+        total = row
+        want_rows = [m.first_row + int(w) for e, m in zip(entries, metas) for w in e.want]
+        max_context = max(m.start + m.count for m in metas)
+        if self._graph_ok(entries, metas):
+            logits = self._step_captured(entries, metas, want_rows, max_context)
+        else:
+            widths = [max(1, max(g.pages_for(m.start + m.count) for m in metas)) for g in cache.groups]
+            offsets = self._layout(total, len(metas), len(want_rows), widths)
+            flat = np.zeros(int(offsets[-1]), dtype=np.int32)
+            self._fill(flat, offsets, entries, metas, want_rows, widths)
+            dev = self._staging.upload(flat)
+            ctx = self._context(dev, offsets, metas, len(want_rows), widths, self.model.workspace, max_context)
+            logits = self.model.forward(ctx, self.views)
         for m in metas:
             cache.advance(m.request, m.start + m.count)
         self.steps += 1
         self.tokens_run += total
         return logits
+
+    # ------------------------------------------------------- captured decoding
+    # A step of single tokens (one per request, each wanting its logits) has the same launches every time,
+    # so it is recorded once per (batch, context bucket) as a HIP graph over buffers of its own and replayed:
+    # the host then only copies the step's integers and starts the graph.
+    GRAPH_MAX_BATCH = 16        # up to here every product is this package's own kernel (no library call is recorded)
+    GRAPH_CONTEXT_BUCKET = 1024
+
+    def _graph_ok(self, entries: Sequence[StepEntry], metas: List[EntryMeta]) -> bool:
+        if not self.use_graphs or self.model.mode != "bfloat16" or len(metas) > self.GRAPH_MAX_BATCH:
+            return False
+        if self.cache.state_runs:   # parts with per-request state may run host code of their own
+            return False
+        return all(m.count == 1 for m in metas) and all(list(e.want) == [0] for e in entries)
+
+    def _step_captured(self, entries: Sequence[StepEntry], metas: List[EntryMeta], want_rows: List[int],
+                       max_context: int) -> torch.Tensor:
+        batch = len(metas)
+        bucket = (max_context + self.GRAPH_CONTEXT_BUCKET - 1) // self.GRAPH_CONTEXT_BUCKET * self.GRAPH_CONTEXT_BUCKET
+        bucket = min(bucket, max(self.max_positions, max_context))
+        key = (batch, bucket)
+        rec = self._graphs.get(key)
+        if rec is None:
+            rec = self._capture(key, entries, metas, want_rows)
+            self._graphs[key] = rec
+        rec.wait()
+        self._fill(rec.host_np, rec.offsets, entries, metas, want_rows, rec.widths)
+        rec.dev.copy_(rec.host, non_blocking=True)
+        rec.graph.replay()
+        rec.mark()
+        return rec.logits.clone()
+
+    def _capture(self, key, entries, metas, want_rows) -> "_Captured":
+        from ..parts.base import Workspace
+
+        batch, bucket = key
+        widths = [max(1, g.pages_for(bucket)) for g in self.cache.groups]
+        offsets = self._layout(batch, batch, batch, widths)
+        n = int(offsets[-1])
+        host = torch.zeros(n, dtype=torch.int32, pin_memory=True)
+        dev = torch.zeros(n, dtype=torch.int32, device=self.device)
+        rec = _Captured(host=host, host_np=host.numpy(), dev=dev, offsets=offsets, widths=widths)
+        workspace = Workspace(self.device)
+        ctx = self._context(dev, offsets, metas, batch, widths, workspace, bucket)
+        self._fill(rec.host_np, offsets, entries, metas, want_rows, widths)
+        dev.copy_(host, non_blocking=True)
+        # an eager run first: it sizes the workspace and lets parts build what depends only on the step's shape
+        self.model.forward(ctx, self.views)
+        torch.cuda.synchronize()
+        ctx.extras = {k: v for k, v in ctx.extras.items() if k.startswith("static:")}
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            rec.logits = self.model.forward(ctx, self.views)
+        rec.graph = graph
+        rec.workspace = workspace
+        rec.context = ctx
+        return rec

@@ -45,6 +45,7 @@ class CausalLM:
         self.device = torch.device(device)
         self.act_dtype = ACT_DTYPES[mode]
         self.workspace = Workspace(self.device)
+        self.options = dict(options or {})
         loader = WeightLoader(source, expected_tensors(spec), mode, self.device, strict=strict)
         build = BuildContext(loader=loader, mode=mode, device=self.device, act_dtype=self.act_dtype,
                              workspace=self.workspace, options=dict(options or {}))

@@ -107,8 +107,8 @@ class PagedAttention(Part):
             return
         group = self.nq // self.nkv
         per = attention_mfma.tokens_per_item(group)
-        key = f"attention.items:{per}"
-        if key not in ctx.extras:  # the same list serves every layer of the step with this grouping
+        key = f"static:attention.items:{per}"
+        if key not in ctx.extras:  # depends only on the step's shape; the same list serves every layer
             flat = attention_mfma.build_items(ctx.entries, per)
             ctx.extras[key] = torch.tensor(flat, dtype=torch.int32, device=q.device)
         items = ctx.extras[key]

@@ -153,3 +153,48 @@ def test_command_line(gpu, model_folders, plain_models, capsys):
                      "--max-new-tokens", "4", "--temperature", "0.7", "--top-k", "20", "--top-p", "0.95",
                      "--sample-seed", "1", "--num-pages", "32"])
     assert code == 0 and len(json.loads(capsys.readouterr().out.splitlines()[0])["output_ids"]) == 4
+
+
+def test_captured_decode_steps_replay_like_eager_ones(gpu, model_folders, plain_logits):
+    """Decode steps are recorded once per (batch, context bucket) and replayed.  Every replay is checked against
+    the eager step and the plain implementation, with eager prompt portions of other requests in between."""
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from test_gpu_model import SPLIT_TOL, close
+
+    cfg, page = TINY["B"]
+    _, model = load_model(model_folders["B"], mode="bfloat16")
+    runners = [ModelRunner(model, page_size=16, num_pages=32, max_requests=4, use_graphs=flag) for flag in (True, False)]
+    ids = {k: token_ids(cfg["vocab_size"], n, seed=90 + n) for k, n in (("a", 60), ("b", 75), ("c", 50))}
+    got = [{k: [] for k in ids} for _ in runners]
+    for which, runner in enumerate(runners):
+        fed = {k: 0 for k in ids}
+
+        def feed(pairs):
+            entries = []
+            for k, n in pairs:
+                if not runner.cache.has_request(k):
+                    runner.add_request(k)
+                runner.reserve(k, fed[k] + n)
+                entries.append(StepEntry(k, ids[k][fed[k]:fed[k] + n], [n - 1]))
+                fed[k] += n
+            logits = runner.step(entries)
+            for row, (k, _) in enumerate(pairs):
+                got[which][k].append((fed[k] - 1, logits[row]))
+
+        feed([("a", 20), ("b", 31)])
+        for _ in range(10):
+            feed([("a", 1), ("b", 1)])                   # recorded at the first, replayed nine times
+        feed([("c", 17)])                                 # eager work between replays
+        for _ in range(8):
+            feed([("a", 1), ("b", 1), ("c", 1)])         # another batch size: another recording
+        feed([("c", 9)])
+        for _ in range(12):
+            feed([("b", 1), ("a", 1)])                   # the first recording again, entries in another order
+        assert runner.use_graphs == (which == 0) and (len(runner._graphs) == 2) == (which == 0)
+    for k in ids:
+        want = plain_logits("B", ids[k])
+        for (pos_g, row_g), (pos_e, row_e) in zip(got[0][k], got[1][k]):
+            assert pos_g == pos_e
+            close(row_g[None], want[pos_g][None], "bfloat16", f"captured {k}@{pos_g}")
+            close(row_g[None], row_e[None], "bfloat16", f"captured against eager {k}@{pos_g}", SPLIT_TOL)
