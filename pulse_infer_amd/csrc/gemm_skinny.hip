@@ -2,11 +2,11 @@
 // cores: the regime of decoding, where the product only has to stream the
 // weight from HBM once.
 //
-// A workgroup of eight wavefronts owns SLABS slabs of 16 weight rows.  Each
-// wavefront takes one eighth of K and runs v_mfma_f32_16x16x32_bf16 with the
+// A workgroup of KW wavefronts owns SLABS slabs of 16 weight rows.  Each
+// wavefront takes its share of K and runs v_mfma_f32_16x16x32_bf16 with the
 // weight slab as the row operand and X^T as the column operand (both are 16-byte
 // loads of 8 consecutive k), so the result is C^T: lane l holds output features
-// 4*(l/16)+i of row l%16.  The eight partial tiles are summed through LDS in
+// 4*(l/16)+i of row l%16.  The wavefronts' partial tiles are summed through LDS in
 // wavefront order, so the result is the same from run to run.  The epilogue
 // stores bfloat16 or float32, adds into a float32 matrix (the residual), or
 // applies SwiGLU to a (gate, up) pair of slabs of a slab-interleaved weight.
@@ -18,8 +18,8 @@
 
 namespace {
 
-constexpr int KWAVES = 8;
 constexpr int UNROLL = 8;
+constexpr int XLDS_BYTES = 16384;  // the most LDS a workgroup takes for X: more costs occupancy and gains nothing
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -33,13 +33,21 @@ __device__ __forceinline__ bf16x8 zeros8() {
     return z;
 }
 
-template <int SLABS, int MT, bool SWIGLU>
-__global__ __launch_bounds__(KWAVES* PULSE_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ X, int64_t ldx,
-                                                                          const bf16_t* __restrict__ W, int64_t ldw,
-                                                                          void* __restrict__ C, int64_t ldc, int M,
-                                                                          int N, int K, int mode) {
+// SLABS slabs of 16 weight rows a workgroup, MT tiles of 16 rows of X, KW wavefronts sharing K.
+// XLDS: X (at most 16 rows, MT == 1) is first copied into LDS in operand order, so that the loop's only global
+// loads are the weight's.  Without it, lanes whose row of X does not exist skip their load: the cost of the X loads
+// is per active lane, and it is what keeps this kernel from the speed of a plain read of the weight.
+template <int SLABS, int MT, int KW, bool SWIGLU, bool XLDS>
+__global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_kernel(const bf16_t* __restrict__ X, int64_t ldx,
+                                                                      const bf16_t* __restrict__ W, int64_t ldw,
+                                                                      void* __restrict__ C, int64_t ldc, int M, int N,
+                                                                      int K, int mode) {
     constexpr int TILES = SLABS * MT;
-    __shared__ float red[KWAVES][TILES][16][17];
+    constexpr int THREADS = KW * PULSE_WAVE;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    // the partial tiles reuse the room of X once every wavefront is done with it
+    float (*red)[TILES][16][17] = reinterpret_cast<float (*)[TILES][16][17]>(smem);
+    bf16x8* xs = reinterpret_cast<bf16x8*>(smem);  // [K / 8][M]
 
     const int tid = threadIdx.x;
     const int wave = tid / PULSE_WAVE;
@@ -49,9 +57,18 @@ __global__ __launch_bounds__(KWAVES* PULSE_WAVE) void gemm_skinny_kernel(const b
     const int n_base = blockIdx.x * SLABS * 16;
 
     const int steps = (K + 31) / 32;
-    const int per = (steps + KWAVES - 1) / KWAVES;
+    const int per = (steps + KW - 1) / KW;
     const int step_begin = wave * per;
     const int step_end = min(steps, step_begin + per);
+
+    if (XLDS) {
+        const int k8s = K / 8;
+        for (int c = tid; c < k8s * M; c += THREADS) {
+            const int m = c / k8s, k8 = c - m * k8s;
+            xs[k8 * M + m] = *reinterpret_cast<const bf16x8*>(X + static_cast<int64_t>(m) * ldx + k8 * 8);
+        }
+        __syncthreads();
+    }
 
     f32x4 acc[SLABS][MT];
 #pragma unroll
@@ -59,13 +76,12 @@ __global__ __launch_bounds__(KWAVES* PULSE_WAVE) void gemm_skinny_kernel(const b
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[s][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // rows beyond N read row 0: their products only reach outputs that are never stored
     const bf16_t* wrow[SLABS];
-    bool wok[SLABS];
 #pragma unroll
     for (int s = 0; s < SLABS; ++s) {
         const int n = n_base + s * 16 + r;
-        wok[s] = n < N;
-        wrow[s] = W + static_cast<int64_t>(wok[s] ? n : 0) * ldw;
+        wrow[s] = W + static_cast<int64_t>(n < N ? n : 0) * ldw;
     }
     const bf16_t* xrow[MT];
     bool xok[MT];
@@ -75,25 +91,27 @@ __global__ __launch_bounds__(KWAVES* PULSE_WAVE) void gemm_skinny_kernel(const b
         xok[mt] = m < M;
         xrow[mt] = X + static_cast<int64_t>(xok[mt] ? m : 0) * ldx;
     }
+    const int xm = r < M ? r : 0;  // XLDS: the row this lane reads (rows that do not exist repeat row 0)
 
-    // UNROLL k-steps at a time: all their loads are issued before the first product waits for one
-    for (int ks = step_begin; ks < step_end; ks += UNROLL) {
+    // Whole groups of UNROLL k-steps first: all their loads are issued before the first product waits for one,
+    // and nothing is done to a loaded value in between (a select on it would make every load wait).
+    const int whole_steps = K / 32;  // steps that lie inside K entirely
+    int ks = step_begin;
+    for (; ks + UNROLL <= min(step_end, whole_steps); ks += UNROLL) {
         bf16x8 xb[UNROLL][MT], wa[UNROLL][SLABS];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int k = (ks + u) * 32 + kg * 8;
-            const bool kok = (ks + u < step_end) && k < K;
-            const int kc = kok ? k : 0;  // always a valid address; what lies beyond K is zeroed below
-            // rows beyond N or M read row 0: their products only reach outputs that are never stored
 #pragma unroll
-            for (int s = 0; s < SLABS; ++s) {
-                wa[u][s] = *reinterpret_cast<const bf16x8*>(wrow[s] + kc);
-                if (!kok) wa[u][s] = zeros8();
-            }
+            for (int s = 0; s < SLABS; ++s) wa[u][s] = *reinterpret_cast<const bf16x8*>(wrow[s] + k);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                xb[u][mt] = *reinterpret_cast<const bf16x8*>(xrow[mt] + kc);
-                if (!kok) xb[u][mt] = zeros8();
+                if (XLDS) {
+                    xb[u][mt] = xs[(k / 8) * M + xm];
+                } else {
+                    xb[u][mt] = zeros8();
+                    if (xok[mt]) xb[u][mt] = *reinterpret_cast<const bf16x8*>(xrow[mt] + k);
+                }
             }
         }
 #pragma unroll
@@ -104,7 +122,25 @@ __global__ __launch_bounds__(KWAVES* PULSE_WAVE) void gemm_skinny_kernel(const b
                 for (int mt = 0; mt < MT; ++mt)
                     acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[u][s], xb[u][mt], acc[s][mt], 0, 0, 0);
     }
+    // what is left, one step at a time; the last step may reach beyond K
+    for (; ks < step_end; ++ks) {
+        const int k = ks * 32 + kg * 8;
+        const bool kok = k < K;
+        const int kc = kok ? k : 0;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            bf16x8 xb = zeros8();
+            if (kok && xok[mt]) xb = XLDS ? xs[(kc / 8) * M + xm] : *reinterpret_cast<const bf16x8*>(xrow[mt] + kc);
+#pragma unroll
+            for (int s = 0; s < SLABS; ++s) {
+                bf16x8 wa = zeros8();
+                if (kok) wa = *reinterpret_cast<const bf16x8*>(wrow[s] + kc);
+                acc[s][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, xb, acc[s][mt], 0, 0, 0);
+            }
+        }
+    }
 
+    if (XLDS) __syncthreads();  // every wavefront has read its part of X; its room now takes the partial tiles
 #pragma unroll
     for (int s = 0; s < SLABS; ++s)
 #pragma unroll
@@ -114,13 +150,13 @@ __global__ __launch_bounds__(KWAVES* PULSE_WAVE) void gemm_skinny_kernel(const b
     __syncthreads();
 
     if (!SWIGLU) {
-        for (int e = tid; e < TILES * 256; e += KWAVES * PULSE_WAVE) {
+        for (int e = tid; e < TILES * 256; e += THREADS) {
             const int tile = e / 256;
             const int m_in = (e % 256) / 16;
             const int n_in = e % 16;
             float v = 0.f;
 #pragma unroll
-            for (int w = 0; w < KWAVES; ++w) v += red[w][tile][n_in][m_in];
+            for (int w = 0; w < KW; ++w) v += red[w][tile][n_in][m_in];
             const int m = (tile % MT) * 16 + m_in;
             const int n = n_base + (tile / MT) * 16 + n_in;
             if (m < M && n < N) {
@@ -133,14 +169,14 @@ __global__ __launch_bounds__(KWAVES* PULSE_WAVE) void gemm_skinny_kernel(const b
     } else {
         // slabs come in (gate, up) pairs; the output has half as many columns
         constexpr int PAIRS = SLABS / 2;
-        for (int e = tid; e < PAIRS * MT * 256; e += KWAVES * PULSE_WAVE) {
+        for (int e = tid; e < PAIRS * MT * 256; e += THREADS) {
             const int pt = e / 256;  // pair * MT + mt
             const int m_in = (e % 256) / 16;
             const int n_in = e % 16;
             const int pair = pt / MT, mt = pt % MT;
             float g = 0.f, u = 0.f;
 #pragma unroll
-            for (int w = 0; w < KWAVES; ++w) {
+            for (int w = 0; w < KW; ++w) {
                 g += red[w][(2 * pair) * MT + mt][n_in][m_in];
                 u += red[w][(2 * pair + 1) * MT + mt][n_in][m_in];
             }
@@ -154,12 +190,19 @@ __global__ __launch_bounds__(KWAVES* PULSE_WAVE) void gemm_skinny_kernel(const b
     }
 }
 
-template <int SLABS, int MT, bool SWIGLU>
-void launch(const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N, int K,
-            int mode, hipStream_t stream) {
+template <int SLABS, int MT, int KW, bool SWIGLU>
+void launch(bool xlds, const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
+            int K, int mode, hipStream_t stream) {
     const unsigned blocks = (N + SLABS * 16 - 1) / (SLABS * 16);
-    hipLaunchKernelGGL((gemm_skinny_kernel<SLABS, MT, SWIGLU>), dim3(blocks), dim3(KWAVES * PULSE_WAVE), 0, stream, X,
-                       ldx, W, ldw, C, ldc, M, N, K, mode);
+    const size_t red_bytes = sizeof(float) * KW * SLABS * MT * 16 * 17;
+    if (MT == 1 && xlds) {
+        const size_t x_bytes = static_cast<size_t>(K) * M * 2;
+        hipLaunchKernelGGL((gemm_skinny_kernel<SLABS, 1, KW, SWIGLU, true>), dim3(blocks), dim3(KW * PULSE_WAVE),
+                           x_bytes > red_bytes ? x_bytes : red_bytes, stream, X, ldx, W, ldw, C, ldc, M, N, K, mode);
+    } else {
+        hipLaunchKernelGGL((gemm_skinny_kernel<SLABS, MT, KW, SWIGLU, false>), dim3(blocks), dim3(KW * PULSE_WAVE),
+                           red_bytes, stream, X, ldx, W, ldw, C, ldc, M, N, K, mode);
+    }
 }
 
 }  // namespace
@@ -185,22 +228,20 @@ extern "C" int pulse_gemm_skinny(const void* X, int64_t ldx, const void* W, int6
     const bf16_t* x = static_cast<const bf16_t*>(X);
     const bf16_t* w = static_cast<const bf16_t*>(W);
     const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-    // more slabs per workgroup reuse X better; fewer give more workgroups.  Aim for at least 512 workgroups.
-    const int slabs_total = (N + 15) / 16;
-    int slabs = 4 / mt;
-    while (slabs > 1 && slabs_total / slabs < 512) slabs /= 2;
-    if (swiglu && slabs < 2) slabs = 2;
+    // X goes through LDS when it is small enough for two workgroups a compute unit
+    const bool xlds = mt == 1 && K % 32 == 0 && static_cast<size_t>(K) * M * 2 <= XLDS_BYTES;
+    const bool wide = N >= 16384;  // enough slabs that pairs of them still fill the chip
     if (swiglu) {
-        if (mt == 1 && slabs == 4) launch<4, 1, true>(x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
-        else if (mt == 1) launch<2, 1, true>(x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
-        else launch<2, 2, true>(x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+        if (mt == 1) launch<2, 1, 4, true>(xlds, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+        else launch<2, 2, 8, true>(false, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+    } else if (mt == 1) {
+        if (wide) launch<2, 1, 4, false>(xlds, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+        else launch<1, 1, 4, false>(xlds, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+    } else if (mt == 2) {
+        if (wide) launch<2, 2, 8, false>(false, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+        else launch<1, 2, 8, false>(false, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
     } else {
-        if (mt == 1 && slabs == 4) launch<4, 1, false>(x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
-        else if (mt == 1 && slabs == 2) launch<2, 1, false>(x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
-        else if (mt == 1) launch<1, 1, false>(x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
-        else if (mt == 2 && slabs == 2) launch<2, 2, false>(x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
-        else if (mt == 2) launch<1, 2, false>(x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
-        else launch<1, 4, false>(x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+        launch<1, 4, 8, false>(false, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
     }
     PULSE_LAUNCH_CHECK("gemm_skinny");
     return 0;
