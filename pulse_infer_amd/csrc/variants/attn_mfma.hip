@@ -43,6 +43,14 @@ constexpr int BLOCK_KEYS = 32;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+// The operands of one 32-key block as they come from memory.
+struct BlockRegs {
+    u32x4 k[2][NCHUNK];  // tile, 32-wide slice of the head: 8 bfloat16 of key row r
+    u32x2 v[2][NDT];     // tile, 16-channel tile: 4 bfloat16 (keys 4kg..4kg+3) of channel row r
+};
 
 struct MfmaArgs {
     const bf16_t* q;
@@ -75,7 +83,14 @@ __device__ __forceinline__ bf16x8 zero8() {
     return z;
 }
 
-__global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_mfma_kernel(MfmaArgs a) {
+// two wavefronts a SIMD (256 registers each) where the head size lets the two register sets fit
+#if PULSE_HEAD_DIM <= 128
+#define PULSE_ATTN_WAVES_PER_EU __attribute__((amdgpu_waves_per_eu(2)))
+#else
+#define PULSE_ATTN_WAVES_PER_EU
+#endif
+
+__global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_mfma_kernel(MfmaArgs a) {
     __shared__ float s_m[WAVES][16];
     __shared__ float s_l[WAVES][16];
     __shared__ float s_o[WAVES][D][17];
@@ -130,10 +145,11 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_mfma_kernel(MfmaArgs a
 
     const int first_block = max(split_begin, lo_item) / BLOCK_KEYS;
     const int last_block = (split_end - 1) / BLOCK_KEYS;
-    for (int b = first_block + wave; b <= last_block; b += WAVES) {
+
+    // Issue every load of a 32-key block: K rows of the two 16-key tiles (a tile never straddles pages:
+    // page_size % 16 == 0) and V rows in the order {tile0: 4kg.., tile1: 4kg..}.  Nothing is done to the values here.
+    auto load_block = [&](int b, BlockRegs& x) {
         const int j0 = b * BLOCK_KEYS;
-        // pages of the two 16-key tiles (a tile never straddles pages: page_size % 16 == 0)
-        int64_t kbase[2], vbase[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int jt = j0 + 16 * t;
@@ -142,33 +158,32 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_mfma_kernel(MfmaArgs a
             page = (page >= 0 && page < a.num_pages) ? page : 0;  // masked keys may sit in pages given back
             const int slot0 = jt % a.page_size;
             const int64_t pg = static_cast<int64_t>(page) * a.nkv + g;
-            kbase[t] = (pg * a.page_size + slot0) * D;
-            vbase[t] = pg * D * a.page_size + slot0;
+            const bf16_t* krow = a.kc + (pg * a.page_size + slot0 + r) * D;
+#pragma unroll
+            for (int ch = 0; ch < NCHUNK; ++ch) {
+                const int off = ch * 32 + kg * 8;
+                x.k[t][ch] = off < D ? *reinterpret_cast<const u32x4*>(krow + off) : u32x4{0u, 0u, 0u, 0u};
+            }
+            const bf16_t* vrow = a.vc + pg * D * a.page_size + slot0 + 4 * kg + static_cast<int64_t>(r) * a.page_size;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+                x.v[t][dt] = *reinterpret_cast<const u32x2*>(vrow + static_cast<int64_t>(dt) * 16 * a.page_size);
         }
+    };
+
+    auto compute_block = [&](int b, const BlockRegs& x) {
+        const int j0 = b * BLOCK_KEYS;
         // S^T = K Q^T
         f32x4 s[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-            const bf16_t* krow = a.kc + kbase[t] + static_cast<int64_t>(r) * D;
 #pragma unroll
-            for (int ch = 0; ch < NCHUNK; ++ch) {
-                const int off = ch * 32 + kg * 8;
-                const bf16x8 ak = off < D ? *reinterpret_cast<const bf16x8*>(krow + off) : zero8();
-                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak, bq[ch], s[t], 0, 0, 0);
-            }
-        }
-        // V^T operands: channel row dt*16 + r, keys {tile0: 4kg.., tile1: 4kg..}
-        bf16x8 av[NDT];
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-            const int64_t ch_off = static_cast<int64_t>(dt * 16 + r) * a.page_size + 4 * kg;
-            const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(a.vc + vbase[0] + ch_off);
-            const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(a.vc + vbase[1] + ch_off);
-            av[dt] = bf16x8{v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+            for (int ch = 0; ch < NCHUNK; ++ch)
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x.k[t][ch]), bq[ch], s[t], 0, 0, 0);
         }
         // scores of this lane: keys j0 + 16t + 4kg + i of column r
-        const bool needs_mask = (j0 + BLOCK_KEYS - 1 > hi) || (j0 < lo_item + 0) || (a.window > 0) || (ntok > 1) ||
+        const bool needs_mask = (j0 + BLOCK_KEYS - 1 > hi) || (j0 < lo_item) || (a.window > 0) || (ntok > 1) ||
                                 (j0 < split_begin) || (j0 + BLOCK_KEYS > split_end);
         float p[2][4];
         float mx = -INFINITY;
@@ -178,8 +193,8 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_mfma_kernel(MfmaArgs a
             for (int i = 0; i < 4; ++i) {
                 const int j = j0 + 16 * t + 4 * kg + i;
                 float v = s[t][i] * a.scale_log2e;
-                if (needs_mask && !(j <= pos_c && j >= lo_c && j >= split_begin && j < split_end)) v = -INFINITY;
-                if (!col_ok) v = -INFINITY;
+                const bool seen = !needs_mask || (j <= pos_c && j >= lo_c && j >= split_begin && j < split_end);
+                v = (seen && col_ok) ? v : -INFINITY;
                 p[t][i] = v;
                 mx = fmaxf(mx, v);
             }
@@ -199,20 +214,40 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_mfma_kernel(MfmaArgs a
             }
         l_part = l_part * alpha + psum;
         m = m_new;
-        if (needs_mask) {
-            // stale values under masked keys must not reach the sum, not even as 0 * (inf or nan)
+        // Stale values under keys that no column of the item may see must not reach the sum, not even as
+        // 0 * (inf or nan): they are cleared by bit masks, one per pair of keys.
+        uint32_t keep[2][2];
 #pragma unroll
-            for (int dt = 0; dt < NDT; ++dt)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int j = j0 + 16 * (e / 4) + 4 * kg + (e % 4);
-                    if (j > hi || j < lo_item) av[dt][e] = (__bf16)0.0f;
-                }
-        }
+            for (int h2 = 0; h2 < 2; ++h2) {
+                const int j = j0 + 16 * t + 4 * kg + 2 * h2;
+                const bool lo_ok = !needs_mask || (j <= hi && j >= lo_item);
+                const bool hi_ok = !needs_mask || (j + 1 <= hi && j + 1 >= lo_item);
+                keep[t][h2] = (lo_ok ? 0x0000ffffu : 0u) | (hi_ok ? 0xffff0000u : 0u);
+            }
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) {
+            const u32x4 words = {x.v[0][dt][0] & keep[0][0], x.v[0][dt][1] & keep[0][1],
+                                 x.v[1][dt][0] & keep[1][0], x.v[1][dt][1] & keep[1][1]};
             acc[dt] = acc[dt] * alpha;
-            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[dt], pb, acc[dt], 0, 0, 0);
+            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, words), pb, acc[dt], 0, 0, 0);
+        }
+    };
+
+    // two register sets in turn: the next block's loads are in flight while this block is computed
+    {
+        BlockRegs xa, xb;
+        int b = first_block + wave;
+        if (b <= last_block) load_block(b, xa);
+        while (b <= last_block) {
+            if (b + WAVES <= last_block) load_block(b + WAVES, xb);
+            compute_block(b, xa);
+            b += WAVES;
+            if (b > last_block) break;
+            if (b + WAVES <= last_block) load_block(b + WAVES, xa);
+            compute_block(b, xb);
+            b += WAVES;
         }
     }
 
@@ -272,17 +307,232 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_mfma_kernel(MfmaArgs a
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Prompt portions: one workgroup per (item, kv head, chunk of 16 heads); its four wavefronts take consecutive
+// sub-items of `per` tokens (16 columns each) and walk the keys together.  Every 32-key block of K and V is copied
+// from its pages into LDS once for all four (two stages, so the next block's loads are in flight while this one
+// is computed), and each wavefront reads its matrix-core operands from there.  No split: a wavefront sees all its
+// keys, so it normalises and writes its columns itself.
+constexpr int KPAD = 8;                    // bfloat16 of padding a key row: 16-byte reads of 16 rows hit 16 bank groups
+constexpr int KROW = D + KPAD;
+constexpr int STAGE_K = BLOCK_KEYS * KROW;  // bfloat16 elements
+constexpr int STAGE_V = 2 * D * 16;
+
+__global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_prefill_kernel(MfmaArgs a, int per) {
+    __shared__ __attribute__((aligned(16))) bf16_t s_k[2][STAGE_K];
+    __shared__ __attribute__((aligned(16))) bf16_t s_v[2][STAGE_V];
+
+    const int item = blockIdx.x;
+    const int g = blockIdx.y / a.head_chunks;
+    const int chunk = blockIdx.y % a.head_chunks;
+    const int tid = threadIdx.x;
+    const int wave = tid / PULSE_WAVE;
+    const int lane = tid % PULSE_WAVE;
+    const int r = lane % 16;
+    const int kg = lane / 16;
+
+    const int row0 = a.items[2 * item];
+    const int ntok = a.items[2 * item + 1];         // at most WAVES * per
+    const int hi = a.positions[row0 + ntok - 1];    // last key of the workgroup
+    const int pos_first = a.positions[row0];
+    const int lo_item = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
+    const int* bt = a.block_table + static_cast<int64_t>(a.token_entry[row0]) * a.bt_width;
+
+    // this wavefront's tokens and this lane's column
+    const int wtok0 = wave * per;
+    const int wntok = max(0, min(per, ntok - wtok0));
+    const int tc = r / a.gp;
+    const int hc = r % a.gp + chunk * 16;
+    const bool col_ok = tc < wntok && hc < a.group;
+    const int col_row = row0 + (col_ok ? wtok0 + tc : 0);
+    const int col_head = g * a.group + (col_ok ? hc : 0);
+    const int pos_c = col_ok ? a.positions[col_row] : -1;
+    const int lo_c = (a.window > 0 && pos_c - a.window + 1 > 0) ? pos_c - a.window + 1 : 0;
+    // keys this wavefront needs at all
+    const int whi = wntok > 0 ? a.positions[row0 + wtok0 + wntok - 1] : -1;
+    const int wpos0 = wntok > 0 ? a.positions[row0 + wtok0] : 0;
+    const int wlo = (a.window > 0 && wpos0 - a.window + 1 > 0) ? wpos0 - a.window + 1 : 0;
+
+    bf16x8 bq[NCHUNK];
+    {
+        const bf16_t* qrow = a.q + static_cast<int64_t>(col_row) * a.q_stride + static_cast<int64_t>(col_head) * D;
+#pragma unroll
+        for (int ch = 0; ch < NCHUNK; ++ch) {
+            const int off = ch * 32 + kg * 8;
+            bq[ch] = (col_ok && off < D) ? *reinterpret_cast<const bf16x8*>(qrow + off) : zero8();
+        }
+    }
+    f32x4 acc[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY;
+    float l_part = 0.f;
+
+    // The copy of a block: K is 32 rows of D, V is 2 tiles of D rows of 16 keys; both in 16-byte pieces.
+    constexpr int K_PIECES = BLOCK_KEYS * D / 8;
+    constexpr int V_PIECES = 2 * D * 16 / 8;
+    constexpr int K_PER = (K_PIECES + WAVES * PULSE_WAVE - 1) / (WAVES * PULSE_WAVE);
+    constexpr int V_PER = (V_PIECES + WAVES * PULSE_WAVE - 1) / (WAVES * PULSE_WAVE);
+    u32x4 kreg[K_PER], vreg[V_PER];
+
+    auto fetch = [&](int b) {
+        const int j0 = b * BLOCK_KEYS;
+        int64_t kbase[2], vbase[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int jt = j0 + 16 * t;
+            const int pi = jt / a.page_size;
+            int page = (jt <= hi && pi < a.bt_width) ? bt[pi] : 0;
+            page = (page >= 0 && page < a.num_pages) ? page : 0;
+            const int slot0 = jt % a.page_size;
+            const int64_t pg = static_cast<int64_t>(page) * a.nkv + g;
+            kbase[t] = (pg * a.page_size + slot0) * D;
+            vbase[t] = pg * D * a.page_size + slot0;
+        }
+#pragma unroll
+        for (int i = 0; i < K_PER; ++i) {
+            const int piece = tid + i * WAVES * PULSE_WAVE;
+            if (piece < K_PIECES) {
+                const int key = piece / (D / 8), c8 = piece % (D / 8);
+                kreg[i] = *reinterpret_cast<const u32x4*>(a.kc + kbase[key / 16] + static_cast<int64_t>(key % 16) * D + c8 * 8);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < V_PER; ++i) {
+            const int piece = tid + i * WAVES * PULSE_WAVE;
+            if (piece < V_PIECES) {
+                const int t = piece / (D * 2), rest = piece % (D * 2);  // D rows * 2 pieces a row
+                const int ch = rest / 2, half = rest % 2;
+                vreg[i] = *reinterpret_cast<const u32x4*>(a.vc + vbase[t] + static_cast<int64_t>(ch) * a.page_size + half * 8);
+            }
+        }
+    };
+    auto stash = [&](int stage) {
+#pragma unroll
+        for (int i = 0; i < K_PER; ++i) {
+            const int piece = tid + i * WAVES * PULSE_WAVE;
+            if (piece < K_PIECES) {
+                const int key = piece / (D / 8), c8 = piece % (D / 8);
+                *reinterpret_cast<u32x4*>(&s_k[stage][key * KROW + c8 * 8]) = kreg[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < V_PER; ++i) {
+            const int piece = tid + i * WAVES * PULSE_WAVE;
+            if (piece < V_PIECES) *reinterpret_cast<u32x4*>(&s_v[stage][piece * 8]) = vreg[i];
+        }
+    };
+
+    auto compute = [&](int b, int stage) {
+        const int j0 = b * BLOCK_KEYS;
+        f32x4 s[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ch = 0; ch < NCHUNK; ++ch) {
+                const int off = ch * 32 + kg * 8;
+                const bf16x8 ak = off < D ? *reinterpret_cast<const bf16x8*>(&s_k[stage][(16 * t + r) * KROW + off]) : zero8();
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak, bq[ch], s[t], 0, 0, 0);
+            }
+        }
+        float p[2][4];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int j = j0 + 16 * t + 4 * kg + i;
+                float v = s[t][i] * a.scale_log2e;
+                v = (col_ok && j <= pos_c && j >= lo_c) ? v : -INFINITY;
+                p[t][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, PULSE_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, PULSE_WAVE));
+        const float m_new = fmaxf(m, mx);
+        const float alpha = (m_new == -INFINITY) ? 1.f : exp2f(m - m_new);
+        float psum = 0.f;
+        bf16x8 pb;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float e = (p[t][i] == -INFINITY) ? 0.f : exp2f(p[t][i] - m_new);
+                psum += e;
+                pb[4 * t + i] = (__bf16)e;
+            }
+        l_part = l_part * alpha + psum;
+        m = m_new;
+        // stale values under keys outside [lo_item, hi] are cleared (see the split kernel)
+        const bool edge = (j0 + BLOCK_KEYS - 1 > hi) || (j0 < lo_item);
+        uint32_t keep[2][2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) {
+                const int j = j0 + 16 * t + 4 * kg + 2 * h2;
+                const bool lo_ok = !edge || (j <= hi && j >= lo_item);
+                const bool hi_ok = !edge || (j + 1 <= hi && j + 1 >= lo_item);
+                keep[t][h2] = (lo_ok ? 0x0000ffffu : 0u) | (hi_ok ? 0xffff0000u : 0u);
+            }
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+            const u32x2 v0 = *reinterpret_cast<const u32x2*>(&s_v[stage][(dt * 16 + r) * 16 + 4 * kg]);
+            const u32x2 v1 = *reinterpret_cast<const u32x2*>(&s_v[stage][D * 16 + (dt * 16 + r) * 16 + 4 * kg]);
+            const u32x4 words = {v0[0] & keep[0][0], v0[1] & keep[0][1], v1[0] & keep[1][0], v1[1] & keep[1][1]};
+            acc[dt] = acc[dt] * alpha;
+            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, words), pb, acc[dt], 0, 0, 0);
+        }
+    };
+
+    const int first_block = lo_item / BLOCK_KEYS;
+    const int last_block = hi / BLOCK_KEYS;
+    fetch(first_block);
+    stash(0);
+    __syncthreads();
+    for (int b = first_block; b <= last_block; ++b) {
+        const int stage = (b - first_block) & 1;
+        if (b < last_block) fetch(b + 1);
+        // a wavefront skips blocks that none of its columns sees (above its diagonal, below its window)
+        if (wntok > 0 && b * BLOCK_KEYS <= whi && b * BLOCK_KEYS + BLOCK_KEYS - 1 >= wlo) compute(b, stage);
+        if (b < last_block) stash(stage ^ 1);
+        __syncthreads();
+    }
+
+    l_part += __shfl_xor(l_part, 16, PULSE_WAVE);
+    l_part += __shfl_xor(l_part, 32, PULSE_WAVE);
+    if (col_ok) {
+        const float inv = l_part > 0.f ? 1.0f / l_part : 0.f;
+        bf16_t* dst = a.out + static_cast<int64_t>(col_row) * a.o_stride + static_cast<int64_t>(col_head) * D;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+            const uint32_t w0 = static_cast<uint32_t>(f32_to_bf16(acc[dt][0] * inv)) |
+                                (static_cast<uint32_t>(f32_to_bf16(acc[dt][1] * inv)) << 16);
+            const uint32_t w1 = static_cast<uint32_t>(f32_to_bf16(acc[dt][2] * inv)) |
+                                (static_cast<uint32_t>(f32_to_bf16(acc[dt][3] * inv)) << 16);
+            *reinterpret_cast<u32x2*>(dst + dt * 16 + 4 * kg) = u32x2{w0, w1};
+        }
+    }
+}
+
 // out[row, head, :] = sum_z w_z o_z / sum_z w_z l_z with w_z = exp2(m_z - max m), over the splits that hold keys of
 // the row.  One workgroup per (row, head); the splits' (m, l) pairs go through LDS so that the loads overlap.
 constexpr int MAX_SPLITS = 1024;
 
 __global__ __launch_bounds__(128) void attn_mfma_reduce_kernel(const float* __restrict__ part_o,
                                                                const float* __restrict__ part_ml,
-                                                               const int* __restrict__ positions, bf16_t* __restrict__ out,
-                                                               int64_t o_stride, int nq, int n_splits, int split_size) {
+                                                               const int* __restrict__ positions,
+                                                               const int* __restrict__ items, int per,
+                                                               bf16_t* __restrict__ out, int64_t o_stride, int nq,
+                                                               int n_splits, int split_size) {
     __shared__ float s_w[MAX_SPLITS];
     __shared__ float s_l[MAX_SPLITS];
-    const int64_t row = blockIdx.x;
+    // only the rows of this launch's items have partial results
+    const int item = blockIdx.x / per;
+    const int tok = blockIdx.x % per;
+    if (tok >= items[2 * item + 1]) return;
+    const int64_t row = items[2 * item] + tok;
     const int head = blockIdx.y;
     const int valid = min(n_splits, positions[row] / split_size + 1);
     const int64_t base = (row * nq + head) * n_splits;
@@ -352,10 +602,49 @@ extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64
                        stream, a);
     PULSE_LAUNCH_CHECK("attn_mfma");
     if (n_splits > 1) {
-        hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(tokens, nq), dim3(128), 0, stream, part_o, part_ml, positions,
-                           a.out, o_stride, nq, n_splits, split_size);
+        const int per = 16 / gp;
+        hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(n_items * per, nq), dim3(128), 0, stream, part_o, part_ml,
+                           positions, items, per, a.out, o_stride, nq, n_splits, split_size);
         PULSE_LAUNCH_CHECK("attn_mfma_reduce");
     }
+    return 0;
+}
+
+// Prompt portions: items of up to 4 * pulse_attn_mfma_tokens_per_item(group) tokens of one request, one workgroup each,
+// keys shared through LDS, no split.
+extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, int64_t o_stride, const void* kcache,
+                                  const void* vcache, const int* positions, const int* token_entry,
+                                  const int* block_table, int bt_width, const int* items, int n_items, int tokens,
+                                  int nq, int nkv, int page_size, int num_pages, float scale, int window,
+                                  hipStream_t stream) {
+    PULSE_REQUIRE(tokens >= 0 && n_items >= 0 && nq > 0 && nkv > 0, "attn_prefill: bad sizes");
+    PULSE_REQUIRE(nq % nkv == 0, "attn_prefill: %d query heads are not a multiple of %d kv heads", nq, nkv);
+    PULSE_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_prefill: page size %d must be a multiple of 16", page_size);
+    PULSE_REQUIRE(num_pages > 0 && bt_width > 0 && window >= 0, "attn_prefill: bad cache geometry");
+    PULSE_REQUIRE(q_stride % 8 == 0 && o_stride % 4 == 0 && q_stride >= static_cast<int64_t>(nq) * D &&
+                  o_stride >= static_cast<int64_t>(nq) * D, "attn_prefill: row strides must cover the heads and keep alignment");
+    PULSE_REQUIRE((reinterpret_cast<uintptr_t>(q) % 16) == 0 && (reinterpret_cast<uintptr_t>(kcache) % 16) == 0 &&
+                  (reinterpret_cast<uintptr_t>(vcache) % 16) == 0 && (reinterpret_cast<uintptr_t>(out) % 8) == 0,
+                  "attn_prefill: pointers must be 16-byte aligned");
+    PULSE_REQUIRE(static_cast<int64_t>(nkv) * ((nq / nkv + 15) / 16) < 65536, "attn_prefill: grid too large");
+    PULSE_REQUIRE(q && out && kcache && vcache && positions && token_entry && block_table && items, "attn_prefill: null pointer");
+    if (tokens == 0 || n_items == 0) return 0;
+    const int group = nq / nkv;
+    int gp = 1;
+    while (gp < group && gp < 16) gp *= 2;
+    MfmaArgs a;
+    a.q = static_cast<const bf16_t*>(q); a.q_stride = q_stride;
+    a.out = static_cast<bf16_t*>(out); a.o_stride = o_stride;
+    a.part_o = nullptr; a.part_ml = nullptr;
+    a.kc = static_cast<const bf16_t*>(kcache); a.vc = static_cast<const bf16_t*>(vcache);
+    a.positions = positions; a.token_entry = token_entry; a.block_table = block_table; a.items = items;
+    a.bt_width = bt_width; a.nq = nq; a.nkv = nkv; a.group = group; a.gp = gp; a.head_chunks = (group + 15) / 16;
+    a.page_size = page_size; a.num_pages = num_pages;
+    a.scale_log2e = scale * 1.4426950408889634f;
+    a.window = window; a.split_size = 0; a.n_splits = 1;
+    hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_items, nkv * a.head_chunks), dim3(WAVES * PULSE_WAVE), 0, stream, a,
+                       16 / gp);
+    PULSE_LAUNCH_CHECK("attn_prefill");
     return 0;
 }
 

@@ -27,6 +27,10 @@ def tokens_per_item(group: int) -> int:
     return 16 // gp
 
 
+PORTION_MIN_TOKENS = 16   # entries with at least this many tokens go to the kernel that shares keys through LDS
+PORTION_WAVES = 4         # wavefronts of its workgroup, each with `tokens_per_item` tokens
+
+
 def build_items(entries: Sequence, tokens_per: int) -> List[int]:
     """Flat [first row, token count] pairs covering every entry of a step."""
     flat: List[int] = []
@@ -34,6 +38,13 @@ def build_items(entries: Sequence, tokens_per: int) -> List[int]:
         for b in range(0, e.count, tokens_per):
             flat.extend((e.first_row + b, min(tokens_per, e.count - b)))
     return flat
+
+
+def split_entries(entries: Sequence):
+    """(single tokens and short portions, long portions)"""
+    short = [e for e in entries if e.count < PORTION_MIN_TOKENS]
+    long = [e for e in entries if e.count >= PORTION_MIN_TOKENS]
+    return short, long
 
 
 def choose_splits(num_items: int, nkv: int, group: int, max_context: int, target_groups: int = 1024) -> Tuple[int, int]:
@@ -78,3 +89,27 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
             _ptr(vcache), _ptr(positions), _ptr(token_entry), _ptr(block_table), _i32(block_table.shape[1]),
             _ptr(items), _i32(n_items), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages), _f32(scale),
             _i32(window), _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml), _stream())
+
+
+def attn_prefill(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
+                 vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
+                 items: torch.Tensor, scale: float, window: int) -> None:
+    """Attention for prompt portions: items of up to 4 * tokens_per_item(group) tokens, keys shared through LDS."""
+    _gpu("attn_prefill", q, out, kcache, vcache, positions, token_entry, block_table, items)
+    tokens = q.shape[0]
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.stride(1) == 1 and out.stride(1) == 1,
+          "attn_prefill: q and out must be bfloat16 matrices with contiguous rows")
+    _need(q.shape[1] >= nq * d and out.shape[1] >= nq * d and out.shape[0] == tokens, "attn_prefill: q/out too narrow")
+    pages, page_size = _check_cache("attn_prefill", kcache, vcache, nkv, d)
+    _need(supported(d, page_size, q.dtype, kcache.dtype), f"attn_prefill: head size {d} / page size {page_size} / "
+          f"{kcache.dtype} is not supported by the matrix-core kernel")
+    _int_vec("attn_prefill: positions", positions, tokens)
+    _int_vec("attn_prefill: token_entry", token_entry, tokens)
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+          "attn_prefill: block_table must be contiguous int32 [entries, width]")
+    _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() % 2 == 0, "attn_prefill: items must be int32 pairs")
+    lib = load_variant("attn_mfma", {"PULSE_HEAD_DIM": d})
+    call_in(lib, "pulse_attn_prefill", _ptr(q), _i64(q.stride(0)), _ptr(out), _i64(out.stride(0)), _ptr(kcache),
+            _ptr(vcache), _ptr(positions), _ptr(token_entry), _ptr(block_table), _i32(block_table.shape[1]),
+            _ptr(items), _i32(items.numel() // 2), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages),
+            _f32(scale), _i32(window), _stream())

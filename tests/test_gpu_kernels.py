@@ -386,7 +386,7 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0):
     q, qref = as_stored(rnd(len(positions), (nq + 2 * nkv) * d, seed=300 + seed), dtype)
     out = torch.zeros(len(positions), nq * d, dtype=dtype, device=DEV)
     max_ctx = max(lens)
-    if split is None:
+    if split is None or split == "portion":
         split_size, n_splits = M.choose_splits(items.numel() // 2, nkv, group, max_ctx)
     else:
         split_size, n_splits = split, (max_ctx + split - 1) // split
@@ -394,9 +394,19 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0):
     part_o = torch.full((rows, d), float("nan"), device=DEV)
     part_ml = torch.full((rows, 2), float("nan"), device=DEV)
     scale = d ** -0.5
-    M.attn_mfma(q, out, nq, nkv, d, kc, vc, torch.tensor(positions, dtype=torch.int32, device=DEV),
-                torch.tensor(entry, dtype=torch.int32, device=DEV), table.to(DEV), items, scale, window, split_size,
-                n_splits, max_ctx, part_o, part_ml)
+    pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    ent_t = torch.tensor(entry, dtype=torch.int32, device=DEV)
+    if split == "portion":
+        # request 0's portion through the kernel that shares keys through LDS, the single tokens through the other
+        big = torch.tensor(M.build_items(entries[:1], M.tokens_per_item(group) * M.PORTION_WAVES), dtype=torch.int32, device=DEV)
+        M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos_t, ent_t, table.to(DEV), big, scale, window)
+        if len(entries) > 1:
+            small = torch.tensor(M.build_items(entries[1:], M.tokens_per_item(group)), dtype=torch.int32, device=DEV)
+            M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, ent_t, table.to(DEV), small, scale, window, split_size,
+                        n_splits, max_ctx, part_o, part_ml)
+    else:
+        M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, ent_t, table.to(DEV), items, scale, window, split_size,
+                    n_splits, max_ctx, part_o, part_ml)
     got = out.cpu().to(F64).reshape(-1, nq, d)
     for t, (p, e) in enumerate(zip(positions, entry)):
         kref, vref = refs[e]
@@ -414,7 +424,7 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0):
     dict(nq=40, nkv=2, d=64, bs=64, window=0, lens=[200, 77], portion=5),              # 20 heads a kv head: two chunks
     dict(nq=16, nkv=1, d=224, bs=16, window=100, lens=[260, 130], portion=18),
 ])
-@pytest.mark.parametrize("split", [None, 32, 128])
+@pytest.mark.parametrize("split", [None, 32, 128, "portion"])
 def test_attn_mfma(k, case, split):
     _mfma_case(k, split=split, **case)
 
