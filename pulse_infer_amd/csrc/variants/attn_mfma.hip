@@ -316,9 +316,12 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
 constexpr int KPAD = 8;                    // bfloat16 of padding a key row: 16-byte reads of 16 rows hit 16 bank groups
 constexpr int KROW = D + KPAD;
 constexpr int STAGE_K = BLOCK_KEYS * KROW;  // bfloat16 elements
-constexpr int STAGE_V = 2 * D * 16;
+// V in LDS, in 8-byte words (4 keys of one channel): [tile][16-channel tile][key group kg][channel row r], padded to
+// 17 words a key group, so that the 16 lanes of one key group read 128 contiguous bytes (no bank conflict).
+constexpr int VGROUP = 17;
+constexpr int STAGE_V = 2 * NDT * 4 * VGROUP * 4;  // bfloat16 elements
 
-__global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_prefill_kernel(MfmaArgs a, int per) {
+__global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_prefill_kernel(MfmaArgs a, int per) {
     __shared__ __attribute__((aligned(16))) bf16_t s_k[2][STAGE_K];
     __shared__ __attribute__((aligned(16))) bf16_t s_v[2][STAGE_V];
 
@@ -419,9 +422,21 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_prefill_kernel(MfmaArg
 #pragma unroll
         for (int i = 0; i < V_PER; ++i) {
             const int piece = tid + i * WAVES * PULSE_WAVE;
-            if (piece < V_PIECES) *reinterpret_cast<u32x4*>(&s_v[stage][piece * 8]) = vreg[i];
+            if (piece < V_PIECES) {
+                const int t = piece / (D * 2), rest = piece % (D * 2);
+                const int ch = rest / 2, half = rest % 2;
+                const int word = ((t * NDT + ch / 16) * 4 + 2 * half) * VGROUP + ch % 16;  // key groups 2*half, 2*half+1
+                *reinterpret_cast<u32x2*>(&s_v[stage][word * 4]) = u32x2{vreg[i][0], vreg[i][1]};
+                *reinterpret_cast<u32x2*>(&s_v[stage][(word + VGROUP) * 4]) = u32x2{vreg[i][2], vreg[i][3]};
+            }
         }
     };
+
+    // lowest position among this wavefront's columns: blocks wholly at or below it (and above every window's
+    // start) need no mask at all
+    const int wmin_pos = wpos0;
+    const int whi_lo = (a.window > 0 && whi - a.window + 1 > 0) ? whi - a.window + 1 : 0;  // highest window start
+    const float c2 = a.scale_log2e;
 
     auto compute = [&](int b, int stage) {
         const int j0 = b * BLOCK_KEYS;
@@ -436,29 +451,37 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_prefill_kernel(MfmaArg
                 s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak, bq[ch], s[t], 0, 0, 0);
             }
         }
+        // the maximum is tracked on the raw scores (the scale is positive); p = exp2((s - m) * scale * log2 e)
+        const bool inner = (j0 + BLOCK_KEYS - 1 <= wmin_pos) && (j0 >= whi_lo);
         float p[2][4];
         float mx = -INFINITY;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int j = j0 + 16 * t + 4 * kg + i;
-                float v = s[t][i] * a.scale_log2e;
-                v = (col_ok && j <= pos_c && j >= lo_c) ? v : -INFINITY;
+                float v = s[t][i];
+                if (!inner) {
+                    const int j = j0 + 16 * t + 4 * kg + i;
+                    v = (col_ok && j <= pos_c && j >= lo_c) ? v : -INFINITY;
+                }
                 p[t][i] = v;
                 mx = fmaxf(mx, v);
             }
+        if (inner && !col_ok) mx = -INFINITY;
         mx = fmaxf(mx, __shfl_xor(mx, 16, PULSE_WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, PULSE_WAVE));
         const float m_new = fmaxf(m, mx);
-        const float alpha = (m_new == -INFINITY) ? 1.f : exp2f(m - m_new);
+        const bool dead = m_new == -INFINITY;  // no key of this column so far
+        const float alpha = dead ? 1.f : __builtin_amdgcn_exp2f((m - m_new) * c2);
+        const float shift = dead ? 0.f : -m_new * c2;
         float psum = 0.f;
         bf16x8 pb;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float e = (p[t][i] == -INFINITY) ? 0.f : exp2f(p[t][i] - m_new);
+                // exp2(-inf) = 0 for masked scores; a dead column keeps -inf + 0 = -inf as well
+                const float e = (inner && !col_ok) ? 0.f : __builtin_amdgcn_exp2f(fmaf(p[t][i], c2, shift));
                 psum += e;
                 pb[4 * t + i] = (__bf16)e;
             }
@@ -466,23 +489,37 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) void attn_prefill_kernel(MfmaArg
         m = m_new;
         // stale values under keys outside [lo_item, hi] are cleared (see the split kernel)
         const bool edge = (j0 + BLOCK_KEYS - 1 > hi) || (j0 < lo_item);
-        uint32_t keep[2][2];
+        // rescale only when some column's maximum moved
+        const bool moved = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
+        if (moved) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+            for (int dt = 0; dt < NDT; ++dt) acc[dt] = acc[dt] * alpha;
+        }
+        if (edge) {
+            uint32_t keep[2][2];
 #pragma unroll
-            for (int h2 = 0; h2 < 2; ++h2) {
-                const int j = j0 + 16 * t + 4 * kg + 2 * h2;
-                const bool lo_ok = !edge || (j <= hi && j >= lo_item);
-                const bool hi_ok = !edge || (j + 1 <= hi && j + 1 >= lo_item);
-                keep[t][h2] = (lo_ok ? 0x0000ffffu : 0u) | (hi_ok ? 0xffff0000u : 0u);
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int h2 = 0; h2 < 2; ++h2) {
+                    const int j = j0 + 16 * t + 4 * kg + 2 * h2;
+                    keep[t][h2] = ((j <= hi && j >= lo_item) ? 0x0000ffffu : 0u) |
+                                  ((j + 1 <= hi && j + 1 >= lo_item) ? 0xffff0000u : 0u);
+                }
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                const u32x2 v0 = *reinterpret_cast<const u32x2*>(&s_v[stage][((dt * 4 + kg) * VGROUP + r) * 4]);
+                const u32x2 v1 = *reinterpret_cast<const u32x2*>(&s_v[stage][(((NDT + dt) * 4 + kg) * VGROUP + r) * 4]);
+                const u32x4 words = {v0[0] & keep[0][0], v0[1] & keep[0][1], v1[0] & keep[1][0], v1[1] & keep[1][1]};
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, words), pb, acc[dt], 0, 0, 0);
             }
+        } else {
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-            const u32x2 v0 = *reinterpret_cast<const u32x2*>(&s_v[stage][(dt * 16 + r) * 16 + 4 * kg]);
-            const u32x2 v1 = *reinterpret_cast<const u32x2*>(&s_v[stage][D * 16 + (dt * 16 + r) * 16 + 4 * kg]);
-            const u32x4 words = {v0[0] & keep[0][0], v0[1] & keep[0][1], v1[0] & keep[1][0], v1[1] & keep[1][1]};
-            acc[dt] = acc[dt] * alpha;
-            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, words), pb, acc[dt], 0, 0, 0);
+            for (int dt = 0; dt < NDT; ++dt) {
+                const u32x2 v0 = *reinterpret_cast<const u32x2*>(&s_v[stage][((dt * 4 + kg) * VGROUP + r) * 4]);
+                const u32x2 v1 = *reinterpret_cast<const u32x2*>(&s_v[stage][(((NDT + dt) * 4 + kg) * VGROUP + r) * 4]);
+                const u32x4 words = {v0[0], v0[1], v1[0], v1[1]};
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, words), pb, acc[dt], 0, 0, 0);
+            }
         }
     };
 
