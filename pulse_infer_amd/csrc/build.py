@@ -63,7 +63,7 @@ def find_hipcc() -> str:
 def _writable(path: str) -> bool:
     try:
         os.makedirs(path, exist_ok=True)
-        probe = os.path.join(path, f".probe{os.getpid()}")
+        probe = os.path.join(path, f".probe{os.getpid()}.{threading.get_ident()}")
         with open(probe, "w"):
             pass
         os.remove(probe)
@@ -209,7 +209,7 @@ def build_variant(source: str, defines: Dict[str, int], force: bool = False, ver
     if verbose:
         threading.Thread(target=ticker, daemon=True).start()
     try:
-        tmp = lib + f".tmp{os.getpid()}"
+        tmp = lib + f".tmp{os.getpid()}.{threading.get_ident()}"
         cmd = [hipcc, *COMMON_FLAGS, "-shared", *[f"-D{k}={v}" for k, v in sorted(defines.items())],
                os.path.join(VARIANT_DIR, source + ".hip"), os.path.join(HERE, "error_text.hip"), "-o", tmp]
         proc = subprocess.run(cmd, capture_output=True, text=True)

@@ -76,6 +76,10 @@ struct MfmaArgs {
     int n_splits;
 };
 
+// A value that is the same in every lane of the wavefront, said so to the compiler: what depends on it becomes
+// scalar work and uniform branches.
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
 __device__ __forceinline__ bf16x8 zero8() {
     bf16x8 z;
 #pragma unroll
@@ -329,17 +333,17 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     const int g = blockIdx.y / a.head_chunks;
     const int chunk = blockIdx.y % a.head_chunks;
     const int tid = threadIdx.x;
-    const int wave = tid / PULSE_WAVE;
+    const int wave = uniform(tid / PULSE_WAVE);
     const int lane = tid % PULSE_WAVE;
     const int r = lane % 16;
     const int kg = lane / 16;
 
-    const int row0 = a.items[2 * item];
-    const int ntok = a.items[2 * item + 1];         // at most WAVES * per
-    const int hi = a.positions[row0 + ntok - 1];    // last key of the workgroup
-    const int pos_first = a.positions[row0];
+    const int row0 = uniform(a.items[2 * item]);
+    const int ntok = uniform(a.items[2 * item + 1]);         // at most WAVES * per
+    const int hi = uniform(a.positions[row0 + ntok - 1]);    // last key of the workgroup
+    const int pos_first = uniform(a.positions[row0]);
     const int lo_item = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
-    const int* bt = a.block_table + static_cast<int64_t>(a.token_entry[row0]) * a.bt_width;
+    const int* bt = a.block_table + static_cast<int64_t>(uniform(a.token_entry[row0])) * a.bt_width;
 
     // this wavefront's tokens and this lane's column
     const int wtok0 = wave * per;
@@ -352,8 +356,8 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     const int pos_c = col_ok ? a.positions[col_row] : -1;
     const int lo_c = (a.window > 0 && pos_c - a.window + 1 > 0) ? pos_c - a.window + 1 : 0;
     // keys this wavefront needs at all
-    const int whi = wntok > 0 ? a.positions[row0 + wtok0 + wntok - 1] : -1;
-    const int wpos0 = wntok > 0 ? a.positions[row0 + wtok0] : 0;
+    const int whi = uniform(wntok > 0 ? a.positions[row0 + wtok0 + wntok - 1] : -1);
+    const int wpos0 = uniform(wntok > 0 ? a.positions[row0 + wtok0] : 0);
     const int wlo = (a.window > 0 && wpos0 - a.window + 1 > 0) ? wpos0 - a.window + 1 : 0;
 
     bf16x8 bq[NCHUNK];
@@ -385,7 +389,7 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
         for (int t = 0; t < 2; ++t) {
             const int jt = j0 + 16 * t;
             const int pi = jt / a.page_size;
-            int page = (jt <= hi && pi < a.bt_width) ? bt[pi] : 0;
+            int page = (jt <= hi && pi < a.bt_width) ? uniform(bt[pi]) : 0;
             page = (page >= 0 && page < a.num_pages) ? page : 0;
             const int slot0 = jt % a.page_size;
             const int64_t pg = static_cast<int64_t>(page) * a.nkv + g;
