@@ -26,7 +26,12 @@ QWEN3_8B = dict(
     num_hidden_layers=36, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
     max_position_embeddings=40960, rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False,
     torch_dtype="bfloat16", use_sliding_window=False)
-FULL_LAYERS = QWEN3_8B["num_hidden_layers"]
+# the other shapes of the benchmark list: selected with --model, never the default
+SHAPES = {
+    "8b": QWEN3_8B,
+    "14b": dict(QWEN3_8B, hidden_size=5120, intermediate_size=17408, num_hidden_layers=40, num_attention_heads=40),
+    "32b": dict(QWEN3_8B, hidden_size=5120, intermediate_size=25600, num_hidden_layers=64, num_attention_heads=64),
+}
 
 
 def parse_args() -> argparse.Namespace:
@@ -36,7 +41,16 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--warmup", type=int, default=8)
     p.add_argument("--batch", type=int, default=8)
     p.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
-    p.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has, if memory or time needs it")
+    p.add_argument("--model", choices=sorted(SHAPES), default="8b", help="layer sizes: Qwen3-8B (the default), 14B or 32B")
+    p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has, if memory or time needs it")
+    p.add_argument("--workload", choices=["decode", "serving"], default="decode",
+                   help="decode: fixed batch at a fixed context; serving: continuous batching of requests with "
+                        "seeded prompt lengths, chunked prefill mixed with decoding")
+    p.add_argument("--requests", type=int, default=32, help="serving: number of requests")
+    p.add_argument("--prompt-range", type=int, nargs=2, default=[128, 2048], help="serving: prompt lengths drawn from [lo, hi]")
+    p.add_argument("--output-tokens", type=int, default=256, help="serving: tokens generated per request")
+    p.add_argument("--chunk", type=int, default=512, help="serving: longest prompt portion in a step")
+    p.add_argument("--temperature", type=float, default=0.7, help="serving: sampling temperature")
     p.add_argument("--prefill-tokens", type=int, default=2048)
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
@@ -67,6 +81,45 @@ def prefill_flops(cfg, tokens: int) -> float:
     return cfg.num_hidden_layers * (2.0 * tokens * linear + attn) + 2.0 * cfg.vocab_size * h
 
 
+def serving(args, cfg, model, full_layers: int) -> int:
+    """Continuous batching end to end: every request through the scheduler, the step function and the sampler."""
+    import torch
+
+    from pulse_infer_amd.engine.engine import ContinuousBatchEngine
+    from pulse_infer_amd.sampling.params import SamplingParams
+
+    gen = torch.Generator().manual_seed(args.seed)
+    lo, hi = args.prompt_range
+    lengths = torch.randint(lo, hi + 1, (args.requests,), generator=gen).tolist()
+    per_request = hi + args.output_tokens + args.page_size
+    pages = args.requests * ((per_request + args.page_size - 1) // args.page_size)
+    engine = ContinuousBatchEngine(model, max_batch_size=args.requests, chunk_size=args.chunk, page_size=args.page_size,
+                                   num_pages=pages, max_sequences=args.requests,
+                                   max_num_batched_tokens=args.chunk + args.requests, seed=args.seed)
+    for i, n in enumerate(lengths):
+        prompt = torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
+        engine.add_request(prompt, args.output_tokens,
+                           SamplingParams(temperature=args.temperature, seed=args.seed + i, ignore_eos=True))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    engine.run_until_complete()
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    stats = engine.get_stats()
+    total = stats.tokens_generated
+    print(json.dumps({
+        "metric": f"qwen3_{args.model}_serving_output_tokens_per_s", "value": round(total / seconds, 2), "unit": "tokens/s",
+        "n_gpus": 1, "steps": stats.num_steps, "warmup": 0, "ms_per_step": round(seconds * 1e3 / max(1, stats.num_steps), 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"model": f"Qwen3-{args.model.upper()} shape, random weights", "global_batch": args.requests,
+                   "seq_len": hi + args.output_tokens, "parallelism": "single GPU", "layers": args.layers,
+                   "layers_full_model": full_layers, "requests": args.requests, "prompt_min": lo, "prompt_max": hi,
+                   "output_tokens": args.output_tokens, "chunk": args.chunk, "temperature": args.temperature,
+                   "prompt_tokens": sum(lengths), "preemptions": stats.num_preemptions},
+        "seconds": round(seconds, 3), "tokens_computed": stats.tokens_computed}))
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -86,11 +139,18 @@ def main() -> int:
 
     torch.backends.cuda.matmul.allow_tf32 = False
     device = torch.device("cuda:0")
-    cfg_dict = dict(QWEN3_8B, num_hidden_layers=args.layers)
+    shape = SHAPES[args.model]
+    full_layers = shape["num_hidden_layers"]
+    if args.layers is None:
+        args.layers = full_layers
+    cfg_dict = dict(shape, num_hidden_layers=args.layers)
     cfg = Qwen3Config.from_dict(cfg_dict, "<bench>")
     element = 2 if args.dtype == "bfloat16" else 4
     source = RandomSource(expected_tensors(cfg.model_spec()), args.seed, 0.02, torch.bfloat16, device=device)
     model = build_model(cfg, source, mode=args.dtype, device=device)
+
+    if args.workload == "serving":
+        return serving(args, cfg, model, full_layers)
 
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     max_batch = max(batches)
@@ -157,13 +217,13 @@ def main() -> int:
     step_bytes = weight_bytes(cfg, element) + args.batch * mean_ctx * kv_bytes_per_token(cfg, element)
     achieved = step_bytes / step_s / 1e9
     result = {
-        "metric": f"qwen3_8b_decode_tokens_per_s_batch{args.batch}", "value": round(value, 2), "unit": "tokens/s",
+        "metric": f"qwen3_{args.model}_decode_tokens_per_s_batch{args.batch}", "value": round(value, 2), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "config": {
-            "model": "Qwen3-8B shape, random weights", "global_batch": args.batch, "seq_len": args.context,
-            "parallelism": "single GPU", "layers": args.layers, "layers_full_model": FULL_LAYERS,
+            "model": f"Qwen3-{args.model.upper()} shape, random weights", "global_batch": args.batch, "seq_len": args.context,
+            "parallelism": "single GPU", "layers": args.layers, "layers_full_model": full_layers,
             "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
             "num_attention_heads": cfg.num_attention_heads, "num_key_value_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "vocab_size": cfg.vocab_size, "rope_theta": cfg.rope_theta,

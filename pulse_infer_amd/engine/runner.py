@@ -225,6 +225,7 @@ class ModelRunner:
     # the host then only copies the step's integers and starts the graph.
     GRAPH_MAX_BATCH = 16        # up to here every product is this package's own kernel (no library call is recorded)
     GRAPH_CONTEXT_BUCKET = 1024
+    GRAPH_LIMIT = 64            # recordings kept
 
     def _graph_ok(self, entries: Sequence[StepEntry], metas: List[EntryMeta]) -> bool:
         if not self.use_graphs or self.model.mode != "bfloat16" or len(metas) > self.GRAPH_MAX_BATCH:
@@ -243,6 +244,8 @@ class ModelRunner:
         if rec is None:
             rec = self._capture(key, entries, metas, want_rows)
             self._graphs[key] = rec
+            if len(self._graphs) > self.GRAPH_LIMIT:   # oldest recording out: contexts move on to higher buckets
+                self._graphs.pop(next(iter(self._graphs)))
         rec.wait()
         self._fill(rec.host_np, rec.offsets, entries, metas, want_rows, rec.widths)
         rec.dev.copy_(rec.host, non_blocking=True)
