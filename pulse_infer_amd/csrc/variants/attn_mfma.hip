@@ -70,6 +70,7 @@ struct MfmaArgs {
     int gp;           // columns per token: the group size rounded up to a power of two, at most 16
     int head_chunks;  // ceil(group / 16)
     int page_size, num_pages;
+    int page_shift;   // log2(page_size) when it is a power of two, else -1
     float scale_log2e;
     int window;
     int split_size;  // multiple of 32
@@ -79,6 +80,18 @@ struct MfmaArgs {
 // A value that is the same in every lane of the wavefront, said so to the compiler: what depends on it becomes
 // scalar work and uniform branches.
 __device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// Page index and slot of a key: a shift when the page size is a power of two (divisions by a run-time
+// number cost dozens of scalar instructions in the inner loop).
+__device__ __forceinline__ void page_of(int j, int page_size, int page_shift, int& pi, int& slot) {
+    if (page_shift >= 0) {
+        pi = j >> page_shift;
+        slot = j & (page_size - 1);
+    } else {
+        pi = j / page_size;
+        slot = j - pi * page_size;
+    }
+}
 
 __device__ __forceinline__ bf16x8 zero8() {
     bf16x8 z;
@@ -157,10 +170,10 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int jt = j0 + 16 * t;
-            const int pi = jt / a.page_size;
+            int pi, slot0;
+            page_of(jt, a.page_size, a.page_shift, pi, slot0);
             int page = (jt <= hi && pi < a.bt_width) ? bt[pi] : 0;
             page = (page >= 0 && page < a.num_pages) ? page : 0;  // masked keys may sit in pages given back
-            const int slot0 = jt % a.page_size;
             const int64_t pg = static_cast<int64_t>(page) * a.nkv + g;
             const bf16_t* krow = a.kc + (pg * a.page_size + slot0 + r) * D;
 #pragma unroll
@@ -388,10 +401,10 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int jt = j0 + 16 * t;
-            const int pi = jt / a.page_size;
+            int pi, slot0;
+            page_of(jt, a.page_size, a.page_shift, pi, slot0);
             int page = (jt <= hi && pi < a.bt_width) ? uniform(bt[pi]) : 0;
             page = (page >= 0 && page < a.num_pages) ? page : 0;
-            const int slot0 = jt % a.page_size;
             const int64_t pg = static_cast<int64_t>(page) * a.nkv + g;
             kbase[t] = (pg * a.page_size + slot0) * D;
             vbase[t] = pg * D * a.page_size + slot0;
@@ -637,6 +650,7 @@ extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64
     a.positions = positions; a.token_entry = token_entry; a.block_table = block_table; a.items = items;
     a.bt_width = bt_width; a.nq = nq; a.nkv = nkv; a.group = group; a.gp = gp; a.head_chunks = (group + 15) / 16;
     a.page_size = page_size; a.num_pages = num_pages;
+    a.page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
     a.scale_log2e = scale * 1.4426950408889634f;
     a.window = window; a.split_size = split_size; a.n_splits = n_splits;
     hipLaunchKernelGGL(attn_mfma_kernel, dim3(n_items, nkv * a.head_chunks, n_splits), dim3(WAVES * PULSE_WAVE), 0,
@@ -681,6 +695,7 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
     a.positions = positions; a.token_entry = token_entry; a.block_table = block_table; a.items = items;
     a.bt_width = bt_width; a.nq = nq; a.nkv = nkv; a.group = group; a.gp = gp; a.head_chunks = (group + 15) / 16;
     a.page_size = page_size; a.num_pages = num_pages;
+    a.page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
     a.scale_log2e = scale * 1.4426950408889634f;
     a.window = window; a.split_size = 0; a.n_splits = 1;
     hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_items, nkv * a.head_chunks), dim3(WAVES * PULSE_WAVE), 0, stream, a,
