@@ -23,6 +23,7 @@ constexpr int XLDS_BYTES = 16384;  // the most LDS a workgroup takes for X: more
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
 
 enum OutMode : int { OUT_BF16 = 0, OUT_F32 = 1, OUT_ADD_F32 = 2 };
 
@@ -31,6 +32,80 @@ __device__ __forceinline__ bf16x8 zeros8() {
 #pragma unroll
     for (int e = 0; e < 8; ++e) z[e] = (__bf16)0.0f;
     return z;
+}
+
+// Lane i of a row of 16 lanes takes the value of lane i + N; lanes without a source take zero.
+template <int N>
+__device__ __forceinline__ int row_shift_left(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, 0x100 + N /* row_shl:N */, 0xF, 0xF, true);
+}
+
+__device__ __forceinline__ int row_shift_left(int v, int n) {
+    switch (n) {  // n is a constant after unrolling: the switch folds to one instruction
+        case 1: return row_shift_left<1>(v);
+        case 2: return row_shift_left<2>(v);
+        case 3: return row_shift_left<3>(v);
+        case 4: return row_shift_left<4>(v);
+        case 5: return row_shift_left<5>(v);
+        case 6: return row_shift_left<6>(v);
+        case 7: return row_shift_left<7>(v);
+        case 8: return row_shift_left<8>(v);
+        case 9: return row_shift_left<9>(v);
+        case 10: return row_shift_left<10>(v);
+        case 11: return row_shift_left<11>(v);
+        case 12: return row_shift_left<12>(v);
+        case 13: return row_shift_left<13>(v);
+        case 14: return row_shift_left<14>(v);
+        case 15: return row_shift_left<15>(v);
+        default: return v;
+    }
+}
+
+// Sum of the wavefronts' partial tiles, in wavefront order, and the store.
+template <int SLABS, int MT, int KW, bool SWIGLU>
+__device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void* __restrict__ C, int64_t ldc, int M, int N,
+                                         int n_base, int mode, int tid) {
+    constexpr int TILES = SLABS * MT;
+    constexpr int THREADS = KW * PULSE_WAVE;
+    if (!SWIGLU) {
+        for (int e = tid; e < TILES * 256; e += THREADS) {
+            const int tile = e / 256;
+            const int m_in = (e % 256) / 16;
+            const int n_in = e % 16;
+            float v = 0.f;
+#pragma unroll
+            for (int w = 0; w < KW; ++w) v += red[w][tile][n_in][m_in];
+            const int m = (tile % MT) * 16 + m_in;
+            const int n = n_base + (tile / MT) * 16 + n_in;
+            if (m < M && n < N) {
+                const int64_t at = static_cast<int64_t>(m) * ldc + n;
+                if (mode == OUT_BF16) static_cast<bf16_t*>(C)[at] = f32_to_bf16(v);
+                else if (mode == OUT_F32) static_cast<float*>(C)[at] = v;
+                else static_cast<float*>(C)[at] += v;
+            }
+        }
+    } else {
+        // slabs come in (gate, up) pairs; the output has half as many columns
+        constexpr int PAIRS = SLABS / 2;
+        for (int e = tid; e < PAIRS * MT * 256; e += THREADS) {
+            const int pt = e / 256;  // pair * MT + mt
+            const int m_in = (e % 256) / 16;
+            const int n_in = e % 16;
+            const int pair = pt / MT, mt = pt % MT;
+            float g = 0.f, u = 0.f;
+#pragma unroll
+            for (int w = 0; w < KW; ++w) {
+                g += red[w][(2 * pair) * MT + mt][n_in][m_in];
+                u += red[w][(2 * pair + 1) * MT + mt][n_in][m_in];
+            }
+            const int m = mt * 16 + m_in;
+            const int n = n_base / 2 + pair * 16 + n_in;
+            if (m < M && 2 * n < N) {  // N counts gate and up rows together
+                const float v = g / (1.0f + expf(-g)) * u;
+                static_cast<bf16_t*>(C)[static_cast<int64_t>(m) * ldc + n] = f32_to_bf16(v);
+            }
+        }
+    }
 }
 
 // SLABS slabs of 16 weight rows a workgroup, MT tiles of 16 rows of X, KW wavefronts sharing K.
@@ -149,45 +224,117 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_kernel(const bf16_
             for (int i = 0; i < 4; ++i) red[wave][s * MT + mt][4 * kg + i][r] = acc[s][mt][i];
     __syncthreads();
 
-    if (!SWIGLU) {
-        for (int e = tid; e < TILES * 256; e += THREADS) {
-            const int tile = e / 256;
-            const int m_in = (e % 256) / 16;
-            const int n_in = e % 16;
-            float v = 0.f;
+    epilogue<SLABS, MT, KW, SWIGLU>(red, C, ldc, M, N, n_base, mode, tid);
+}
+
+// The streaming kernel for at most 16 rows of X when K is a multiple of 256 * KW (every wavefront then runs whole
+// groups of UNROLL k-steps).  Two things set it apart from the kernel above:
+//
+//  * Weight loads cover whole 128-byte lines.  Two k-steps (64 values of k) are fetched by two loads of 8 rows x
+//    128 bytes each instead of two loads of 16 rows x 64 bytes: load 0 takes rows 0-7, load 1 rows 8-15; a lane in the
+//    lower half of its row of 16 lanes fetches 16 bytes of the first k-step from load 0 and of the second from load
+//    1, a lane in the upper half the other way round.  One select a register and one rotation by 8 lanes (DPP) then
+//    put every value where the matrix-core operand expects it.
+//  * X loads are packed.  With M <= 16 / PACK rows, the 16 column lanes of the X^T operand hold PACK consecutive
+//    k-steps of the same rows (lane c: row c % (16 / PACK), k-step c / (16 / PACK)), so one load serves PACK steps
+//    and a DPP shift hands each step its columns.  Columns beyond M read as zero.
+//
+// Both only change which lane fetches what; every product and the order of the sums are those of the kernel above.
+template <int SLABS, int KW, int PACK, bool SWIGLU>
+__global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(const bf16_t* __restrict__ X, int64_t ldx,
+                                                                             const bf16_t* __restrict__ W, int64_t ldw,
+                                                                             void* __restrict__ C, int64_t ldc, int M,
+                                                                             int N, int K, int mode) {
+    static_assert(PACK == 1 || PACK == 2 || PACK == 4 || PACK == 8, "PACK k-steps a load of X");
+    static_assert(UNROLL % 2 == 0 && UNROLL % PACK == 0, "groups hold whole pairs and whole packs");
+    constexpr int MP = 16 / PACK;  // rows of X a pack has room for
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    float (*red)[SLABS][16][17] = reinterpret_cast<float (*)[SLABS][16][17]>(smem);
+
+    const int tid = threadIdx.x;
+    const int wave = tid / PULSE_WAVE;
+    const int lane = tid % PULSE_WAVE;
+    const int r = lane % 16;
+    const int kg = lane / 16;
+    const int n_base = blockIdx.x * SLABS * 16;
+    const int per = K / 32 / KW;  // a multiple of UNROLL (checked by the caller)
+    const int step_begin = wave * per;
+    const bool low = r < 8;
+
+    f32x4 acc[SLABS];
 #pragma unroll
-            for (int w = 0; w < KW; ++w) v += red[w][tile][n_in][m_in];
-            const int m = (tile % MT) * 16 + m_in;
-            const int n = n_base + (tile / MT) * 16 + n_in;
-            if (m < M && n < N) {
-                const int64_t at = static_cast<int64_t>(m) * ldc + n;
-                if (mode == OUT_BF16) static_cast<bf16_t*>(C)[at] = f32_to_bf16(v);
-                else if (mode == OUT_F32) static_cast<float*>(C)[at] = v;
-                else static_cast<float*>(C)[at] += v;
-            }
-        }
-    } else {
-        // slabs come in (gate, up) pairs; the output has half as many columns
-        constexpr int PAIRS = SLABS / 2;
-        for (int e = tid; e < PAIRS * MT * 256; e += THREADS) {
-            const int pt = e / 256;  // pair * MT + mt
-            const int m_in = (e % 256) / 16;
-            const int n_in = e % 16;
-            const int pair = pt / MT, mt = pt % MT;
-            float g = 0.f, u = 0.f;
+    for (int s = 0; s < SLABS; ++s) acc[s] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // rows beyond N repeat the last row: their products only reach outputs that are never stored
+    const bf16_t* w0[SLABS];
+    const bf16_t* w1[SLABS];
 #pragma unroll
-            for (int w = 0; w < KW; ++w) {
-                g += red[w][(2 * pair) * MT + mt][n_in][m_in];
-                u += red[w][(2 * pair + 1) * MT + mt][n_in][m_in];
-            }
-            const int m = mt * 16 + m_in;
-            const int n = n_base / 2 + pair * 16 + n_in;
-            if (m < M && 2 * n < N) {  // N counts gate and up rows together
-                const float v = g / (1.0f + expf(-g)) * u;
-                static_cast<bf16_t*>(C)[static_cast<int64_t>(m) * ldc + n] = f32_to_bf16(v);
-            }
-        }
+    for (int s = 0; s < SLABS; ++s) {
+        const int n0 = min(n_base + s * 16 + (r & 7), N - 1);
+        const int n1 = min(n_base + s * 16 + 8 + (r & 7), N - 1);
+        w0[s] = W + static_cast<int64_t>(n0) * ldw + (kg + (low ? 0 : 4)) * 8;
+        w1[s] = W + static_cast<int64_t>(n1) * ldw + (kg + (low ? 4 : 0)) * 8;
     }
+    const int xr = r % MP;
+    const bool xok = xr < M;
+    const bf16_t* xrow = X + static_cast<int64_t>(xok ? xr : 0) * ldx + (r / MP) * 32 + kg * 8;
+
+    for (int ks = step_begin; ks < step_begin + per; ks += UNROLL) {
+        bf16x8 xb[UNROLL], wa[UNROLL][SLABS];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int pair_k = ((ks + u) & ~1) * 32;
+#pragma unroll
+            for (int s = 0; s < SLABS; ++s)
+                wa[u][s] = *reinterpret_cast<const bf16x8*>(((u & 1) ? w1[s] : w0[s]) + pair_k);
+            if (u % PACK == 0) {
+                xb[u] = zeros8();
+                if (xok) xb[u] = *reinterpret_cast<const bf16x8*>(xrow + (ks + u) * 32);
+            }
+        }
+        // every load of the group is on its way; now the lane exchanges
+#pragma unroll
+        for (int u = 0; u < UNROLL; u += 2) {
+#pragma unroll
+            for (int s = 0; s < SLABS; ++s) {
+                const i32x4 l0 = __builtin_bit_cast(i32x4, wa[u][s]);
+                const i32x4 l1 = __builtin_bit_cast(i32x4, wa[u + 1][s]);
+                i32x4 a0, a1;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    a0[e] = low ? l0[e] : l1[e];
+                    const int other = low ? l1[e] : l0[e];
+                    a1[e] = __builtin_amdgcn_mov_dpp(other, 0x128 /* row_ror:8 */, 0xF, 0xF, true);
+                }
+                wa[u][s] = __builtin_bit_cast(bf16x8, a0);
+                wa[u + 1][s] = __builtin_bit_cast(bf16x8, a1);
+            }
+        }
+        if (PACK > 1) {
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                if (u % PACK != 0) {
+                    const i32x4 src = __builtin_bit_cast(i32x4, xb[u - u % PACK]);
+                    i32x4 moved;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) moved[e] = row_shift_left(src[e], (u % PACK) * MP);
+                    xb[u] = __builtin_bit_cast(bf16x8, moved);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+            for (int s = 0; s < SLABS; ++s)
+                acc[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[u][s], xb[u], acc[s], 0, 0, 0);
+    }
+
+#pragma unroll
+    for (int s = 0; s < SLABS; ++s)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[wave][s][4 * kg + i][r] = acc[s][i];
+    __syncthreads();
+    epilogue<SLABS, 1, KW, SWIGLU>(red, C, ldc, M, N, n_base, mode, tid);
 }
 
 template <int SLABS, int MT, int KW, bool SWIGLU>
@@ -205,12 +352,32 @@ void launch(bool xlds, const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ld
     }
 }
 
+
+template <int SLABS, int KW, bool SWIGLU>
+void launch_stream(int pack, const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
+                   int K, int mode, hipStream_t stream) {
+    const dim3 grid((N + SLABS * 16 - 1) / (SLABS * 16)), block(KW * PULSE_WAVE);
+    const size_t red_bytes = sizeof(float) * KW * SLABS * 16 * 17;
+#define PULSE_STREAM(P)                                                                                               \
+    hipLaunchKernelGGL((gemm_skinny_stream_kernel<SLABS, KW, P, SWIGLU>), grid, block, red_bytes, stream, X, ldx, W, ldw, \
+                       C, ldc, M, N, K, mode)
+    if (pack == 8) PULSE_STREAM(8);
+    else if (pack == 4) PULSE_STREAM(4);
+    else if (pack == 2) PULSE_STREAM(2);
+    else PULSE_STREAM(1);
+#undef PULSE_STREAM
+}
+
+// The most k-steps one load of X can serve for M rows.
+int pack_for(int M) { return M <= 2 ? 8 : (M <= 4 ? 4 : (M <= 8 ? 2 : 1)); }
+
 }  // namespace
 
 // mode: 0 store bfloat16, 1 store float32, 2 add into float32.  swiglu != 0: W holds gate and up rows interleaved in
-// slabs of 16 (gate slab, up slab, ...), N counts both, C is bfloat16 [M, N / 2] = silu(gate) * up.
+// slabs of 16 (gate slab, up slab, ...), N counts both, C is bfloat16 [M, N / 2] = silu(gate) * up.  tune: 0 lets the
+// entry point choose the kernel.
 extern "C" int pulse_gemm_skinny(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
-                                 int N, int K, int mode, int swiglu, hipStream_t stream) {
+                                 int N, int K, int mode, int swiglu, int tune, hipStream_t stream) {
     PULSE_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: sizes M=%d (at most 64) N=%d K=%d", M, N, K);
     PULSE_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K,
                   "gemm_skinny: K and the row strides must be multiples of 8 (16-byte loads)");
@@ -228,9 +395,39 @@ extern "C" int pulse_gemm_skinny(const void* X, int64_t ldx, const void* W, int6
     const bf16_t* x = static_cast<const bf16_t*>(X);
     const bf16_t* w = static_cast<const bf16_t*>(W);
     const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+    const bool wide = N >= 16384;  // enough slabs that pairs of them still fill the chip
+    // tune (tests and measurements): decimal digits S K P, S slabs (1, 2), K wavefronts (4, 8), P = 1 + log2 of the
+    // k-steps a load of X serves (1..4), all for the streaming kernel; 9 asks for the general kernel.
+    int t_slabs = 0, t_kw = 0, t_pack = 0;
+    if (tune > 0 && tune != 9) {
+        t_slabs = tune / 100, t_kw = tune / 10 % 10, t_pack = 1 << (tune % 10 - 1);
+        PULSE_REQUIRE((t_slabs == 1 || t_slabs == 2) && (t_kw == 4 || t_kw == 8) && tune % 10 >= 1 && tune % 10 <= 4,
+                      "gemm_skinny: unknown tuning %d", tune);
+        PULSE_REQUIRE(mt == 1 && K % (256 * t_kw) == 0 && M <= 16 / t_pack && (!swiglu || t_slabs == 2),
+                      "gemm_skinny: tuning %d does not fit M=%d K=%d", tune, M, K);
+    }
+    if (mt == 1 && tune != 9 && (t_kw ? true : K % 1024 == 0)) {
+        // the streaming kernel: pairs of slabs when there are many (or, from 8 rows of X on, enough of them: a
+        // pair shares its loads of X), else single slabs with more wavefronts along K
+        const bool pairs = swiglu || wide || (N >= 6144 && M >= 8);
+        const int slabs = t_slabs ? t_slabs : (pairs ? 2 : 1);
+        const int kw = t_kw ? t_kw : ((K % 2048 == 0 && !pairs) ? 8 : 4);
+        const int pack = t_pack ? t_pack : pack_for(M);
+        if (swiglu) {
+            if (kw == 8) launch_stream<2, 8, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+            else launch_stream<2, 4, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+        } else if (slabs == 2) {
+            if (kw == 8) launch_stream<2, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+            else launch_stream<2, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+        } else {
+            if (kw == 8) launch_stream<1, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+            else launch_stream<1, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+        }
+        PULSE_LAUNCH_CHECK("gemm_skinny");
+        return 0;
+    }
     // X goes through LDS when it is small enough for two workgroups a compute unit
     const bool xlds = mt == 1 && K % 32 == 0 && static_cast<size_t>(K) * M * 2 <= XLDS_BYTES;
-    const bool wide = N >= 16384;  // enough slabs that pairs of them still fill the chip
     if (swiglu) {
         if (mt == 1) launch<2, 1, 4, true>(xlds, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
         else launch<2, 2, 8, true>(false, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);

@@ -163,11 +163,13 @@ def gemm_skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
             and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool = False, swiglu: bool = False) -> None:
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool = False, swiglu: bool = False,
+                tune: int = 0) -> None:
     """out = a @ w^T for at most 64 rows of bfloat16, float32 accumulation on the matrix cores.
 
     ``out`` bfloat16 or float32 is stored; with ``add`` (float32 only) the product is added to it.  With
     ``swiglu`` the weight holds gate and up rows in alternating slabs of 16 and out is silu(gate) * up.
+    ``tune`` picks a kernel variant by hand (tests and measurements); 0 lets the library choose.
     """
     _gpu("gemm_skinny", a, w, out)
     _need(gemm_skinny_ok(a, w), "gemm_skinny: needs bfloat16 operands with at most 64 rows, K a multiple of 8, "
@@ -188,7 +190,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool =
               "gemm_skinny: the SwiGLU epilogue needs at most 32 rows, N a multiple of 32 and bfloat16 output")
     call("pulse_gemm_skinny", _ptr(a), _i64(a.stride(0) if m > 1 else k), _ptr(w), _i64(w.stride(0) if n > 1 else k),
          _ptr(out), _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode),
-         _i32(1 if swiglu else 0), _stream())
+         _i32(1 if swiglu else 0), _i32(tune), _stream())
 
 
 def _check_cache(what: str, kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, d: int):

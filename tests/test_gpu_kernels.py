@@ -471,8 +471,42 @@ def test_gemm_skinny(k, m, n, kk):
         assert torch.equal(again, out32)
 
 
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 7, 8, 11, 16])
+@pytest.mark.parametrize("n,kk", [(40, 2048), (509, 1024), (96, 3072), (33, 4096)])
+def test_gemm_skinny_streaming_variants(k, m, n, kk):
+    """Every variant of the streaming kernel (slabs, wavefronts, k-steps a load of X) against the general kernel
+    and float64: a lane that fetched the wrong row or k-step would change the sums."""
+    a, aref = as_stored(rnd(m, kk, seed=76), torch.bfloat16)
+    w, wref = as_stored(rnd(n, kk, seed=77), torch.bfloat16)
+    want = aref @ wref.T
+    general = torch.empty(m, n, device=DEV)
+    k.gemm_skinny(a, w, general, tune=9)
+    assert torch.allclose(general.cpu().to(F64), want, atol=2e-3 * math.sqrt(kk), rtol=1e-5)
+    ran = 0
+    for slabs in (1, 2):
+        for kw in (4, 8):
+            if kk % (256 * kw):
+                continue
+            for p in (1, 2, 3, 4):
+                if m > 16 >> (p - 1):
+                    continue
+                out = torch.full((m, n), float("nan"), device=DEV)
+                k.gemm_skinny(a, w, out, tune=slabs * 100 + kw * 10 + p)
+                if kw == 4:      # the same split of K as the general kernel: the same sums in the same order
+                    assert torch.equal(out, general), (slabs, kw, p)
+                else:
+                    assert torch.allclose(out.cpu().to(F64), want, atol=2e-3 * math.sqrt(kk), rtol=1e-5), (slabs, kw, p)
+                ran += 1
+    assert ran >= 2
+    auto = torch.empty(m, n, device=DEV)
+    k.gemm_skinny(a, w, auto)
+    assert torch.allclose(auto.cpu().to(F64), want, atol=2e-3 * math.sqrt(kk), rtol=1e-5)
+    with pytest.raises(Exception, match="does not fit|unknown tuning"):
+        k.gemm_skinny(a, w, auto, tune=184 if m > 2 else 777)
+
+
 @pytest.mark.parametrize("m", [1, 8, 20, 32])
-@pytest.mark.parametrize("inter,kk", [(32, 64), (224, 96), (176, 80), (12288 // 8, 256)])
+@pytest.mark.parametrize("inter,kk", [(32, 64), (224, 96), (176, 80), (12288 // 8, 256), (48, 2048), (176, 1024)])
 def test_gemm_skinny_swiglu(k, m, inter, kk):
     a, aref = as_stored(rnd(m, kk, seed=73), torch.bfloat16)
     gate, gref = as_stored(rnd(inter, kk, seed=74, scale=kk ** -0.5), torch.bfloat16)
