@@ -230,14 +230,16 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_kernel(const bf16_
 // The streaming kernel for at most 16 rows of X when K is a multiple of 256 * KW (every wavefront then runs whole
 // groups of UNROLL k-steps).  Two things set it apart from the kernel above:
 //
-//  * Weight loads cover whole 128-byte lines.  Two k-steps (64 values of k) are fetched by two loads of 8 rows x
-//    128 bytes each instead of two loads of 16 rows x 64 bytes: load 0 takes rows 0-7, load 1 rows 8-15; a lane in the
-//    lower half of its row of 16 lanes fetches 16 bytes of the first k-step from load 0 and of the second from load
-//    1, a lane in the upper half the other way round.  One select a register and one rotation by 8 lanes (DPP) then
-//    put every value where the matrix-core operand expects it.
+//  * Weight loads are contiguous.  The matrix-core operand wants 16 rows x 16 bytes from every 16 consecutive
+//    lanes, which costs a memory request a lane.  Here 16 consecutive lanes fetch two whole 128-byte lines
+//    instead: two k-steps (64 values of k) of a slab are two loads of 8 rows x 128 bytes, load h giving lane
+//    (q = lane / 16, i = lane % 16) row 2q + i/8 + 8h and the i%8-th 16 bytes of the line.  A DPP move by four
+//    lanes then trades the halves of the lines between the two registers (register = k-step afterwards), and one
+//    ds_bpermute a register brings every value to the lane whose row and k-group the operand expects.
 //  * X loads are packed.  With M <= 16 / PACK rows, the 16 column lanes of the X^T operand hold PACK consecutive
 //    k-steps of the same rows (lane c: row c % (16 / PACK), k-step c / (16 / PACK)), so one load serves PACK steps
-//    and a DPP shift hands each step its columns.  Columns beyond M read as zero.
+//    and a DPP shift hands each step its columns.  Columns beyond M read as zero.  (Contiguous loads of X with a
+//    ds_bpermute a step were measured too and gain nothing.)
 //
 // Both only change which lane fetches what; every product and the order of the sums are those of the kernel above.
 template <int SLABS, int KW, int PACK, bool SWIGLU>
@@ -259,7 +261,6 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
     const int n_base = blockIdx.x * SLABS * 16;
     const int per = K / 32 / KW;  // a multiple of UNROLL (checked by the caller)
     const int step_begin = wave * per;
-    const bool low = r < 8;
 
     f32x4 acc[SLABS];
 #pragma unroll
@@ -270,11 +271,13 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
     const bf16_t* w1[SLABS];
 #pragma unroll
     for (int s = 0; s < SLABS; ++s) {
-        const int n0 = min(n_base + s * 16 + (r & 7), N - 1);
-        const int n1 = min(n_base + s * 16 + 8 + (r & 7), N - 1);
-        w0[s] = W + static_cast<int64_t>(n0) * ldw + (kg + (low ? 0 : 4)) * 8;
-        w1[s] = W + static_cast<int64_t>(n1) * ldw + (kg + (low ? 4 : 0)) * 8;
+        const int row = n_base + s * 16 + 2 * kg + (r >> 3);
+        w0[s] = W + static_cast<int64_t>(min(row, N - 1)) * ldw + (r & 7) * 8;
+        w1[s] = W + static_cast<int64_t>(min(row + 8, N - 1)) * ldw + (r & 7) * 8;
     }
+    // after the exchange of halves, lane (q, i) holds row 2q + i/8 + 8 * (i/4 % 2) and k-group i % 4 of the step;
+    // the operand's lane (kg, r) takes it from there
+    const int source_lane = 16 * ((r >> 1) & 3) + 8 * (r & 1) + 4 * (r >> 3) + kg;
     const int xr = r % MP;
     const bool xok = xr < M;
     const bf16_t* xrow = X + static_cast<int64_t>(xok ? xr : 0) * ldx + (r / MP) * 32 + kg * 8;
@@ -302,9 +305,12 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
                 i32x4 a0, a1;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    a0[e] = low ? l0[e] : l1[e];
-                    const int other = low ? l1[e] : l0[e];
-                    a1[e] = __builtin_amdgcn_mov_dpp(other, 0x128 /* row_ror:8 */, 0xF, 0xF, true);
+                    // lanes 4-7 and 12-15 of a row of 16 take the first half-line of rows 8-15 from four lanes below
+                    const int first = __builtin_amdgcn_update_dpp(l0[e], l1[e], 0x114 /* row_shr:4 */, 0xF, 0xA, false);
+                    // lanes 0-3 and 8-11 take the second half-line of rows 0-7 from four lanes above
+                    const int second = __builtin_amdgcn_update_dpp(l1[e], l0[e], 0x104 /* row_shl:4 */, 0xF, 0x5, false);
+                    a0[e] = __builtin_amdgcn_ds_bpermute(source_lane * 4, first);
+                    a1[e] = __builtin_amdgcn_ds_bpermute(source_lane * 4, second);
                 }
                 wa[u][s] = __builtin_bit_cast(bf16x8, a0);
                 wa[u + 1][s] = __builtin_bit_cast(bf16x8, a1);
