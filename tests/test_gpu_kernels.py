@@ -149,6 +149,9 @@ def _tables(k, positions, theta, rot):
     dict(nq=4, nkv=1, d=80, rot=32, pairing="interleaved", norm=True, bs=8),    # partial rotation, tail untouched
     dict(nq=3, nkv=3, d=160, rot=160, pairing="half", norm=False, bs=16),       # other pairing, no norm, > 128 channels
     dict(nq=2, nkv=1, d=32, rot=0, pairing="interleaved", norm=True, bs=2),     # no position encoding at all
+    dict(nq=7, nkv=7, d=64, rot=32, pairing="half", norm=True, bs=16),          # other pairing, partial rotation
+    dict(nq=5, nkv=1, d=128, rot=128, pairing="interleaved", norm=True, bs=16), # heads no multiple of a wavefront's share
+    dict(nq=2, nkv=2, d=20, rot=12, pairing="half", norm=True, bs=4),           # sizes only the element-wise kernel takes
 ])
 def test_qk_rope_kv(k, dtype, case):
     nq, nkv, d, rot, bs = case["nq"], case["nkv"], case["d"], case["rot"], case["bs"]
