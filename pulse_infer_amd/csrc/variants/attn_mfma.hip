@@ -39,6 +39,11 @@ constexpr int NCHUNK = (D + 31) / 32;  // 32-wide slices of the q.k contraction
 constexpr int NDT = D / 16;            // 16-channel tiles of the output
 constexpr int WAVES = 4;
 constexpr int BLOCK_KEYS = 32;
+// Column tiles a wavefront takes in the prompt-portion kernel: two while the accumulators of both fit the registers.
+#define PULSE_WIDE (PULSE_HEAD_DIM == 32 || PULSE_HEAD_DIM == 64 || PULSE_HEAD_DIM == 128)
+constexpr int PREFILL_TILES = PULSE_WIDE ? 2 : 1;
+constexpr int WIDE_NW = 4;   // wavefronts of the wide prompt-portion kernel
+constexpr int WIDE_CT = 2;   // column tiles each takes
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -570,6 +575,301 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     }
 }
 
+#if PULSE_WIDE
+// ---------------------------------------------------------------------------------------------------------
+// Prompt portions, wide: the same scheme with CT column tiles a wavefront (CT * 16 / G' tokens) and blocks of
+// KT * 16 keys, so that every K and V operand read from LDS feeds CT products and the work around a block (the
+// addresses, the loop, the barriers) is spread over CT * KT / 2 times as many scores.  The latencies inside a
+// block's chain, not the matrix cores, bound this kernel, so the copy must stay out of that chain: K and V go from
+// memory straight into LDS (global_load_lds_dwordx4: 16 bytes a lane, lane i to the wavefront's LDS base + 16 i),
+// two stages, the next block on its way while this one is computed, with no register in between.
+//
+// LDS holds 16-byte pieces without padding; which piece a lane fetches is chosen so that the matrix-core operand
+// reads are free of bank conflicts:
+//   K: piece c of key j (P = D / 8 pieces a key) sits at slot j * P + (c + rot(j)) % P, rot(j) = (j * P / 16) % P, so
+//      the 16 keys that 16 consecutive lanes read for one c lie in 16 different 16-byte bank groups;
+//   V: a tile of 16 keys is D channel rows of 32 bytes; the piece (channel ch, half h) sits at slot
+//      (ch / 16) * 32 + h * 16 + ch % 16, so the 16 channel rows of one half are 256 contiguous bytes.
+// Needs D in {32, 64, 128} (P a power of two, whole 1 KB chunks a tile).
+//
+// The loads are written in assembly: the compiler knows nothing of them (it would wait for every one before any LDS
+// read), so the waits for them are written here too.  Its own vector loads inside the loop (the block table) only
+// ever make it wait longer, never shorter: the counter runs in issue order.
+template <int CT, int KT, int NW>
+struct WideShape {
+    static constexpr int BK = KT * 16;                    // keys a block
+    static constexpr int P = D / 8;                       // 16-byte pieces a key row
+    static constexpr int STAGE_K = BK * D;                // bfloat16 elements
+    static constexpr int STAGE_V = KT * D * 16;
+    static constexpr int STAGE = STAGE_K + STAGE_V;
+    static constexpr int TILE_CHUNKS = 16 * P / 64;       // 1 KB chunks (one load of a wavefront) of a key tile; as many of a value tile
+    static_assert(KT == NW, "a wavefront copies one key tile and one value tile of every block");
+};
+
+// 16 bytes a lane from memory straight into LDS: lane i's piece lands at lds_base + 16 i (a wavefront-wide address).
+__device__ __forceinline__ void load_to_lds(const void* from, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_base), "v"(from) : "memory", "m0");
+}
+
+template <int CT, int KT, int NW>
+__global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_prefill_wide_kernel(MfmaArgs a, int per) {
+    using Shape = WideShape<CT, KT, NW>;
+    constexpr int BK = Shape::BK;
+    static_assert(KT % 2 == 0, "the second product takes pairs of key tiles");
+    static_assert(D == 32 || D == 64 || D == 128, "whole 1 KB chunks and a power of two of pieces a key");
+    constexpr int P = Shape::P;
+    __shared__ __attribute__((aligned(1024))) bf16_t s_kv[2 * Shape::STAGE];  // stage: K block, then V block
+
+    // The second half of the kv heads walks the items backwards: a long item (a late portion of a prompt) then
+    // shares its compute unit with a short one instead of another long one, and the longest workgroups, which set
+    // the kernel's time, run at a lone workgroup's speed.
+    const int item = (blockIdx.y * 2 / gridDim.y) & 1 ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
+    const int g = blockIdx.y / a.head_chunks;
+    const int chunk = blockIdx.y % a.head_chunks;
+    const int tid = threadIdx.x;
+    const int wave = uniform(tid / PULSE_WAVE);
+    const int lane = tid % PULSE_WAVE;
+    const int r = lane % 16;
+    const int kg = lane / 16;
+
+    const int row0 = uniform(a.items[2 * item]);
+    const int ntok = uniform(a.items[2 * item + 1]);         // at most NW * CT * per
+    const int hi = uniform(a.positions[row0 + ntok - 1]);    // last key of the workgroup
+    const int pos_first = uniform(a.positions[row0]);
+    const int lo_item = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
+    const int* bt = a.block_table + static_cast<int64_t>(uniform(a.token_entry[row0])) * a.bt_width;
+
+    // this wavefront's column tiles and this lane's column in each
+    const int tc = r / a.gp;
+    const int hc = r % a.gp + chunk * 16;
+    bool col_ok[CT];
+    int col_row[CT], pos_c[CT], lo_c[CT];
+    int t_hi[CT], t_pos0[CT], t_lo[CT], t_hi_lo[CT];  // per tile: last and first position, lowest and highest window start
+    bool t_any[CT];
+    int col_head = g * a.group;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int wtok0 = (wave * CT + ct) * per;
+        const int wntok = max(0, min(per, ntok - wtok0));
+        t_any[ct] = wntok > 0;
+        col_ok[ct] = tc < wntok && hc < a.group;
+        col_row[ct] = row0 + (col_ok[ct] ? wtok0 + tc : 0);
+        pos_c[ct] = col_ok[ct] ? a.positions[col_row[ct]] : -1;
+        lo_c[ct] = (a.window > 0 && pos_c[ct] - a.window + 1 > 0) ? pos_c[ct] - a.window + 1 : 0;
+        t_hi[ct] = uniform(wntok > 0 ? a.positions[row0 + wtok0 + wntok - 1] : -1);
+        t_pos0[ct] = uniform(wntok > 0 ? a.positions[row0 + wtok0] : 0);
+        t_lo[ct] = (a.window > 0 && t_pos0[ct] - a.window + 1 > 0) ? t_pos0[ct] - a.window + 1 : 0;
+        t_hi_lo[ct] = (a.window > 0 && t_hi[ct] - a.window + 1 > 0) ? t_hi[ct] - a.window + 1 : 0;
+    }
+    if (hc < a.group) col_head += hc;
+    // keys this wavefront needs at all: from its first tile's window to its last tile's diagonal
+    int w_hi = -1;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) w_hi = max(w_hi, t_hi[ct]);
+    const int w_lo = t_lo[0];
+
+    bf16x8 bq[CT][NCHUNK];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const bf16_t* qrow = a.q + static_cast<int64_t>(col_row[ct]) * a.q_stride + static_cast<int64_t>(col_head) * D;
+#pragma unroll
+        for (int ch = 0; ch < NCHUNK; ++ch) {
+            const int off = ch * 32 + kg * 8;
+            bq[ct][ch] = (col_ok[ct] && off < D) ? *reinterpret_cast<const bf16x8*>(qrow + off) : zero8();
+        }
+    }
+    f32x4 acc[CT][NDT];
+    float m[CT], l_part[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) acc[ct][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        m[ct] = -INFINITY;
+        l_part[ct] = 0.f;
+    }
+
+    // The copy of a block: wavefront w brings key tile w and value tile w, in 1 KB chunks (one load each).  What a
+    // lane fetches of a chunk does not depend on the block: its offsets are computed once.  Only the page of the
+    // wavefront's tile changes from block to block.
+    const uint32_t lds0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+        (void __attribute__((address_space(3)))*)(&s_kv[0])));  // the array's address inside LDS
+    int k_from[Shape::TILE_CHUNKS], v_from[Shape::TILE_CHUNKS];
+#pragma unroll
+    for (int i = 0; i < Shape::TILE_CHUNKS; ++i) {
+        const int slot = 64 * i + lane;         // within the tile's 16 * P slots
+        const int key = slot / P, pos = slot % P;
+        const int c8 = (pos - (key * P / 16) % P + P) % P;
+        k_from[i] = key * D + c8 * 8;
+        const int blk = slot / 32, half = (slot / 16) % 2, chr = slot % 16;
+        v_from[i] = (blk * 16 + chr) * a.page_size + half * 8;
+    }
+    // The page of this wavefront's tile of block b: read from the block table without a branch (an index beyond
+    // the table reads its last entry; what it gives is not used) one block ahead of the copy that needs it.
+    auto page_ahead = [&](int b) {
+        int pi, slot0;
+        page_of(b * BK + 16 * wave, a.page_size, a.page_shift, pi, slot0);
+        // volatile: the load stays here, a block ahead of its use (the compiler would move it next to the use and
+        // wait for it there); it is said to be uniform only where it is used, not to wait here either
+        return *static_cast<const volatile int*>(bt + min(pi, a.bt_width - 1));
+    };
+    const int64_t page_elems = static_cast<int64_t>(a.nkv) * a.page_size * D;  // of K and of V alike
+    const int head_elems = g * a.page_size * D;
+    auto fetch = [&](int b, int page_read, int stage) {
+        const int jt = b * BK + 16 * wave;
+        int pi, slot0;
+        page_of(jt, a.page_size, a.page_shift, pi, slot0);
+        int page = (jt <= hi && pi < a.bt_width) ? uniform(page_read) : 0;
+        page = (page >= 0 && page < a.num_pages) ? page : 0;
+        const int64_t base = page * page_elems + head_elems;
+        const bf16_t* kfrom = a.kc + base + slot0 * D;
+        const bf16_t* vfrom = a.vc + base + slot0;
+        const uint32_t to = lds0 + stage * (Shape::STAGE * 2) + wave * (Shape::TILE_CHUNKS * 1024);
+#pragma unroll
+        for (int i = 0; i < Shape::TILE_CHUNKS; ++i) load_to_lds(kfrom + k_from[i], to + i * 1024);
+#pragma unroll
+        for (int i = 0; i < Shape::TILE_CHUNKS; ++i) load_to_lds(vfrom + v_from[i], to + Shape::STAGE_K * 2 + i * 1024);
+    };
+    // operand reads: K piece 4 ch + kg of key 16 t + r, V words of channel row 16 dt + r
+    int k_at[NCHUNK];
+#pragma unroll
+    for (int ch = 0; ch < NCHUNK; ++ch) k_at[ch] = (r * P + (4 * ch + kg + (r * P / 16) % P) % P) * 8;
+    const int v_at = ((kg >> 1) * 16 + r) * 8 + (kg & 1) * 4;
+
+    const float c2 = a.scale_log2e;
+    auto compute = [&](int b, int stage) {
+        const int j0 = b * BK;
+        const bf16_t* s_k = s_kv + stage * Shape::STAGE;
+        const bf16_t* s_v = s_k + Shape::STAGE_K;
+        f32x4 s[CT][KT];
+#pragma unroll
+        for (int t = 0; t < KT; ++t) {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) s[ct][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ch = 0; ch < NCHUNK; ++ch) {
+                const int off = ch * 32 + kg * 8;
+                const bf16x8 ak = off < D ? *reinterpret_cast<const bf16x8*>(&s_k[16 * t * D + k_at[ch]]) : zero8();
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct)
+                    s[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak, bq[ct][ch], s[ct][t], 0, 0, 0);
+            }
+        }
+        // the maximum is tracked on the raw scores (the scale is positive); p = exp2((s - m) * scale * log2 e)
+        bf16x8 pb[CT][KT / 2];
+        bool moved = false;
+        float alpha[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            // The mask without a branch: key j0 + 16 t + 4 kg + i is seen when 16 t + i lies in [lim_lo, lim_hi]
+            // (a compare with a constant and a select a score; a branch a score costs a lone wavefront more).
+            const int lim_hi = col_ok[ct] ? pos_c[ct] - j0 - 4 * kg : -1;
+            const int lim_lo = lo_c[ct] - j0 - 4 * kg;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < KT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float v = (16 * t + i <= lim_hi && 16 * t + i >= lim_lo) ? s[ct][t][i] : -INFINITY;
+                    s[ct][t][i] = v;
+                    mx = fmaxf(mx, v);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, PULSE_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, PULSE_WAVE));
+            const float m_new = fmaxf(m[ct], mx);
+            const bool dead = m_new == -INFINITY;  // no key of this column so far
+            alpha[ct] = dead ? 1.f : __builtin_amdgcn_exp2f((m[ct] - m_new) * c2);
+            const float shift = dead ? 0.f : -m_new * c2;
+            float psum = 0.f;
+#pragma unroll
+            for (int t = 0; t < KT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    // exp2(-inf) = 0 for masked scores; a dead column keeps -inf + 0 = -inf as well
+                    const float e = __builtin_amdgcn_exp2f(fmaf(s[ct][t][i], c2, shift));
+                    psum += e;
+                    pb[ct][t / 2][4 * (t % 2) + i] = (__bf16)e;
+                }
+            l_part[ct] = l_part[ct] * alpha[ct] + psum;
+            m[ct] = m_new;
+            moved = moved || alpha[ct] != 1.f;
+        }
+        // rescale only when some column's maximum moved
+        if (__builtin_amdgcn_ballot_w64(moved) != 0) {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt) acc[ct][dt] = acc[ct][dt] * alpha[ct];
+        }
+        // stale values under keys outside [lo_item, hi] are cleared (see the split kernel)
+        const bool edge = (j0 + BK - 1 > hi) || (j0 < lo_item);
+#pragma unroll
+        for (int ks = 0; ks < KT / 2; ++ks) {
+            uint32_t keep[2][2] = {{0xffffffffu, 0xffffffffu}, {0xffffffffu, 0xffffffffu}};
+            if (edge) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int h2 = 0; h2 < 2; ++h2) {
+                        const int j = j0 + 16 * (2 * ks + t) + 4 * kg + 2 * h2;
+                        keep[t][h2] = ((j <= hi && j >= lo_item) ? 0x0000ffffu : 0u) |
+                                      ((j + 1 <= hi && j + 1 >= lo_item) ? 0xffff0000u : 0u);
+                    }
+            }
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                const u32x2 v0 = *reinterpret_cast<const u32x2*>(&s_v[(2 * ks) * D * 16 + dt * 256 + v_at]);
+                const u32x2 v1 = *reinterpret_cast<const u32x2*>(&s_v[(2 * ks + 1) * D * 16 + dt * 256 + v_at]);
+                u32x4 words = {v0[0], v0[1], v1[0], v1[1]};
+                if (edge) words = u32x4{v0[0] & keep[0][0], v0[1] & keep[0][1], v1[0] & keep[1][0], v1[1] & keep[1][1]};
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct)
+                    acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, words), pb[ct][ks],
+                                                                          acc[ct][dt], 0, 0, 0);
+            }
+        }
+    };
+
+    const int first_block = lo_item / BK;
+    const int last_block = hi / BK;
+    fetch(first_block, page_ahead(first_block), 0);
+    int page_next = page_ahead(first_block + 1);
+    for (int b = first_block; b <= last_block; ++b) {
+        const int stage = (b - first_block) & 1;
+        // This block's loads were issued a block ago; nothing else is in flight, so the wait does not depend on a
+        // count of loads.
+        asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+        __syncthreads();  // every wavefront's part of this block has landed
+        if (b < last_block) {
+            fetch(b + 1, page_next, stage ^ 1);  // that stage was read a block ago; the barrier that ended that block released it
+            page_next = page_ahead(b + 2);       // used an iteration later
+        }
+        // a wavefront skips blocks that none of its columns sees (above its diagonal, below its window)
+        if (w_hi >= 0 && b * BK <= w_hi && b * BK + BK - 1 >= w_lo) compute(b, stage);
+        __syncthreads();  // everybody has read this block
+    }
+
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        float l = l_part[ct];
+        l += __shfl_xor(l, 16, PULSE_WAVE);
+        l += __shfl_xor(l, 32, PULSE_WAVE);
+        if (col_ok[ct]) {
+            const float inv = l > 0.f ? 1.0f / l : 0.f;
+            bf16_t* dst = a.out + static_cast<int64_t>(col_row[ct]) * a.o_stride + static_cast<int64_t>(col_head) * D;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                const uint32_t w0 = static_cast<uint32_t>(f32_to_bf16(acc[ct][dt][0] * inv)) |
+                                    (static_cast<uint32_t>(f32_to_bf16(acc[ct][dt][1] * inv)) << 16);
+                const uint32_t w1 = static_cast<uint32_t>(f32_to_bf16(acc[ct][dt][2] * inv)) |
+                                    (static_cast<uint32_t>(f32_to_bf16(acc[ct][dt][3] * inv)) << 16);
+                *reinterpret_cast<u32x2*>(dst + dt * 16 + 4 * kg) = u32x2{w0, w1};
+            }
+        }
+    }
+}
+
+#endif  // PULSE_WIDE
+
 // out[row, head, :] = sum_z w_z o_z / sum_z w_z l_z with w_z = exp2(m_z - max m), over the splits that hold keys of
 // the row.  One workgroup per (row, head); the splits' (m, l) pairs go through LDS so that the loads overlap.
 constexpr int MAX_SPLITS = 1024;
@@ -698,11 +998,19 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
     a.page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
     a.scale_log2e = scale * 1.4426950408889634f;
     a.window = window; a.split_size = 0; a.n_splits = 1;
+#if PULSE_WIDE
+    hipLaunchKernelGGL((attn_prefill_wide_kernel<WIDE_CT, 4, WIDE_NW>), dim3(n_items, nkv * a.head_chunks),
+                       dim3(WIDE_NW * PULSE_WAVE), 0, stream, a, 16 / gp);
+#else
     hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_items, nkv * a.head_chunks), dim3(WAVES * PULSE_WAVE), 0, stream, a,
                        16 / gp);
+#endif
     PULSE_LAUNCH_CHECK("attn_prefill");
     return 0;
 }
+
+// Column tiles a wavefront of the prompt-portion kernel takes: its items hold 4 * this * tokens_per_item tokens.
+extern "C" int pulse_attn_prefill_tiles() { return PREFILL_TILES; }
 
 // Columns per token and tokens per item for a group size: the host builds its item list with these.
 extern "C" int pulse_attn_mfma_tokens_per_item(int group) {

@@ -28,7 +28,13 @@ def tokens_per_item(group: int) -> int:
 
 
 PORTION_MIN_TOKENS = 16   # entries with at least this many tokens go to the kernel that shares keys through LDS
-PORTION_WAVES = 4         # wavefronts of its workgroup, each with `tokens_per_item` tokens
+PORTION_WAVES = 4         # wavefronts of its workgroup
+
+
+def portion_tokens(group: int, head_dim: int) -> int:
+    """Tokens of one work item of the prompt-portion kernel: its four wavefronts take one or two column tiles of
+    ``tokens_per_item`` tokens each (two for the head sizes its wide variant takes)."""
+    return tokens_per_item(group) * PORTION_WAVES * (2 if head_dim in (32, 64, 128) else 1)
 
 
 def build_items(entries: Sequence, tokens_per: int) -> List[int]:
@@ -47,7 +53,7 @@ def split_entries(entries: Sequence):
     return short, long
 
 
-def choose_splits(num_items: int, nkv: int, group: int, max_context: int, target_groups: int = 1024) -> Tuple[int, int]:
+def choose_splits(num_items: int, nkv: int, group: int, max_context: int, target_groups: int = 512) -> Tuple[int, int]:
     """(split_size, n_splits): enough workgroups to fill the chip, whole contexts when there are plenty already."""
     groups = num_items * nkv * ((group + 15) // 16)
     whole = (max_context + BLOCK_KEYS - 1) // BLOCK_KEYS * BLOCK_KEYS
@@ -94,7 +100,7 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
 def attn_prefill(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
                  vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
                  items: torch.Tensor, scale: float, window: int) -> None:
-    """Attention for prompt portions: items of up to 4 * tokens_per_item(group) tokens, keys shared through LDS."""
+    """Attention for prompt portions: items of up to portion_tokens(group, d) tokens, keys shared through LDS."""
     _gpu("attn_prefill", q, out, kcache, vcache, positions, token_entry, block_table, items)
     tokens = q.shape[0]
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.stride(1) == 1 and out.stride(1) == 1,

@@ -107,13 +107,14 @@ class PagedAttention(Part):
             return
         group = self.nq // self.nkv
         per = attention_mfma.tokens_per_item(group)
-        key = f"static:attention.items:{per}"
+        portion = attention_mfma.portion_tokens(group, self.d)
+        key = f"static:attention.items:{per}:{portion}"
         if key not in ctx.extras:  # depends only on the step's shape; the same lists serve every layer
             short, long = attention_mfma.split_entries(ctx.entries)
             dev = lambda flat: torch.tensor(flat, dtype=torch.int32, device=q.device) if flat else None
             ctx.extras[key] = (
                 dev(attention_mfma.build_items(short, per)),
-                dev(attention_mfma.build_items(long, per * attention_mfma.PORTION_WAVES)),
+                dev(attention_mfma.build_items(long, portion)),
                 max((e.start + e.count for e in short), default=0))
         short_items, long_items, short_context = ctx.extras[key]
         if long_items is not None:

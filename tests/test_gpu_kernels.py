@@ -401,7 +401,7 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0):
     ent_t = torch.tensor(entry, dtype=torch.int32, device=DEV)
     if split == "portion":
         # request 0's portion through the kernel that shares keys through LDS, the single tokens through the other
-        big = torch.tensor(M.build_items(entries[:1], M.tokens_per_item(group) * M.PORTION_WAVES), dtype=torch.int32, device=DEV)
+        big = torch.tensor(M.build_items(entries[:1], M.portion_tokens(group, d)), dtype=torch.int32, device=DEV)
         M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos_t, ent_t, table.to(DEV), big, scale, window)
         if len(entries) > 1:
             small = torch.tensor(M.build_items(entries[1:], M.tokens_per_item(group)), dtype=torch.int32, device=DEV)
@@ -423,6 +423,9 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0):
     dict(nq=6, nkv=1, d=32, bs=16, window=0, lens=[150, 1, 64, 65], portion=70),      # 6 heads: 8 columns a token
     dict(nq=6, nkv=3, d=48, bs=32, window=24, lens=[170, 90, 24, 25], portion=40),     # window, head size 48
     dict(nq=32, nkv=8, d=128, bs=16, window=0, lens=[300, 513, 512, 31], portion=37),
+    dict(nq=8, nkv=2, d=64, bs=32, window=40, lens=[333, 64], portion=150),              # wide portions: window, 32-key pages
+    dict(nq=2, nkv=2, d=32, bs=16, window=0, lens=[190, 17], portion=129),               # one head a kv head: 16 tokens a tile
+    dict(nq=16, nkv=2, d=128, bs=64, window=0, lens=[257, 100], portion=257),            # a whole prompt from position 0
     dict(nq=3, nkv=3, d=80, bs=16, window=0, lens=[97, 40], portion=1),                # no grouping: 16 tokens an item
     dict(nq=40, nkv=2, d=64, bs=64, window=0, lens=[200, 77], portion=5),              # 20 heads a kv head: two chunks
     dict(nq=16, nkv=1, d=224, bs=16, window=100, lens=[260, 130], portion=18),
