@@ -4,9 +4,9 @@ Three products stand behind it:
 
 * few rows (decoding, short portions) of bfloat16: this package's weight-streaming
   matrix-core kernel, which can also add into the float32 residual or apply SwiGLU;
-* many rows of bfloat16: the vendor library's product (torch.matmul, i.e.
-  hipBLASLt/rocBLAS, float32 accumulation), as the reference uses cuBLAS
-  (src/ops/kernels/cuda/matmul_kernel.cu:132-154);
+* many rows of bfloat16: the vendor library's product (torch.matmul / torch.mm,
+  i.e. hipBLASLt/rocBLAS, float32 accumulation, bfloat16 or float32 output), as
+  the reference uses cuBLAS (src/ops/kernels/cuda/matmul_kernel.cu:132-154);
 * the float32 run, and any weight kept in 32-bit: this package's own
   fused-multiply-add kernel, with no reduced-precision mode anywhere.
 """
@@ -32,14 +32,18 @@ class Linear:
         """``out`` [M, out_features] receives the product; its storage type is bfloat16 or float32."""
         w = self.weight if rows is None else self.weight[:rows]
         if self.library and x.dtype == torch.bfloat16:
-            few = x.shape[0] <= kernels.SKINNY_FAST_ROWS or out.dtype != torch.bfloat16
+            few = x.shape[0] <= kernels.SKINNY_FAST_ROWS
             if few and kernels.gemm_skinny_ok(x, w):
                 kernels.gemm_skinny(x, w, out)
                 return out
             if out.dtype == torch.bfloat16:
                 torch.matmul(x, w.t(), out=out)
                 return out
-            if w.shape[1] % 8 == 0:  # float32 results of many rows: the few-rows kernel, 64 rows at a time
+            if out.dtype == torch.float32 and out.is_contiguous():
+                # float32 results of many rows (logits): the library's product with a float32 output
+                torch.mm(x, w.t(), out_dtype=torch.float32, out=out)
+                return out
+            if w.shape[1] % 8 == 0:  # otherwise the few-rows kernel, 64 rows at a time
                 for r0 in range(0, x.shape[0], kernels.SKINNY_MAX_ROWS):
                     kernels.gemm_skinny(x[r0:r0 + kernels.SKINNY_MAX_ROWS], w, out[r0:r0 + kernels.SKINNY_MAX_ROWS])
                 return out
