@@ -169,6 +169,53 @@ def test_mixed_batches_with_page_reuse(engines, plain_logits, name, page, dtype)
         close(torch.cat(parts), plain_logits(name, ids[k]), dtype, f"{name} mixed request {k}")
 
 
+# The layer sizes of the benchmark's model (Qwen3-8B: 32 query heads over 8 kv heads of 128, hidden 4096, feed-forward
+# 12288) with two layers and a small vocabulary: the sizes at which the serving kernels run (the streaming product with
+# K = 4096 and 12288, 128-wide heads in groups of four), against the plain implementation.
+LAYER_SHAPE = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=1031, hidden_size=4096, intermediate_size=12288,
+    num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128, max_position_embeddings=4096,
+    rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False, torch_dtype="bfloat16", attention_bias=False,
+    use_sliding_window=False, hidden_act="silu")
+
+
+@pytest.fixture(scope="module")
+def layer_shape(tmp_path_factory):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from plain.qwen3_plain import PlainQwen3
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.weights import write_model_folder
+
+    folder = str(tmp_path_factory.mktemp("layer_shape"))
+    write_model_folder(Qwen3Config.from_dict(LAYER_SHAPE), folder, seed=41)
+    ids = token_ids(LAYER_SHAPE["vocab_size"], 150, seed=42)
+    want = PlainQwen3.from_folder(folder).logits(ids)
+    return folder, ids, want
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_benchmark_layer_sizes(layer_shape, dtype):
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+
+    folder, ids, want = layer_shape
+    _, model = load_model(folder, mode=dtype)
+    runner = ModelRunner(model, page_size=16, num_pages=24, max_requests=4)
+    whole = run_alone(runner, ids, [len(ids)])
+    close(whole, want, dtype, "layer sizes, whole")
+    tail = run_alone(runner, ids, [len(ids) - 32] + [1] * 32)
+    close(tail, want, dtype, "layer sizes, last 32 one by one")
+    close(tail, whole, dtype, "layer sizes, tail against whole", SPLIT_TOL)
+    portions = run_alone(runner, ids, [40, 2, 17, 64, 3, 5, 19])
+    close(portions, want, dtype, "layer sizes, portions")
+    close(portions, whole, dtype, "layer sizes, portions against whole", SPLIT_TOL)
+    if dtype == "bfloat16":
+        assert len(runner._graphs) >= 1            # the single tokens ran as recorded steps
+    del runner, model
+    torch.cuda.empty_cache()
+
+
 def test_step_refuses_what_it_cannot_run(engines):
     from pulse_infer_amd.engine.runner import StepEntry, StepError
 
