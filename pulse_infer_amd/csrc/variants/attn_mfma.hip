@@ -67,9 +67,8 @@ struct MfmaArgs {
     const bf16_t* kc;
     const bf16_t* vc;
     const int* positions;
-    const int* token_entry;
     const int* block_table;
-    const int* items;  // [n_items, 2]: first token row, number of tokens
+    const int* items;  // [n_items, 4]: first token row, number of tokens, row of the block table, 0
     int bt_width;
     int nq, nkv, group;
     int gp;           // columns per token: the group size rounded up to a power of two, at most 16
@@ -127,12 +126,15 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     const int r = lane % 16;   // operand row / result column
     const int kg = lane / 16;  // contraction group / result row group
 
-    const int row0 = a.items[2 * item];
-    const int ntok = a.items[2 * item + 1];
+    // Everything the first loads of keys need comes with the item (the block table's row too), so that the chain of
+    // dependent trips to memory before a workgroup streams is item -> block table -> keys.  The positions (which only
+    // decide masks and the end of the walk) and q travel at the same time.
+    const int row0 = a.items[4 * item];
+    const int ntok = a.items[4 * item + 1];
+    const int* bt = a.block_table + static_cast<int64_t>(a.items[4 * item + 2]) * a.bt_width;
     const int hi = a.positions[row0 + ntok - 1];    // last key any column of the item may see
     const int split_begin = split * a.split_size;
-    if (split_begin > hi) return;                   // nothing here; the merge does not read this split
-    const int split_end = min(split_begin + a.split_size, hi + 1);
+    int split_end = 0;                              // set once hi has arrived
 
     // this lane's column: a token of the item and a head of the group
     const int tc = r / a.gp;
@@ -145,8 +147,6 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     // lowest key any column needs (the first token's window)
     const int pos_first = a.positions[row0];
     const int lo_item = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
-
-    const int* bt = a.block_table + static_cast<int64_t>(a.token_entry[row0]) * a.bt_width;
 
     // Q^T operand: column r, contraction elements ch*32 + kg*8 ..
     bf16x8 bq[NCHUNK];
@@ -165,11 +165,9 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     float m = -INFINITY;
     float l_part = 0.f;
 
-    const int first_block = max(split_begin, lo_item) / BLOCK_KEYS;
-    const int last_block = (split_end - 1) / BLOCK_KEYS;
-
     // Issue every load of a 32-key block: K rows of the two 16-key tiles (a tile never straddles pages:
     // page_size % 16 == 0) and V rows in the order {tile0: 4kg.., tile1: 4kg..}.  Nothing is done to the values here.
+    // A page that the table does not hold (-1, or beyond its width) reads page 0: those keys are masked.
     auto load_block = [&](int b, BlockRegs& x) {
         const int j0 = b * BLOCK_KEYS;
 #pragma unroll
@@ -177,7 +175,7 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
             const int jt = j0 + 16 * t;
             int pi, slot0;
             page_of(jt, a.page_size, a.page_shift, pi, slot0);
-            int page = (jt <= hi && pi < a.bt_width) ? bt[pi] : 0;
+            int page = pi < a.bt_width ? bt[pi] : 0;
             page = (page >= 0 && page < a.num_pages) ? page : 0;  // masked keys may sit in pages given back
             const int64_t pg = static_cast<int64_t>(page) * a.nkv + g;
             const bf16_t* krow = a.kc + (pg * a.page_size + slot0 + r) * D;
@@ -257,11 +255,21 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
         }
     };
 
-    // two register sets in turn: the next block's loads are in flight while this block is computed
+    // two register sets in turn: the next block's loads are in flight while this block is computed.  Without a window
+    // the first block is known from the split alone: its loads go out before the positions have arrived.
     {
         BlockRegs xa, xb;
-        int b = first_block + wave;
-        if (b <= last_block) load_block(b, xa);
+        const bool early = a.window == 0;
+        int b = split_begin / BLOCK_KEYS + wave;
+        if (early && b <= (split_begin + a.split_size - 1) / BLOCK_KEYS) load_block(b, xa);
+        if (split_begin > hi) return;                   // nothing here; the merge does not read this split
+        split_end = min(split_begin + a.split_size, hi + 1);
+        const int first_block = max(split_begin, lo_item) / BLOCK_KEYS;
+        const int last_block = (split_end - 1) / BLOCK_KEYS;
+        if (!early) {
+            b = first_block + wave;
+            if (b <= last_block) load_block(b, xa);
+        }
         while (b <= last_block) {
             if (b + WAVES <= last_block) load_block(b + WAVES, xb);
             compute_block(b, xa);
@@ -356,12 +364,12 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     const int r = lane % 16;
     const int kg = lane / 16;
 
-    const int row0 = uniform(a.items[2 * item]);
-    const int ntok = uniform(a.items[2 * item + 1]);         // at most WAVES * per
+    const int row0 = uniform(a.items[4 * item]);
+    const int ntok = uniform(a.items[4 * item + 1]);         // at most WAVES * per
     const int hi = uniform(a.positions[row0 + ntok - 1]);    // last key of the workgroup
     const int pos_first = uniform(a.positions[row0]);
     const int lo_item = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
-    const int* bt = a.block_table + static_cast<int64_t>(uniform(a.token_entry[row0])) * a.bt_width;
+    const int* bt = a.block_table + static_cast<int64_t>(uniform(a.items[4 * item + 2])) * a.bt_width;
 
     // this wavefront's tokens and this lane's column
     const int wtok0 = wave * per;
@@ -632,12 +640,12 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_p
     const int r = lane % 16;
     const int kg = lane / 16;
 
-    const int row0 = uniform(a.items[2 * item]);
-    const int ntok = uniform(a.items[2 * item + 1]);         // at most NW * CT * per
+    const int row0 = uniform(a.items[4 * item]);
+    const int ntok = uniform(a.items[4 * item + 1]);         // at most NW * CT * per
     const int hi = uniform(a.positions[row0 + ntok - 1]);    // last key of the workgroup
     const int pos_first = uniform(a.positions[row0]);
     const int lo_item = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
-    const int* bt = a.block_table + static_cast<int64_t>(uniform(a.token_entry[row0])) * a.bt_width;
+    const int* bt = a.block_table + static_cast<int64_t>(uniform(a.items[4 * item + 2])) * a.bt_width;
 
     // this wavefront's column tiles and this lane's column in each
     const int tc = r / a.gp;
@@ -885,8 +893,8 @@ __global__ __launch_bounds__(128) void attn_mfma_reduce_kernel(const float* __re
     // only the rows of this launch's items have partial results
     const int item = blockIdx.x / per;
     const int tok = blockIdx.x % per;
-    if (tok >= items[2 * item + 1]) return;
-    const int64_t row = items[2 * item] + tok;
+    if (tok >= items[4 * item + 1]) return;
+    const int64_t row = items[4 * item] + tok;
     const int head = blockIdx.y;
     const int valid = min(n_splits, positions[row] / split_size + 1);
     const int64_t base = (row * nq + head) * n_splits;
@@ -918,8 +926,8 @@ extern "C" int pulse_attn_mfma_head_dim() { return D; }
 
 // Scratch needed for `tokens` rows cut into `n_splits`: floats of part_o and of part_ml.
 extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_stride, const void* kcache,
-                               const void* vcache, const int* positions, const int* token_entry,
-                               const int* block_table, int bt_width, const int* items, int n_items, int tokens, int nq,
+                               const void* vcache, const int* positions, const int* block_table, int bt_width,
+                               const int* items, int n_items, int tokens, int nq,
                                int nkv, int page_size, int num_pages, float scale, int window, int split_size,
                                int n_splits, int max_context, float* part_o, float* part_ml, hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && n_items >= 0 && nq > 0 && nkv > 0, "attn_mfma: bad sizes");
@@ -937,7 +945,7 @@ extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64
     PULSE_REQUIRE(n_splits == 1 || (part_o && part_ml), "attn_mfma: scratch is missing");
     PULSE_REQUIRE(n_splits <= MAX_SPLITS, "attn_mfma: at most %d splits, got %d", MAX_SPLITS, n_splits);
     PULSE_REQUIRE(n_splits < 65536 && static_cast<int64_t>(nkv) * ((nq / nkv + 15) / 16) < 65536, "attn_mfma: grid too large");
-    PULSE_REQUIRE(q && out && kcache && vcache && positions && token_entry && block_table && items, "attn_mfma: null pointer");
+    PULSE_REQUIRE(q && out && kcache && vcache && positions && block_table && items, "attn_mfma: null pointer");
     if (tokens == 0 || n_items == 0) return 0;
     const int group = nq / nkv;
     int gp = 1;
@@ -947,7 +955,7 @@ extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64
     a.out = static_cast<bf16_t*>(out); a.o_stride = o_stride;
     a.part_o = part_o; a.part_ml = part_ml;
     a.kc = static_cast<const bf16_t*>(kcache); a.vc = static_cast<const bf16_t*>(vcache);
-    a.positions = positions; a.token_entry = token_entry; a.block_table = block_table; a.items = items;
+    a.positions = positions; a.block_table = block_table; a.items = items;
     a.bt_width = bt_width; a.nq = nq; a.nkv = nkv; a.group = group; a.gp = gp; a.head_chunks = (group + 15) / 16;
     a.page_size = page_size; a.num_pages = num_pages;
     a.page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
@@ -968,8 +976,8 @@ extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64
 // Prompt portions: items of up to 4 * pulse_attn_mfma_tokens_per_item(group) tokens of one request, one workgroup each,
 // keys shared through LDS, no split.
 extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, int64_t o_stride, const void* kcache,
-                                  const void* vcache, const int* positions, const int* token_entry,
-                                  const int* block_table, int bt_width, const int* items, int n_items, int tokens,
+                                  const void* vcache, const int* positions, const int* block_table, int bt_width,
+                                  const int* items, int n_items, int tokens,
                                   int nq, int nkv, int page_size, int num_pages, float scale, int window,
                                   hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && n_items >= 0 && nq > 0 && nkv > 0, "attn_prefill: bad sizes");
@@ -982,7 +990,7 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
                   (reinterpret_cast<uintptr_t>(vcache) % 16) == 0 && (reinterpret_cast<uintptr_t>(out) % 8) == 0,
                   "attn_prefill: pointers must be 16-byte aligned");
     PULSE_REQUIRE(static_cast<int64_t>(nkv) * ((nq / nkv + 15) / 16) < 65536, "attn_prefill: grid too large");
-    PULSE_REQUIRE(q && out && kcache && vcache && positions && token_entry && block_table && items, "attn_prefill: null pointer");
+    PULSE_REQUIRE(q && out && kcache && vcache && positions && block_table && items, "attn_prefill: null pointer");
     if (tokens == 0 || n_items == 0) return 0;
     const int group = nq / nkv;
     int gp = 1;
@@ -992,7 +1000,7 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
     a.out = static_cast<bf16_t*>(out); a.o_stride = o_stride;
     a.part_o = nullptr; a.part_ml = nullptr;
     a.kc = static_cast<const bf16_t*>(kcache); a.vc = static_cast<const bf16_t*>(vcache);
-    a.positions = positions; a.token_entry = token_entry; a.block_table = block_table; a.items = items;
+    a.positions = positions; a.block_table = block_table; a.items = items;
     a.bt_width = bt_width; a.nq = nq; a.nkv = nkv; a.group = group; a.gp = gp; a.head_chunks = (group + 15) / 16;
     a.page_size = page_size; a.num_pages = num_pages;
     a.page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;

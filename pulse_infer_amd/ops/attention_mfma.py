@@ -37,19 +37,26 @@ def portion_tokens(group: int, head_dim: int) -> int:
     return tokens_per_item(group) * PORTION_WAVES * (2 if head_dim in (32, 64, 128) else 1)
 
 
+ITEM_INTS = 4
+
+
 def build_items(entries: Sequence, tokens_per: int) -> List[int]:
-    """Flat [first row, token count] pairs covering every entry of a step."""
+    """Flat [first row, token count, row of the block table, 0] quadruples covering the given entries of a step.
+
+    ``entries`` are (index of the entry in the step, entry) pairs: the index is the entry's row of the block table
+    (what ``token_entry`` holds for its tokens), so that a kernel finds the table with the item alone."""
     flat: List[int] = []
-    for e in entries:
+    for index, e in entries:
         for b in range(0, e.count, tokens_per):
-            flat.extend((e.first_row + b, min(tokens_per, e.count - b)))
+            flat.extend((e.first_row + b, min(tokens_per, e.count - b), index, 0))
     return flat
 
 
 def split_entries(entries: Sequence):
-    """(single tokens and short portions, long portions)"""
-    short = [e for e in entries if e.count < PORTION_MIN_TOKENS]
-    long = [e for e in entries if e.count >= PORTION_MIN_TOKENS]
+    """(single tokens and short portions, long portions), each as (index in the step, entry) pairs"""
+    numbered = list(enumerate(entries))
+    short = [(i, e) for i, e in numbered if e.count < PORTION_MIN_TOKENS]
+    long = [(i, e) for i, e in numbered if e.count >= PORTION_MIN_TOKENS]
     return short, long
 
 
@@ -68,10 +75,10 @@ def choose_splits(num_items: int, nkv: int, group: int, max_context: int, target
 
 
 def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
-              vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
+              vcache: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
               items: torch.Tensor, scale: float, window: int, split_size: int, n_splits: int, max_context: int,
               part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor]) -> None:
-    _gpu("attn_mfma", q, out, kcache, vcache, positions, token_entry, block_table, items, part_o, part_ml)
+    _gpu("attn_mfma", q, out, kcache, vcache, positions, block_table, items, part_o, part_ml)
     tokens = q.shape[0]
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.stride(1) == 1 and out.stride(1) == 1,
           "attn_mfma: q and out must be bfloat16 matrices with contiguous rows")
@@ -80,11 +87,11 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
     _need(supported(d, page_size, q.dtype, kcache.dtype), f"attn_mfma: head size {d} / page size {page_size} / "
           f"{kcache.dtype} is not supported by the matrix-core kernel")
     _int_vec("attn_mfma: positions", positions, tokens)
-    _int_vec("attn_mfma: token_entry", token_entry, tokens)
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
           "attn_mfma: block_table must be contiguous int32 [entries, width]")
-    _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() % 2 == 0, "attn_mfma: items must be int32 pairs")
-    n_items = items.numel() // 2
+    _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() % ITEM_INTS == 0,
+          "attn_mfma: items must be int32 quadruples")
+    n_items = items.numel() // ITEM_INTS
     if n_splits > 1:
         need = tokens * nq * n_splits
         _need(part_o is not None and part_ml is not None and part_o.dtype == torch.float32
@@ -92,16 +99,16 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
               "attn_mfma: scratch for the split results is too small")
     lib = load_variant("attn_mfma", {"PULSE_HEAD_DIM": d})
     call_in(lib, "pulse_attn_mfma", _ptr(q), _i64(q.stride(0)), _ptr(out), _i64(out.stride(0)), _ptr(kcache),
-            _ptr(vcache), _ptr(positions), _ptr(token_entry), _ptr(block_table), _i32(block_table.shape[1]),
+            _ptr(vcache), _ptr(positions), _ptr(block_table), _i32(block_table.shape[1]),
             _ptr(items), _i32(n_items), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages), _f32(scale),
             _i32(window), _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml), _stream())
 
 
 def attn_prefill(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
-                 vcache: torch.Tensor, positions: torch.Tensor, token_entry: torch.Tensor, block_table: torch.Tensor,
+                 vcache: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
                  items: torch.Tensor, scale: float, window: int) -> None:
     """Attention for prompt portions: items of up to portion_tokens(group, d) tokens, keys shared through LDS."""
-    _gpu("attn_prefill", q, out, kcache, vcache, positions, token_entry, block_table, items)
+    _gpu("attn_prefill", q, out, kcache, vcache, positions, block_table, items)
     tokens = q.shape[0]
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.stride(1) == 1 and out.stride(1) == 1,
           "attn_prefill: q and out must be bfloat16 matrices with contiguous rows")
@@ -110,12 +117,12 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, 
     _need(supported(d, page_size, q.dtype, kcache.dtype), f"attn_prefill: head size {d} / page size {page_size} / "
           f"{kcache.dtype} is not supported by the matrix-core kernel")
     _int_vec("attn_prefill: positions", positions, tokens)
-    _int_vec("attn_prefill: token_entry", token_entry, tokens)
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
           "attn_prefill: block_table must be contiguous int32 [entries, width]")
-    _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() % 2 == 0, "attn_prefill: items must be int32 pairs")
+    _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() % ITEM_INTS == 0,
+          "attn_prefill: items must be int32 quadruples")
     lib = load_variant("attn_mfma", {"PULSE_HEAD_DIM": d})
     call_in(lib, "pulse_attn_prefill", _ptr(q), _i64(q.stride(0)), _ptr(out), _i64(out.stride(0)), _ptr(kcache),
-            _ptr(vcache), _ptr(positions), _ptr(token_entry), _ptr(block_table), _i32(block_table.shape[1]),
-            _ptr(items), _i32(items.numel() // 2), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages),
+            _ptr(vcache), _ptr(positions), _ptr(block_table), _i32(block_table.shape[1]),
+            _ptr(items), _i32(items.numel() // ITEM_INTS), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages),
             _f32(scale), _i32(window), _stream())

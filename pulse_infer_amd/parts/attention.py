@@ -115,20 +115,21 @@ class PagedAttention(Part):
             ctx.extras[key] = (
                 dev(attention_mfma.build_items(short, per)),
                 dev(attention_mfma.build_items(long, portion)),
-                max((e.start + e.count for e in short), default=0))
+                max((e.start + e.count for _, e in short), default=0))
         short_items, long_items, short_context = ctx.extras[key]
         if long_items is not None:
             attention_mfma.attn_prefill(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
-                                        ctx.token_entry, table, long_items, self.scale, window)
+                                        table, long_items, self.scale, window)
         if short_items is not None:
             # a recorded step passes its context bucket as max_context: its splits must cover that
             max_context = ctx.max_context if long_items is None else short_context
-            split_size, n_splits = attention_mfma.choose_splits(short_items.numel() // 2, self.nkv, group, max_context)
+            split_size, n_splits = attention_mfma.choose_splits(short_items.numel() // attention_mfma.ITEM_INTS, self.nkv, group,
+                                                                      max_context)
             part_o = part_ml = None
             if n_splits > 1:
                 rows = ctx.num_tokens * self.nq * n_splits
                 part_o = ctx.workspace.buffer("attention.part_o", rows, self.d, torch.float32)
                 part_ml = ctx.workspace.buffer("attention.part_ml", rows, 2, torch.float32)
             attention_mfma.attn_mfma(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
-                                     ctx.token_entry, table, short_items, self.scale, window, split_size, n_splits,
+                                     table, short_items, self.scale, window, split_size, n_splits,
                                      max_context, part_o, part_ml)

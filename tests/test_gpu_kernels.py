@@ -385,12 +385,13 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0):
             self.first_row, self.count = first_row, count
     entries = [E(0, portion)] + [E(portion + i, 1) for i in range(len(lens) - 1)]
     group = nq // nkv
-    items = torch.tensor(M.build_items(entries, M.tokens_per_item(group)), dtype=torch.int32, device=DEV)
+    numbered = list(enumerate(entries))                 # (row of the block table, entry)
+    items = torch.tensor(M.build_items(numbered, M.tokens_per_item(group)), dtype=torch.int32, device=DEV)
     q, qref = as_stored(rnd(len(positions), (nq + 2 * nkv) * d, seed=300 + seed), dtype)
     out = torch.zeros(len(positions), nq * d, dtype=dtype, device=DEV)
     max_ctx = max(lens)
     if split is None or split == "portion":
-        split_size, n_splits = M.choose_splits(items.numel() // 2, nkv, group, max_ctx)
+        split_size, n_splits = M.choose_splits(items.numel() // M.ITEM_INTS, nkv, group, max_ctx)
     else:
         split_size, n_splits = split, (max_ctx + split - 1) // split
     rows = len(positions) * nq * n_splits
@@ -398,17 +399,16 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0):
     part_ml = torch.full((rows, 2), float("nan"), device=DEV)
     scale = d ** -0.5
     pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
-    ent_t = torch.tensor(entry, dtype=torch.int32, device=DEV)
     if split == "portion":
         # request 0's portion through the kernel that shares keys through LDS, the single tokens through the other
-        big = torch.tensor(M.build_items(entries[:1], M.portion_tokens(group, d)), dtype=torch.int32, device=DEV)
-        M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos_t, ent_t, table.to(DEV), big, scale, window)
+        big = torch.tensor(M.build_items(numbered[:1], M.portion_tokens(group, d)), dtype=torch.int32, device=DEV)
+        M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), big, scale, window)
         if len(entries) > 1:
-            small = torch.tensor(M.build_items(entries[1:], M.tokens_per_item(group)), dtype=torch.int32, device=DEV)
-            M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, ent_t, table.to(DEV), small, scale, window, split_size,
+            small = torch.tensor(M.build_items(numbered[1:], M.tokens_per_item(group)), dtype=torch.int32, device=DEV)
+            M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), small, scale, window, split_size,
                         n_splits, max_ctx, part_o, part_ml)
     else:
-        M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, ent_t, table.to(DEV), items, scale, window, split_size,
+        M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), items, scale, window, split_size,
                     n_splits, max_ctx, part_o, part_ml)
     got = out.cpu().to(F64).reshape(-1, nq, d)
     for t, (p, e) in enumerate(zip(positions, entry)):
@@ -446,8 +446,8 @@ def test_attn_mfma_refuses_other_sizes(k):
     z = torch.zeros(1, dtype=torch.int32, device=DEV)
     with pytest.raises(KernelError, match="not supported"):
         M.attn_mfma(torch.zeros(1, 64, dtype=torch.bfloat16, device=DEV), torch.zeros(1, 64, dtype=torch.bfloat16, device=DEV),
-                    1, 1, 64, kc, vc, z, z, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
-                    torch.tensor([0, 1], dtype=torch.int32, device=DEV), 1.0, 0, 32, 1, 1, None, None)
+                    1, 1, 64, kc, vc, z, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+                    torch.tensor([0, 1, 0, 0], dtype=torch.int32, device=DEV), 1.0, 0, 32, 1, 1, None, None)
 
 
 # ------------------------------------------------------------ few-rows product
