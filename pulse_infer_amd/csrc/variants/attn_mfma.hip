@@ -148,16 +148,16 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     const int pos_first = a.positions[row0];
     const int lo_item = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
 
-    // Q^T operand: column r, contraction elements ch*32 + kg*8 ..
+    // Q^T operand: column r, contraction elements ch*32 + kg*8 ..; loaded below, after the first keys are asked for
     bf16x8 bq[NCHUNK];
-    {
+    auto load_q = [&]() {
         const bf16_t* qrow = a.q + static_cast<int64_t>(col_row) * a.q_stride + static_cast<int64_t>(col_head) * D;
 #pragma unroll
         for (int ch = 0; ch < NCHUNK; ++ch) {
             const int off = ch * 32 + kg * 8;
             bq[ch] = (col_ok && off < D) ? *reinterpret_cast<const bf16x8*>(qrow + off) : zero8();
         }
-    }
+    };
 
     f32x4 acc[NDT];
 #pragma unroll
@@ -262,6 +262,7 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
         const bool early = a.window == 0;
         int b = split_begin / BLOCK_KEYS + wave;
         if (early && b <= (split_begin + a.split_size - 1) / BLOCK_KEYS) load_block(b, xa);
+        load_q();   // behind the keys' pages in the queue: results come back in the order asked for
         if (split_begin > hi) return;                   // nothing here; the merge does not read this split
         split_end = min(split_begin + a.split_size, hi + 1);
         const int first_block = max(split_begin, lo_item) / BLOCK_KEYS;
