@@ -61,10 +61,12 @@ __device__ __forceinline__ int row_shift_left(int v, int n) {
     }
 }
 
-// Sum of the wavefronts' partial tiles, in wavefront order, and the store.
+// Sum of the wavefronts' partial tiles, in wavefront order, and the store.  With `sumsq` (adding into a float32
+// matrix only) every slab also leaves the sum of squares of its 16 new values of each row, sumsq[row * parts + slab
+// number]: what a following RMSNorm needs of the row, so that the product after it can normalise by itself.
 template <int SLABS, int MT, int KW, bool SWIGLU>
 __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void* __restrict__ C, int64_t ldc, int M, int N,
-                                         int n_base, int mode, int tid) {
+                                         int n_base, int mode, int tid, float* __restrict__ sumsq = nullptr, int parts = 0) {
     constexpr int TILES = SLABS * MT;
     constexpr int THREADS = KW * PULSE_WAVE;
     if (!SWIGLU) {
@@ -77,11 +79,23 @@ __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void*
             for (int w = 0; w < KW; ++w) v += red[w][tile][n_in][m_in];
             const int m = (tile % MT) * 16 + m_in;
             const int n = n_base + (tile / MT) * 16 + n_in;
+            float updated = 0.f;
             if (m < M && n < N) {
                 const int64_t at = static_cast<int64_t>(m) * ldc + n;
                 if (mode == OUT_BF16) static_cast<bf16_t*>(C)[at] = f32_to_bf16(v);
                 else if (mode == OUT_F32) static_cast<float*>(C)[at] = v;
-                else static_cast<float*>(C)[at] += v;
+                else {
+                    updated = static_cast<float*>(C)[at] + v;
+                    static_cast<float*>(C)[at] = updated;
+                }
+            }
+            if (sumsq) {  // the 16 lanes of a row of lanes hold the 16 columns of one row of the tile
+                float sq = updated * updated;
+                sq += __shfl_xor(sq, 8, 16);
+                sq += __shfl_xor(sq, 4, 16);
+                sq += __shfl_xor(sq, 2, 16);
+                sq += __shfl_xor(sq, 1, 16);
+                if (n_in == 0 && m < M) sumsq[static_cast<int64_t>(m) * parts + n_base / 16 + tile / MT] = sq;
             }
         }
     } else {
@@ -242,11 +256,24 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_kernel(const bf16_
 //    ds_bpermute a step were measured too and gain nothing.)
 //
 // Both only change which lane fetches what; every product and the order of the sums are those of the kernel above.
-template <int SLABS, int KW, int PACK, bool SWIGLU>
+//
+// NORMED: X is not given; the float32 residual H is, with the row sums of squares that the product before left
+// (`sumsq`, `parts` of them a row) and the RMSNorm weight: x = bfloat16(h / sqrt(mean(h^2) + eps) * w) is formed here,
+// as the norm kernel forms it, and that kernel's launch is saved.
+struct NormInput {
+    const float* h;        // [M, K] float32, row stride ldx
+    const float* sumsq;    // [M, parts]
+    const bf16_t* weight;  // [K]
+    int parts;
+    float eps;
+};
+
+template <int SLABS, int KW, int PACK, bool SWIGLU, bool NORMED>
 __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(const bf16_t* __restrict__ X, int64_t ldx,
                                                                              const bf16_t* __restrict__ W, int64_t ldw,
                                                                              void* __restrict__ C, int64_t ldc, int M,
-                                                                             int N, int K, int mode) {
+                                                                             int N, int K, int mode, NormInput norm,
+                                                                             float* __restrict__ sumsq_out, int parts_out) {
     static_assert(PACK == 1 || PACK == 2 || PACK == 4 || PACK == 8, "PACK k-steps a load of X");
     static_assert(UNROLL % 2 == 0 && UNROLL % PACK == 0, "groups hold whole pairs and whole packs");
     constexpr int MP = 16 / PACK;  // rows of X a pack has room for
@@ -280,10 +307,28 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
     const int source_lane = 16 * ((r >> 1) & 3) + 8 * (r & 1) + 4 * (r >> 3) + kg;
     const int xr = r % MP;
     const bool xok = xr < M;
-    const bf16_t* xrow = X + static_cast<int64_t>(xok ? xr : 0) * ldx + (r / MP) * 32 + kg * 8;
+    const int x_at = (r / MP) * 32 + kg * 8;
+    const bf16_t* xrow = NORMED ? nullptr : X + static_cast<int64_t>(xok ? xr : 0) * ldx + x_at;
+    const float* hrow = NORMED ? norm.h + static_cast<int64_t>(xok ? xr : 0) * ldx + x_at : nullptr;
+    const bf16_t* nrow = NORMED ? norm.weight + x_at : nullptr;
+    float rstd = 0.f;
+    if (NORMED) {
+        // 1 / sqrt(mean(h^2) + eps) of every row from the parts; a wavefront takes rows wave, wave + KW, ..
+        __shared__ float s_rstd[16];
+        for (int m = wave; m < M; m += KW) {
+            float sum = 0.f;
+            for (int p = lane; p < norm.parts; p += PULSE_WAVE) sum += norm.sumsq[static_cast<int64_t>(m) * norm.parts + p];
+            sum = wave_sum(sum);
+            if (lane == 0) s_rstd[m] = 1.0f / sqrtf(sum / static_cast<float>(K) + norm.eps);
+        }
+        __syncthreads();
+        rstd = xok ? s_rstd[xr] : 0.f;
+    }
 
     for (int ks = step_begin; ks < step_begin + per; ks += UNROLL) {
         bf16x8 xb[UNROLL], wa[UNROLL][SLABS];
+        f32x4 hraw[NORMED ? UNROLL / PACK : 1][2];
+        bf16x8 nraw[NORMED ? UNROLL / PACK : 1];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int pair_k = ((ks + u) & ~1) * 32;
@@ -291,8 +336,17 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
             for (int s = 0; s < SLABS; ++s)
                 wa[u][s] = *reinterpret_cast<const bf16x8*>(((u & 1) ? w1[s] : w0[s]) + pair_k);
             if (u % PACK == 0) {
-                xb[u] = zeros8();
-                if (xok) xb[u] = *reinterpret_cast<const bf16x8*>(xrow + (ks + u) * 32);
+                if (NORMED) {
+                    hraw[u / PACK][0] = hraw[u / PACK][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+                    if (xok) {
+                        hraw[u / PACK][0] = *reinterpret_cast<const f32x4*>(hrow + (ks + u) * 32);
+                        hraw[u / PACK][1] = *reinterpret_cast<const f32x4*>(hrow + (ks + u) * 32 + 4);
+                    }
+                    nraw[u / PACK] = *reinterpret_cast<const bf16x8*>(nrow + (ks + u) * 32);
+                } else {
+                    xb[u] = zeros8();
+                    if (xok) xb[u] = *reinterpret_cast<const bf16x8*>(xrow + (ks + u) * 32);
+                }
             }
         }
         // every load of the group is on its way; now the lane exchanges
@@ -314,6 +368,18 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
                 }
                 wa[u][s] = __builtin_bit_cast(bf16x8, a0);
                 wa[u + 1][s] = __builtin_bit_cast(bf16x8, a1);
+            }
+        }
+        if (NORMED) {
+#pragma unroll
+            for (int u = 0; u < UNROLL; u += PACK) {
+                bf16x8 x;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float hv = hraw[u / PACK][e / 4][e % 4];
+                    x[e] = (__bf16)(hv * rstd * static_cast<float>(nraw[u / PACK][e]));  // as the norm kernel: (h * inv) * w, one rounding
+                }
+                xb[u] = x;
             }
         }
         if (PACK > 1) {
@@ -340,7 +406,7 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
 #pragma unroll
         for (int i = 0; i < 4; ++i) red[wave][s][4 * kg + i][r] = acc[s][i];
     __syncthreads();
-    epilogue<SLABS, 1, KW, SWIGLU>(red, C, ldc, M, N, n_base, mode, tid);
+    epilogue<SLABS, 1, KW, SWIGLU>(red, C, ldc, M, N, n_base, mode, tid, sumsq_out, parts_out);
 }
 
 template <int SLABS, int MT, int KW, bool SWIGLU>
@@ -361,16 +427,23 @@ void launch(bool xlds, const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ld
 
 template <int SLABS, int KW, bool SWIGLU>
 void launch_stream(int pack, const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
-                   int K, int mode, hipStream_t stream) {
+                   int K, int mode, const NormInput& norm, float* sumsq_out, int parts_out, hipStream_t stream) {
     const dim3 grid((N + SLABS * 16 - 1) / (SLABS * 16)), block(KW * PULSE_WAVE);
     const size_t red_bytes = sizeof(float) * KW * SLABS * 16 * 17;
-#define PULSE_STREAM(P)                                                                                               \
-    hipLaunchKernelGGL((gemm_skinny_stream_kernel<SLABS, KW, P, SWIGLU>), grid, block, red_bytes, stream, X, ldx, W, ldw, \
-                       C, ldc, M, N, K, mode)
-    if (pack == 8) PULSE_STREAM(8);
-    else if (pack == 4) PULSE_STREAM(4);
-    else if (pack == 2) PULSE_STREAM(2);
-    else PULSE_STREAM(1);
+#define PULSE_STREAM(P, NORMED)                                                                                          \
+    hipLaunchKernelGGL((gemm_skinny_stream_kernel<SLABS, KW, P, SWIGLU, NORMED>), grid, block, red_bytes, stream, X, ldx, \
+                       W, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out)
+    if (norm.h) {
+        if (pack == 8) PULSE_STREAM(8, true);
+        else if (pack == 4) PULSE_STREAM(4, true);
+        else if (pack == 2) PULSE_STREAM(2, true);
+        else PULSE_STREAM(1, true);
+    } else {
+        if (pack == 8) PULSE_STREAM(8, false);
+        else if (pack == 4) PULSE_STREAM(4, false);
+        else if (pack == 2) PULSE_STREAM(2, false);
+        else PULSE_STREAM(1, false);
+    }
 #undef PULSE_STREAM
 }
 
@@ -382,10 +455,31 @@ int pack_for(int M) { return M <= 2 ? 8 : (M <= 4 ? 4 : (M <= 8 ? 2 : 1)); }
 // mode: 0 store bfloat16, 1 store float32, 2 add into float32.  swiglu != 0: W holds gate and up rows interleaved in
 // slabs of 16 (gate slab, up slab, ...), N counts both, C is bfloat16 [M, N / 2] = silu(gate) * up.  tune: 0 lets the
 // entry point choose the kernel.
-extern "C" int pulse_gemm_skinny(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
-                                 int N, int K, int mode, int swiglu, int tune, hipStream_t stream) {
+// The same with the two fusions of the streaming kernel (M <= 16, K a multiple of 1024), each optional:
+//   norm_h != null: X is not read; x = bfloat16(norm_h / sqrt(mean(norm_h^2) + eps) * norm_w) is formed in the kernel
+//     from the float32 matrix norm_h [M, K] (row stride ldx), its row sums of squares norm_sumsq [M, norm_parts] (any
+//     split of the row into parts) and the bfloat16 weight norm_w [K];
+//   sumsq_out != null (mode 2 only): besides adding into C, leave sumsq_out[row * parts + slab] = sum of squares of the
+//     new values of C[row, 16 slab .. 16 slab + 15], parts = ceil(N / 16).
+// pulse_gemm_skinny_fusable says whether the streaming kernel takes a shape.
+extern "C" int pulse_gemm_skinny_fusable(int M, int N, int K) { return M >= 1 && M <= 16 && N > 0 && K > 0 && K % 1024 == 0; }
+
+extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
+                                       int N, int K, int mode, int swiglu, int tune, const float* norm_h,
+                                       const float* norm_sumsq, int norm_parts, const void* norm_w, float norm_eps,
+                                       float* sumsq_out, hipStream_t stream) {
+    const bool fused = norm_h != nullptr || sumsq_out != nullptr;
+    if (fused) {
+        PULSE_REQUIRE(pulse_gemm_skinny_fusable(M, N, K) && tune != 9, "gemm_skinny: M=%d N=%d K=%d cannot take the fused kernel", M, N, K);
+        PULSE_REQUIRE(sumsq_out == nullptr || (mode == OUT_ADD_F32 && !swiglu), "gemm_skinny: row sums of squares come with adding into float32 only");
+        PULSE_REQUIRE(norm_h == nullptr || (norm_sumsq && norm_w && norm_parts > 0 && ldx % 4 == 0 && ldx >= K &&
+                                            (reinterpret_cast<uintptr_t>(norm_h) % 16) == 0 &&
+                                            (reinterpret_cast<uintptr_t>(norm_w) % 16) == 0),
+                      "gemm_skinny: the norm's inputs are missing or misaligned");
+    }
+    if (norm_h) X = norm_h;  // only for the checks below: a non-null, aligned pointer with a fitting stride
     PULSE_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: sizes M=%d (at most 64) N=%d K=%d", M, N, K);
-    PULSE_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K,
+    PULSE_REQUIRE(K % 8 == 0 && (norm_h || ldx % 8 == 0) && ldw % 8 == 0 && ldx >= K && ldw >= K,
                   "gemm_skinny: K and the row strides must be multiples of 8 (16-byte loads)");
     PULSE_REQUIRE((reinterpret_cast<uintptr_t>(X) % 16) == 0 && (reinterpret_cast<uintptr_t>(W) % 16) == 0,
                   "gemm_skinny: operands must be 16-byte aligned");
@@ -398,7 +492,9 @@ extern "C" int pulse_gemm_skinny(const void* X, int64_t ldx, const void* W, int6
         PULSE_REQUIRE(ldc >= N, "gemm_skinny: output row stride too small");
     }
     if (M == 0) return 0;
-    const bf16_t* x = static_cast<const bf16_t*>(X);
+    const bf16_t* x = norm_h ? nullptr : static_cast<const bf16_t*>(X);
+    NormInput norm{norm_h, norm_sumsq, static_cast<const bf16_t*>(norm_w), norm_parts, norm_eps};
+    const int parts_out = (N + 15) / 16;
     const bf16_t* w = static_cast<const bf16_t*>(W);
     const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
     const bool wide = N >= 16384;  // enough slabs that pairs of them still fill the chip
@@ -420,18 +516,19 @@ extern "C" int pulse_gemm_skinny(const void* X, int64_t ldx, const void* W, int6
         const int kw = t_kw ? t_kw : ((K % 2048 == 0 && !pairs) ? 8 : 4);
         const int pack = t_pack ? t_pack : pack_for(M);
         if (swiglu) {
-            if (kw == 8) launch_stream<2, 8, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
-            else launch_stream<2, 4, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+            if (kw == 8) launch_stream<2, 8, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
+            else launch_stream<2, 4, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
         } else if (slabs == 2) {
-            if (kw == 8) launch_stream<2, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
-            else launch_stream<2, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+            if (kw == 8) launch_stream<2, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
+            else launch_stream<2, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
         } else {
-            if (kw == 8) launch_stream<1, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
-            else launch_stream<1, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, stream);
+            if (kw == 8) launch_stream<1, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
+            else launch_stream<1, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
         }
         PULSE_LAUNCH_CHECK("gemm_skinny");
         return 0;
     }
+    PULSE_REQUIRE(!fused, "gemm_skinny: K=%d takes no fused kernel", K);
     // X goes through LDS when it is small enough for two workgroups a compute unit
     const bool xlds = mt == 1 && K % 32 == 0 && static_cast<size_t>(K) * M * 2 <= XLDS_BYTES;
     if (swiglu) {
@@ -448,4 +545,10 @@ extern "C" int pulse_gemm_skinny(const void* X, int64_t ldx, const void* W, int6
     }
     PULSE_LAUNCH_CHECK("gemm_skinny");
     return 0;
+}
+
+extern "C" int pulse_gemm_skinny(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
+                                 int N, int K, int mode, int swiglu, int tune, hipStream_t stream) {
+    return pulse_gemm_skinny_fused(X, ldx, W, ldw, C, ldc, M, N, K, mode, swiglu, tune, nullptr, nullptr, 0, nullptr, 0.f,
+                                   nullptr, stream);
 }

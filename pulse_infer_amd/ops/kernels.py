@@ -163,18 +163,44 @@ def gemm_skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
             and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
-def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool = False, swiglu: bool = False,
-                tune: int = 0) -> None:
+def gemm_skinny_fusable(m: int, n: int, k: int) -> bool:
+    """Whether the few-rows product can take its input as (residual, row sums of squares, norm weight) and leave
+    row sums of squares of what it adds into (the streaming kernel's shapes)."""
+    return 1 <= m <= SKINNY_FAST_ROWS and n > 0 and k > 0 and k % 1024 == 0   # as pulse_gemm_skinny_fusable
+
+
+def gemm_skinny(a: Optional[torch.Tensor], w: torch.Tensor, out: torch.Tensor, add: bool = False, swiglu: bool = False,
+                tune: int = 0, norm: Optional[tuple] = None, sumsq_out: Optional[torch.Tensor] = None) -> None:
     """out = a @ w^T for at most 64 rows of bfloat16, float32 accumulation on the matrix cores.
 
     ``out`` bfloat16 or float32 is stored; with ``add`` (float32 only) the product is added to it.  With
     ``swiglu`` the weight holds gate and up rows in alternating slabs of 16 and out is silu(gate) * up.
     ``tune`` picks a kernel variant by hand (tests and measurements); 0 lets the library choose.
+
+    Two fusions for shapes that ``gemm_skinny_fusable`` accepts.  ``norm = (h, sumsq, weight, eps)`` instead of
+    ``a``: the input is RMSNorm(h) * weight, formed inside the kernel from the float32 matrix ``h`` and the sums of
+    squares of its rows, given in parts ``sumsq`` [M, parts].  ``sumsq_out`` [M, ceil(N / 16)] with ``add``: the
+    kernel also leaves the sums of squares of the rows of the updated ``out``, 16 columns a part.
     """
-    _gpu("gemm_skinny", a, w, out)
-    _need(gemm_skinny_ok(a, w), "gemm_skinny: needs bfloat16 operands with at most 64 rows, K a multiple of 8, "
-          "contiguous 16-byte aligned rows")
-    m, k = a.shape
+    if norm is not None:
+        h, sumsq, nweight, eps = norm
+        _gpu("gemm_skinny", h, sumsq, nweight, w, out, sumsq_out)
+        _need(a is None, "gemm_skinny: give either the input or what it is the norm of")
+        _need(h.dtype == torch.float32 and h.dim() == 2 and h.stride(1) == 1 and w.dim() == 2 and h.shape[1] == w.shape[1],
+              "gemm_skinny: the norm's input must be a float32 matrix with the weight's inner size")
+        m, k = h.shape
+        _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[0] >= m and sumsq.is_contiguous(),
+              "gemm_skinny: the row sums of squares must be a contiguous float32 [M, parts]")
+        _need(nweight.dtype == torch.bfloat16 and nweight.numel() == k and nweight.is_contiguous(),
+              "gemm_skinny: the fused norm takes a bfloat16 weight of the inner size")
+        _need(w.dtype == torch.bfloat16 and w.stride(1) == 1 and w.data_ptr() % 16 == 0, "gemm_skinny: bad weight")
+        ldx = h.stride(0) if m > 1 else k
+    else:
+        _gpu("gemm_skinny", a, w, out, sumsq_out)
+        _need(gemm_skinny_ok(a, w), "gemm_skinny: needs bfloat16 operands with at most 64 rows, K a multiple of 8, "
+              "contiguous 16-byte aligned rows")
+        m, k = a.shape
+        ldx = a.stride(0) if m > 1 else k
     n, k2 = w.shape
     _need(k == k2, f"gemm_skinny: inner sizes differ: a is [{m}, {k}], w is [{n}, {k2}]")
     cols = n // 2 if swiglu else n
@@ -188,9 +214,20 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool =
     if swiglu:
         _need(m <= SKINNY_SWIGLU_MAX_ROWS and n % 32 == 0 and out.dtype == torch.bfloat16,
               "gemm_skinny: the SwiGLU epilogue needs at most 32 rows, N a multiple of 32 and bfloat16 output")
-    call("pulse_gemm_skinny", _ptr(a), _i64(a.stride(0) if m > 1 else k), _ptr(w), _i64(w.stride(0) if n > 1 else k),
-         _ptr(out), _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode),
-         _i32(1 if swiglu else 0), _i32(tune), _stream())
+    if norm is not None or sumsq_out is not None:
+        _need(gemm_skinny_fusable(m, n, k), f"gemm_skinny: M={m} N={n} K={k} cannot take the fused kernel")
+    if sumsq_out is not None:
+        _need(add and sumsq_out.dtype == torch.float32 and sumsq_out.is_contiguous() and sumsq_out.dim() == 2
+              and sumsq_out.shape[0] >= m and sumsq_out.shape[1] == (n + 15) // 16,
+              "gemm_skinny: sumsq_out must be a contiguous float32 [M, ceil(N / 16)] and comes with add")
+    if norm is not None:
+        call("pulse_gemm_skinny_fused", _ptr(None), _i64(ldx), _ptr(w), _i64(w.stride(0) if n > 1 else k), _ptr(out),
+             _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0),
+             _i32(tune), _ptr(h), _ptr(sumsq), _i32(sumsq.shape[1]), _ptr(nweight), _f32(eps), _ptr(sumsq_out), _stream())
+    else:
+        call("pulse_gemm_skinny_fused", _ptr(a), _i64(ldx), _ptr(w), _i64(w.stride(0) if n > 1 else k), _ptr(out),
+             _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0),
+             _i32(tune), _ptr(None), _ptr(None), _i32(0), _ptr(None), _f32(0.0), _ptr(sumsq_out), _stream())
 
 
 def _check_cache(what: str, kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, d: int):

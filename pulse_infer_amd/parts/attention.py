@@ -21,7 +21,7 @@ import torch
 from ..cache.manager import PagedKVSpec
 from ..ops import attention_mfma, kernels
 from ..weights.store import TensorSpec
-from .base import MIXERS, BuildContext, PagedCacheView, Part, StepContext
+from .base import MIXERS, BuildContext, LazyNorm, PagedCacheView, Part, StepContext
 from .linear import Linear
 
 
@@ -72,15 +72,17 @@ class PagedAttention(Part):
         return PagedKVSpec(self.nkv, self.d, int(self.window) if self.window is not None else None)
 
     accepts_residual = True
+    accepts_lazy_input = True   # the first product may compute the norm before it by itself
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, cache: PagedCacheView,
-                residual: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    def forward(self, x, ctx: StepContext, cache: PagedCacheView, residual: Optional[torch.Tensor] = None):
         tokens = x.shape[0]
         ws = ctx.workspace
         write = cache.writable
         q_cols = self.nq * self.d
         cols = (self.nq + 2 * self.nkv) * self.d if write else q_cols
         qkv = ws.buffer("attention.qkv", tokens, cols, self.act_dtype)
+        if isinstance(x, LazyNorm) and not self.qkv.takes_lazy(x, rows=None if write else q_cols):
+            x = x.materialize(ws.buffer("attention.normed", tokens, self.hidden, self.act_dtype))
         self.qkv.forward(x, qkv, rows=None if write else q_cols)
         tables = ctx.position_product(self.position, self.encodings) if self.position is not None else None
         table = ctx.block_tables[cache.group]
@@ -93,7 +95,7 @@ class PagedAttention(Part):
         self.attend(qkv, attn, ctx, cache, table)
         out = ws.buffer("attention.proj", tokens, self.hidden, self.act_dtype)
         if residual is not None:
-            return self.o.add_into(attn, residual, out)
+            return self.o.add_into(attn, residual, out, ws)
         return self.o.forward(attn, out)
 
     def attend(self, q: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: PagedCacheView,

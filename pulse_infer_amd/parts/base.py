@@ -152,23 +152,70 @@ class StepContext:
         return self.extras[key]
 
 
+@dataclass
+class RowStats:
+    """What a part that added into the residual itself knows about the new rows: their sums of squares, in parts
+    (``sumsq`` [rows, parts] float32).  A norm that only needs that of a row can then be left to its consumer."""
+
+    sumsq: torch.Tensor
+
+
+@dataclass
+class LazyNorm:
+    """A normalised input that has not been computed: norm(h) * weight, for a consumer whose first product can form
+    it by itself (``accepts_lazy_input``).  ``materialize`` computes it the ordinary way."""
+
+    h: torch.Tensor
+    sumsq: torch.Tensor
+    weight: torch.Tensor
+    eps: float
+    norm: Any
+
+    @property
+    def shape(self):
+        return self.h.shape
+
+    def materialize(self, out: torch.Tensor) -> torch.Tensor:
+        return self.norm.apply(self.h, None, out)
+
+
 class ResidualStream:
     """The float32 residual ``h`` and the update that has not been added to it yet.
 
-    Adding is deferred so that it happens inside the next norm's kernel.
+    Adding is deferred so that it happens inside the next norm's kernel.  A part that added its result itself may
+    hand back ``RowStats`` of the new ``h``; they stay valid until ``h`` changes again.
     """
+
+    # Up to here a consumer that forms the norm itself is faster than the norm's kernel followed by it (measured:
+    # 6% of a decoding step at 2 rows, 1.6% at 8; with more rows every k-step of the product reads the float32
+    # residual and the norm's kernel wins).
+    LAZY_MAX_ROWS = 8
 
     def __init__(self, h: torch.Tensor):
         self.h = h
         self.pending: Optional[torch.Tensor] = None
+        self.stats: Optional[RowStats] = None
 
     def normed(self, norm: Any, out: torch.Tensor) -> torch.Tensor:
         norm.apply(self.h, self.pending, out)
         self.pending = None
         return out
 
-    def push(self, delta: Optional[torch.Tensor]) -> None:
-        """Hand over an update; None means the part has already added it to ``h``."""
+    def lazy(self, norm: Any) -> Optional[LazyNorm]:
+        """The norm of the current ``h`` as something a consumer can compute itself, if the norm allows that and the
+        rows' statistics are at hand."""
+        if self.pending is not None or self.stats is None or not hasattr(norm, "lazy"):
+            return None
+        if self.h.shape[0] > self.LAZY_MAX_ROWS:
+            return None
+        return norm.lazy(self.h, self.stats)
+
+    def push(self, delta: Any) -> None:
+        """Hand over an update; None or RowStats mean the part has already added it to ``h``."""
+        if isinstance(delta, RowStats):
+            self.stats = delta
+            return
+        self.stats = None
         if delta is None:
             return
         if self.pending is not None:

@@ -45,15 +45,23 @@ class PreNormBlock(Part):
     def cache_spec(self) -> Optional[Any]:
         return self.mixer.cache_spec()
 
-    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Any) -> None:
+    def _input(self, stream: ResidualStream, norm: Any, part: Any, ctx: StepContext) -> Any:
+        """norm(h) for ``part``: left to the part's first product where that is possible, else computed here."""
+        if getattr(part, "accepts_lazy_input", False):
+            lazy = stream.lazy(norm)
+            if lazy is not None:
+                return lazy
         x = ctx.workspace.buffer("block.normed", ctx.num_tokens, self.hidden, self.act_dtype)
-        stream.normed(self.mixer_norm, x)
-        # a part that says so may add its result into the residual itself and return None
+        return stream.normed(norm, x)
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Any) -> None:
+        x = self._input(stream, self.mixer_norm, self.mixer, ctx)
+        # a part that says so may add its result into the residual itself and return None (or the new rows' statistics)
         if getattr(self.mixer, "accepts_residual", False):
             stream.push(self.mixer.forward(x, ctx, cache, residual=stream.h))
         else:
             stream.push(self.mixer.forward(x, ctx, cache))
-        stream.normed(self.ffn_norm, x)
+        x = self._input(stream, self.ffn_norm, self.ffn, ctx)
         if getattr(self.ffn, "accepts_residual", False):
             stream.push(self.ffn.forward(x, ctx, residual=stream.h))
         else:

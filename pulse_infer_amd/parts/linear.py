@@ -17,6 +17,7 @@ from typing import Optional
 import torch
 
 from ..ops import kernels
+from .base import LazyNorm, RowStats, Workspace
 
 
 class Linear:
@@ -28,9 +29,22 @@ class Linear:
         self.mode = mode
         self.library = mode == "bfloat16" and weight.dtype == torch.bfloat16
 
-    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[int] = None) -> torch.Tensor:
-        """``out`` [M, out_features] receives the product; its storage type is bfloat16 or float32."""
+    def takes_lazy(self, x: LazyNorm, rows: Optional[int] = None) -> bool:
+        """Whether the product can form this not yet computed input by itself."""
+        n = self.out_features if rows is None else rows
+        return (self.library and kernels.gemm_skinny_fusable(x.shape[0], n, self.in_features)
+                and x.h.stride(1) == 1 and self.weight.stride(1) == 1)
+
+    def forward(self, x, out: torch.Tensor, rows: Optional[int] = None, swiglu: bool = False) -> torch.Tensor:
+        """``out`` [M, out_features] receives the product; its storage type is bfloat16 or float32.  ``x`` may be a
+        ``LazyNorm`` that ``takes_lazy`` accepted.  ``swiglu``: few rows of a slab-interleaved gate/up weight only."""
         w = self.weight if rows is None else self.weight[:rows]
+        if isinstance(x, LazyNorm):
+            kernels.gemm_skinny(None, w, out, swiglu=swiglu, norm=(x.h, x.sumsq, x.weight, x.eps))
+            return out
+        if swiglu:
+            kernels.gemm_skinny(x, w, out, swiglu=True)
+            return out
         if self.library and x.dtype == torch.bfloat16:
             few = x.shape[0] <= kernels.SKINNY_FAST_ROWS
             if few and kernels.gemm_skinny_ok(x, w):
@@ -50,11 +64,18 @@ class Linear:
         kernels.gemm_f32(x, w, out)
         return out
 
-    def add_into(self, x: torch.Tensor, residual: torch.Tensor, scratch: torch.Tensor) -> Optional[torch.Tensor]:
-        """residual += x W^T where the kernel can do that itself (returns None); otherwise the product is
-        written to ``scratch`` and returned for the caller to add."""
+    def add_into(self, x: torch.Tensor, residual: torch.Tensor, scratch: torch.Tensor,
+                 workspace: Optional[Workspace] = None):
+        """residual += x W^T where the kernel can do that itself: returns None, or, given a workspace and a shape the
+        fused kernel takes, the ``RowStats`` of the updated rows.  Otherwise the product is written to ``scratch`` and
+        returned for the caller to add."""
         if (self.library and x.dtype == torch.bfloat16 and x.shape[0] <= kernels.SKINNY_FAST_ROWS
                 and kernels.gemm_skinny_ok(x, self.weight)):
+            if workspace is not None and kernels.gemm_skinny_fusable(x.shape[0], self.out_features, self.in_features):
+                sums = workspace.buffer(f"linear.sumsq.{self.out_features}", x.shape[0], (self.out_features + 15) // 16,
+                                        torch.float32)
+                kernels.gemm_skinny(x, self.weight, residual, add=True, sumsq_out=sums)
+                return RowStats(sums)
             kernels.gemm_skinny(x, self.weight, residual, add=True)
             return None
         return self.forward(x, scratch)

@@ -10,7 +10,7 @@ import torch
 
 from ..ops import kernels
 from ..weights.store import TensorSpec
-from .base import FEED_FORWARDS, BuildContext, Part, StepContext
+from .base import FEED_FORWARDS, BuildContext, LazyNorm, Part, StepContext
 from .linear import Linear
 
 
@@ -50,18 +50,23 @@ class GatedMLP(Part):
         self.act_dtype = build.act_dtype
 
     accepts_residual = True
+    accepts_lazy_input = True   # the first product may compute the norm before it by itself
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, residual: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    def forward(self, x, ctx: StepContext, residual: Optional[torch.Tensor] = None):
         tokens = x.shape[0]
         ws = ctx.workspace
         z = ws.buffer("mlp.act", tokens, self.inter, self.act_dtype)
-        if (self.slab and tokens <= kernels.SKINNY_FAST_ROWS and kernels.gemm_skinny_ok(x, self.gate_up.weight)):
-            kernels.gemm_skinny(x, self.gate_up.weight, z, swiglu=True)
+        if isinstance(x, LazyNorm) and not (self.slab and self.gate_up.takes_lazy(x)):
+            x = x.materialize(ws.buffer("mlp.normed", tokens, self.hidden, self.act_dtype))
+        if isinstance(x, LazyNorm):
+            self.gate_up.forward(x, z, swiglu=True)
+        elif (self.slab and tokens <= kernels.SKINNY_FAST_ROWS and kernels.gemm_skinny_ok(x, self.gate_up.weight)):
+            self.gate_up.forward(x, z, swiglu=True)
         else:
             gu = ws.buffer("mlp.gate_up", tokens, 2 * self.inter, self.act_dtype)
             self.gate_up.forward(x, gu)
             kernels.swiglu(gu, z, slab=self.slab)
         out = ws.buffer("mlp.out", tokens, self.hidden, self.act_dtype)
         if residual is not None:
-            return self.down.add_into(z, residual, out)
+            return self.down.add_into(z, residual, out, ws)
         return self.down.forward(z, out)

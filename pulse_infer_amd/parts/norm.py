@@ -8,7 +8,7 @@ import torch
 
 from ..ops import kernels
 from ..weights.store import TensorSpec
-from .base import NORMS, BuildContext, Part
+from .base import NORMS, BuildContext, LazyNorm, Part, RowStats
 
 
 @NORMS.register("rmsnorm")
@@ -27,3 +27,9 @@ class RMSNorm(Part):
         """out = norm(h + delta) * w; h keeps the sum unless rows are gathered."""
         kernels.add_rmsnorm(h, delta, self.weight, self.eps, out, rows=rows)
         return out
+
+    def lazy(self, h: torch.Tensor, stats: RowStats) -> Optional[LazyNorm]:
+        """This norm as an input that its consumer computes (it needs the rows' sums of squares only)."""
+        if self.weight.dtype != torch.bfloat16:
+            return None
+        return LazyNorm(h, stats.sumsq, self.weight, self.eps, self)

@@ -511,6 +511,43 @@ def test_gemm_skinny_streaming_variants(k, m, n, kk):
         k.gemm_skinny(a, w, auto, tune=184 if m > 2 else 777)
 
 
+@pytest.mark.parametrize("m", [1, 3, 8, 13, 16])
+@pytest.mark.parametrize("n,kk,swiglu", [(48, 1024, False), (4096 + 32, 2048, False), (96, 3072, True)])
+def test_gemm_skinny_fused_norm_and_row_sums(k, m, n, kk, swiglu):
+    """The product that normalises its input itself, from the float32 residual and the row sums of squares that the
+    product before it left, against the norm kernel followed by the plain product; and those row sums themselves."""
+    eps = 3e-6
+    h = (rnd(m, kk, seed=80) * 3).to(DEV)
+    nw, _ = as_stored(1 + 0.1 * rnd(kk, seed=81), torch.bfloat16)
+    w, wref = as_stored(rnd(n, kk, seed=82, scale=kk ** -0.5), torch.bfloat16)
+    # 1. adding into the residual leaves the sums of squares of the new rows, 16 columns a part
+    a, aref = as_stored(rnd(m, 2048, seed=83), torch.bfloat16)
+    wo, woref = as_stored(rnd(kk, 2048, seed=84, scale=2048 ** -0.5), torch.bfloat16)
+    sums = torch.full((m, kk // 16), float("nan"), device=DEV)
+    plain = h.clone()
+    k.gemm_skinny(a, wo, plain, add=True)
+    k.gemm_skinny(a, wo, h, add=True, sumsq_out=sums)
+    assert torch.equal(h, plain)
+    want_sums = (h.cpu().to(F64) ** 2).view(m, kk // 16, 16).sum(-1)
+    assert torch.allclose(sums.cpu().to(F64), want_sums, rtol=1e-5, atol=1e-6)
+    # 2. the product of the normalised residual
+    x = torch.empty(m, kk, dtype=torch.bfloat16, device=DEV)
+    k.add_rmsnorm(h, None, nw, eps, x)
+    cols = n // 2 if swiglu else n
+    want = torch.empty(m, cols, dtype=torch.bfloat16, device=DEV)
+    k.gemm_skinny(x, w, want, swiglu=swiglu)
+    got = torch.full_like(want, float("nan"))
+    k.gemm_skinny(None, w, got, swiglu=swiglu, norm=(h, sums, nw, eps))
+    # the same formula; the norm's 1 / sqrt comes from sums taken in another order, which may move a bfloat16 input
+    # by one unit in the last place
+    scale = float(want.float().abs().max())
+    assert float((got.float() - want.float()).abs().max()) <= 2e-2 * scale
+    assert float((got.float() - want.float()).abs().mean()) <= 2e-3 * scale
+    from pulse_infer_amd.ops import KernelError
+    with pytest.raises(KernelError, match="fused"):
+        k.gemm_skinny(None, w[:, :512].contiguous(), got, swiglu=swiglu, norm=(h[:, :512].contiguous(), sums, nw[:512].contiguous(), eps))
+
+
 @pytest.mark.parametrize("m", [1, 8, 20, 32])
 @pytest.mark.parametrize("inter,kk", [(32, 64), (224, 96), (176, 80), (12288 // 8, 256), (48, 2048), (176, 1024)])
 def test_gemm_skinny_swiglu(k, m, inter, kk):
