@@ -1,6 +1,6 @@
 """Each part alone against its plain formula, models whose order names a layer twice or shares a cache,
-and a toy mixer with state of its own that is registered, built and stepped from here without a change
-to the framework's files."""
+and toy parts (a mixer with state of its own, a feed-forward that routes tokens to experts, another position
+encoding) that are registered, built and stepped from here without a change to the framework's files."""
 import math
 
 import pytest
@@ -308,3 +308,172 @@ def test_order_may_name_a_layer_twice_and_share_a_cache(gpu, tmp_path):
     h = h + P.gated_mlp(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
     want = P.linear(P.rms_norm(h, w["model.norm.weight"], eps), w["model.embed_tokens.weight"])
     close(torch.cat(outs), want, "float32", "shared order")
+
+
+# ------------------------------------------- a routed feed-forward and another position encoding, as toys
+ROUTED = {"experts": 5, "top_k": 2, "expert_size": 24}
+BANDS = {"factor": 4.0, "theta": 500.0}
+
+
+def register_routed_toys():
+    """A feed-forward that routes each token to its best experts, and a rotary encoding whose slow half of the
+    frequencies sees positions divided by a factor (pairs (i, i + d/2)); an architecture uses the first in its odd
+    layers and the second in its even layers, beside the ordinary parts."""
+    from pulse_infer_amd.config import Qwen3Config, register_architecture
+    from pulse_infer_amd.models.spec import LayerSpec, PartSpec
+    from pulse_infer_amd.parts.base import FEED_FORWARDS, POSITIONS, Part
+    from pulse_infer_amd.parts.rope import PAIRINGS, RotationTables
+    from pulse_infer_amd.weights import TensorSpec
+
+    @FEED_FORWARDS.register("toy_routed", replace=True)
+    class RoutedExperts(Part):
+        """y = sum over the top_k experts e of softmax(router logits of those)_e * W2_e relu(W1_e x); router in float32."""
+
+        @classmethod
+        def weight_specs(cls, params):
+            hidden, size = params["hidden_size"], params["expert_size"]
+            specs = {"router.weight": TensorSpec((params["experts"], hidden), fan_in=hidden)}
+            for e in range(params["experts"]):
+                specs[f"experts.{e}.w1.weight"] = TensorSpec((size, hidden), fan_in=hidden)
+                specs[f"experts.{e}.w2.weight"] = TensorSpec((hidden, size), fan_in=size)
+            return specs
+
+        def __init__(self, params, prefix, build):
+            self.top_k = params["top_k"]
+            get = lambda name: build.loader.get(f"{prefix}.{name}").float()
+            self.router = get("router.weight")
+            self.w1 = torch.stack([get(f"experts.{e}.w1.weight") for e in range(params["experts"])])
+            self.w2 = torch.stack([get(f"experts.{e}.w2.weight") for e in range(params["experts"])])
+            self.act = build.act_dtype
+
+        def forward(self, x, ctx):
+            x = x.float()
+            top, chosen = (x @ self.router.t()).topk(self.top_k, dim=-1)
+            share = torch.softmax(top, dim=-1)
+            out = torch.zeros_like(x)
+            for e in range(self.w1.shape[0]):                       # tokens grouped by expert
+                rows, slot = (chosen == e).nonzero(as_tuple=True)
+                if rows.numel():
+                    y = torch.relu(x[rows] @ self.w1[e].t()) @ self.w2[e].t()
+                    out.index_add_(0, rows, y * share[rows, slot].unsqueeze(1))
+            return out.to(self.act)
+
+    @POSITIONS.register("toy_banded_rope", replace=True)
+    class BandedRotary(Part):
+        def __init__(self, params, build):
+            self.dim, self.factor = params["rotary_dim"], params["factor"]
+            half = self.dim // 2
+            inv = torch.tensor(params["theta"], dtype=F64) ** (-torch.arange(half, dtype=F64) * 2.0 / self.dim)
+            inv[half // 2:] /= self.factor
+            self.inv_freq = inv.to(build.device)
+
+        def prepare(self, ctx):
+            angle = ctx.positions.to(F64).unsqueeze(1) * self.inv_freq
+            return RotationTables(torch.cos(angle).float().contiguous(), torch.sin(angle).float().contiguous(),
+                                  self.dim, PAIRINGS["half"])
+
+    class RoutedConfig(Qwen3Config):
+        def model_spec(self):
+            base = super().model_spec()
+            base.positions["bands"] = PartSpec("toy_banded_rope", dict(BANDS, rotary_dim=self.head_dim))
+            layers = []
+            for i, layer in enumerate(base.layers):
+                mixer, ffn = layer.mixer, layer.ffn
+                if i % 2 == 0:
+                    mixer = PartSpec("attention", dict(mixer.params, position="bands"))
+                else:
+                    ffn = PartSpec("toy_routed", dict(ROUTED, hidden_size=self.hidden_size, prefix="moe"))
+                layers.append(LayerSpec(layer.prefix, mixer, ffn, layer.norm, layer.block))
+            base.layers = layers
+            base.architecture = "RoutedToyForCausalLM"
+            return base
+
+    register_architecture("RoutedToyForCausalLM", RoutedConfig, replace=True)
+    return RoutedConfig
+
+
+def plain_routed_logits(plain, ids):
+    c, w = plain.c, plain.w
+    nq, nkv, d, eps = c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"], c["rms_norm_eps"]
+    t = len(ids)
+    pos = list(range(t))
+    h = P.embedding(w["model.embed_tokens.weight"], ids)
+    margins = []
+
+    def banded(x):  # complex multiplication of (x[i], x[i + d/2]) by e^(i angle)
+        half = d // 2
+        inv = torch.tensor(BANDS["theta"], dtype=F64) ** (-torch.arange(half, dtype=F64) * 2.0 / d)
+        inv[half // 2:] /= BANDS["factor"]
+        turn = torch.polar(torch.ones(t, half, dtype=F64), torch.tensor(pos, dtype=F64).unsqueeze(1) * inv).unsqueeze(1)
+        z = torch.complex(x[..., :half], x[..., half:]) * turn
+        return torch.cat([z.real, z.imag], dim=-1)
+
+    for i in range(c["num_hidden_layers"]):
+        p = f"model.layers.{i}."
+        a = P.rms_norm(h, w[p + "input_layernorm.weight"], eps)
+        q = P.rms_norm(P.linear(a, w[p + "self_attn.q_proj.weight"]).view(t, nq, d), w[p + "self_attn.q_norm.weight"], eps)
+        k = P.rms_norm(P.linear(a, w[p + "self_attn.k_proj.weight"]).view(t, nkv, d), w[p + "self_attn.k_norm.weight"], eps)
+        v = P.linear(a, w[p + "self_attn.v_proj.weight"]).view(t, nkv, d)
+        q, k = (banded(q), banded(k)) if i % 2 == 0 else (P.rope(q, pos, c["rope_theta"]), P.rope(k, pos, c["rope_theta"]))
+        o = P.causal_attention(q, k, v, d ** -0.5)
+        h = h + P.linear(o.reshape(t, nq * d), w[p + "self_attn.o_proj.weight"])
+        m = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)
+        if i % 2 == 0:
+            h = h + P.gated_mlp(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+            continue
+        rows = []
+        for row in m:                                                # token by token, expert by expert
+            scores = w[p + "moe.router.weight"] @ row
+            order = sorted(range(ROUTED["experts"]), key=lambda e: -scores[e].item())
+            margins.append((scores[order[ROUTED["top_k"] - 1]] - scores[order[ROUTED["top_k"]]]).item())
+            best = order[:ROUTED["top_k"]]
+            share = torch.softmax(torch.stack([scores[e] for e in best]), dim=0)
+            rows.append(sum(share[j] * (w[p + f"moe.experts.{e}.w2.weight"] @ torch.relu(w[p + f"moe.experts.{e}.w1.weight"] @ row))
+                            for j, e in enumerate(best)))
+        h = h + torch.stack(rows)
+    return P.linear(P.rms_norm(h, w["model.norm.weight"], eps), w["lm_head.weight"]), min(margins)
+
+
+def test_a_toy_routed_feed_forward_and_another_position_encoding(gpu, tmp_path):
+    from conftest import TINY_B
+    from pulse_infer_amd.config import unregister_architecture
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.parts.base import FEED_FORWARDS, POSITIONS
+    from pulse_infer_amd.weights import write_model_folder
+    from test_gpu_model import close
+
+    config = register_routed_toys()
+    try:
+        cfg = config.from_dict(dict(TINY_B, architectures=["RoutedToyForCausalLM"], num_hidden_layers=4))
+        cfg.architecture = "RoutedToyForCausalLM"
+        folder = write_model_folder(cfg, str(tmp_path / "routed"), seed=33)
+        plain = P.PlainQwen3.from_folder(folder)
+        assert f"model.layers.1.moe.experts.{ROUTED['experts'] - 1}.w2.weight" in plain.w
+        assert "model.layers.1.mlp.gate_proj.weight" not in plain.w
+        _, model = load_model(folder, mode="float32")
+        assert type(model.blocks[1].ffn).__name__ == "RoutedExperts" and model.blocks[0].mixer.position == "bands"
+        runner = ModelRunner(model, page_size=16, num_pages=12, max_requests=2)
+        ids = {k: token_ids(cfg.vocab_size, n, seed=80 + n) for k, n in (("a", 45), ("b", 27))}
+        got, fed = {k: [] for k in ids}, {k: 0 for k in ids}
+        for step in ([("a", 9), ("b", 2)], [("a", 1), ("b", 14)], [("a", 33), ("b", 1)], [("a", 2), ("b", 10)]):
+            entries = []
+            for k, n in step:
+                if not runner.cache.has_request(k):
+                    runner.add_request(k)
+                runner.reserve(k, fed[k] + n)
+                entries.append(StepEntry(k, ids[k][fed[k]:fed[k] + n], list(range(n))))
+                fed[k] += n
+            logits = runner.step(entries)
+            row = 0
+            for k, n in step:
+                got[k].append(logits[row:row + n])
+                row += n
+        for k in ids:
+            want, margin = plain_routed_logits(plain, ids[k])
+            assert margin > 1e-4, "two experts score alike for a token: choose another seed, the choice is not pinned"
+            close(torch.cat(got[k]), want, "float32", f"routed toy request {k}")
+    finally:
+        unregister_architecture("RoutedToyForCausalLM")
+        FEED_FORWARDS.unregister("toy_routed")
+        POSITIONS.unregister("toy_banded_rope")
