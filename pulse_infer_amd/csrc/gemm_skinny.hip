@@ -312,18 +312,7 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
     const float* hrow = NORMED ? norm.h + static_cast<int64_t>(xok ? xr : 0) * ldx + x_at : nullptr;
     const bf16_t* nrow = NORMED ? norm.weight + x_at : nullptr;
     float rstd = 0.f;
-    if (NORMED) {
-        // 1 / sqrt(mean(h^2) + eps) of every row from the parts; a wavefront takes rows wave, wave + KW, ..
-        __shared__ float s_rstd[16];
-        for (int m = wave; m < M; m += KW) {
-            float sum = 0.f;
-            for (int p = lane; p < norm.parts; p += PULSE_WAVE) sum += norm.sumsq[static_cast<int64_t>(m) * norm.parts + p];
-            sum = wave_sum(sum);
-            if (lane == 0) s_rstd[m] = 1.0f / sqrtf(sum / static_cast<float>(K) + norm.eps);
-        }
-        __syncthreads();
-        rstd = xok ? s_rstd[xr] : 0.f;
-    }
+    __shared__ float s_rstd[16];
 
     for (int ks = step_begin; ks < step_begin + per; ks += UNROLL) {
         bf16x8 xb[UNROLL], wa[UNROLL][SLABS];
@@ -348,6 +337,18 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
                     if (xok) xb[u] = *reinterpret_cast<const bf16x8*>(xrow + (ks + u) * 32);
                 }
             }
+        }
+        if (NORMED && ks == step_begin) {
+            // 1 / sqrt(mean(h^2) + eps) of every row from the parts; a wavefront takes rows wave, wave + KW, ..  This
+            // stands behind the first group's loads so that its own round trip to memory runs beside theirs.
+            for (int m = wave; m < M; m += KW) {
+                float sum = 0.f;
+                for (int p = lane; p < norm.parts; p += PULSE_WAVE) sum += norm.sumsq[static_cast<int64_t>(m) * norm.parts + p];
+                sum = wave_sum(sum);
+                if (lane == 0) s_rstd[m] = 1.0f / sqrtf(sum / static_cast<float>(K) + norm.eps);
+            }
+            __syncthreads();
+            rstd = xok ? s_rstd[xr] : 0.f;
         }
         // every load of the group is on its way; now the lane exchanges
 #pragma unroll
