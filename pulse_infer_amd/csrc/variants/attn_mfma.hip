@@ -79,6 +79,16 @@ struct MfmaArgs {
     int window;
     int split_size;  // multiple of 32
     int n_splits;
+    // Only for the kernel that prepares q and the step's own key itself (decoded tokens): then q points at the raw
+    // projection output [T, (nq + 2 nkv) D] (q heads, k heads, v heads), as the kernel of qk_rope_kv.hip takes it.
+    const bf16_t* q_w;     // per-head RMSNorm weights [D], or null for no norm
+    const bf16_t* k_w;
+    const float* cos_t;    // [T, rotary_dim / 2], or null for no rotation
+    const float* sin_t;
+    float eps;
+    int rotary_dim;        // multiple of 8
+    int pairing;           // 0: (2i, 2i+1)   1: (i, i + rotary_dim / 2), rotary_dim a multiple of 64
+    int new_key;           // 1: the token's key and value are prepared, used and written to their page here
 };
 
 // A value that is the same in every lane of the wavefront, said so to the compiler: what depends on it becomes
@@ -104,6 +114,80 @@ __device__ __forceinline__ bf16x8 zero8() {
     return z;
 }
 
+// What the preparation of a head needs besides the head: norm weight, cos and sin of this lane's slices (for pairs
+// (2i, 2i+1) the four angles of a slice, for pairs (i, i + rotary_dim / 2) the eight of a slice of the first half).
+struct HeadTables {
+    bf16x8 w[NCHUNK];
+    float cs[NCHUNK][8];
+    float sn[NCHUNK][8];
+};
+
+// Rotation of the pairs (i, i + 32 SHIFT): the partner slice lies SHIFT chunks further on, in the same lane.
+template <int SHIFT>
+__device__ __forceinline__ void rotate_halves(float (&f)[NCHUNK][8], const HeadTables& tb) {
+#pragma unroll
+    for (int ch = 0; ch < SHIFT; ++ch) {
+        if (ch + SHIFT >= NCHUNK) continue;
+        constexpr int LAST = NCHUNK - 1;
+        const int c2 = ch + SHIFT < NCHUNK ? ch + SHIFT : LAST;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float va = f[ch][e], vb = f[c2][e];
+            f[ch][e] = va * tb.cs[ch][e] - vb * tb.sn[ch][e];
+            f[c2][e] = va * tb.sn[ch][e] + vb * tb.cs[ch][e];
+        }
+    }
+}
+
+// Per-head RMSNorm and rotation of one head whose 8-element slices ch*32 + kg*8.. sit in the four lanes kg = 0..3
+// of a column, with the arithmetic of qk_rope_kv.hip: float32, (x * inv) * w, then the rotation, one rounding.
+__device__ __forceinline__ void prepare_head(bf16x8 (&x)[NCHUNK], const HeadTables& tb, bool normed, bool rotated,
+                                             float eps, int rot, int pairing, int kg) {
+    float f[NCHUNK][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < NCHUNK; ++ch)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            f[ch][e] = static_cast<float>(x[ch][e]);
+            ss += f[ch][e] * f[ch][e];
+        }
+    if (normed) {
+        ss += __shfl_xor(ss, 16, PULSE_WAVE);
+        ss += __shfl_xor(ss, 32, PULSE_WAVE);
+        const float inv = 1.0f / sqrtf(ss / static_cast<float>(D) + eps);
+#pragma unroll
+        for (int ch = 0; ch < NCHUNK; ++ch)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[ch][e] = f[ch][e] * inv * static_cast<float>(tb.w[ch][e]);
+    }
+    if (rotated) {
+        if (pairing == 0) {
+#pragma unroll
+            for (int ch = 0; ch < NCHUNK; ++ch)
+                if (ch * 32 + kg * 8 < rot) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float va = f[ch][2 * i], vb = f[ch][2 * i + 1];
+                        f[ch][2 * i] = va * tb.cs[ch][i] - vb * tb.sn[ch][i];
+                        f[ch][2 * i + 1] = va * tb.sn[ch][i] + vb * tb.cs[ch][i];
+                    }
+                }
+        } else {
+            switch (rot / 64) {
+                case 1: rotate_halves<1>(f, tb); break;
+                case 2: rotate_halves<2>(f, tb); break;
+                case 3: rotate_halves<3>(f, tb); break;
+                default: break;
+            }
+        }
+    }
+#pragma unroll
+    for (int ch = 0; ch < NCHUNK; ++ch)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[ch][e] = (__bf16)f[ch][e];
+}
+
 // two wavefronts a SIMD (256 registers each) where the head size lets the two register sets fit
 #if PULSE_HEAD_DIM <= 128
 #define PULSE_ATTN_WAVES_PER_EU __attribute__((amdgpu_waves_per_eu(2)))
@@ -111,6 +195,11 @@ __device__ __forceinline__ bf16x8 zero8() {
 #define PULSE_ATTN_WAVES_PER_EU
 #endif
 
+// FUSED: the items are decoded tokens (one token each) whose q, and whose own key and value if a.new_key, are still
+// raw in the projection output.  Every workgroup prepares its q heads itself; the workgroup whose split holds the
+// token's position also prepares the token's key, puts key and value into the registers of the block they belong
+// to (their page is written from here and never read back), so that the launch before this one is saved.
+template <bool FUSED>
 __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_mfma_kernel(MfmaArgs a) {
     __shared__ float s_m[WAVES][16];
     __shared__ float s_l[WAVES][16];
@@ -150,12 +239,127 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
 
     // Q^T operand: column r, contraction elements ch*32 + kg*8 ..; loaded below, after the first keys are asked for
     bf16x8 bq[NCHUNK];
+    bf16x8 knew[NCHUNK];   // FUSED: slice kg of the token's own key, the same in the 16 lanes of a kg
+    bf16x8 kwt[NCHUNK];    // and of the key norm's weight
+    constexpr int VPL = (D + PULSE_WAVE - 1) / PULSE_WAVE;
+    bf16_t vown[VPL];      // FUSED: channels lane, lane + 64, .. of the token's own value
+    int own_page = -1;     // FUSED: the page the token's key and value go to (asked for early, used at the end)
+    HeadTables tb;
     auto load_q = [&]() {
         const bf16_t* qrow = a.q + static_cast<int64_t>(col_row) * a.q_stride + static_cast<int64_t>(col_head) * D;
 #pragma unroll
         for (int ch = 0; ch < NCHUNK; ++ch) {
             const int off = ch * 32 + kg * 8;
             bq[ch] = (col_ok && off < D) ? *reinterpret_cast<const bf16x8*>(qrow + off) : zero8();
+        }
+        if (FUSED) {
+            // everything the preparation needs is asked for here, behind the first keys: the raw key of the token,
+            // the norm weights' slices, the slices of the token's cos and sin rows
+            const bf16_t* krow = a.q + static_cast<int64_t>(row0) * a.q_stride + static_cast<int64_t>(a.nq + g) * D;
+            const int half = a.rotary_dim / 2;
+            const float* cos_row = a.cos_t ? a.cos_t + static_cast<int64_t>(row0) * half : nullptr;
+            const float* sin_row = a.sin_t ? a.sin_t + static_cast<int64_t>(row0) * half : nullptr;
+            const bf16_t* vraw = a.q + static_cast<int64_t>(row0) * a.q_stride + static_cast<int64_t>(a.nq + a.nkv + g) * D;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) vown[i] = (a.new_key && lane + i * PULSE_WAVE < D) ? vraw[lane + i * PULSE_WAVE] : 0;
+#pragma unroll
+            for (int ch = 0; ch < NCHUNK; ++ch) {
+                const int off = ch * 32 + kg * 8;
+                knew[ch] = (a.new_key && off < D) ? *reinterpret_cast<const bf16x8*>(krow + off) : zero8();
+                tb.w[ch] = (a.q_w && off < D) ? *reinterpret_cast<const bf16x8*>(a.q_w + off) : zero8();
+                kwt[ch] = (a.new_key && a.k_w && off < D) ? *reinterpret_cast<const bf16x8*>(a.k_w + off) : zero8();
+                // pairs (2i, 2i+1): the slice's four angles; pairs (i, i + half): the eight of a slice of the first half
+                f32x4 c0 = {1.f, 1.f, 1.f, 1.f}, c1 = c0, s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0;
+                if (cos_row && off < (a.pairing == 0 ? a.rotary_dim : half)) {
+                    const int at = a.pairing == 0 ? off / 2 : off;
+                    c0 = *reinterpret_cast<const f32x4*>(cos_row + at);
+                    s0 = *reinterpret_cast<const f32x4*>(sin_row + at);
+                    if (a.pairing != 0) {
+                        c1 = *reinterpret_cast<const f32x4*>(cos_row + at + 4);
+                        s1 = *reinterpret_cast<const f32x4*>(sin_row + at + 4);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    tb.cs[ch][i] = c0[i]; tb.cs[ch][4 + i] = c1[i];
+                    tb.sn[ch][i] = s0[i]; tb.sn[ch][4 + i] = s1[i];
+                }
+            }
+        }
+    };
+    // FUSED: the token's key and value wait in LDS, a copy for each wavefront (so that no barrier is needed), until
+    // the block they belong to is computed.
+    __shared__ u32x4 s_newk[FUSED ? WAVES : 1][D / 8];
+    __shared__ bf16_t s_newv[FUSED ? WAVES : 1][D];
+    u32x4* stash_k = s_newk[FUSED ? wave : 0];
+    bf16_t* stash_v = s_newv[FUSED ? wave : 0];
+    auto prepare = [&](bool own_key) {
+        prepare_head(bq, tb, a.q_w != nullptr, a.cos_t != nullptr, a.eps, a.rotary_dim, a.pairing, kg);
+        if (!col_ok) {
+#pragma unroll
+            for (int ch = 0; ch < NCHUNK; ++ch) bq[ch] = zero8();
+        }
+        if (!own_key) return;
+        // the key's norm weight takes the place of q's; cos and sin are the token's for both
+#pragma unroll
+        for (int ch = 0; ch < NCHUNK; ++ch) tb.w[ch] = kwt[ch];
+        prepare_head(knew, tb, a.k_w != nullptr, a.cos_t != nullptr, a.eps, a.rotary_dim, a.pairing, kg);
+        if (r == 0) {
+#pragma unroll
+            for (int ch = 0; ch < NCHUNK; ++ch) {
+                const int off = ch * 32 + kg * 8;
+                if (off < D) stash_k[off / 8] = __builtin_bit_cast(u32x4, knew[ch]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VPL; ++i)
+            if (lane + i * PULSE_WAVE < D) stash_v[lane + i * PULSE_WAVE] = vown[i];
+        // where key and value go, for the steps to come: asked for now, written when the walk over the keys is over
+        int pi, slot;
+        page_of(hi, a.page_size, a.page_shift, pi, slot);
+        own_page = pi < a.bt_width ? bt[pi] : -1;
+    };
+    // FUSED: the first wavefront of the split that holds the token writes its key and value to their page
+    auto store_own = [&]() {
+        if (wave != 0 || own_page < 0 || own_page >= a.num_pages) return;
+        int pi, slot;
+        page_of(hi, a.page_size, a.page_shift, pi, slot);
+        const int64_t pg = static_cast<int64_t>(own_page) * a.nkv + g;
+        bf16_t* kdst = const_cast<bf16_t*>(a.kc) + (pg * a.page_size + slot) * D;
+        bf16_t* vdst = const_cast<bf16_t*>(a.vc) + pg * D * a.page_size + slot;
+        if (r == 0) {
+#pragma unroll
+            for (int ch = 0; ch < NCHUNK; ++ch) {
+                const int off = ch * 32 + kg * 8;
+                if (off < D) *reinterpret_cast<u32x4*>(kdst + off) = stash_k[off / 8];
+            }
+        }
+        for (int c = lane; c < D; c += PULSE_WAVE) vdst[static_cast<int64_t>(c) * a.page_size] = stash_v[c];
+    };
+    // FUSED: key `hi` of block `b` comes from the stash, not from its page
+    auto patch = [&](BlockRegs& x) {
+        const int tpos = (hi % BLOCK_KEYS) / 16;
+        const int rpos = hi % 16;
+        const int word = (hi % 4) / 2;
+        const uint32_t sh = (hi % 2) * 16;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            if (t != tpos) continue;
+#pragma unroll
+            for (int ch = 0; ch < NCHUNK; ++ch) {
+                const int off = ch * 32 + kg * 8;
+                if (off < D && r == rpos) x.k[t][ch] = stash_k[off / 8];
+            }
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) {
+                const uint32_t v = stash_v[dt * 16 + r];
+                if (kg == rpos / 4) {
+                    const uint32_t old = word == 0 ? x.v[t][dt][0] : x.v[t][dt][1];
+                    const uint32_t neu = (old & ~(0xffffu << sh)) | (v << sh);
+                    if (word == 0) x.v[t][dt][0] = neu;
+                    else x.v[t][dt][1] = neu;
+                }
+            }
         }
     };
 
@@ -267,19 +471,26 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
         split_end = min(split_begin + a.split_size, hi + 1);
         const int first_block = max(split_begin, lo_item) / BLOCK_KEYS;
         const int last_block = (split_end - 1) / BLOCK_KEYS;
+        // FUSED: the split that holds the token's position (the last one with keys) has its key to prepare
+        const bool own_key = FUSED && a.new_key && hi < split_begin + a.split_size;
+        const int own_block = own_key ? hi / BLOCK_KEYS : -1;
+        if (FUSED) prepare(own_key);
         if (!early) {
             b = first_block + wave;
             if (b <= last_block) load_block(b, xa);
         }
         while (b <= last_block) {
             if (b + WAVES <= last_block) load_block(b + WAVES, xb);
+            if (FUSED && b == own_block) patch(xa);
             compute_block(b, xa);
             b += WAVES;
             if (b > last_block) break;
             if (b + WAVES <= last_block) load_block(b + WAVES, xa);
+            if (FUSED && b == own_block) patch(xb);
             compute_block(b, xb);
             b += WAVES;
         }
+        if (FUSED && own_key) store_own();
     }
 
     // the column's sum sits in four lanes
@@ -925,12 +1136,22 @@ __global__ __launch_bounds__(128) void attn_mfma_reduce_kernel(const float* __re
 
 extern "C" int pulse_attn_mfma_head_dim() { return D; }
 
-// Scratch needed for `tokens` rows cut into `n_splits`: floats of part_o and of part_ml.
-extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_stride, const void* kcache,
-                               const void* vcache, const int* positions, const int* block_table, int bt_width,
-                               const int* items, int n_items, int tokens, int nq,
-                               int nkv, int page_size, int num_pages, float scale, int window, int split_size,
-                               int n_splits, int max_context, float* part_o, float* part_ml, hipStream_t stream) {
+namespace {
+
+struct Preparation {
+    const void* q_w;
+    const void* k_w;
+    const float* cos_t;
+    const float* sin_t;
+    float eps;
+    int rotary_dim, pairing, new_key;
+};
+
+int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_stride, const void* kcache,
+                     const void* vcache, const int* positions, const int* block_table, int bt_width, const int* items,
+                     int n_items, int tokens, int nq, int nkv, int page_size, int num_pages, float scale, int window,
+                     int split_size, int n_splits, int max_context, float* part_o, float* part_ml,
+                     const Preparation* prep, hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && n_items >= 0 && nq > 0 && nkv > 0, "attn_mfma: bad sizes");
     PULSE_REQUIRE(nq % nkv == 0, "attn_mfma: %d query heads are not a multiple of %d kv heads", nq, nkv);
     PULSE_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_mfma: page size %d must be a multiple of 16", page_size);
@@ -962,8 +1183,17 @@ extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64
     a.page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
     a.scale_log2e = scale * 1.4426950408889634f;
     a.window = window; a.split_size = split_size; a.n_splits = n_splits;
-    hipLaunchKernelGGL(attn_mfma_kernel, dim3(n_items, nkv * a.head_chunks, n_splits), dim3(WAVES * PULSE_WAVE), 0,
-                       stream, a);
+    a.q_w = a.k_w = nullptr; a.cos_t = a.sin_t = nullptr; a.eps = 0.f; a.rotary_dim = 0; a.pairing = 0; a.new_key = 0;
+    if (prep) {
+        a.q_w = static_cast<const bf16_t*>(prep->q_w); a.k_w = static_cast<const bf16_t*>(prep->k_w);
+        a.cos_t = prep->cos_t; a.sin_t = prep->sin_t; a.eps = prep->eps; a.rotary_dim = prep->rotary_dim;
+        a.pairing = prep->pairing; a.new_key = prep->new_key;
+        hipLaunchKernelGGL(attn_mfma_kernel<true>, dim3(n_items, nkv * a.head_chunks, n_splits), dim3(WAVES * PULSE_WAVE),
+                           0, stream, a);
+    } else {
+        hipLaunchKernelGGL(attn_mfma_kernel<false>, dim3(n_items, nkv * a.head_chunks, n_splits), dim3(WAVES * PULSE_WAVE),
+                           0, stream, a);
+    }
     PULSE_LAUNCH_CHECK("attn_mfma");
     if (n_splits > 1) {
         const int per = 16 / gp;
@@ -972,6 +1202,56 @@ extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64
         PULSE_LAUNCH_CHECK("attn_mfma_reduce");
     }
     return 0;
+}
+
+}  // namespace
+
+// Scratch needed for `tokens` rows cut into `n_splits`: tokens * nq * n_splits * D floats of part_o, * 2 of part_ml.
+extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_stride, const void* kcache,
+                               const void* vcache, const int* positions, const int* block_table, int bt_width,
+                               const int* items, int n_items, int tokens, int nq,
+                               int nkv, int page_size, int num_pages, float scale, int window, int split_size,
+                               int n_splits, int max_context, float* part_o, float* part_ml, hipStream_t stream) {
+    return launch_attn_mfma(q, q_stride, out, o_stride, kcache, vcache, positions, block_table, bt_width, items, n_items,
+                            tokens, nq, nkv, page_size, num_pages, scale, window, split_size, n_splits, max_context,
+                            part_o, part_ml, nullptr, stream);
+}
+
+// Whether pulse_attn_decode takes a rotation: whole 8-element slices, and for pairs (i, i + rotary_dim / 2) a
+// partner slice in the same lane.
+extern "C" int pulse_attn_decode_takes(int rotary_dim, int pairing) {
+    if (rotary_dim == 0) return 1;
+    if (rotary_dim < 0 || rotary_dim > D || rotary_dim % 8) return 0;
+    return pairing == 0 || (pairing == 1 && rotary_dim % 64 == 0);
+}
+
+// Attention for decoded tokens straight from the raw projection output: every item holds ONE token; qkv is
+// [tokens, (nq + 2 nkv) D] bfloat16 (q heads, k heads, v heads; row stride qkv_stride).  Per-head RMSNorm (q_w, k_w
+// bfloat16 [D], or null) and rotation (cos_t, sin_t float32 [tokens, rotary_dim / 2], or null) of q and, with new_key,
+// of the token's key happen inside; with new_key the key and the value are also written to the token's page (kcache
+// and vcache are written then).  Without new_key the pages already hold the token (a run that reads another run's
+// cache).  The rest as pulse_attn_mfma.
+extern "C" int pulse_attn_decode(const void* qkv, int64_t qkv_stride, void* out, int64_t o_stride, void* kcache,
+                                 void* vcache, const int* positions, const int* block_table, int bt_width,
+                                 const int* items, int n_items, int tokens, int nq, int nkv, int page_size,
+                                 int num_pages, float scale, int window, int split_size, int n_splits, int max_context,
+                                 float* part_o, float* part_ml, const void* q_w, const void* k_w, float eps,
+                                 const float* cos_t, const float* sin_t, int rotary_dim, int pairing, int new_key,
+                                 hipStream_t stream) {
+    PULSE_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode: cos and sin come together");
+    if (!cos_t) rotary_dim = 0;
+    PULSE_REQUIRE(pulse_attn_decode_takes(rotary_dim, pairing), "attn_decode: rotation of %d channels with pairing %d is not "
+                  "supported for head size %d", rotary_dim, pairing, D);
+    PULSE_REQUIRE((reinterpret_cast<uintptr_t>(q_w) % 16) == 0 && (reinterpret_cast<uintptr_t>(k_w) % 16) == 0 &&
+                  (reinterpret_cast<uintptr_t>(cos_t) % 16) == 0 && (reinterpret_cast<uintptr_t>(sin_t) % 16) == 0,
+                  "attn_decode: norm weights and rotation tables must be 16-byte aligned");
+    PULSE_REQUIRE(nq > 0 && nkv > 0 && qkv_stride >= static_cast<int64_t>(nq + (new_key ? 2 * nkv : 0)) * D,
+                  "attn_decode: the projection output's rows are too short");
+    PULSE_REQUIRE(n_items == tokens, "attn_decode: %d items for %d tokens (every item holds one token)", n_items, tokens);
+    Preparation prep{q_w, k_w, cos_t, sin_t, eps, rotary_dim, pairing, new_key ? 1 : 0};
+    return launch_attn_mfma(qkv, qkv_stride, out, o_stride, kcache, vcache, positions, block_table, bt_width, items,
+                            n_items, tokens, nq, nkv, page_size, num_pages, scale, window, split_size, n_splits,
+                            max_context, part_o, part_ml, &prep, stream);
 }
 
 // Prompt portions: items of up to 4 * pulse_attn_mfma_tokens_per_item(group) tokens of one request, one workgroup each,

@@ -126,3 +126,55 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, 
             _ptr(vcache), _ptr(positions), _ptr(block_table), _i32(block_table.shape[1]),
             _ptr(items), _i32(items.numel() // ITEM_INTS), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages),
             _f32(scale), _i32(window), _stream())
+
+
+def decode_takes(d: int, rotary_dim: int, pairing: int) -> bool:
+    """Whether ``attn_decode`` can rotate ``rotary_dim`` channels with this pairing for head size ``d``."""
+    lib = load_variant("attn_mfma", {"PULSE_HEAD_DIM": d})
+    return bool(lib.pulse_attn_decode_takes(int(rotary_dim), int(pairing)))
+
+
+def attn_decode(qkv: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
+                vcache: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor, items: torch.Tensor,
+                scale: float, window: int, split_size: int, n_splits: int, max_context: int,
+                part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor], q_w: Optional[torch.Tensor],
+                k_w: Optional[torch.Tensor], eps: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                rotary_dim: int, pairing: int, new_key: bool) -> None:
+    """Attention for decoded tokens from the raw projection output ``qkv`` [tokens, (nq + 2 nkv) d]: per-head norm
+    and rotation of q and of the token's own key happen inside the kernel; with ``new_key`` key and value are also
+    written to the token's page.  Every item must hold one token."""
+    _gpu("attn_decode", qkv, out, kcache, vcache, positions, block_table, items, part_o, part_ml, q_w, k_w, cos, sin)
+    tokens = qkv.shape[0]
+    _need(qkv.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and qkv.stride(1) == 1 and out.stride(1) == 1,
+          "attn_decode: qkv and out must be bfloat16 matrices with contiguous rows")
+    _need(qkv.shape[1] >= (nq + (2 * nkv if new_key else 0)) * d and out.shape[1] >= nq * d and out.shape[0] == tokens,
+          "attn_decode: qkv/out too narrow")
+    pages, page_size = _check_cache("attn_decode", kcache, vcache, nkv, d)
+    _need(supported(d, page_size, qkv.dtype, kcache.dtype), f"attn_decode: head size {d} / page size {page_size} / "
+          f"{kcache.dtype} is not supported by the matrix-core kernel")
+    _int_vec("attn_decode: positions", positions, tokens)
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
+          "attn_decode: block_table must be contiguous int32 [entries, width]")
+    _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() == ITEM_INTS * tokens,
+          "attn_decode: one int32 quadruple for every token")
+    for name, w in (("q_w", q_w), ("k_w", k_w)):
+        _need(w is None or (w.dtype == torch.bfloat16 and w.numel() == d and w.is_contiguous()),
+              f"attn_decode: {name} must hold {d} bfloat16 values")
+    _need((cos is None) == (sin is None), "attn_decode: cos and sin come together")
+    if cos is not None:
+        half = rotary_dim // 2
+        for name, t in (("cos", cos), ("sin", sin)):
+            _need(t.dtype == torch.float32 and t.is_contiguous() and t.dim() == 2 and t.shape[0] >= tokens
+                  and t.shape[1] == half, f"attn_decode: {name} must be float32 [tokens, {half}]")
+    if n_splits > 1:
+        need = tokens * nq * n_splits
+        _need(part_o is not None and part_ml is not None and part_o.dtype == torch.float32
+              and part_ml.dtype == torch.float32 and part_o.numel() >= need * d and part_ml.numel() >= need * 2,
+              "attn_decode: scratch for the split results is too small")
+    lib = load_variant("attn_mfma", {"PULSE_HEAD_DIM": d})
+    call_in(lib, "pulse_attn_decode", _ptr(qkv), _i64(qkv.stride(0)), _ptr(out), _i64(out.stride(0)), _ptr(kcache),
+            _ptr(vcache), _ptr(positions), _ptr(block_table), _i32(block_table.shape[1]), _ptr(items), _i32(tokens),
+            _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages), _f32(scale), _i32(window),
+            _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml), _ptr(q_w), _ptr(k_w),
+            _f32(eps), _ptr(cos), _ptr(sin), _i32(rotary_dim if cos is not None else 0), _i32(pairing),
+            _i32(1 if new_key else 0), _stream())

@@ -86,24 +86,48 @@ class PagedAttention(Part):
         self.qkv.forward(x, qkv, rows=None if write else q_cols)
         tables = ctx.position_product(self.position, self.encodings) if self.position is not None else None
         table = ctx.block_tables[cache.group]
-        kernels.qk_rope_kv(
-            qkv, self.nq, self.nkv, self.d, self.q_w, self.k_w, self.eps,
-            tables.cos if tables is not None else None, tables.sin if tables is not None else None,
-            tables.rotary_dim if tables is not None else 0, tables.pairing if tables is not None else 0,
-            cache.keys, cache.values, ctx.positions, ctx.token_entry, table, write_kv=write)
         attn = ws.buffer("attention.out", tokens, q_cols, self.act_dtype)
-        self.attend(qkv, attn, ctx, cache, table)
+        if self.decodes_from_raw(ctx, cache, qkv, tables):
+            # decoded tokens only: the attention kernel prepares q and each token's own key itself
+            self.attend(qkv, attn, ctx, cache, table, raw=(tables, write))
+        else:
+            kernels.qk_rope_kv(
+                qkv, self.nq, self.nkv, self.d, self.q_w, self.k_w, self.eps,
+                tables.cos if tables is not None else None, tables.sin if tables is not None else None,
+                tables.rotary_dim if tables is not None else 0, tables.pairing if tables is not None else 0,
+                cache.keys, cache.values, ctx.positions, ctx.token_entry, table, write_kv=write)
+            self.attend(qkv, attn, ctx, cache, table)
         out = ws.buffer("attention.proj", tokens, self.hidden, self.act_dtype)
         if residual is not None:
             return self.o.add_into(attn, residual, out, ws)
         return self.o.forward(attn, out)
 
+    def uses_matrix_cores(self, q: torch.Tensor, cache: PagedCacheView) -> bool:
+        return (self.options.get("attention", "auto") != "generic"
+                and attention_mfma.supported(self.d, cache.page_size, q.dtype, cache.keys.dtype))
+
+    def decodes_from_raw(self, ctx: StepContext, cache: PagedCacheView, qkv: torch.Tensor, tables: Any) -> bool:
+        """Whether this step's attention can start from the raw projection output: every entry is one decoded
+        token, the matrix-core kernel takes the sizes, and norm weights and rotation are of the kinds it prepares."""
+        if self.options.get("decode_from_raw", True) is False or not self.uses_matrix_cores(qkv, cache):
+            return False
+        if "static:attention.single_tokens" not in ctx.extras:
+            ctx.extras["static:attention.single_tokens"] = all(e.count == 1 for e in ctx.entries)
+        if not ctx.extras["static:attention.single_tokens"]:
+            return False
+        if any(w is not None and w.dtype != torch.bfloat16 for w in (self.q_w, self.k_w)):
+            return False
+        if tables is None:
+            return True
+        return (tables.cos.dtype == torch.float32 and tables.cos.is_contiguous() and tables.sin.is_contiguous()
+                and attention_mfma.decode_takes(self.d, tables.rotary_dim, tables.pairing))
+
     def attend(self, q: torch.Tensor, out: torch.Tensor, ctx: StepContext, cache: PagedCacheView,
-               table: torch.Tensor) -> None:
+               table: torch.Tensor, raw: Optional[tuple] = None) -> None:
+        """out = attention of the step's tokens over the cache.  ``raw = (rotation tables, write)``: q is the raw
+        projection output of decoded tokens, which the kernel prepares itself (see ``decodes_from_raw``)."""
         window = int(self.window) if self.window is not None else 0
-        use_mfma = (self.options.get("attention", "auto") != "generic"
-                    and attention_mfma.supported(self.d, cache.page_size, q.dtype, cache.keys.dtype))
-        if not use_mfma:
+        if not self.uses_matrix_cores(q, cache):
             kernels.attn_generic(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
                                  ctx.token_entry, table, self.scale, window)
             return
@@ -132,6 +156,15 @@ class PagedAttention(Part):
                 rows = ctx.num_tokens * self.nq * n_splits
                 part_o = ctx.workspace.buffer("attention.part_o", rows, self.d, torch.float32)
                 part_ml = ctx.workspace.buffer("attention.part_ml", rows, 2, torch.float32)
+            if raw is not None:
+                tables, write = raw
+                attention_mfma.attn_decode(
+                    q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions, table, short_items,
+                    self.scale, window, split_size, n_splits, max_context, part_o, part_ml, self.q_w, self.k_w,
+                    self.eps, tables.cos if tables is not None else None, tables.sin if tables is not None else None,
+                    tables.rotary_dim if tables is not None else 0, tables.pairing if tables is not None else 0,
+                    new_key=write)
+                return
             attention_mfma.attn_mfma(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
                                      table, short_items, self.scale, window, split_size, n_splits,
                                      max_context, part_o, part_ml)

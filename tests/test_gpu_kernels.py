@@ -450,6 +450,113 @@ def test_attn_mfma_refuses_other_sizes(k):
                     torch.tensor([0, 1, 0, 0], dtype=torch.int32, device=DEV), 1.0, 0, 32, 1, 1, None, None)
 
 
+@pytest.mark.parametrize("case", [
+    dict(nq=32, nkv=8, d=128, rot=128, pairing="interleaved", norm=True, bs=16, window=0, lens=[300, 1, 513, 512, 33]),
+    dict(nq=8, nkv=2, d=64, rot=64, pairing="half", norm=True, bs=32, window=40, lens=[333, 64, 40, 41]),
+    dict(nq=6, nkv=3, d=48, rot=16, pairing="interleaved", norm=True, bs=16, window=0, lens=[170, 17, 16]),
+    dict(nq=6, nkv=1, d=32, rot=0, pairing="interleaved", norm=False, bs=16, window=0, lens=[150, 2]),
+    dict(nq=4, nkv=4, d=128, rot=64, pairing="half", norm=False, bs=64, window=0, lens=[97, 200]),
+    dict(nq=16, nkv=1, d=224, rot=224, pairing="interleaved", norm=True, bs=16, window=100, lens=[260, 130]),
+])
+@pytest.mark.parametrize("split", [None, 32, 128])
+@pytest.mark.parametrize("new_key", [True, False])
+def test_attn_decode_from_raw(k, case, split, new_key):
+    """Decoded tokens straight from the raw projection output: per-head norm, rotation, the token's own key and
+    value (used from registers, written to the page) inside the attention kernel, against the plain formulas and
+    against what the separate preparation kernel writes.  With new_key False the pages already hold the token."""
+    from pulse_infer_amd.ops import attention_mfma as M
+    nq, nkv, d, rot, bs, window, lens = (case[x] for x in ("nq", "nkv", "d", "rot", "bs", "window", "lens"))
+    pairing = 0 if case["pairing"] == "interleaved" else 1
+    dtype, eps, theta, scale = torch.bfloat16, 3e-5, 9e3, d ** -0.5
+    assert M.decode_takes(d, rot, pairing)
+    n = len(lens)
+    pages_per = [(c + bs - 1) // bs for c in lens]
+    total = sum(pages_per) + 2
+    perm = torch.randperm(total, generator=torch.Generator().manual_seed(5)).tolist()
+    kc, vc = _cache(total, nkv, bs, d, dtype)
+    kc.normal_()                                   # stale data, also in the slot the new key goes to
+    vc.normal_()
+    table = torch.full((n, max(pages_per)), -1, dtype=torch.int32)
+    positions = [c - 1 for c in lens]
+    qkv, ref = as_stored(rnd(n, (nq + 2 * nkv) * d + 8, seed=41), dtype)
+    qw, qwref = as_stored(1 + 0.1 * rnd(d, seed=42), dtype)
+    kw, kwref = as_stored(1 + 0.1 * rnd(d, seed=43), dtype)
+    if not case["norm"]:
+        qw = kw = None
+    cos, sin = _tables(k, positions, theta, rot) if rot else (None, None)
+    q = ref[:, :nq * d].reshape(n, nq, d)
+    knew = ref[:, nq * d:(nq + nkv) * d].reshape(n, nkv, d)
+    vnew = ref[:, (nq + nkv) * d:(nq + 2 * nkv) * d].reshape(n, nkv, d)
+    if case["norm"]:
+        q, knew = P.rms_norm(q, qwref, eps), P.rms_norm(knew, kwref, eps)
+    if rot:
+        q = P.rope(q, positions, theta, rot, case["pairing"])
+        knew = P.rope(knew, positions, theta, rot, case["pairing"])
+    knew = knew.to(dtype).to(F64)                  # keys are stored rounded
+    refs, start = [], 0
+    for r, c in enumerate(lens):
+        pages = perm[start:start + pages_per[r]]
+        start += pages_per[r]
+        table[r, :len(pages)] = torch.tensor(pages, dtype=torch.int32)
+        ks, kref = as_stored(rnd(c, nkv, d, seed=100 + 7 * r), dtype)
+        vs, vref = as_stored(rnd(c, nkv, d, seed=200 + 7 * r), dtype)
+        kref[c - 1], vref[c - 1] = knew[r], vnew[r]
+        if not new_key:                            # the pages already hold the token
+            ks[c - 1], vs[c - 1] = knew[r].to(dtype), vnew[r].to(dtype)
+        _fill_cache(kc, vc, ks[:c if not new_key else c - 1], vs[:c if not new_key else c - 1], pages, bs)
+        refs.append((kref, vref))
+    before_k, before_v = kc.clone(), vc.clone()
+
+    class E:
+        def __init__(self, first_row, count):
+            self.first_row, self.count = first_row, count
+    group = nq // nkv
+    items = torch.tensor(M.build_items(list(enumerate(E(i, 1) for i in range(n))), M.tokens_per_item(group)),
+                         dtype=torch.int32, device=DEV)
+    max_ctx = max(lens)
+    if split is None:
+        split_size, n_splits = M.choose_splits(n, nkv, group, max_ctx)
+    else:
+        split_size, n_splits = split, (max_ctx + split - 1) // split
+    part_o = torch.full((n * nq * n_splits, d), float("nan"), device=DEV)
+    part_ml = torch.full((n * nq * n_splits, 2), float("nan"), device=DEV)
+    out = torch.zeros(n, nq * d, dtype=dtype, device=DEV)
+    pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    raw = qkv.clone()
+    M.attn_decode(qkv, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), items, scale, window, split_size, n_splits,
+                  max_ctx, part_o, part_ml, qw, kw, eps, cos, sin, rot, pairing, new_key)
+    assert torch.equal(qkv, raw)                   # the projection output stays raw
+    got = out.cpu().to(F64).reshape(n, nq, d)
+    for t, p in enumerate(positions):
+        kref, vref = refs[t]
+        want = P.causal_attention(q[t:t + 1], kref[:p + 1], vref[:p + 1], scale, window or None, [p])
+        assert torch.allclose(got[t], want[0], atol=2e-2, rtol=2e-2), (t, p, float((got[t] - want[0]).abs().max()))
+    # the pages: the token's slot holds its key and value, nothing else has changed
+    touched = torch.zeros(kc.shape[0], bs, dtype=torch.bool)
+    kcpu, vcpu = kc.cpu().to(F64), vc.cpu().to(F64)
+    for t, p in enumerate(positions):
+        page, slot = int(table[t, p // bs]), p % bs
+        touched[page, slot] = new_key
+        assert torch.allclose(kcpu[page, :, slot, :], knew[t], atol=2e-2, rtol=2e-2)
+        assert torch.equal(vcpu[page, :, :, slot], vnew[t])
+    same = ~touched.unsqueeze(1).expand(-1, nkv, -1)
+    assert torch.equal(kc.cpu()[same], before_k.cpu()[same])
+    assert torch.equal(vc.cpu().transpose(2, 3)[same], before_v.cpu().transpose(2, 3)[same])
+    if new_key:
+        # the separate preparation kernel writes the same pages (up to the last bit of a sum in another order)
+        k.qk_rope_kv(raw, nq, nkv, d, qw, kw, eps, cos, sin, rot, pairing, before_k, before_v, pos_t,
+                     torch.arange(n, dtype=torch.int32, device=DEV), table.to(DEV))
+        assert torch.allclose(kc.float(), before_k.float(), atol=0, rtol=2 ** -7) and torch.equal(vc, before_v)
+
+
+def test_attn_decode_refuses_rotations_it_cannot_prepare(k):
+    from pulse_infer_amd.ops import attention_mfma as M
+    assert M.decode_takes(128, 128, 0) and M.decode_takes(128, 64, 1) and M.decode_takes(64, 0, 0)
+    assert not M.decode_takes(128, 12, 0)          # slices of 8 channels are rotated whole
+    assert not M.decode_takes(128, 32, 1)          # the partner of a channel must lie in the same lane
+    assert not M.decode_takes(64, 128, 0)
+
+
 # ------------------------------------------------------------ few-rows product
 @pytest.mark.parametrize("m", [1, 8, 16, 17, 33, 64])
 @pytest.mark.parametrize("n,kk", [(48, 64), (509, 96), (4096 + 16, 200), (96, 4096)])
