@@ -1091,17 +1091,23 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_p
 #endif  // PULSE_WIDE
 
 // out[row, head, :] = sum_z w_z o_z / sum_z w_z l_z with w_z = exp2(m_z - max m), over the splits that hold keys of
-// the row.  One workgroup per (row, head); the splits' (m, l) pairs go through LDS so that the loads overlap.
+// the row.  One workgroup per (row, head); the splits' (m, l) pairs go through LDS, and the partial outputs of the
+// first splits are asked for before anything waits, so that the kernel is little more than two trips to memory.
 constexpr int MAX_SPLITS = 1024;
 
-__global__ __launch_bounds__(128) void attn_mfma_reduce_kernel(const float* __restrict__ part_o,
-                                                               const float* __restrict__ part_ml,
-                                                               const int* __restrict__ positions,
-                                                               const int* __restrict__ items, int per,
-                                                               bf16_t* __restrict__ out, int64_t o_stride, int nq,
-                                                               int n_splits, int split_size) {
+constexpr int REDUCE_THREADS = 256;
+constexpr int REDUCE_QUADS = D / 4;                              // float4 pieces of a head
+constexpr int REDUCE_GROUPS = REDUCE_THREADS / REDUCE_QUADS;     // groups of threads that share the splits out
+
+__global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const float* __restrict__ part_o,
+                                                                         const float* __restrict__ part_ml,
+                                                                         const int* __restrict__ positions,
+                                                                         const int* __restrict__ items, int per,
+                                                                         bf16_t* __restrict__ out, int64_t o_stride, int nq,
+                                                                         int n_splits, int split_size) {
     __shared__ float s_w[MAX_SPLITS];
     __shared__ float s_l[MAX_SPLITS];
+    __shared__ f32x4 s_acc[REDUCE_GROUPS][REDUCE_QUADS];
     // only the rows of this launch's items have partial results
     const int item = blockIdx.x / per;
     const int tok = blockIdx.x % per;
@@ -1110,9 +1116,23 @@ __global__ __launch_bounds__(128) void attn_mfma_reduce_kernel(const float* __re
     const int head = blockIdx.y;
     const int valid = min(n_splits, positions[row] / split_size + 1);
     const int64_t base = (row * nq + head) * n_splits;
-    for (int z = threadIdx.x; z < valid; z += blockDim.x) {
+    for (int z = threadIdx.x; z < valid; z += REDUCE_THREADS) {
         s_w[z] = part_ml[2 * (base + z)];
         s_l[z] = part_ml[2 * (base + z) + 1];
+    }
+    // group `grp` of threads takes splits grp, grp + REDUCE_GROUPS, ..; a thread four channels of them.  The partial
+    // outputs are asked for before the weights are known, eight splits of a group at a time.
+    const int quad = threadIdx.x % REDUCE_QUADS;
+    const int grp = threadIdx.x / REDUCE_QUADS;
+    const bool works = grp < REDUCE_GROUPS;
+    constexpr int AHEAD = 8;
+    f32x4 first[AHEAD];
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) {
+        const int z = grp + i * REDUCE_GROUPS;
+        // a split without keys of the row left nothing behind: what is read there is not used (z < valid below)
+        first[i] = (works && z < n_splits) ? *reinterpret_cast<const f32x4*>(part_o + (base + z) * D + 4 * quad)
+                                           : f32x4{0.f, 0.f, 0.f, 0.f};
     }
     __syncthreads();
     float mm = -INFINITY;
@@ -1120,15 +1140,28 @@ __global__ __launch_bounds__(128) void attn_mfma_reduce_kernel(const float* __re
     float ll = 0.f;
     for (int z = 0; z < valid; ++z) ll += (s_w[z] == -INFINITY ? 0.f : exp2f(s_w[z] - mm)) * s_l[z];
     const float inv = ll > 0.f ? 1.0f / ll : 0.f;
-    bf16_t* dst = out + row * o_stride + static_cast<int64_t>(head) * D;
-    for (int ch = threadIdx.x; ch < D; ch += blockDim.x) {
-        float v = 0.f;
-#pragma unroll 4
-        for (int z = 0; z < valid; ++z) {
-            const float wz = s_w[z] == -INFINITY ? 0.f : exp2f(s_w[z] - mm);
-            v += wz * part_o[(base + z) * D + ch];
+    if (works) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < AHEAD; ++i) {
+            const int z = grp + i * REDUCE_GROUPS;
+            if (z < valid) acc += first[i] * (s_w[z] == -INFINITY ? 0.f : exp2f(s_w[z] - mm));
         }
-        dst[ch] = f32_to_bf16(v * inv);
+        for (int z = grp + AHEAD * REDUCE_GROUPS; z < valid; z += REDUCE_GROUPS) {
+            const float wz = s_w[z] == -INFINITY ? 0.f : exp2f(s_w[z] - mm);
+            acc += *reinterpret_cast<const f32x4*>(part_o + (base + z) * D + 4 * quad) * wz;
+        }
+        s_acc[grp][quad] = acc;
+    }
+    __syncthreads();
+    // the groups' sums in a fixed order
+    if (threadIdx.x < REDUCE_QUADS) {
+        f32x4 v = s_acc[0][quad];
+#pragma unroll
+        for (int gi = 1; gi < REDUCE_GROUPS; ++gi) v += s_acc[gi][quad];
+        bf16_t* dst = out + row * o_stride + static_cast<int64_t>(head) * D + 4 * quad;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dst[e] = f32_to_bf16(v[e] * inv);
     }
 }
 
@@ -1164,7 +1197,8 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
                   "attn_mfma: split size %d must be a positive multiple of %d", split_size, BLOCK_KEYS);
     PULSE_REQUIRE(static_cast<int64_t>(n_splits) * split_size >= max_context,
                   "attn_mfma: %d splits of %d keys do not cover a context of %d", n_splits, split_size, max_context);
-    PULSE_REQUIRE(n_splits == 1 || (part_o && part_ml), "attn_mfma: scratch is missing");
+    PULSE_REQUIRE(n_splits == 1 || (part_o && part_ml && (reinterpret_cast<uintptr_t>(part_o) % 16) == 0),
+                  "attn_mfma: scratch is missing or not 16-byte aligned");
     PULSE_REQUIRE(n_splits <= MAX_SPLITS, "attn_mfma: at most %d splits, got %d", MAX_SPLITS, n_splits);
     PULSE_REQUIRE(n_splits < 65536 && static_cast<int64_t>(nkv) * ((nq / nkv + 15) / 16) < 65536, "attn_mfma: grid too large");
     PULSE_REQUIRE(q && out && kcache && vcache && positions && block_table && items, "attn_mfma: null pointer");
@@ -1197,7 +1231,7 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
     PULSE_LAUNCH_CHECK("attn_mfma");
     if (n_splits > 1) {
         const int per = 16 / gp;
-        hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(n_items * per, nq), dim3(128), 0, stream, part_o, part_ml,
+        hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(n_items * per, nq), dim3(REDUCE_THREADS), 0, stream, part_o, part_ml,
                            positions, items, per, a.out, o_stride, nq, n_splits, split_size);
         PULSE_LAUNCH_CHECK("attn_mfma_reduce");
     }
