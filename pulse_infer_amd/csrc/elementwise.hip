@@ -46,7 +46,7 @@ extern "C" int pulse_embed_gather(const int* ids, const void* table, int table_d
 // (formula: src/ops/kernels/cuda/rmsnorm_kernel.cu:97-157; the reference adds the
 // residual in a separate kernel, src/ops/kernels/cuda/add_kernel.cu:73-92)
 template <typename TD, typename TW, typename TY>
-__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, int parts, int64_t part_stride,
                                    const int* __restrict__ rows, const TW* __restrict__ w,
                                    TY* __restrict__ y, int hidden, float eps, int write_back) {
     __shared__ float scratch[16];
@@ -57,7 +57,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
     float ss = 0.f;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = hrow[i];
-        if (drow) v += to_f32<TD>(drow[i]);
+        if (drow)
+            for (int p = 0; p < parts; ++p) v += to_f32<TD>(drow[p * part_stride + i]);
         ss += v * v;
     }
     ss = block_sum(ss, scratch);
@@ -65,7 +66,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
     TY* yrow = y + static_cast<int64_t>(r) * hidden;
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
         float v = hrow[i];
-        if (drow) v += to_f32<TD>(drow[i]);
+        if (drow)
+            for (int p = 0; p < parts; ++p) v += to_f32<TD>(drow[p * part_stride + i]);
         if (write_back) hrow[i] = v;
         yrow[i] = from_f32<TY>(v * inv * to_f32<TW>(w[i]));
     }
@@ -91,6 +93,7 @@ template <> __device__ __forceinline__ ushort4 narrow4<bf16_t>(float4 v) {
 
 template <typename TD, typename TW, typename TY>
 __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+                                                              int parts, int64_t part_stride,
                                                               const int* __restrict__ rows, const TW* __restrict__ w,
                                                               TY* __restrict__ y, int hidden, float eps, int write_back) {
     __shared__ float scratch[16];
@@ -103,18 +106,34 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     float4* hrow = reinterpret_cast<float4*>(h + s * hidden);
     const VD* drow = delta ? reinterpret_cast<const VD*>(delta + s * hidden) : nullptr;
     float4 v[RMS_CHUNKS];
+#pragma unroll
+    for (int c = 0; c < RMS_CHUNKS; ++c) {
+        const int i = threadIdx.x + c * 256;
+        if (i < nvec) v[c] = hrow[i];
+    }
+    if (drow) {
+        // The parts of an update (shares of a product's inner dimension) are added in their order; the loads of
+        // several parts are asked for before the first is added, since few rows are bound by the trips to memory.
+#pragma unroll 8
+        for (int p = 0; p < parts; ++p) {
+            float4 d[RMS_CHUNKS];
+#pragma unroll
+            for (int c = 0; c < RMS_CHUNKS; ++c) {
+                const int i = threadIdx.x + c * 256;
+                if (i < nvec) d[c] = widen4(drow[p * (part_stride / 4) + i]);
+            }
+#pragma unroll
+            for (int c = 0; c < RMS_CHUNKS; ++c) {
+                const int i = threadIdx.x + c * 256;
+                if (i < nvec) { v[c].x += d[c].x; v[c].y += d[c].y; v[c].z += d[c].z; v[c].w += d[c].w; }
+            }
+        }
+    }
     float ss = 0.f;
 #pragma unroll
     for (int c = 0; c < RMS_CHUNKS; ++c) {
         const int i = threadIdx.x + c * 256;
-        if (i < nvec) {
-            v[c] = hrow[i];
-            if (drow) {
-                const float4 d = widen4(drow[i]);
-                v[c].x += d.x; v[c].y += d.y; v[c].z += d.z; v[c].w += d.w;
-            }
-            ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
-        }
+        if (i < nvec) ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
     }
     ss = block_sum(ss, scratch);
     const float inv = 1.0f / sqrtf(ss / static_cast<float>(hidden) + eps);
@@ -132,9 +151,12 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     }
 }
 
-extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, const int* rows,
-                                 const void* w, int w_dtype, void* y, int y_dtype, int out_rows,
+// delta may come in `parts` (>= 1) matrices of the shape of h, `part_stride` elements apart: h + their sum, added in
+// order, is what is normalised (the shares of a product whose inner dimension was split).
+extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, int parts, int64_t part_stride,
+                                 const int* rows, const void* w, int w_dtype, void* y, int y_dtype, int out_rows,
                                  int hidden, float eps, int write_back, hipStream_t stream) {
+    PULSE_REQUIRE(parts >= 1 && (parts == 1 || (delta && part_stride % 4 == 0)), "add_rmsnorm: bad parts of the update");
     PULSE_REQUIRE(out_rows >= 0 && hidden > 0, "add_rmsnorm: bad sizes rows=%d H=%d", out_rows, hidden);
     PULSE_REQUIRE(pulse_dtype_ok(delta_dtype) && pulse_dtype_ok(w_dtype) && pulse_dtype_ok(y_dtype),
                   "add_rmsnorm: bad dtype tag");
@@ -146,12 +168,12 @@ extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, c
     if (hidden % 4 == 0 && hidden <= 256 * 4 * RMS_CHUNKS && aligned) {
         PULSE_DISPATCH_DTYPE(delta_dtype, TD, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(y_dtype, TY,
             hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY>), dim3(out_rows), dim3(256), 0, stream, h,
-                               static_cast<const TD*>(delta), rows, static_cast<const TW*>(w),
+                               static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
                                static_cast<TY*>(y), hidden, eps, write_back))));
     } else {
         PULSE_DISPATCH_DTYPE(delta_dtype, TD, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(y_dtype, TY,
             hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, TY>), dim3(out_rows), dim3(256), 0, stream, h,
-                               static_cast<const TD*>(delta), rows, static_cast<const TW*>(w),
+                               static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
                                static_cast<TY*>(y), hidden, eps, write_back))));
     }
     PULSE_LAUNCH_CHECK("add_rmsnorm");
@@ -161,19 +183,23 @@ extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, c
 // -------------------------------------------------------------- residual add
 // h += delta (used where no norm follows).
 template <typename TD>
-__global__ void residual_add_kernel(float* __restrict__ h, const TD* __restrict__ delta, int64_t n) {
+__global__ void residual_add_kernel(float* __restrict__ h, const TD* __restrict__ delta, int parts, int64_t n) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i < n) h[i] += to_f32<TD>(delta[i]);
+    if (i >= n) return;
+    float v = h[i];
+    for (int p = 0; p < parts; ++p) v += to_f32<TD>(delta[p * n + i]);
+    h[i] = v;
 }
 
-extern "C" int pulse_residual_add(float* h, const void* delta, int delta_dtype, int64_t n, hipStream_t stream) {
-    PULSE_REQUIRE(n >= 0 && pulse_dtype_ok(delta_dtype) && h && delta, "residual_add: bad arguments");
+// delta holds `parts` (>= 1) arrays of n values one after the other; they are added in order.
+extern "C" int pulse_residual_add(float* h, const void* delta, int delta_dtype, int parts, int64_t n, hipStream_t stream) {
+    PULSE_REQUIRE(n >= 0 && parts >= 1 && pulse_dtype_ok(delta_dtype) && h && delta, "residual_add: bad arguments");
     if (n == 0) return 0;
     const int64_t blocks = (n + 255) / 256;
     PULSE_REQUIRE(blocks < (1ll << 31), "residual_add: too many elements (%lld)", static_cast<long long>(n));
     PULSE_DISPATCH_DTYPE(delta_dtype, TD,
         hipLaunchKernelGGL(residual_add_kernel<TD>, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream, h,
-                           static_cast<const TD*>(delta), n));
+                           static_cast<const TD*>(delta), parts, n));
     PULSE_LAUNCH_CHECK("residual_add");
     return 0;
 }

@@ -1,0 +1,273 @@
+// C[M, N] = X[M, K] * W[N, K]^T in bfloat16 on the matrix cores for 9 to 64 rows: the regime of decoding with
+// many requests, where the product still only has to stream the weight from HBM once, but X is too large to be
+// fetched again by every wavefront.
+//
+// A workgroup of four wavefronts owns 64 weight rows (16 a wavefront) and a share of K (grid.y splits K when the
+// weight has too few rows to fill the chip otherwise).  The wavefronts walk K together in chunks of 128: the
+// chunk of X (up to 64 rows) goes through LDS once for all four, two stages, one barrier a chunk; each wavefront
+// streams its 16 weight rows straight into registers, whole 128-byte lines per 16 lanes, and brings them into the
+// matrix-core layout with DPP and ds_bpermute as the few-rows kernel does.  The weight slab is the row operand and
+// X^T the column operand of v_mfma_f32_16x16x32_bf16, so lane l holds output features 4*(l/16)+i of row l%16.
+//
+// Epilogues: bfloat16 store; SwiGLU of a slab-interleaved (gate, up) weight; float32 partial sums [split, M, N] that a
+// consumer adds up in split order (so the result is the same from run to run).  Accumulation is float32
+// (reference: cublasGemmEx with CUBLAS_COMPUTE_32F, src/ops/kernels/cuda/matmul_kernel.cu:132-154).
+#include "common.h"
+
+#include <math.h>
+
+#include <type_traits>
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+
+constexpr int KC = 128;        // k of a chunk: four steps of the matrix-core instruction
+constexpr int XROW = KC + 8;   // bfloat16 a row of X takes in LDS: 16 bytes of padding spread the rows over the banks
+
+enum MidMode : int { MID_BF16 = 0, MID_PARTS = 1 };
+
+__device__ __forceinline__ bf16x8 zeros8() {
+    bf16x8 z;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) z[e] = (__bf16)0.0f;
+    return z;
+}
+
+// NW wavefronts of 16 weight rows each a workgroup; MT tiles of 16 rows of X.
+template <int NW, int MT, bool SWIGLU>
+__global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* __restrict__ X, int64_t ldx,
+                                                                    const bf16_t* __restrict__ W, int64_t ldw,
+                                                                    void* __restrict__ C, int64_t ldc, int M, int N,
+                                                                    int k_len, int mode) {
+    __shared__ __attribute__((aligned(16))) bf16_t s_x[2][16 * MT * XROW];
+    __shared__ f32x4 s_up[SWIGLU ? NW / 2 : 1][MT][PULSE_WAVE];
+    static_assert(!SWIGLU || NW % 2 == 0, "gate and up slabs come in pairs");
+    constexpr int NT = 16 * NW;                                  // weight rows of a workgroup
+    constexpr int THREADS = NW * PULSE_WAVE;
+    constexpr int XP = (256 * MT + THREADS - 1) / THREADS;       // 16-byte pieces of a chunk of X a thread stages
+
+    const int tid = threadIdx.x;
+    const int wave = tid / PULSE_WAVE;
+    const int lane = tid % PULSE_WAVE;
+    const int r = lane % 16;
+    const int kg = lane / 16;
+    const int n_base = blockIdx.x * NT;
+    const int split = blockIdx.y;
+    const int64_t k0 = static_cast<int64_t>(split) * k_len;
+    const int chunks = k_len / KC;
+
+    // Weight loads: 16 consecutive lanes fetch two whole 128-byte lines (rows 2kg + r/8 and that + 8, piece r%8);
+    // rows beyond N repeat the last row: their products only reach outputs that are never stored.
+    const int wrow = n_base + 16 * wave + 2 * kg + (r >> 3);
+    const bf16_t* w0 = W + static_cast<int64_t>(min(wrow, N - 1)) * ldw + k0 + (r & 7) * 8;
+    const bf16_t* w1 = W + static_cast<int64_t>(min(wrow + 8, N - 1)) * ldw + k0 + (r & 7) * 8;
+    // after the exchange of halves, lane (q, i) holds row 2q + i/8 + 8 * (i/4 % 2) and k-group i % 4 of a step;
+    // the operand's lane (kg, r) takes it from there
+    const int source_lane = 16 * ((r >> 1) & 3) + 8 * (r & 1) + 4 * (r >> 3) + kg;
+
+    // X pieces (16 bytes) of a chunk that this thread stages: piece p = tid + THREADS i is row p / 16, columns
+    // 8 (p % 16)..; xdst < 0: no such piece
+    const bf16_t* xsrc[XP];
+    int xdst[XP];
+#pragma unroll
+    for (int i = 0; i < XP; ++i) {
+        const int p = tid + THREADS * i;
+        const int xr = p / 16, xc = p % 16;
+        xsrc[i] = (xr < M && p < 256 * MT) ? X + static_cast<int64_t>(xr) * ldx + k0 + xc * 8 : nullptr;
+        xdst[i] = p < 256 * MT ? xr * XROW + xc * 8 : -1;
+    }
+
+    f32x4 acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // Loads run ahead of their use by more than a trip to memory: the weight RING - 1 chunks (a ring of register
+    // sets), X two chunks (two sets; X comes from L2 for every workgroup but the first).
+    constexpr int RING = 4;
+    bf16x8 xg[2][XP];
+    bf16x8 wr[RING][4];
+    auto load_x = [&](int c, bf16x8 (&x)[XP]) {
+#pragma unroll
+        for (int i = 0; i < XP; ++i)
+            x[i] = (xsrc[i] && c < chunks) ? *reinterpret_cast<const bf16x8*>(xsrc[i] + static_cast<int64_t>(c) * KC) : zeros8();
+    };
+    auto load_w = [&](int c, bf16x8 (&w)[4]) {
+        if (c >= chunks) return;
+#pragma unroll
+        for (int pair = 0; pair < 2; ++pair) {
+            w[2 * pair] = *reinterpret_cast<const bf16x8*>(w0 + static_cast<int64_t>(c) * KC + pair * 64);
+            w[2 * pair + 1] = *reinterpret_cast<const bf16x8*>(w1 + static_cast<int64_t>(c) * KC + pair * 64);
+        }
+    };
+    // One chunk (J = its number modulo RING, which names its register sets): X into its stage, loads for later chunks
+    // on their way, then the products of this one.
+    auto body = [&](auto J, int c) {
+        constexpr int j = decltype(J)::value;
+        bf16_t* stage = s_x[c & 1];
+#pragma unroll
+        for (int i = 0; i < XP; ++i)
+            if (xdst[i] >= 0) *reinterpret_cast<bf16x8*>(stage + xdst[i]) = xg[j % 2][i];
+        // Everybody has left the chunk before the last one (they passed the barrier of the last one), whose stage
+        // this is; after this barrier everybody sees this chunk.
+        __syncthreads();
+        load_x(c + 2, xg[j % 2]);
+        load_w(c + RING - 1, wr[(j + RING - 1) % RING]);
+#pragma unroll
+        for (int pair = 0; pair < 2; ++pair) {
+            const i32x4 l0 = __builtin_bit_cast(i32x4, wr[j][2 * pair]);
+            const i32x4 l1 = __builtin_bit_cast(i32x4, wr[j][2 * pair + 1]);
+            i32x4 a0, a1;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                // lanes 4-7 and 12-15 of a row of 16 take the first half-line of rows 8-15 from four lanes below
+                const int first = __builtin_amdgcn_update_dpp(l0[e], l1[e], 0x114 /* row_shr:4 */, 0xF, 0xA, false);
+                // lanes 0-3 and 8-11 take the second half-line of rows 0-7 from four lanes above
+                const int second = __builtin_amdgcn_update_dpp(l1[e], l0[e], 0x104 /* row_shl:4 */, 0xF, 0x5, false);
+                a0[e] = __builtin_amdgcn_ds_bpermute(source_lane * 4, first);
+                a1[e] = __builtin_amdgcn_ds_bpermute(source_lane * 4, second);
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const bf16x8 a = __builtin_bit_cast(bf16x8, h == 0 ? a0 : a1);
+                const int ks = 2 * pair + h;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const bf16x8 xb = *reinterpret_cast<const bf16x8*>(stage + (16 * mt + r) * XROW + ks * 32 + kg * 8);
+                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, xb, acc[mt], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    static_assert(RING == 4, "the loop below names the four sets");
+    load_x(0, xg[0]);
+    load_w(0, wr[0]);
+    load_x(1, xg[1]);
+    load_w(1, wr[1]);
+    load_w(2, wr[2]);
+    for (int c = 0; c < chunks; c += RING) {
+        body(std::integral_constant<int, 0>{}, c);
+        if (c + 1 < chunks) body(std::integral_constant<int, 1>{}, c + 1);
+        if (c + 2 < chunks) body(std::integral_constant<int, 2>{}, c + 2);
+        if (c + 3 < chunks) body(std::integral_constant<int, 3>{}, c + 3);
+    }
+
+    // lane (kg, r) holds features n_base + 16 wave + 4 kg + i of row 16 mt + r
+    if (!SWIGLU) {
+        const int n = n_base + 16 * wave + 4 * kg;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = 16 * mt + r;
+            if (m >= M || n >= N) continue;
+            if (mode == MID_PARTS) {
+                float* dst = static_cast<float*>(C) + (static_cast<int64_t>(split) * M + m) * ldc + n;
+                if (n + 3 < N) *reinterpret_cast<f32x4*>(dst) = acc[mt];
+                else
+                    for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = acc[mt][i];
+            } else {
+                bf16_t* dst = static_cast<bf16_t*>(C) + static_cast<int64_t>(m) * ldc + n;
+                if (n + 3 < N) {
+                    bf16x4 v;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = (__bf16)acc[mt][i];
+                    *reinterpret_cast<bf16x4*>(dst) = v;
+                } else {
+                    for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = f32_to_bf16(acc[mt][i]);
+                }
+            }
+        }
+    } else {
+        // even wavefronts hold gate slabs, odd ones the up slabs beside them; the output has half as many columns
+        if (wave & 1) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) s_up[wave / 2][mt][lane] = acc[mt];
+        }
+        __syncthreads();
+        if (!(wave & 1)) {
+            const int n = n_base / 2 + 16 * (wave / 2) + 4 * kg;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int m = 16 * mt + r;
+                if (m >= M || 2 * n >= N) continue;
+                const f32x4 up = s_up[wave / 2][mt][lane];
+                bf16_t* dst = static_cast<bf16_t*>(C) + static_cast<int64_t>(m) * ldc + n;
+                bf16x4 v;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float g = acc[mt][i];
+                    v[i] = (__bf16)(g / (1.0f + expf(-g)) * up[i]);
+                }
+                *reinterpret_cast<bf16x4*>(dst) = v;   // N is a multiple of 32: whole groups of four
+            }
+        }
+    }
+}
+
+template <int NW, int MT>
+void launch_mid(const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
+                int k_len, int splits, int mode, bool swiglu, hipStream_t stream) {
+    const dim3 grid((N + 16 * NW - 1) / (16 * NW), splits);
+    const dim3 block(NW * PULSE_WAVE);
+    if constexpr (NW % 2 == 0) {
+        if (swiglu) {
+            hipLaunchKernelGGL((gemm_mid_kernel<NW, MT, true>), grid, block, 0, stream, X, ldx, W, ldw, C, ldc, M, N, k_len, mode);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((gemm_mid_kernel<NW, MT, false>), grid, block, 0, stream, X, ldx, W, ldw, C, ldc, M, N, k_len, mode);
+}
+
+template <int NW>
+void launch_rows(const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
+                 int k_len, int splits, int mode, bool swiglu, hipStream_t stream) {
+    if (M <= 16) launch_mid<NW, 1>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+    else if (M <= 32) launch_mid<NW, 2>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+    else if (M <= 48) launch_mid<NW, 3>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+    else launch_mid<NW, 4>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+}
+
+}  // namespace
+
+// Whether pulse_gemm_mid takes a shape: 1..64 rows, K cut into `splits` shares that are multiples of 128.
+extern "C" int pulse_gemm_mid_takes(int M, int N, int K, int splits) {
+    return M >= 1 && M <= 64 && N > 0 && K > 0 && splits >= 1 && splits <= 64 && K % splits == 0 && (K / splits) % KC == 0;
+}
+
+// mode 0: C is bfloat16 [M, N] (splits must be 1).  mode 1: C is float32 [splits, M, N] (row stride ldc), the partial
+// products of the shares of K, to be added up by the consumer in split order.  swiglu != 0 (mode 0, splits 1): W holds
+// gate and up rows interleaved in slabs of 16 (gate slab, up slab, ...), N counts both, C is bfloat16 [M, N / 2] =
+// silu(gate) * up.
+// waves: wavefronts (of 16 weight rows) a workgroup, 2, 3, 4 or 6; 0 lets the entry point choose.
+extern "C" int pulse_gemm_mid(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
+                              int K, int mode, int swiglu, int splits, int waves, hipStream_t stream) {
+    PULSE_REQUIRE(pulse_gemm_mid_takes(M, N, K, splits), "gemm_mid: M=%d (1..64) N=%d K=%d in %d shares (multiples of %d)",
+                  M, N, K, splits, KC);
+    PULSE_REQUIRE(X && W && C, "gemm_mid: null pointer");
+    PULSE_REQUIRE(ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K, "gemm_mid: the row strides must be multiples of 8 and cover K");
+    PULSE_REQUIRE((reinterpret_cast<uintptr_t>(X) % 16) == 0 && (reinterpret_cast<uintptr_t>(W) % 16) == 0 &&
+                  (reinterpret_cast<uintptr_t>(C) % 16) == 0, "gemm_mid: operands must be 16-byte aligned");
+    PULSE_REQUIRE(mode == MID_BF16 || mode == MID_PARTS, "gemm_mid: unknown output mode %d", mode);
+    PULSE_REQUIRE(mode == MID_PARTS || splits == 1, "gemm_mid: a bfloat16 result needs all of K in one share");
+    PULSE_REQUIRE(ldc % 4 == 0, "gemm_mid: the output's row stride must be a multiple of 4");
+    if (swiglu) {
+        PULSE_REQUIRE(mode == MID_BF16 && N % 32 == 0 && ldc >= N / 2, "gemm_mid: SwiGLU needs N %% 32 == 0 and bfloat16 output");
+    } else {
+        PULSE_REQUIRE(ldc >= N, "gemm_mid: output row stride too small");
+    }
+    const bf16_t* x = static_cast<const bf16_t*>(X);
+    const bf16_t* w = static_cast<const bf16_t*>(W);
+    const int k_len = K / splits;
+    if (waves == 0) waves = 4;
+    PULSE_REQUIRE(waves == 2 || waves == 3 || waves == 4 || waves == 6, "gemm_mid: 2, 3, 4 or 6 wavefronts a workgroup, got %d", waves);
+    PULSE_REQUIRE(!swiglu || waves % 2 == 0, "gemm_mid: SwiGLU needs an even number of wavefronts");
+    if (waves == 2) launch_rows<2>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
+    else if (waves == 3) launch_rows<3>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
+    else if (waves == 4) launch_rows<4>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
+    else launch_rows<6>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
+    PULSE_LAUNCH_CHECK("gemm_mid");
+    return 0;
+}

@@ -82,7 +82,6 @@ class CausalLM:
         if ctx.num_wanted == 0:
             return logits
         x = ws.buffer("model.final", ctx.num_wanted, self.hidden_size, self.act_dtype)
-        self.final_norm.apply(stream.h, stream.pending, x, rows=ctx.want_rows)
-        stream.pending = None
+        self.final_norm.apply(stream.h, stream.pending_for(self.final_norm), x, rows=ctx.want_rows)
         self.head.forward(x, logits)
         return logits

@@ -78,7 +78,8 @@ def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, bad_
 
 def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
                 out: torch.Tensor, rows: Optional[torch.Tensor] = None, write_back: bool = True) -> None:
-    """out[r] = rmsnorm(h[s] + delta[s]) * weight, s = rows[r] or r; with write_back h[s] keeps the sum."""
+    """out[r] = rmsnorm(h[s] + delta[s]) * weight, s = rows[r] or r; with write_back h[s] keeps the sum.
+    ``delta`` may be float32 [parts, T, H]: the shares of a product whose inner dimension was split, added in order."""
     _gpu("add_rmsnorm", h, delta, weight, out, rows)
     _need(h.dtype == torch.float32 and h.dim() == 2 and h.is_contiguous(), "add_rmsnorm: h must be contiguous float32 [T, H]")
     hidden = h.shape[1]
@@ -86,21 +87,31 @@ def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
     if rows is not None:
         _int_vec("add_rmsnorm: rows", rows)
         write_back = False
+    parts = 1
     if delta is not None:
-        _need(delta.shape == h.shape and delta.is_contiguous(), "add_rmsnorm: delta must match h")
+        if delta.dim() == 3:
+            parts = delta.shape[0]
+            _need(parts >= 1 and delta.shape[1:] == h.shape and delta.is_contiguous() and delta.dtype == torch.float32
+                  and hidden % 4 == 0, "add_rmsnorm: an update in parts must be contiguous float32 [parts, T, H], H % 4 == 0")
+        else:
+            _need(delta.shape == h.shape and delta.is_contiguous(), "add_rmsnorm: delta must match h")
     _need(weight.numel() == hidden and weight.is_contiguous(), f"add_rmsnorm: weight must hold {hidden} values")
     _need(out.is_contiguous() and tuple(out.shape) == (n_out, hidden),
           f"add_rmsnorm: out must be [{n_out}, {hidden}], got {tuple(out.shape)}")
     call("pulse_add_rmsnorm", _ptr(h), _ptr(delta), _i32(_tag(delta, "add_rmsnorm") if delta is not None else 0),
-         _ptr(rows), _ptr(weight), _i32(_tag(weight, "add_rmsnorm")), _ptr(out), _i32(_tag(out, "add_rmsnorm")),
+         _i32(parts), _i64(h.numel()), _ptr(rows), _ptr(weight), _i32(_tag(weight, "add_rmsnorm")), _ptr(out), _i32(_tag(out, "add_rmsnorm")),
          _i32(n_out), _i32(hidden), _f32(eps), _i32(1 if (write_back and delta is not None) else 0), _stream())
 
 
 def residual_add(h: torch.Tensor, delta: torch.Tensor) -> None:
+    """h += delta; ``delta`` of the shape of h, or [parts, *h.shape] (added in order)."""
     _gpu("residual_add", h, delta)
-    _need(h.dtype == torch.float32 and h.is_contiguous() and delta.is_contiguous() and h.shape == delta.shape,
-          "residual_add: h must be contiguous float32 and delta of the same shape")
-    call("pulse_residual_add", _ptr(h), _ptr(delta), _i32(_tag(delta, "residual_add")), _i64(h.numel()), _stream())
+    parts = delta.shape[0] if delta.dim() == h.dim() + 1 else 1
+    _need(h.dtype == torch.float32 and h.is_contiguous() and delta.is_contiguous()
+          and (delta.shape == h.shape or delta.shape[1:] == h.shape),
+          "residual_add: h must be contiguous float32 and delta of the same shape (or several of them)")
+    call("pulse_residual_add", _ptr(h), _ptr(delta), _i32(_tag(delta, "residual_add")), _i32(parts), _i64(h.numel()),
+         _stream())
 
 
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor, slab: int = 0) -> None:
@@ -228,6 +239,39 @@ def gemm_skinny(a: Optional[torch.Tensor], w: torch.Tensor, out: torch.Tensor, a
         call("pulse_gemm_skinny_fused", _ptr(a), _i64(ldx), _ptr(w), _i64(w.stride(0) if n > 1 else k), _ptr(out),
              _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0),
              _i32(tune), _ptr(None), _ptr(None), _i32(0), _ptr(None), _f32(0.0), _ptr(sumsq_out), _stream())
+
+
+def gemm_mid_takes(m: int, n: int, k: int, splits: int = 1) -> bool:
+    """Whether ``gemm_mid`` takes a shape (as pulse_gemm_mid_takes)."""
+    return 1 <= m <= 64 and n > 0 and k > 0 and 1 <= splits <= 64 and k % splits == 0 and (k // splits) % 128 == 0
+
+
+def gemm_mid(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False, splits: int = 1,
+             waves: int = 0) -> None:
+    """a @ w^T for up to 64 rows of bfloat16 with X shared through LDS (the regime of 9 to 64 rows).
+
+    ``out`` bfloat16 [M, N]: the product (``splits`` must be 1); with ``swiglu`` the weight holds gate and up rows in
+    alternating slabs of 16 and out [M, N / 2] is silu(gate) * up.  ``out`` float32 [splits, M, N]: the partial
+    products of ``splits`` equal shares of K, which the consumer adds up in order."""
+    _gpu("gemm_mid", a, w, out)
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and w.dim() == 2
+          and a.stride(1) == 1 and w.stride(1) == 1, "gemm_mid: a and w must be bfloat16 matrices with contiguous rows")
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k, f"gemm_mid: inner sizes differ ({k} and {w.shape[1]})")
+    _need(gemm_mid_takes(m, n, k, splits), f"gemm_mid: M={m} N={n} K={k} in {splits} shares is not a shape it takes")
+    if out.dtype == torch.float32:
+        _need(not swiglu and out.is_contiguous() and tuple(out.shape) == (splits, m, n),
+              f"gemm_mid: partial sums go to a contiguous float32 [{splits}, {m}, {n}]")
+        mode, ldc = 1, n
+    else:
+        cols = n // 2 if swiglu else n
+        _need(out.dtype == torch.bfloat16 and splits == 1 and out.dim() == 2 and out.shape[0] == m
+              and out.shape[1] == cols and out.stride(1) == 1, f"gemm_mid: out must be bfloat16 [{m}, {cols}]")
+        mode, ldc = 0, (out.stride(0) if m > 1 else cols)
+    call("pulse_gemm_mid", _ptr(a), _i64(a.stride(0) if m > 1 else k), _ptr(w), _i64(w.stride(0) if n > 1 else k),
+         _ptr(out), _i64(ldc), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0), _i32(splits), _i32(waves),
+         _stream())
 
 
 def _check_cache(what: str, kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, d: int):

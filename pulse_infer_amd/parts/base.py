@@ -196,9 +196,18 @@ class ResidualStream:
         self.pending: Optional[torch.Tensor] = None
         self.stats: Optional[RowStats] = None
 
+    def pending_for(self, norm: Any) -> Optional[torch.Tensor]:
+        """The update not yet added, in a form ``norm`` takes: an update in parts ([parts, T, H] float32, the shares of
+        a product whose inner dimension was split) is added to ``h`` first unless the norm says ``takes_parts``."""
+        pending, self.pending = self.pending, None
+        if pending is not None and pending.dim() == 3 and not getattr(norm, "takes_parts", False):
+            from ..ops import kernels
+            kernels.residual_add(self.h, pending)
+            return None
+        return pending
+
     def normed(self, norm: Any, out: torch.Tensor) -> torch.Tensor:
-        norm.apply(self.h, self.pending, out)
-        self.pending = None
+        norm.apply(self.h, self.pending_for(norm), out)
         return out
 
     def lazy(self, norm: Any) -> Optional[LazyNorm]:
@@ -211,7 +220,8 @@ class ResidualStream:
         return norm.lazy(self.h, self.stats)
 
     def push(self, delta: Any) -> None:
-        """Hand over an update; None or RowStats mean the part has already added it to ``h``."""
+        """Hand over an update ([T, H], or [parts, T, H] float32 to be added in order); None or RowStats mean the part
+        has already added it to ``h``."""
         if isinstance(delta, RowStats):
             self.stats = delta
             return

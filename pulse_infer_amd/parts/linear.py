@@ -43,7 +43,10 @@ class Linear:
             kernels.gemm_skinny(None, w, out, swiglu=swiglu, norm=(x.h, x.sumsq, x.weight, x.eps))
             return out
         if swiglu:
-            kernels.gemm_skinny(x, w, out, swiglu=True)
+            if x.shape[0] > kernels.SKINNY_FAST_ROWS:
+                kernels.gemm_mid(x, w, out, swiglu=True)
+            else:
+                kernels.gemm_skinny(x, w, out, swiglu=True)
             return out
         if self.library and x.dtype == torch.bfloat16:
             few = x.shape[0] <= kernels.SKINNY_FAST_ROWS
@@ -78,4 +81,38 @@ class Linear:
                 return RowStats(sums)
             kernels.gemm_skinny(x, self.weight, residual, add=True)
             return None
+        splits = self.shares_for(x)
+        if workspace is not None and splits:
+            # 17 to 64 rows: the product's inner dimension is shared out over workgroups; the shares' float32 results
+            # are the update, which the next norm adds up in order
+            rows = x.shape[0]
+            parts = workspace.buffer(f"linear.parts.{self.out_features}.{self.in_features}", splits * rows,
+                                     self.out_features, torch.float32).view(splits, rows, self.out_features)
+            kernels.gemm_mid(x, self.weight, parts, splits=splits)
+            return parts
         return self.forward(x, scratch)
+
+    MID_ROWS = (17, 64)          # where the product with X shared through LDS beats the library's (with SwiGLU inside)
+    SHARES_FROM_ROWS = 49        # from here on sharing out the inner dimension pays (measured: a decoding step of the
+                                 # 8B shape is 1-5% slower with it at 20 to 48 rows, 3% faster at 64: the norm that
+                                 # adds the parts up runs on one compute unit a row)
+    MID_WORKGROUPS = 512         # workgroups wanted of it (64 weight rows times a share of the inner dimension each)
+
+    def takes_mid(self, x: torch.Tensor) -> bool:
+        return (self.library and x.dtype == torch.bfloat16 and self.MID_ROWS[0] <= x.shape[0] <= self.MID_ROWS[1]
+                and kernels.gemm_skinny_ok(x, self.weight))
+
+    def shares_for(self, x: torch.Tensor) -> int:
+        """Into how many shares the inner dimension is cut for an update in parts; 0: not this product."""
+        if not self.takes_mid(x) or x.shape[0] < self.SHARES_FROM_ROWS or self.out_features % 4:
+            return 0
+        tiles = (self.out_features + 63) // 64
+        best = 0
+        for splits in range(1, 17):
+            # a share of at least 1024: every further part costs the norm that adds them up about 0.5 us
+            if self.in_features % splits or (self.in_features // splits) % 128 or self.in_features // splits < 1024:
+                continue
+            best = splits
+            if tiles * splits >= self.MID_WORKGROUPS:
+                break
+        return best

@@ -62,6 +62,9 @@ class GatedMLP(Part):
             self.gate_up.forward(x, z, swiglu=True)
         elif (self.slab and tokens <= kernels.SKINNY_FAST_ROWS and kernels.gemm_skinny_ok(x, self.gate_up.weight)):
             self.gate_up.forward(x, z, swiglu=True)
+        elif (self.slab and self.gate_up.takes_mid(x) and (2 * self.inter) % 32 == 0
+              and kernels.gemm_mid_takes(tokens, 2 * self.inter, self.hidden)):
+            self.gate_up.forward(x, z, swiglu=True)   # 17 to 64 rows: X shared through LDS, SwiGLU in the epilogue
         else:
             gu = ws.buffer("mlp.gate_up", tokens, 2 * self.inter, self.act_dtype)
             self.gate_up.forward(x, gu)

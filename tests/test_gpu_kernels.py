@@ -687,6 +687,98 @@ def test_gemm_skinny_refuses(k):
         k.gemm_skinny(a[:4], w, torch.zeros(4, 32, dtype=torch.bfloat16, device=DEV), add=True)
 
 
+@pytest.mark.parametrize("m", [1, 16, 17, 33, 48, 64])
+@pytest.mark.parametrize("n,kk", [(200, 128), (4096 + 16, 384), (96, 4096), (64, 1536)])
+def test_gemm_mid(k, m, n, kk):
+    """The product for 17 to 64 rows (X shared through LDS) at every workgroup shape, whole and in shares of the
+    inner dimension, against float64: a wavefront that took another's weight rows, a piece of X staged to the wrong
+    place or a chunk used before it had landed would change the sums."""
+    a, aref = as_stored(rnd(m, kk, seed=90), torch.bfloat16)
+    w, wref = as_stored(rnd(n, kk, seed=91), torch.bfloat16)
+    want = aref @ wref.T
+    first = None
+    for waves in (0, 2, 3, 4, 6):
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+        k.gemm_mid(a, w, out, waves=waves)
+        assert torch.allclose(out.cpu().to(F64), want, atol=3e-2 * math.sqrt(kk / 128), rtol=1e-2), waves
+        first = out if first is None else first
+        assert torch.equal(out, first)                      # the sums do not depend on the workgroup's shape
+    for splits in (1, 2, 3, 4, 12):
+        if not k.gemm_mid_takes(m, n, kk, splits):
+            continue
+        parts = torch.full((splits, m, n), float("nan"), device=DEV)
+        k.gemm_mid(a, w, parts, splits=splits)
+        share = kk // splits
+        for s_ in range(splits):                            # every share is the product over its part of K
+            part = aref[:, s_ * share:(s_ + 1) * share] @ wref[:, s_ * share:(s_ + 1) * share].T
+            assert torch.allclose(parts[s_].cpu().to(F64), part, atol=2e-3 * math.sqrt(share), rtol=1e-5), (splits, s_)
+        again = torch.empty_like(parts)
+        k.gemm_mid(a, w, again, splits=splits, waves=2)
+        assert torch.equal(again, parts)
+    if m > 1:                                                # strided rows (a view into a wider buffer)
+        wide = torch.zeros(m, kk + 24, dtype=torch.bfloat16, device=DEV)
+        wide[:, :kk] = a
+        out = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+        k.gemm_mid(wide[:, :kk], w, out)
+        assert torch.equal(out, first)
+
+
+@pytest.mark.parametrize("m", [3, 17, 40, 64])
+@pytest.mark.parametrize("inter,kk", [(48, 128), (1008, 256), (96, 2048)])
+def test_gemm_mid_swiglu(k, m, inter, kk):
+    a, aref = as_stored(rnd(m, kk, seed=93), torch.bfloat16)
+    gate, gref = as_stored(rnd(inter, kk, seed=94, scale=kk ** -0.5), torch.bfloat16)
+    up, uref = as_stored(rnd(inter, kk, seed=95, scale=kk ** -0.5), torch.bfloat16)
+    mixed = torch.stack([gate.view(-1, 16, kk), up.view(-1, 16, kk)], dim=1).reshape(2 * inter, kk).contiguous()
+    want = P.silu(aref @ gref.T) * (aref @ uref.T)
+    for waves in (0, 2, 4, 6):
+        out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+        k.gemm_mid(a, mixed, out, swiglu=True, waves=waves)
+        assert torch.allclose(out.cpu().to(F64), want, atol=1e-2, rtol=1e-2), waves
+
+
+def test_gemm_mid_refuses(k):
+    from pulse_infer_amd.ops import KernelError
+    a = torch.zeros(65, 256, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(64, 256, dtype=torch.bfloat16, device=DEV)
+    assert k.gemm_mid_takes(64, 64, 256) and not k.gemm_mid_takes(65, 64, 256)
+    assert not k.gemm_mid_takes(8, 64, 192) and not k.gemm_mid_takes(8, 64, 256, 3) and k.gemm_mid_takes(8, 64, 256, 2)
+    with pytest.raises(KernelError, match="not a shape"):
+        k.gemm_mid(a, w, torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(KernelError, match="partial sums"):
+        k.gemm_mid(a[:8], w, torch.zeros(8, 64, device=DEV), splits=2)
+    with pytest.raises(KernelError, match="bfloat16"):
+        k.gemm_mid(a[:8], w, torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV), splits=2)
+    with pytest.raises(KernelError, match="wavefronts"):
+        k.gemm_mid(a[:8], w, torch.zeros(8, 32, dtype=torch.bfloat16, device=DEV), swiglu=True, waves=3)
+
+
+@pytest.mark.parametrize("hidden", [48, 4096])
+def test_an_update_in_parts_is_added_in_order(k, hidden):
+    """h + the parts of an update (the shares of a product whose inner dimension was split), in the norm's kernel
+    and in the plain addition, with and without gathered rows."""
+    rows, parts, eps = 20, 5, 1e-5
+    h0 = rnd(rows, hidden, seed=96).to(DEV)
+    delta = rnd(parts, rows, hidden, seed=97).to(DEV)
+    w, wref = as_stored(1 + 0.1 * rnd(hidden, seed=98), torch.bfloat16)
+    total = h0.clone()
+    for p_ in range(parts):
+        total += delta[p_]                                  # float32, in order: the kernel's own sums
+    h = h0.clone()
+    out = torch.empty(rows, hidden, dtype=torch.bfloat16, device=DEV)
+    k.add_rmsnorm(h, delta, w, eps, out)
+    assert torch.equal(h, total)
+    assert torch.allclose(out.cpu().to(F64), P.rms_norm(total.cpu().to(F64), wref, eps), **tol(torch.bfloat16))
+    pick = torch.tensor([19, 0, 7], dtype=torch.int32, device=DEV)
+    h = h0.clone()
+    some = torch.empty(3, hidden, dtype=torch.bfloat16, device=DEV)
+    k.add_rmsnorm(h, delta, w, eps, some, rows=pick)
+    assert torch.equal(h, h0) and torch.equal(some, out[pick.long()])
+    h = h0.clone()
+    k.residual_add(h, delta)
+    assert torch.equal(h, total)
+
+
 def test_two_stage_argmax(k):
     for rows, vocab in ((1, 5), (3, 2048), (8, 151936), (5, 4097)):
         logits = rnd(rows, vocab, seed=80 + rows).to(DEV)
