@@ -91,8 +91,10 @@ template <> __device__ __forceinline__ ushort4 narrow4<bf16_t>(float4 v) {
     return make_ushort4(f32_to_bf16(v.x), f32_to_bf16(v.y), f32_to_bf16(v.z), f32_to_bf16(v.w));
 }
 
-template <typename TD, typename TW, typename TY>
-__global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
+// THREADS threads a row: 256, or 1024 for few rows and for an update in parts (a row then has enough loads in
+// flight to be read at more than the rate of one wavefront's round trips).
+template <typename TD, typename TW, typename TY, int THREADS>
+__global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                                               int parts, int64_t part_stride,
                                                               const int* __restrict__ rows, const TW* __restrict__ w,
                                                               TY* __restrict__ y, int hidden, float eps, int write_back) {
@@ -105,10 +107,11 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     const int nvec = hidden / 4;
     float4* hrow = reinterpret_cast<float4*>(h + s * hidden);
     const VD* drow = delta ? reinterpret_cast<const VD*>(delta + s * hidden) : nullptr;
-    float4 v[RMS_CHUNKS];
+    constexpr int CHUNKS = RMS_CHUNKS * 256 / THREADS;
+    float4 v[CHUNKS];
 #pragma unroll
-    for (int c = 0; c < RMS_CHUNKS; ++c) {
-        const int i = threadIdx.x + c * 256;
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * THREADS;
         if (i < nvec) v[c] = hrow[i];
     }
     if (drow) {
@@ -116,23 +119,23 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
         // several parts are asked for before the first is added, since few rows are bound by the trips to memory.
 #pragma unroll 8
         for (int p = 0; p < parts; ++p) {
-            float4 d[RMS_CHUNKS];
+            float4 d[CHUNKS];
 #pragma unroll
-            for (int c = 0; c < RMS_CHUNKS; ++c) {
-                const int i = threadIdx.x + c * 256;
+            for (int c = 0; c < CHUNKS; ++c) {
+                const int i = threadIdx.x + c * THREADS;
                 if (i < nvec) d[c] = widen4(drow[p * (part_stride / 4) + i]);
             }
 #pragma unroll
-            for (int c = 0; c < RMS_CHUNKS; ++c) {
-                const int i = threadIdx.x + c * 256;
+            for (int c = 0; c < CHUNKS; ++c) {
+                const int i = threadIdx.x + c * THREADS;
                 if (i < nvec) { v[c].x += d[c].x; v[c].y += d[c].y; v[c].z += d[c].z; v[c].w += d[c].w; }
             }
         }
     }
     float ss = 0.f;
 #pragma unroll
-    for (int c = 0; c < RMS_CHUNKS; ++c) {
-        const int i = threadIdx.x + c * 256;
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * THREADS;
         if (i < nvec) ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
     }
     ss = block_sum(ss, scratch);
@@ -140,8 +143,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_vec_kernel(float* __restrict_
     VY* yrow = reinterpret_cast<VY*>(y + static_cast<int64_t>(r) * hidden);
     const VW* wv = reinterpret_cast<const VW*>(w);
 #pragma unroll
-    for (int c = 0; c < RMS_CHUNKS; ++c) {
-        const int i = threadIdx.x + c * 256;
+    for (int c = 0; c < CHUNKS; ++c) {
+        const int i = threadIdx.x + c * THREADS;
         if (i < nvec) {
             if (write_back) hrow[i] = v[c];
             const float4 ww = widen4(wv[i]);
@@ -167,9 +170,14 @@ extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, i
                          (reinterpret_cast<uintptr_t>(w) % 16 == 0) && (reinterpret_cast<uintptr_t>(delta) % 16 == 0);
     if (hidden % 4 == 0 && hidden <= 256 * 4 * RMS_CHUNKS && aligned) {
         PULSE_DISPATCH_DTYPE(delta_dtype, TD, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(y_dtype, TY,
-            hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY>), dim3(out_rows), dim3(256), 0, stream, h,
-                               static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
-                               static_cast<TY*>(y), hidden, eps, write_back))));
+            if (parts > 1 || (out_rows <= 256 && hidden >= 2048))   // few rows: bound by round trips, not by bandwidth
+                hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 1024>), dim3(out_rows), dim3(1024), 0, stream, h,
+                                   static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
+                                   static_cast<TY*>(y), hidden, eps, write_back);
+            else
+                hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 256>), dim3(out_rows), dim3(256), 0, stream, h,
+                                   static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
+                                   static_cast<TY*>(y), hidden, eps, write_back))));
     } else {
         PULSE_DISPATCH_DTYPE(delta_dtype, TD, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(y_dtype, TY,
             hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TW, TY>), dim3(out_rows), dim3(256), 0, stream, h,

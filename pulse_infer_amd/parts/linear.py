@@ -93,9 +93,9 @@ class Linear:
         return self.forward(x, scratch)
 
     MID_ROWS = (17, 64)          # where the product with X shared through LDS beats the library's (with SwiGLU inside)
-    SHARES_FROM_ROWS = 49        # from here on sharing out the inner dimension pays (measured: a decoding step of the
-                                 # 8B shape is 1-5% slower with it at 20 to 48 rows, 3% faster at 64: the norm that
-                                 # adds the parts up runs on one compute unit a row)
+    SHARES_FROM_ROWS = 17        # from here on the inner dimension of a product that adds into the residual is shared
+                                 # out over workgroups (measured on the 8B shape: a decoding step gains 1% at 17 to 32
+                                 # rows, 4% at 48, 6% at 64)
     MID_WORKGROUPS = 512         # workgroups wanted of it (64 weight rows times a share of the inner dimension each)
 
     def takes_mid(self, x: torch.Tensor) -> bool:
