@@ -69,9 +69,18 @@ class Linear:
 
     def add_into(self, x: torch.Tensor, residual: torch.Tensor, scratch: torch.Tensor,
                  workspace: Optional[Workspace] = None):
-        """residual += x W^T where the kernel can do that itself: returns None, or, given a workspace and a shape the
-        fused kernel takes, the ``RowStats`` of the updated rows.  Otherwise the product is written to ``scratch`` and
-        returned for the caller to add."""
+        """residual += x W^T, in one of four ways.  Few rows: the kernel adds into the residual itself and None is
+        returned, or, given a workspace and a shape the fused kernel takes, the ``RowStats`` of the updated rows.  Up to
+        64 rows, given a workspace: the product's inner dimension is shared out over workgroups and the shares' float32
+        results [parts, rows, out] are returned as the update, which the next norm adds up in order.  Otherwise the
+        product is written to ``scratch`` and returned for the caller to add."""
+        splits = self.shares_for(x) if workspace is not None else 0
+        if splits:
+            rows = x.shape[0]
+            parts = workspace.buffer(f"linear.parts.{self.out_features}.{self.in_features}", splits * rows,
+                                     self.out_features, torch.float32).view(splits, rows, self.out_features)
+            kernels.gemm_mid(x, self.weight, parts, splits=splits)
+            return parts
         if (self.library and x.dtype == torch.bfloat16 and x.shape[0] <= kernels.SKINNY_FAST_ROWS
                 and kernels.gemm_skinny_ok(x, self.weight)):
             if workspace is not None and kernels.gemm_skinny_fusable(x.shape[0], self.out_features, self.in_features):
@@ -81,15 +90,6 @@ class Linear:
                 return RowStats(sums)
             kernels.gemm_skinny(x, self.weight, residual, add=True)
             return None
-        splits = self.shares_for(x)
-        if workspace is not None and splits:
-            # 17 to 64 rows: the product's inner dimension is shared out over workgroups; the shares' float32 results
-            # are the update, which the next norm adds up in order
-            rows = x.shape[0]
-            parts = workspace.buffer(f"linear.parts.{self.out_features}.{self.in_features}", splits * rows,
-                                     self.out_features, torch.float32).view(splits, rows, self.out_features)
-            kernels.gemm_mid(x, self.weight, parts, splits=splits)
-            return parts
         return self.forward(x, scratch)
 
     MID_ROWS = (17, 64)          # where the product with X shared through LDS beats the library's (with SwiGLU inside)
@@ -104,7 +104,8 @@ class Linear:
 
     def shares_for(self, x: torch.Tensor) -> int:
         """Into how many shares the inner dimension is cut for an update in parts; 0: not this product."""
-        if not self.takes_mid(x) or x.shape[0] < self.SHARES_FROM_ROWS or self.out_features % 4:
+        if not (self.library and x.dtype == torch.bfloat16 and self.SHARES_FROM_ROWS <= x.shape[0] <= self.MID_ROWS[1]
+                and kernels.gemm_skinny_ok(x, self.weight)) or self.out_features % 4:
             return 0
         tiles = (self.out_features + 63) // 64
         best = 0
