@@ -93,7 +93,8 @@ template <> __device__ __forceinline__ ushort4 narrow4<bf16_t>(float4 v) {
 
 // THREADS threads a row: 256, or 1024 for few rows and for an update in parts (a row then has enough loads in
 // flight to be read at more than the rate of one wavefront's round trips).
-template <typename TD, typename TW, typename TY, int THREADS>
+// PARTS: the update may come in parts (kept apart so that the kernel for one update needs no more registers than it did).
+template <typename TD, typename TW, typename TY, int THREADS, bool PARTS>
 __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restrict__ h, const TD* __restrict__ delta,
                                                               int parts, int64_t part_stride,
                                                               const int* __restrict__ rows, const TW* __restrict__ w,
@@ -109,12 +110,26 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
     const VD* drow = delta ? reinterpret_cast<const VD*>(delta + s * hidden) : nullptr;
     constexpr int CHUNKS = RMS_CHUNKS * 256 / THREADS;
     float4 v[CHUNKS];
+    float ss = 0.f;
+    if (!PARTS) {
 #pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-        const int i = threadIdx.x + c * THREADS;
-        if (i < nvec) v[c] = hrow[i];
-    }
-    if (drow) {
+        for (int c = 0; c < CHUNKS; ++c) {
+            const int i = threadIdx.x + c * THREADS;
+            if (i < nvec) {
+                v[c] = hrow[i];
+                if (drow) {
+                    const float4 d = widen4(drow[i]);
+                    v[c].x += d.x; v[c].y += d.y; v[c].z += d.z; v[c].w += d.w;
+                }
+                ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < CHUNKS; ++c) {
+            const int i = threadIdx.x + c * THREADS;
+            if (i < nvec) v[c] = hrow[i];
+        }
         // The parts of an update (shares of a product's inner dimension) are added in their order; the loads of
         // several parts are asked for before the first is added, since few rows are bound by the trips to memory.
 #pragma unroll 8
@@ -131,12 +146,11 @@ __global__ __launch_bounds__(THREADS) void add_rmsnorm_vec_kernel(float* __restr
                 if (i < nvec) { v[c].x += d[c].x; v[c].y += d[c].y; v[c].z += d[c].z; v[c].w += d[c].w; }
             }
         }
-    }
-    float ss = 0.f;
 #pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-        const int i = threadIdx.x + c * THREADS;
-        if (i < nvec) ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
+        for (int c = 0; c < CHUNKS; ++c) {
+            const int i = threadIdx.x + c * THREADS;
+            if (i < nvec) ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
+        }
     }
     ss = block_sum(ss, scratch);
     const float inv = 1.0f / sqrtf(ss / static_cast<float>(hidden) + eps);
@@ -170,12 +184,16 @@ extern "C" int pulse_add_rmsnorm(float* h, const void* delta, int delta_dtype, i
                          (reinterpret_cast<uintptr_t>(w) % 16 == 0) && (reinterpret_cast<uintptr_t>(delta) % 16 == 0);
     if (hidden % 4 == 0 && hidden <= 256 * 4 * RMS_CHUNKS && aligned) {
         PULSE_DISPATCH_DTYPE(delta_dtype, TD, PULSE_DISPATCH_DTYPE(w_dtype, TW, PULSE_DISPATCH_DTYPE(y_dtype, TY,
-            if (parts > 1 || (out_rows <= 256 && hidden >= 2048))   // few rows: bound by round trips, not by bandwidth
-                hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 1024>), dim3(out_rows), dim3(1024), 0, stream, h,
+            if (parts > 1)
+                hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 1024, true>), dim3(out_rows), dim3(1024), 0, stream, h,
+                                   static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
+                                   static_cast<TY*>(y), hidden, eps, write_back);
+            else if (out_rows <= 256 && hidden >= 2048)   // few rows: bound by round trips, not by bandwidth
+                hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 1024, false>), dim3(out_rows), dim3(1024), 0, stream, h,
                                    static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
                                    static_cast<TY*>(y), hidden, eps, write_back);
             else
-                hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 256>), dim3(out_rows), dim3(256), 0, stream, h,
+                hipLaunchKernelGGL((add_rmsnorm_vec_kernel<TD, TW, TY, 256, false>), dim3(out_rows), dim3(256), 0, stream, h,
                                    static_cast<const TD*>(delta), parts, part_stride, rows, static_cast<const TW*>(w),
                                    static_cast<TY*>(y), hidden, eps, write_back))));
     } else {
