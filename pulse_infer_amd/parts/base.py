@@ -186,10 +186,10 @@ class ResidualStream:
     hand back ``RowStats`` of the new ``h``; they stay valid until ``h`` changes again.
     """
 
-    # Up to here a consumer that forms the norm itself is faster than the norm's kernel followed by it (measured:
-    # 6% of a decoding step at 2 rows, 1.6% at 8; with more rows every k-step of the product reads the float32
-    # residual and the norm's kernel wins).
-    LAZY_MAX_ROWS = 8
+    # Up to here a consumer that forms the norm itself is faster than the norm's kernel followed by it (measured on a
+    # decoding step: 5% at 1 row, 0.3% at 6; at 8 rows the norm's kernel wins by 2.5%: every k-step of the product
+    # reads the float32 residual then).
+    LAZY_MAX_ROWS = 6
 
     def __init__(self, h: torch.Tensor):
         self.h = h

@@ -17,7 +17,7 @@ from typing import Optional
 import torch
 
 from ..ops import kernels
-from .base import LazyNorm, RowStats, Workspace
+from .base import LazyNorm, ResidualStream, RowStats, Workspace
 
 
 class Linear:
@@ -83,7 +83,8 @@ class Linear:
             return parts
         if (self.library and x.dtype == torch.bfloat16 and x.shape[0] <= kernels.SKINNY_FAST_ROWS
                 and kernels.gemm_skinny_ok(x, self.weight)):
-            if workspace is not None and kernels.gemm_skinny_fusable(x.shape[0], self.out_features, self.in_features):
+            if (workspace is not None and x.shape[0] <= ResidualStream.LAZY_MAX_ROWS   # nobody would use them otherwise
+                    and kernels.gemm_skinny_fusable(x.shape[0], self.out_features, self.in_features)):
                 sums = workspace.buffer(f"linear.sumsq.{self.out_features}", x.shape[0], (self.out_features + 15) // 16,
                                         torch.float32)
                 kernels.gemm_skinny(x, self.weight, residual, add=True, sumsq_out=sums)
