@@ -457,6 +457,7 @@ def test_attn_mfma_refuses_other_sizes(k):
     dict(nq=6, nkv=1, d=32, rot=0, pairing="interleaved", norm=False, bs=16, window=0, lens=[150, 2]),
     dict(nq=4, nkv=4, d=128, rot=64, pairing="half", norm=False, bs=64, window=0, lens=[97, 200]),
     dict(nq=16, nkv=1, d=224, rot=224, pairing="interleaved", norm=True, bs=16, window=100, lens=[260, 130]),
+    dict(nq=40, nkv=2, d=64, rot=32, pairing="interleaved", norm=True, bs=64, window=0, lens=[200, 77, 64]),  # 20 heads a kv head: two chunks
 ])
 @pytest.mark.parametrize("split", [None, 32, 128])
 @pytest.mark.parametrize("new_key", [True, False])
