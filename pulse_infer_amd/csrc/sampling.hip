@@ -11,6 +11,10 @@
 //   6. top-p in (0, 1): keep the most likely tokens whose mass first reaches
 //      top_p of the total;
 //   7. draw: u * (kept mass), walked along the cumulative sum.
+// With top-k (or top-p alone on a peaked row) the row is read three times: the maximum, a histogram of the values
+// that locates the k-th largest, and the collection of what lies at or above its bin; the rest happens on that
+// short list in LDS.  Rows that do not fit (many equal values, a flat row under top-p alone) take passes over the
+// whole vocabulary for every bit of a threshold, with the same result.
 // Differences, both of measure zero or none in distribution: the kept sets are
 // found as thresholds (tokens equal to the threshold are all kept), and the
 // cumulative walk runs in vocabulary order rather than sorted order.  The
@@ -48,6 +52,18 @@ struct RowView {
 
 __device__ float block_sum_f(float v, float* scratch) { return block_sum(v, scratch); }
 
+__device__ float block_max_f(float v, float* scratch) {
+    const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, PULSE_WAVE));
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float m = scratch[0];
+    for (int w = 1; w < SAMPLE_WAVES; ++w) m = fmaxf(m, scratch[w]);
+    return m;
+}
+
 __device__ int block_sum_i(int v, int* scratch) {
     const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
 #pragma unroll
@@ -77,6 +93,40 @@ __device__ void block_argmax(float& v, int& idx, float* sv, int* si) {
         if (sv[w] > v || (sv[w] == v && si[w] < idx)) { v = sv[w]; idx = si[w]; }
 }
 
+// ---- the walk along the cumulative sum, a wavefront over 64 consecutive entries at a time ---------------------
+// `weight(i)` is the weight of entry i of [begin, end) (0 for what is not kept), entries in vocabulary order.  The
+// wavefront finds the first entry at which the running sum exceeds `rest` and returns its number, or -1 if the sum
+// never gets there (rounding); `last` is the last entry with a weight.  Every lane returns the same.
+template <typename Weight>
+__device__ int wave_walk(int begin, int end, float rest, Weight weight, int& last) {
+    const int lane = threadIdx.x % PULSE_WAVE;
+    float run = 0.f;
+    last = -1;
+    for (int base = begin; base < end; base += PULSE_WAVE) {
+        const int i = base + lane;
+        const float w = i < end ? weight(i) : 0.f;
+        const unsigned long long has = __ballot(w > 0.f);
+        if (has == 0ull) continue;
+        last = base + (63 - __builtin_clzll(has));
+        // inclusive prefix over the lanes, in lane order
+        float pre = w;
+#pragma unroll
+        for (int off = 1; off < PULSE_WAVE; off <<= 1) {
+            const float up = __shfl_up(pre, off, PULSE_WAVE);
+            if (lane >= off) pre += up;
+        }
+        const unsigned long long hit = __ballot(w > 0.f && rest < run + pre);
+        if (hit != 0ull) return base + __builtin_ctzll(hit);
+        run += __shfl(pre, PULSE_WAVE - 1, PULSE_WAVE);
+    }
+    return -1;
+}
+
+constexpr int HIST_BINS = 2048;                         // bins of the value histogram that locates the k-th largest
+constexpr int WAVE_CAP = 128;                           // candidates a wavefront may collect
+constexpr int LIST_CAP = SAMPLE_WAVES * WAVE_CAP;       // candidates of a row
+constexpr int LIST_PER_LANE = LIST_CAP / PULSE_WAVE;
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ uniform,
@@ -84,11 +134,18 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const uint32_t* __restrict__ banned, int mask_words, int* __restrict__ out) {
     __shared__ float sf[SAMPLE_WAVES];
     __shared__ int si[SAMPLE_WAVES];
-    __shared__ float chunk_sum[SAMPLE_THREADS];
-    __shared__ int chosen_thread;
-    __shared__ float chosen_rest;
+    __shared__ int hist[HIST_BINS];
+    __shared__ int wave_bins[SAMPLE_WAVES];
+    __shared__ int region_i[SAMPLE_WAVES][WAVE_CAP];
+    __shared__ float region_x[SAMPLE_WAVES][WAVE_CAP];
+    __shared__ int region_n[SAMPLE_WAVES];
+    __shared__ int list_i[LIST_CAP];
+    __shared__ float list_x[LIST_CAP];
+    __shared__ float part_sum[SAMPLE_WAVES];
+    __shared__ int list_done;
 
     const int r = blockIdx.x;
+    const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
     RowView row;
     row.logits = logits + r * row_stride;
     row.vocab = vocab;
@@ -97,12 +154,13 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     row.seen = (seen_masks && seen_row && seen_row[r] >= 0 && row.penalty > 0.f)
                    ? seen_masks + static_cast<int64_t>(seen_row[r]) * mask_words : nullptr;
 
-    // largest logit, lowest index among equals
-    float best = -INFINITY;
+    // largest logit, lowest index among equals; the smallest number too (the histogram's range)
+    float best = -INFINITY, lowest = INFINITY;
     int best_i = 0x7fffffff;
     for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
         const float x = row.at(i);
         if (x > best) { best = x; best_i = i; }
+        if (x != -INFINITY) lowest = fminf(lowest, x);
     }
     block_argmax(best, best_i, sf, si);
     if (best_i == 0x7fffffff) {  // everything banned or NaN
@@ -114,10 +172,167 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         if (threadIdx.x == 0) out[r] = best_i;
         return;
     }
+    const float inv_t = 1.0f / temp;
+    const int k = top_k ? top_k[r] : 0;
+    const float p = top_p ? top_p[r] : 0.f;
+    const bool use_p = p > 0.f && p < 1.f;
+    // each wavefront owns a contiguous part of the vocabulary, walked 64 entries at a time
+    const int part = ((vocab + SAMPLE_WAVES - 1) / SAMPLE_WAVES + PULSE_WAVE - 1) / PULSE_WAVE * PULSE_WAVE;
+    const int part_begin = min(vocab, wave * part), part_end = min(vocab, wave * part + part);
 
+    // ---- with top-k: locate the k-th largest with a histogram over [lowest, best], collect what lies at or above
+    // its bin (in vocabulary order), and finish on that short list in LDS.  Falls through to the passes over the
+    // whole vocabulary when the list would not fit (many equal values) or the range is empty.
+    // Top-p alone takes the same way with the LIST_TRY largest values, if their mass reaches top_p of the whole.
+    constexpr int LIST_TRY = 1024;
+    const bool by_k = k > 0 && k < vocab;
+    const int k_list = by_k ? k : min(vocab - 1, LIST_TRY);
+    if (by_k || (use_p && k_list > 0)) {
+        float whole = 0.f;   // without top-k: the mass of the whole vocabulary, which top_p refers to
+        if (!by_k) {
+            float mass = 0.f;
+            for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
+                const float x = row.at(i);
+                if (x != -INFINITY) mass += expf((x - best) * inv_t);
+            }
+            whole = block_sum_f(mass, sf);
+        }
+        lowest = -block_max_f(-lowest, sf);
+        const float scale = static_cast<float>(HIST_BINS) / (best - lowest);
+        const bool ranged = best > lowest && scale < INFINITY;
+        auto bin_of = [&](float x) { return min(HIST_BINS - 1, static_cast<int>((best - x) * scale)); };  // 0: the largest values
+        int edge = -1, listed = 0;
+        if (ranged) {
+            for (int b = threadIdx.x; b < HIST_BINS; b += SAMPLE_THREADS) hist[b] = 0;
+            __syncthreads();
+            for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
+                const float x = row.at(i);
+                if (x != -INFINITY) atomicAdd(&hist[bin_of(x)], 1);
+            }
+            __syncthreads();
+            // the bin in which the count from the top reaches k: first by wavefronts' shares of the bins, then by bins
+            constexpr int SHARE = HIST_BINS / SAMPLE_WAVES;
+            int mine = 0;
+            for (int b = wave * SHARE + lane; b < (wave + 1) * SHARE; b += PULSE_WAVE) mine += hist[b];
+#pragma unroll
+            for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) mine += __shfl_xor(mine, off, PULSE_WAVE);
+            if (lane == 0) wave_bins[wave] = mine;
+            __syncthreads();
+            int w = 0;
+            while (w < SAMPLE_WAVES && listed + wave_bins[w] < k_list) listed += wave_bins[w++];
+            if (w < SAMPLE_WAVES) {
+                int b = w * SHARE;
+                while (listed + hist[b] < k_list) listed += hist[b++];
+                listed += hist[b];
+                edge = b;
+            }
+        }
+        if (edge >= 0 && listed <= LIST_CAP) {
+            int count = 0;
+            for (int base = part_begin; base < part_end; base += PULSE_WAVE) {
+                const int i = base + lane;
+                const float x = i < part_end ? row.at(i) : -INFINITY;
+                const bool in = x != -INFINITY && bin_of(x) <= edge;
+                const unsigned long long mask = __ballot(in);
+                const int at = count + __builtin_popcountll(mask & ((1ull << lane) - 1ull));
+                if (in && at < WAVE_CAP) { region_i[wave][at] = i; region_x[wave][at] = x; }
+                count += __builtin_popcountll(mask);
+            }
+            if (lane == 0) region_n[wave] = count;
+            __syncthreads();
+            bool fits = true;
+            for (int w = 0; w < SAMPLE_WAVES; ++w) fits = fits && region_n[w] <= WAVE_CAP;
+            if (fits) {
+                // one list, in vocabulary order
+                int n = 0;
+                for (int w = 0; w < SAMPLE_WAVES; ++w) {
+                    for (int e = threadIdx.x; e < region_n[w]; e += SAMPLE_THREADS) {
+                        list_i[n + e] = region_i[w][e];
+                        list_x[n + e] = region_x[w][e];
+                    }
+                    n += region_n[w];
+                }
+                __syncthreads();
+                // the first wavefront finishes alone (lane l holds entries l, l + 64, ..); the others wait for its word
+                if (wave == 0) {
+                auto lane_sum_i = [&](int v) {
+#pragma unroll
+                    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, PULSE_WAVE);
+                    return v;
+                };
+                auto lane_sum_f = [&](float v) {
+#pragma unroll
+                    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, PULSE_WAVE);
+                    return v;
+                };
+                uint32_t keys[LIST_PER_LANE];
+                float wts[LIST_PER_LANE];
+#pragma unroll
+                for (int j = 0; j < LIST_PER_LANE; ++j) {
+                    const int e = lane + j * PULSE_WAVE;
+                    keys[j] = e < n ? order_key(list_x[e]) : 0u;
+                    wts[j] = e < n ? expf((list_x[e] - best) * inv_t) : 0.f;
+                }
+                // the k-th largest key, bit by bit
+                uint32_t keep = 0u;
+                if (by_k) {
+                    for (int bit = 31; bit >= 0; --bit) {
+                        const uint32_t cand = keep | (1u << bit);
+                        int c = 0;
+#pragma unroll
+                        for (int j = 0; j < LIST_PER_LANE; ++j) c += (lane + j * PULSE_WAVE < n && keys[j] >= cand) ? 1 : 0;
+                        if (lane_sum_i(c) >= k) keep = cand;
+                    }
+                }
+                bool enough = true;
+                if (use_p) {
+                    float mass = 0.f;
+#pragma unroll
+                    for (int j = 0; j < LIST_PER_LANE; ++j) mass += keys[j] >= keep ? wts[j] : 0.f;
+                    mass = lane_sum_f(mass);
+                    const float want = p * (by_k ? mass : whole);
+                    enough = by_k || mass >= want;   // without top-k the list must hold all of the top_p set
+                    uint32_t thr = 0u;
+                    for (int bit = 31; bit >= 0; --bit) {
+                        const uint32_t cand = thr | (1u << bit);
+                        const uint32_t lim = cand > keep ? cand : keep;
+                        float part_mass = 0.f;
+#pragma unroll
+                        for (int j = 0; j < LIST_PER_LANE; ++j) part_mass += keys[j] >= lim ? wts[j] : 0.f;
+                        if (lane_sum_f(part_mass) >= want) thr = cand;
+                    }
+                    if (thr > keep) keep = thr;
+                }
+                if (!enough) {   // (only without top-k) the list is too short: the passes over the whole vocabulary
+                    if (lane == 0) list_done = 0;
+                } else {
+                // what is kept, as weights in the list's place of x, then the walk
+                float kept = 0.f;
+#pragma unroll
+                for (int j = 0; j < LIST_PER_LANE; ++j) {
+                    const int e = lane + j * PULSE_WAVE;
+                    const float w = (e < n && keys[j] >= keep) ? wts[j] : 0.f;
+                    if (e < n) list_x[e] = w;
+                    kept += w;
+                }
+                kept = lane_sum_f(kept);
+                int last;
+                const int e = wave_walk(0, n, uniform[r] * kept, [&](int q) { return list_x[q]; }, last);
+                if (lane == 0) {
+                    out[r] = e >= 0 ? list_i[e] : (last >= 0 ? list_i[last] : best_i);
+                    list_done = 1;
+                }
+                }
+                }
+                __syncthreads();
+                if (list_done) return;
+            }
+        }
+    }
+
+    // ---- passes over the whole vocabulary
     // top-k threshold: the k-th largest key, found bit by bit
     uint32_t keep = 0u;
-    const int k = top_k ? top_k[r] : 0;
     if (k > 0 && k < vocab) {
         for (int bit = 31; bit >= 0; --bit) {
             const uint32_t cand = keep | (1u << bit);
@@ -126,71 +341,54 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
             if (block_sum_i(count, si) >= k) keep = cand;
         }
     }
-    const float inv_t = 1.0f / temp;
-    // total mass of what top-k keeps
-    float mass = 0.f;
-    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
+    auto weight = [&](int i) {
         const float x = row.at(i);
-        if (x != -INFINITY && order_key(x) >= keep) mass += expf((x - best) * inv_t);
-    }
-    float total = block_sum_f(mass, sf);
-
-    const float p = top_p ? top_p[r] : 0.f;
-    if (p > 0.f && p < 1.f) {
-        const float want = p * total;
+        return (x != -INFINITY && order_key(x) >= keep) ? expf((x - best) * inv_t) : 0.f;
+    };
+    if (use_p) {
+        float mass = 0.f;
+        for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) mass += weight(i);
+        const float want = p * block_sum_f(mass, sf);
         uint32_t thr = 0u;
         for (int bit = 31; bit >= 0; --bit) {
             const uint32_t cand = thr | (1u << bit);
             const uint32_t lim = cand > keep ? cand : keep;
-            float part = 0.f;
+            float part_mass = 0.f;
             for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
                 const float x = row.at(i);
-                if (x != -INFINITY && order_key(x) >= lim) part += expf((x - best) * inv_t);
+                if (x != -INFINITY && order_key(x) >= lim) part_mass += expf((x - best) * inv_t);
             }
-            if (block_sum_f(part, sf) >= want) thr = cand;
+            if (block_sum_f(part_mass, sf) >= want) thr = cand;
         }
         if (thr > keep) keep = thr;
     }
-
-    // cumulative walk in vocabulary order over contiguous chunks
-    const int chunk = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
-    const int begin = threadIdx.x * chunk;
-    const int end = min(vocab, begin + chunk);
+    // the kept mass of every wavefront's part, then the part in which the draw falls is walked by its wavefront
     float mine = 0.f;
-    for (int i = begin; i < end; ++i) {
-        const float x = row.at(i);
-        if (x != -INFINITY && order_key(x) >= keep) mine += expf((x - best) * inv_t);
-    }
-    chunk_sum[threadIdx.x] = mine;
+    for (int i = part_begin + lane; i < part_end; i += PULSE_WAVE) mine += weight(i);
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) mine += __shfl_xor(mine, off, PULSE_WAVE);
+    if (lane == 0) part_sum[wave] = mine;
     __syncthreads();
-    if (threadIdx.x == 0) {
-        float kept = 0.f;
-        for (int i = 0; i < SAMPLE_THREADS; ++i) kept += chunk_sum[i];
-        const float target = uniform[r] * kept;
-        float run = 0.f;
-        int who = -1;
-        for (int i = 0; i < SAMPLE_THREADS; ++i) {
-            if (chunk_sum[i] > 0.f && target < run + chunk_sum[i]) { who = i; break; }
-            run += chunk_sum[i];
+    float kept = 0.f;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) kept += part_sum[w];
+    const float target = uniform[r] * kept;
+    float run = 0.f;
+    int who = -1, last_part = -1;
+    for (int w = 0; w < SAMPLE_WAVES; ++w) {
+        if (part_sum[w] > 0.f) {
+            last_part = w;
+            if (who < 0 && target < run + part_sum[w]) who = w;
         }
-        chosen_thread = who;
-        chosen_rest = target - run;
-        if (who < 0) out[r] = best_i;  // rounding left the target beyond the last chunk
+        if (who < 0) run += part_sum[w];
     }
-    __syncthreads();
-    if (static_cast<int>(threadIdx.x) == chosen_thread) {
-        float run = 0.f;
-        int pick = -1, last = -1;
-        for (int i = begin; i < end; ++i) {
-            const float x = row.at(i);
-            if (x != -INFINITY && order_key(x) >= keep) {
-                run += expf((x - best) * inv_t);
-                last = i;
-                if (chosen_rest < run) { pick = i; break; }
-            }
-        }
-        out[r] = pick >= 0 ? pick : (last >= 0 ? last : best_i);
+    if (who < 0) {  // rounding left the target beyond the last part: its last kept entry
+        who = last_part;
+        run = INFINITY;
     }
+    if (wave != who) return;
+    int last;
+    const int e = wave_walk(part_begin, part_end, run == INFINITY ? INFINITY : target - run, weight, last);
+    if (lane == 0) out[r] = e >= 0 ? e : (last >= 0 ? last : best_i);
 }
 
 __global__ void mark_seen_kernel(uint32_t* __restrict__ masks, int mask_words, const int* __restrict__ rows,

@@ -340,6 +340,66 @@ def test_top_k_top_p_penalty_and_banned(k):
     assert greedy[0].item() == second
 
 
+@pytest.mark.parametrize("mode", ["temperature", "top_k", "top_k_top_p", "top_p", "top_p_peaked", "ties", "penalty"])
+def test_sampling_at_a_real_vocabulary(k, mode):
+    """The draw of every row against the same steps in float64: kept set by thresholds (top-k, then top-p on what
+    top-k kept), cumulative walk in vocabulary order.  The chosen token must be kept and the draw must fall into its
+    interval of the cumulative sum (up to float32 rounding of the sums)."""
+    vocab, rows = 151936, 48
+    gen = torch.Generator().manual_seed(11)
+    # flat enough that top-p alone needs thousands of tokens (the passes over the whole vocabulary), or peaked so that
+    # a thousand hold its mass (the short list)
+    logits = torch.randn(rows, vocab, generator=gen) * (8.0 if mode == "top_p_peaked" else 2.5)
+    if mode == "ties":                       # the k-th largest value many times: all of its copies are kept
+        logits[:, ::97] = 6.0
+    temp = 0.7
+    top_k = {"top_k": 20, "top_k_top_p": 50, "ties": 40, "penalty": 20}.get(mode, 0)
+    top_p = {"top_k_top_p": 0.9, "top_p": 0.8, "top_p_peaked": 0.9, "penalty": 0.95}.get(mode, 0.0)
+    uniform = torch.rand(rows, generator=gen)
+    dev = lambda t: t.to(DEV)
+    kw = dict(temperature=dev(torch.full((rows,), temp)), uniform=dev(uniform))
+    if top_k:
+        kw["top_k"] = dev(torch.full((rows,), top_k, dtype=torch.int32))
+    if top_p:
+        kw["top_p"] = dev(torch.full((rows,), top_p))
+    ref = logits.to(F64).clone()
+    if mode == "penalty":
+        words = (vocab + 31) // 32
+        seen = torch.zeros(rows, words, dtype=torch.int32, device=DEV)
+        best = torch.argmax(logits, dim=1).to(torch.int32)
+        k.mark_seen(seen, torch.arange(rows, dtype=torch.int32, device=DEV), dev(best), vocab)
+        kw.update(penalty=dev(torch.full((rows,), 1.5)), seen_row=torch.arange(rows, dtype=torch.int32, device=DEV),
+                  seen_masks=seen)
+        ref[torch.arange(rows), best.long()] -= 1.5
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    k.sample(dev(logits), out, **kw)
+    got = out.cpu().tolist()
+    for r in range(rows):
+        x = ref[r]
+        kept = torch.ones(vocab, dtype=torch.bool)
+        if top_k:
+            kept &= x >= torch.topk(x, top_k).values[-1]
+        w = torch.where(kept, torch.exp((x - x.max()) / temp), torch.zeros_like(x))
+        if top_p:
+            order = torch.argsort(w, descending=True)
+            csum = torch.cumsum(w[order], 0)
+            cut = int((csum < top_p * w.sum()).sum())                # the first place where the mass reaches p
+            kept &= x >= x[order[cut]]
+            w = torch.where(kept, w, torch.zeros_like(w))
+        cum = torch.cumsum(w, 0)
+        target = float(uniform[r]) * float(cum[-1])
+        t = got[r]
+        slack = 2e-5 * float(cum[-1])
+        assert kept[t], (mode, r, t)
+        assert float(cum[t]) - float(w[t]) - slack <= target <= float(cum[t]) + slack, (mode, r, t)
+    again = torch.empty(1, dtype=torch.int32, device=DEV)            # a row's draw does not depend on the other rows
+    one = {n: v[5:6] for n, v in kw.items() if n not in ("seen_masks",)}
+    if "seen_masks" in kw:
+        one["seen_masks"] = kw["seen_masks"]
+    k.sample(dev(logits[5:6]), again, **one)
+    assert again.item() == got[5]
+
+
 def test_kernels_refuse_what_they_cannot_do(k):
     from pulse_infer_amd.ops import KernelError
     with pytest.raises(KernelError, match="GPU"):
