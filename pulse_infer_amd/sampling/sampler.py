@@ -9,6 +9,7 @@ from __future__ import annotations
 
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..ops import kernels
@@ -47,9 +48,8 @@ class Sampler:
     def note_tokens(self, slots: Sequence[int], tokens: Sequence[int]) -> None:
         if self.seen is None or not slots:
             return
-        rows = torch.tensor(list(slots), dtype=torch.int32, device=self.device)
-        toks = torch.tensor(list(tokens), dtype=torch.int32, device=self.device)
-        kernels.mark_seen(self.seen, rows, toks, self.vocab)
+        both = torch.tensor([list(slots), list(tokens)], dtype=torch.int32).to(self.device)   # one upload
+        kernels.mark_seen(self.seen, both[0], both[1], self.vocab)
 
     # ---------------------------------------------------------------- sampling
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], slots: Sequence[int],
@@ -66,17 +66,22 @@ class Sampler:
                 self._part_idx = torch.empty(need, dtype=torch.int32, device=self.device)
             kernels.argmax(logits, out, self._part_val, self._part_idx)
             return out.tolist()
-        temperature = torch.tensor([p.temperature for p in params], dtype=torch.float32, device=self.device)
-        top_k = torch.tensor([p.top_k for p in params], dtype=torch.int32, device=self.device)
-        top_p = torch.tensor([p.top_p for p in params], dtype=torch.float32, device=self.device)
-        uniform = torch.tensor(
-            [uniform_for(p.seed if p.seed is not None else d, c) for p, c, d in zip(params, counters, default_seeds)],
-            dtype=torch.float32, device=self.device)
-        penalty = seen_row = None
-        if self.seen is not None and any(p.presence_penalty > 0.0 for p in params):
-            penalty = torch.tensor([p.presence_penalty for p in params], dtype=torch.float32, device=self.device)
-            seen_row = torch.tensor([s if p.presence_penalty > 0.0 else -1 for p, s in zip(params, slots)],
-                                    dtype=torch.int32, device=self.device)
+        # every per-row option in one upload: rows of a [6, R] int32 array, the float ones as their bit patterns
+        use_penalty = self.seen is not None and any(p.presence_penalty > 0.0 for p in params)
+        host = np.empty((6, rows), dtype=np.int32)
+        as_float = host.view(np.float32)
+        as_float[0] = [p.temperature for p in params]
+        host[1] = [p.top_k for p in params]
+        as_float[2] = [p.top_p for p in params]
+        as_float[3] = [uniform_for(p.seed if p.seed is not None else d, c)
+                       for p, c, d in zip(params, counters, default_seeds)]
+        as_float[4] = [p.presence_penalty for p in params]
+        host[5] = [s if p.presence_penalty > 0.0 else -1 for p, s in zip(params, slots)]
+        dev = torch.from_numpy(host).to(self.device)
+        temperature, top_p, uniform = (dev[i].view(torch.float32) for i in (0, 2, 3))
+        top_k = dev[1]
+        penalty = dev[4].view(torch.float32) if use_penalty else None
+        seen_row = dev[5] if use_penalty else None
         kernels.sample(logits, out, temperature=temperature, top_k=top_k, top_p=top_p, uniform=uniform,
                        penalty=penalty, seen_row=seen_row, seen_masks=self.seen if penalty is not None else None,
                        banned=self.banned)
