@@ -1,10 +1,11 @@
-// C[M, N] = X[M, K] * W[N, K]^T in bfloat16 on the matrix cores for 9 to 64 rows: the regime of decoding with
-// many requests, where the product still only has to stream the weight from HBM once, but X is too large to be
-// fetched again by every wavefront.
+// C[M, N] = X[M, K] * W[N, K]^T in bfloat16 on the matrix cores for 17 to 192 rows: the regime of decoding with
+// many requests and of short prompt portions, where the product still only has to stream the weight from HBM once,
+// but X is too large to be fetched again by every wavefront.
 //
 // A workgroup of four wavefronts owns 64 weight rows (16 a wavefront) and a share of K (grid.y splits K when the
-// weight has too few rows to fill the chip otherwise).  The wavefronts walk K together in chunks of 128: the
-// chunk of X (up to 64 rows) goes through LDS once for all four, two stages, one barrier a chunk; each wavefront
+// weight has too few rows to fill the chip otherwise).  The wavefronts walk K together in chunks of 128 (64 from
+// 65 rows on, so that two stages of X fit LDS): the chunk of X goes through LDS once for all four, two stages, one
+// barrier a chunk; each wavefront
 // streams its 16 weight rows straight into registers, whole 128-byte lines per 16 lanes, and brings them into the
 // matrix-core layout with DPP and ds_bpermute as the few-rows kernel does.  The weight slab is the row operand and
 // X^T the column operand of v_mfma_f32_16x16x32_bf16, so lane l holds output features 4*(l/16)+i of row l%16.
@@ -17,6 +18,7 @@
 #include <math.h>
 
 #include <type_traits>
+#include <utility>
 
 namespace {
 
@@ -25,8 +27,17 @@ typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
 
-constexpr int KC = 128;        // k of a chunk: four steps of the matrix-core instruction
-constexpr int XROW = KC + 8;   // bfloat16 a row of X takes in LDS: 16 bytes of padding spread the rows over the banks
+constexpr int KC_MIN = 128;    // what a share of K must be a multiple of
+
+template <class F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+// f(integral_constant<int, 0>), .., f(integral_constant<int, N - 1>)
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
 
 enum MidMode : int { MID_BF16 = 0, MID_PARTS = 1 };
 
@@ -37,18 +48,25 @@ __device__ __forceinline__ bf16x8 zeros8() {
     return z;
 }
 
-// NW wavefronts of 16 weight rows each a workgroup; MT tiles of 16 rows of X.
-template <int NW, int MT, bool SWIGLU>
+// NW wavefronts of 16 weight rows each a workgroup; MT tiles of 16 rows of X; KC k a chunk (steps of 32).
+template <int NW, int MT, int KC, bool SWIGLU>
 __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* __restrict__ X, int64_t ldx,
                                                                     const bf16_t* __restrict__ W, int64_t ldw,
                                                                     void* __restrict__ C, int64_t ldc, int M, int N,
                                                                     int k_len, int mode) {
+    constexpr int XROW = KC + 8;   // bfloat16 a row of X takes in LDS: 16 bytes of padding spread the rows over the banks
     __shared__ __attribute__((aligned(16))) bf16_t s_x[2][16 * MT * XROW];
-    __shared__ f32x4 s_up[SWIGLU ? NW / 2 : 1][MT][PULSE_WAVE];
     static_assert(!SWIGLU || NW % 2 == 0, "gate and up slabs come in pairs");
+    static_assert(KC == 64 || KC == 128, "a chunk is one or two pairs of steps");
+    static_assert(sizeof(f32x4) * (NW / 2) * MT * PULSE_WAVE <= sizeof(bf16_t) * 2 * 16 * MT * XROW,
+                  "the up slabs' results take the place of the stages of X at the end");
     constexpr int NT = 16 * NW;                                  // weight rows of a workgroup
     constexpr int THREADS = NW * PULSE_WAVE;
-    constexpr int XP = (256 * MT + THREADS - 1) / THREADS;       // 16-byte pieces of a chunk of X a thread stages
+    constexpr int ROWP = KC / 8;                                 // 16-byte pieces of a row of a chunk of X
+    constexpr int PIECES = 16 * MT * ROWP;
+    constexpr int XP = (PIECES + THREADS - 1) / THREADS;         // pieces a thread stages
+    constexpr int PAIRS = KC / 64;                               // pairs of steps a chunk
+    constexpr int RING = 512 / KC;                               // register sets of weight chunks: loads run RING - 1 ahead
 
     const int tid = threadIdx.x;
     const int wave = tid / PULSE_WAVE;
@@ -69,16 +87,16 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
     // the operand's lane (kg, r) takes it from there
     const int source_lane = 16 * ((r >> 1) & 3) + 8 * (r & 1) + 4 * (r >> 3) + kg;
 
-    // X pieces (16 bytes) of a chunk that this thread stages: piece p = tid + THREADS i is row p / 16, columns
-    // 8 (p % 16)..; xdst < 0: no such piece
+    // X pieces (16 bytes) of a chunk that this thread stages: piece p = tid + THREADS i is row p / ROWP, columns
+    // 8 (p % ROWP)..; xdst < 0: no such piece
     const bf16_t* xsrc[XP];
     int xdst[XP];
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
         const int p = tid + THREADS * i;
-        const int xr = p / 16, xc = p % 16;
-        xsrc[i] = (xr < M && p < 256 * MT) ? X + static_cast<int64_t>(xr) * ldx + k0 + xc * 8 : nullptr;
-        xdst[i] = p < 256 * MT ? xr * XROW + xc * 8 : -1;
+        const int xr = p / ROWP, xc = p % ROWP;
+        xsrc[i] = (xr < M && p < PIECES) ? X + static_cast<int64_t>(xr) * ldx + k0 + xc * 8 : nullptr;
+        xdst[i] = p < PIECES ? xr * XROW + xc * 8 : -1;
     }
 
     f32x4 acc[MT];
@@ -87,18 +105,17 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
 
     // Loads run ahead of their use by more than a trip to memory: the weight RING - 1 chunks (a ring of register
     // sets), X two chunks (two sets; X comes from L2 for every workgroup but the first).
-    constexpr int RING = 4;
     bf16x8 xg[2][XP];
-    bf16x8 wr[RING][4];
+    bf16x8 wr[RING][2 * PAIRS];
     auto load_x = [&](int c, bf16x8 (&x)[XP]) {
 #pragma unroll
         for (int i = 0; i < XP; ++i)
             x[i] = (xsrc[i] && c < chunks) ? *reinterpret_cast<const bf16x8*>(xsrc[i] + static_cast<int64_t>(c) * KC) : zeros8();
     };
-    auto load_w = [&](int c, bf16x8 (&w)[4]) {
+    auto load_w = [&](int c, bf16x8 (&w)[2 * PAIRS]) {
         if (c >= chunks) return;
 #pragma unroll
-        for (int pair = 0; pair < 2; ++pair) {
+        for (int pair = 0; pair < PAIRS; ++pair) {
             w[2 * pair] = *reinterpret_cast<const bf16x8*>(w0 + static_cast<int64_t>(c) * KC + pair * 64);
             w[2 * pair + 1] = *reinterpret_cast<const bf16x8*>(w1 + static_cast<int64_t>(c) * KC + pair * 64);
         }
@@ -117,7 +134,7 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
         load_x(c + 2, xg[j % 2]);
         load_w(c + RING - 1, wr[(j + RING - 1) % RING]);
 #pragma unroll
-        for (int pair = 0; pair < 2; ++pair) {
+        for (int pair = 0; pair < PAIRS; ++pair) {
             const i32x4 l0 = __builtin_bit_cast(i32x4, wr[j][2 * pair]);
             const i32x4 l1 = __builtin_bit_cast(i32x4, wr[j][2 * pair + 1]);
             i32x4 a0, a1;
@@ -143,18 +160,14 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
         }
     };
 
-    static_assert(RING == 4, "the loop below names the four sets");
     load_x(0, xg[0]);
     load_w(0, wr[0]);
     load_x(1, xg[1]);
-    load_w(1, wr[1]);
-    load_w(2, wr[2]);
-    for (int c = 0; c < chunks; c += RING) {
-        body(std::integral_constant<int, 0>{}, c);
-        if (c + 1 < chunks) body(std::integral_constant<int, 1>{}, c + 1);
-        if (c + 2 < chunks) body(std::integral_constant<int, 2>{}, c + 2);
-        if (c + 3 < chunks) body(std::integral_constant<int, 3>{}, c + 3);
-    }
+    static_for<RING - 2>([&](auto J) { load_w(decltype(J)::value + 1, wr[decltype(J)::value + 1]); });
+    for (int c = 0; c < chunks; c += RING)
+        static_for<RING>([&](auto J) {
+            if (c + decltype(J)::value < chunks) body(J, c + decltype(J)::value);
+        });
 
     // lane (kg, r) holds features n_base + 16 wave + 4 kg + i of row 16 mt + r
     if (!SWIGLU) {
@@ -181,7 +194,10 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
             }
         }
     } else {
-        // even wavefronts hold gate slabs, odd ones the up slabs beside them; the output has half as many columns
+        // even wavefronts hold gate slabs, odd ones the up slabs beside them; the output has half as many columns.
+        // The up slabs' results go through the memory of the stages of X, which everybody has left after a barrier.
+        f32x4 (*s_up)[MT][PULSE_WAVE] = reinterpret_cast<f32x4 (*)[MT][PULSE_WAVE]>(&s_x[0][0]);
+        __syncthreads();
         if (wave & 1) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) s_up[wave / 2][mt][lane] = acc[mt];
@@ -207,18 +223,18 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
     }
 }
 
-template <int NW, int MT>
+template <int NW, int MT, int KC = 128>
 void launch_mid(const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
                 int k_len, int splits, int mode, bool swiglu, hipStream_t stream) {
     const dim3 grid((N + 16 * NW - 1) / (16 * NW), splits);
     const dim3 block(NW * PULSE_WAVE);
     if constexpr (NW % 2 == 0) {
         if (swiglu) {
-            hipLaunchKernelGGL((gemm_mid_kernel<NW, MT, true>), grid, block, 0, stream, X, ldx, W, ldw, C, ldc, M, N, k_len, mode);
+            hipLaunchKernelGGL((gemm_mid_kernel<NW, MT, KC, true>), grid, block, 0, stream, X, ldx, W, ldw, C, ldc, M, N, k_len, mode);
             return;
         }
     }
-    hipLaunchKernelGGL((gemm_mid_kernel<NW, MT, false>), grid, block, 0, stream, X, ldx, W, ldw, C, ldc, M, N, k_len, mode);
+    hipLaunchKernelGGL((gemm_mid_kernel<NW, MT, KC, false>), grid, block, 0, stream, X, ldx, W, ldw, C, ldc, M, N, k_len, mode);
 }
 
 template <int NW>
@@ -230,22 +246,31 @@ void launch_rows(const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, voi
     else launch_mid<NW, 4>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
 }
 
+// 65 to 192 rows: four wavefronts, chunks of 64 k, rows rounded up to 32
+void launch_many_rows(const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
+                      int k_len, int splits, int mode, bool swiglu, hipStream_t stream) {
+    if (M <= 96) launch_mid<4, 6, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+    else if (M <= 128) launch_mid<4, 8, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+    else if (M <= 160) launch_mid<4, 10, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+    else launch_mid<4, 12, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+}
+
 }  // namespace
 
-// Whether pulse_gemm_mid takes a shape: 1..64 rows, K cut into `splits` shares that are multiples of 128.
+// Whether pulse_gemm_mid takes a shape: 1..192 rows, K cut into `splits` shares that are multiples of 128.
 extern "C" int pulse_gemm_mid_takes(int M, int N, int K, int splits) {
-    return M >= 1 && M <= 64 && N > 0 && K > 0 && splits >= 1 && splits <= 64 && K % splits == 0 && (K / splits) % KC == 0;
+    return M >= 1 && M <= 192 && N > 0 && K > 0 && splits >= 1 && splits <= 64 && K % splits == 0 && (K / splits) % KC_MIN == 0;
 }
 
 // mode 0: C is bfloat16 [M, N] (splits must be 1).  mode 1: C is float32 [splits, M, N] (row stride ldc), the partial
 // products of the shares of K, to be added up by the consumer in split order.  swiglu != 0 (mode 0, splits 1): W holds
 // gate and up rows interleaved in slabs of 16 (gate slab, up slab, ...), N counts both, C is bfloat16 [M, N / 2] =
 // silu(gate) * up.
-// waves: wavefronts (of 16 weight rows) a workgroup, 2, 3, 4 or 6; 0 lets the entry point choose.
+// waves: wavefronts (of 16 weight rows) a workgroup, 2, 3, 4 or 6 (4 only above 64 rows); 0 lets the entry point choose.
 extern "C" int pulse_gemm_mid(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
                               int K, int mode, int swiglu, int splits, int waves, hipStream_t stream) {
-    PULSE_REQUIRE(pulse_gemm_mid_takes(M, N, K, splits), "gemm_mid: M=%d (1..64) N=%d K=%d in %d shares (multiples of %d)",
-                  M, N, K, splits, KC);
+    PULSE_REQUIRE(pulse_gemm_mid_takes(M, N, K, splits), "gemm_mid: M=%d (1..192) N=%d K=%d in %d shares (multiples of %d)",
+                  M, N, K, splits, KC_MIN);
     PULSE_REQUIRE(X && W && C, "gemm_mid: null pointer");
     PULSE_REQUIRE(ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K, "gemm_mid: the row strides must be multiples of 8 and cover K");
     PULSE_REQUIRE((reinterpret_cast<uintptr_t>(X) % 16) == 0 && (reinterpret_cast<uintptr_t>(W) % 16) == 0 &&
@@ -264,7 +289,9 @@ extern "C" int pulse_gemm_mid(const void* X, int64_t ldx, const void* W, int64_t
     if (waves == 0) waves = 4;
     PULSE_REQUIRE(waves == 2 || waves == 3 || waves == 4 || waves == 6, "gemm_mid: 2, 3, 4 or 6 wavefronts a workgroup, got %d", waves);
     PULSE_REQUIRE(!swiglu || waves % 2 == 0, "gemm_mid: SwiGLU needs an even number of wavefronts");
-    if (waves == 2) launch_rows<2>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
+    PULSE_REQUIRE(M <= 64 || waves == 4, "gemm_mid: more than 64 rows take 4 wavefronts a workgroup, got %d", waves);
+    if (M > 64) launch_many_rows(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
+    else if (waves == 2) launch_rows<2>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
     else if (waves == 3) launch_rows<3>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
     else if (waves == 4) launch_rows<4>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
     else launch_rows<6>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);

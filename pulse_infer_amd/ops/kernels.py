@@ -241,14 +241,17 @@ def gemm_skinny(a: Optional[torch.Tensor], w: torch.Tensor, out: torch.Tensor, a
              _i32(tune), _ptr(None), _ptr(None), _i32(0), _ptr(None), _f32(0.0), _ptr(sumsq_out), _stream())
 
 
+MID_MAX_ROWS = 192
+
+
 def gemm_mid_takes(m: int, n: int, k: int, splits: int = 1) -> bool:
     """Whether ``gemm_mid`` takes a shape (as pulse_gemm_mid_takes)."""
-    return 1 <= m <= 64 and n > 0 and k > 0 and 1 <= splits <= 64 and k % splits == 0 and (k // splits) % 128 == 0
+    return 1 <= m <= MID_MAX_ROWS and n > 0 and k > 0 and 1 <= splits <= 64 and k % splits == 0 and (k // splits) % 128 == 0
 
 
 def gemm_mid(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False, splits: int = 1,
              waves: int = 0) -> None:
-    """a @ w^T for up to 64 rows of bfloat16 with X shared through LDS (the regime of 9 to 64 rows).
+    """a @ w^T for up to 192 rows of bfloat16 with X shared through LDS (the regime of 17 to 192 rows).
 
     ``out`` bfloat16 [M, N]: the product (``splits`` must be 1); with ``swiglu`` the weight holds gate and up rows in
     alternating slabs of 16 and out [M, N / 2] is silu(gate) * up.  ``out`` float32 [splits, M, N]: the partial

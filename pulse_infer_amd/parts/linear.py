@@ -93,20 +93,29 @@ class Linear:
             return None
         return self.forward(x, scratch)
 
-    MID_ROWS = (17, 64)          # where the product with X shared through LDS beats the library's (with SwiGLU inside)
-    SHARES_FROM_ROWS = 17        # from here on the inner dimension of a product that adds into the residual is shared
-                                 # out over workgroups (measured on the 8B shape: a decoding step gains 1% at 17 to 32
-                                 # rows, 4% at 48, 6% at 64)
+    MID_ROWS = (17, 64)          # where the product with X shared through LDS and SwiGLU inside beats the library's
+                                 # product followed by the SwiGLU kernel
+    SHARES_ROWS = (17, 192)      # where a product that adds into the residual has its inner dimension shared out over
+                                 # workgroups (measured on the 8B shape: a decoding step gains 1% at 17 to 32 rows, 4% at
+                                 # 48, 6% at 64; at 96 to 192 rows the library takes 22 to 33 us for o and 55 to 90 us
+                                 # for down, the shared-out product 16 to 22 and 33 to 47)
     MID_WORKGROUPS = 512         # workgroups wanted of it (64 weight rows times a share of the inner dimension each)
+
+    def operands_ok(self, x: torch.Tensor) -> bool:
+        """Contiguous, aligned bfloat16 rows of a length the kernels' 16-byte loads take."""
+        w = self.weight
+        return (x.dim() == 2 and x.shape[1] % 8 == 0 and x.stride(1) == 1 and w.stride(1) == 1
+                and (x.shape[0] <= 1 or x.stride(0) % 8 == 0) and (w.shape[0] <= 1 or w.stride(0) % 8 == 0)
+                and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
     def takes_mid(self, x: torch.Tensor) -> bool:
         return (self.library and x.dtype == torch.bfloat16 and self.MID_ROWS[0] <= x.shape[0] <= self.MID_ROWS[1]
-                and kernels.gemm_skinny_ok(x, self.weight))
+                and self.operands_ok(x))
 
     def shares_for(self, x: torch.Tensor) -> int:
         """Into how many shares the inner dimension is cut for an update in parts; 0: not this product."""
-        if not (self.library and x.dtype == torch.bfloat16 and self.SHARES_FROM_ROWS <= x.shape[0] <= self.MID_ROWS[1]
-                and kernels.gemm_skinny_ok(x, self.weight)) or self.out_features % 4:
+        if not (self.library and x.dtype == torch.bfloat16 and self.SHARES_ROWS[0] <= x.shape[0] <= self.SHARES_ROWS[1]
+                and self.operands_ok(x)) or self.out_features % 4:
             return 0
         tiles = (self.out_features + 63) // 64
         best = 0
