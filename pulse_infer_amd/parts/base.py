@@ -70,15 +70,25 @@ class Workspace:
     def __init__(self, device: torch.device):
         self.device = device
         self._flat: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self._views: Dict[Tuple[str, torch.dtype, int, int], torch.Tensor] = {}   # what buffer() handed out before
 
     def buffer(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
+        view = self._views.get((name, dtype, rows, cols))
+        if view is not None:
+            return view
         need = max(1, rows * cols)
         key = (name, dtype)
         flat = self._flat.get(key)
         if flat is None or flat.numel() < need:
             flat = torch.empty(need, dtype=dtype, device=self.device)
             self._flat[key] = flat
-        return flat[: rows * cols].view(rows, cols)
+            for old in [k for k in self._views if k[0] == name and k[1] == dtype]:   # views of the buffer it replaces
+                del self._views[old]
+        view = flat[: rows * cols].view(rows, cols)
+        if len(self._views) >= 4096:   # steps of ever new sizes: start over rather than grow without end
+            self._views.clear()
+        self._views[(name, dtype, rows, cols)] = view
+        return view
 
 
 @dataclass
