@@ -16,8 +16,10 @@ What the reference leaves out is decided here:
   preempted: its pages and slot are given back, it returns to the front of the
   waiting queue and is later computed again from its first token (prompt and
   generated tokens alike), which reproduces what it had.  A prefill portion is
-  shortened rather than preempting anyone.  A request that could never fit the
-  pool or the model's positions is refused at ``add_request``.
+  shortened rather than preempting anyone; only when every running request is
+  still in its prompt and none can get a page (they hold each other's) does the
+  newest give way too.  A request that could never fit the pool or the model's
+  positions is refused at ``add_request``.
   (The reference aborts the whole run when pages run out,
   src/runtime/block_manager.cpp:44-46, src/scheduler/continuous_batch_engine.cpp:98-101.)
 """
@@ -153,6 +155,20 @@ class ContinuousBatchScheduler:
 
     def schedule_next_batch(self) -> ScheduledBatch:
         batch = ScheduledBatch()
+        while True:
+            self._fill(batch)
+            if not batch.empty() or not (self.running or self.waiting):
+                return batch
+            if len(self.running) > 1:
+                # every running request waits for pages that the others hold (all of them still in their prompts):
+                # the newest gives way, as when a decoding request needs a page
+                self._preempt(self.running[-1], batch)
+                continue
+            raise SchedulerError("nothing can be scheduled although requests remain: the cache pool cannot hold "
+                                 "the first portion of the next request")
+
+    def _fill(self, batch: ScheduledBatch) -> None:
+        """One pass of the three phases, adding to ``batch``."""
         budget = self.max_num_batched_tokens
 
         # 1. running requests that decode: one token each, preempting the newest when pages run out
@@ -223,10 +239,6 @@ class ContinuousBatchScheduler:
                                                    count == request.num_pending_tokens))
             budget -= count
 
-        if batch.empty() and (self.running or self.waiting):
-            raise SchedulerError("nothing can be scheduled although requests remain: the cache pool cannot hold "
-                                 "the first portion of the next request")
-        return batch
 
     def update_after_step(self, finished_ids: Sequence[int]) -> None:
         """Take finished requests out of the running list and give their cache back

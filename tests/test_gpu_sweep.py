@@ -1,0 +1,102 @@
+"""A sweep over seeded random configurations of the architecture (head sizes in steps of 16, any grouping of heads,
+windows on some layers, widths that are multiples of 128 so that every product kernel has its turn, vocabularies that
+are no power of two, several page sizes): the engine whole, with the last 32 tokens one by one and in portions of
+17 to 150 tokens, against the plain implementation in 32-bit and in bfloat16; and continuous batching with small
+portions and a pool so tight that requests are preempted, in 32-bit against each request alone and against the plain
+implementation's greedy choice."""
+import random
+
+import pytest
+import torch
+
+from conftest import token_ids
+from plain.qwen3_plain import PlainQwen3
+from test_gpu_model import TOL, SPLIT_TOL, close, run_alone
+
+pytestmark = pytest.mark.gpu
+
+
+def random_config(rng, hidden_choices, max_positions=1024):
+    d = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
+    nkv = rng.choice([1, 2, 3, 4])
+    group = rng.choice([1, 2, 3, 4, 5, 7, 8])
+    window = rng.choice([None, None, 20, 70])
+    cfg = dict(architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=rng.choice([300, 1000, 2053]),
+               hidden_size=rng.choice(hidden_choices), intermediate_size=rng.choice([128, 160, 256, 1056]),
+               num_hidden_layers=rng.choice([1, 2, 3]), num_attention_heads=nkv * group, num_key_value_heads=nkv,
+               head_dim=d, max_position_embeddings=max_positions, rms_norm_eps=rng.choice([1e-6, 1e-5]),
+               rope_theta=rng.choice([1e4, 1e6]), tie_word_embeddings=rng.random() < 0.5, torch_dtype="bfloat16",
+               attention_bias=False, hidden_act="silu", use_sliding_window=window is not None)
+    if window is not None:
+        cfg.update(sliding_window=window, max_window_layers=rng.choice([0, 1]))
+    return cfg
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configurations_whole_tail_and_portions(tmp_path, seed):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.weights import write_model_folder
+
+    rng = random.Random(1000 + seed)
+    cfg = random_config(rng, [128, 256, 384, 1024])
+    page, length = rng.choice([16, 32, 64]), rng.choice([90, 200, 333])
+    folder = write_model_folder(Qwen3Config.from_dict(cfg), str(tmp_path / "m"), seed=seed)
+    ids = token_ids(cfg["vocab_size"], length, seed=seed)
+    want = PlainQwen3.from_folder(folder).logits(ids)
+    what = f"{cfg} page {page} length {length}"
+    for dtype in ("float32", "bfloat16"):
+        _, model = load_model(folder, mode=dtype)
+        runner = ModelRunner(model, page_size=page, num_pages=(length + page - 1) // page + 2, max_requests=2)
+        whole = run_alone(runner, ids, [length])
+        close(whole, want, dtype, f"whole: {what}")
+        tail = run_alone(runner, ids, [length - 32] + [1] * 32)
+        close(tail, want, dtype, f"tail: {what}")
+        close(tail, whole, dtype, f"tail against whole: {what}", SPLIT_TOL)
+        cuts, left, sizes = [], length, [40, 2, 17, 64, 3, 100, 5, 19, 150]
+        while left:
+            n = min(sizes[len(cuts) % len(sizes)], left)
+            if left - n == 1:
+                n += 1
+            cuts.append(n)
+            left -= n
+        portions = run_alone(runner, ids, cuts)
+        close(portions, want, dtype, f"portions {cuts}: {what}")
+        close(portions, whole, dtype, f"portions against whole: {what}", SPLIT_TOL)
+        del runner, model
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_configurations_continuous_batching_and_preemption(tmp_path, seed):
+    """In 32-bit the greedy choice does not depend on the batch: what a request generates beside others, in small
+    portions, and after being preempted and recomputed, is what it generates alone and what the plain
+    implementation generates."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from pulse_infer_amd import LLM
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.weights import write_model_folder
+
+    rng = random.Random(2000 + seed)
+    cfg = random_config(rng, [128, 256], max_positions=512)
+    page = rng.choice([16, 32])
+    folder = write_model_folder(Qwen3Config.from_dict(cfg), str(tmp_path / "m"), seed=50 + seed)
+    prompts = [token_ids(cfg["vocab_size"], rng.choice([1, 5, 18, 40, 77]), seed=seed * 10 + i)
+               for i in range(rng.choice([3, 5, 7]))]
+    new = rng.choice([8, 20])
+    make = lambda **kw: LLM.from_pretrained(folder, dtype="float32", page_size=page, **kw)
+    alone = [make(max_batch_size=1, chunk_size=256, num_pages=64).generate([p], max_new_tokens=new, ignore_eos=True)[0]
+             for p in prompts]
+    plain = PlainQwen3.from_folder(folder)
+    assert alone[:2] == [plain.greedy(p, new) for p in prompts[:2]]
+    roomy = make(max_batch_size=4, chunk_size=rng.choice([8, 16, 50]), num_pages=64,
+                 max_num_batched_tokens=rng.choice([24, 64]))
+    assert roomy.generate(prompts, max_new_tokens=new, ignore_eos=True) == alone
+    need = max((len(p) + new + page - 1) // page for p in prompts)
+    tight = make(max_batch_size=4, chunk_size=16, num_pages=need + 2)       # room for little more than one request
+    assert tight.generate(prompts, max_new_tokens=new, ignore_eos=True) == alone
+    tight.engine.runner.cache.check()

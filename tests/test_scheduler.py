@@ -165,3 +165,29 @@ def test_a_lone_request_that_outgrows_the_pool_is_an_error_not_a_hang():
     s.get_request(a).add_sampled_token(1, [])
     with pytest.raises(SchedulerError, match="too small"):
         s.schedule_next_batch()
+
+
+def test_prompts_that_hold_each_others_pages_do_not_stall():
+    """Three long prompts admitted together fill the pool while all of them are still in their prompts: none can get
+    another page.  The newest gives way (twice if need be) and every request finishes with what it generates alone."""
+    c = _cache(pages=8)            # 32 tokens
+    s = ContinuousBatchScheduler(4, 4, chunk_size=4, cache=c, max_positions=64)
+    ids = [s.add_request(list(range(20)), 2) for _ in range(3)]     # each needs 6 pages in the end
+    steps, preempted, done = 0, 0, set()
+    while s.has_work():
+        batch = s.schedule_next_batch()
+        assert not batch.empty()
+        preempted += len(batch.preempted)
+        finished = []
+        for p in batch.portions:
+            p.request.add_computed_tokens(len(p.tokens))
+            if p.samples and not p.request.add_sampled_token(5, []):
+                finished.append(p.request.request_id)
+        s.update_after_step(finished)
+        done.update(finished)
+        c.check()
+        steps += 1
+        assert steps < 200, "the scheduler goes round in circles"
+    assert done == set(ids) and preempted >= 1
+    assert all(s.get_request(i).generated_tokens == [5, 5] for i in ids)
+    assert c.free_pages() == [8]
