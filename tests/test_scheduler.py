@@ -191,3 +191,63 @@ def test_prompts_that_hold_each_others_pages_do_not_stall():
     assert done == set(ids) and preempted >= 1
     assert all(s.get_request(i).generated_tokens == [5, 5] for i in ids)
     assert c.free_pages() == [8]
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_workloads_always_finish(seed):
+    """Random pools (one group with all keys, sometimes a windowed one beside it), portions, budgets, batch limits and
+    requests that arrive while others run: every step schedules something, the cache stays consistent, every
+    request ends with exactly the tokens it was allowed, and nothing is left in the pool."""
+    import random
+    rng = random.Random(seed)
+    page = rng.choice([1, 4, 16])
+    specs = [PagedKVSpec(1, 8)] + ([PagedKVSpec(1, 8, window=rng.choice([3, 10, 40]))] if rng.random() < 0.4 else [])
+    longest = rng.choice([12, 40, 90])
+    pages = (longest + 8 + page - 1) // page + rng.choice([0, 1, 3, 20])
+    slots = rng.choice([1, 2, 4, 8])
+    c = CacheManager(specs, page_size=page, num_pages=pages, max_requests=slots)
+    budget = rng.choice([None, 5, 17, 64])
+    s = ContinuousBatchScheduler(rng.choice([1, 2, 4, 8]), rng.choice([1, 2, 8]), chunk_size=rng.choice([1, 3, 8, 32]),
+                                 max_num_batched_tokens=budget, cache=c, max_positions=256)
+    eos = [7]
+    todo = [(rng.randint(1, longest), rng.randint(0, 8)) for _ in range(rng.randint(1, 12))]
+    ids, allowed = [], {}
+
+    def add():
+        n, new = todo.pop()
+        rid = s.add_request([rng.randint(0, 6) for _ in range(n)], new,
+                            SamplingParams(ignore_eos=rng.random() < 0.5))
+        ids.append(rid)
+        allowed[rid] = new
+
+    for _ in range(min(len(todo), rng.randint(1, 4))):
+        add()
+    steps = 0
+    while s.has_work() or todo:
+        if todo and (not s.has_work() or rng.random() < 0.3):
+            add()
+        batch = s.schedule_next_batch()
+        assert not batch.empty()
+        if budget is not None:
+            assert batch.num_tokens() <= budget
+        finished = []
+        for p in batch.portions:
+            assert c.reserved(p.request.request_id) >= p.start + len(p.tokens)
+            p.request.add_computed_tokens(len(p.tokens))
+            c.advance(p.request.request_id, p.start + len(p.tokens))
+            if p.samples:
+                if not p.request.can_generate_more:
+                    p.request.finish("length")
+                    finished.append(p.request.request_id)
+                elif not p.request.add_sampled_token(rng.choice([1, 2, 7]), eos):
+                    finished.append(p.request.request_id)
+        s.update_after_step(finished)
+        c.check()
+        steps += 1
+        assert steps < 5000, "the scheduler goes round in circles"
+    for rid in ids:
+        r = s.get_request(rid)
+        assert r.is_finished and len(r.generated_tokens) <= allowed[rid]
+        if r.finish_reason == "length":
+            assert len(r.generated_tokens) == allowed[rid]
+    assert c.free_pages() == [pages] * len(specs) and c.slots.num_free == slots
