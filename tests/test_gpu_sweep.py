@@ -100,3 +100,47 @@ def test_random_configurations_continuous_batching_and_preemption(tmp_path, seed
     tight = make(max_batch_size=4, chunk_size=16, num_pages=need + 2)       # room for little more than one request
     assert tight.generate(prompts, max_new_tokens=new, ignore_eos=True) == alone
     tight.engine.runner.cache.check()
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_configurations_mixed_batches_with_page_reuse(tmp_path, seed):
+    """Up to four live requests, portions of some beside single tokens of others, in a pool of 256 tokens whose
+    pages are used again, for random configurations in both storage types."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.weights import write_model_folder
+    from test_gpu_model import mixed_trace
+
+    rng = random.Random(3000 + seed)
+    cfg = random_config(rng, [128, 256, 1024])
+    page = rng.choice([16, 32, 64])
+    folder = write_model_folder(Qwen3Config.from_dict(cfg), str(tmp_path / "m"), seed=70 + seed)
+    plain = PlainQwen3.from_folder(folder)
+    ids, steps = mixed_trace(cfg["vocab_size"], seed=20 + seed)
+    want = {k: plain.logits(v) for k, v in ids.items()}
+    for dtype in ("float32", "bfloat16"):
+        _, model = load_model(folder, mode=dtype)
+        runner = ModelRunner(model, page_size=page, num_pages=256 // page, max_requests=4)
+        got = {k: [] for k in ids}
+        for step in steps:
+            entries = []
+            for e in step["entries"]:
+                if not runner.cache.has_request(e["id"]):
+                    runner.add_request(e["id"])
+                runner.reserve(e["id"], runner.cache.computed(e["id"]) + len(e["tokens"]))
+                entries.append(StepEntry(e["id"], e["tokens"], e["want"]))
+            logits = runner.step(entries)
+            row = 0
+            for e in step["entries"]:
+                got[e["id"]].append(logits[row:row + len(e["want"])])
+                row += len(e["want"])
+            for k in step["end"]:
+                runner.free_request(k)
+            runner.cache.check()
+        for k, parts in got.items():
+            close(torch.cat(parts), want[k], dtype, f"mixed request {k}: {cfg} page {page}")
+        del runner, model
+    torch.cuda.empty_cache()
