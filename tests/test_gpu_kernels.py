@@ -495,6 +495,66 @@ def test_attn_mfma(k, case, split):
     _mfma_case(k, split=split, **case)
 
 
+@pytest.mark.parametrize("path", ["decode", "decode_raw", "portion"])
+def test_attn_mfma_one_far_key_in_a_long_context(k, path):
+    """A context of 20,000 keys (scattered pages, many splits) in which one key's score stands out: the output is that
+    key's value wherever it lies (the first block, a page's edge, a split's edge, the far end), and not when a window
+    excludes it.  Through the kernel for decoded tokens, the same from the raw projection output, and the kernel for
+    prompt portions (its last 40 tokens)."""
+    from pulse_infer_amd.ops import attention_mfma as M
+    nq, nkv, d, bs, n = 8, 2, 128, 16, 20000
+    dtype = torch.bfloat16
+    pages = torch.randperm(n // bs + 1, generator=torch.Generator().manual_seed(8)).tolist()
+    table = torch.tensor([pages], dtype=torch.int32, device=DEV)
+    group = nq // nkv
+    rows = 1 if path != "portion" else 40
+    positions = list(range(n - rows, n))
+    pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
+
+    class E:
+        def __init__(self, first_row, count):
+            self.first_row, self.count = first_row, count
+    per = M.tokens_per_item(group) if path != "portion" else M.portion_tokens(group, d)
+    items = torch.tensor(M.build_items([(0, E(0, rows))], per), dtype=torch.int32, device=DEV)
+    split_size, n_splits = M.choose_splits(1, nkv, group, n)
+    assert n_splits > 8
+    part_o = torch.empty(rows * nq * n_splits, d, device=DEV)
+    part_ml = torch.empty(rows * nq * n_splits, 2, device=DEV)
+    kc, vc = _cache(len(pages), nkv, bs, d, dtype)
+    ks, _ = as_stored(rnd(n, nkv, d, seed=50, scale=0.05), dtype)
+    vs, vref = as_stored(rnd(n, nkv, d, seed=51), dtype)
+    order = torch.tensor(pages, device=DEV)[torch.arange(n, device=DEV) // bs]          # page of every key
+    slots = torch.arange(n, device=DEV) % bs
+    kc[order, :, slots, :] = ks
+    vc[order, :, :, slots] = vs
+    spike = torch.zeros(nkv, d, dtype=dtype, device=DEV)
+    spike[:, 0] = 40.0
+    for target, window, seen in ((0, 0, True), (31, 0, True), (32, 0, True), (split_size - 1, 0, True),
+                                 (split_size, 0, True), (bs * 700 - 1, 0, True), (n - 3000, 3000 + rows, True),
+                                 (n - 3001 - rows, 3000, False), (n - rows - 1, 0, True)):
+        page, slot = pages[target // bs], target % bs
+        kept = kc[page, :, slot, :].clone()
+        kc[page, :, slot, :] = spike
+        qv = rnd(rows, (nq + 2 * nkv) * d, seed=52, scale=0.05)
+        qv[:, 0:nq * d:d] = 40.0                                   # channel 0 of every query head
+        qv[:, nq * d:] = 0                                          # (raw path) the tokens' own keys and values: nothing
+        q, qref = as_stored(qv, dtype)
+        out = torch.zeros(rows, nq * d, dtype=dtype, device=DEV)
+        if path == "portion":
+            M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos_t, table, items, 1.0, window)
+        elif path == "decode":
+            M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, table, items, 1.0, window, split_size, n_splits, n,
+                        part_o, part_ml)
+        else:
+            M.attn_decode(q, out, nq, nkv, d, kc, vc, pos_t, table, items, 1.0, window, split_size, n_splits, n,
+                          part_o, part_ml, None, None, 0.0, None, None, 0, 0, False)
+        got = out.cpu().to(F64).reshape(rows, nq, d)
+        heads = torch.arange(nq) // group
+        close = torch.allclose(got[-1], vref[target][heads], atol=2e-2)
+        assert close == seen, (path, target, window)
+        kc[page, :, slot, :] = kept
+
+
 def test_attn_mfma_refuses_other_sizes(k):
     from pulse_infer_amd.ops import KernelError
     from pulse_infer_amd.ops import attention_mfma as M
