@@ -110,6 +110,7 @@ class ModelRunner:
         self._staging = _Staging(self.device)
         self.use_graphs = bool(use_graphs) and model.options.get("decode_graph", True)
         self._graphs: dict = {}
+        self._graph_seen: dict = {}
         self.max_positions = model.spec.max_positions
         self.steps = 0
         self.tokens_run = 0
@@ -203,7 +204,7 @@ class ModelRunner:
         total = row
         want_rows = [m.first_row + int(w) for e, m in zip(entries, metas) for w in e.want]
         max_context = max(m.start + m.count for m in metas)
-        if self._graph_ok(entries, metas):
+        if self._graph_ok(entries, metas) and self._graph_ready(len(metas), max_context):
             logits = self._step_captured(entries, metas, want_rows, max_context)
         else:
             widths = [max(1, max(g.pages_for(m.start + m.count) for m in metas)) for g in cache.groups]
@@ -226,6 +227,7 @@ class ModelRunner:
     GRAPH_MAX_BATCH = 16        # up to here every product is this package's own kernel (no library call is recorded)
     GRAPH_CONTEXT_BUCKET = 1024
     GRAPH_LIMIT = 64            # recordings kept
+    GRAPH_AFTER_STEPS = 4       # a (batch, context bucket) is recorded when it comes for this many-th time
 
     def _graph_ok(self, entries: Sequence[StepEntry], metas: List[EntryMeta]) -> bool:
         if not self.use_graphs or self.model.mode != "bfloat16" or len(metas) > self.GRAPH_MAX_BATCH:
@@ -234,12 +236,23 @@ class ModelRunner:
             return False
         return all(m.count == 1 for m in metas) and all(list(e.want) == [0] for e in entries)
 
+    def _graph_key(self, batch: int, max_context: int):
+        bucket = (max_context + self.GRAPH_CONTEXT_BUCKET - 1) // self.GRAPH_CONTEXT_BUCKET * self.GRAPH_CONTEXT_BUCKET
+        return batch, min(bucket, max(self.max_positions, max_context))
+
+    def _graph_ready(self, batch: int, max_context: int) -> bool:
+        """A shape is recorded when it comes for the GRAPH_AFTER_STEPS-th time: recording costs about as much as a
+        dozen steps, which a shape that a draining batch passes through once or twice never pays back."""
+        key = self._graph_key(batch, max_context)
+        if key in self._graphs:
+            return True
+        seen = self._graph_seen.get(key, 0) + 1
+        self._graph_seen[key] = seen
+        return seen >= self.GRAPH_AFTER_STEPS
+
     def _step_captured(self, entries: Sequence[StepEntry], metas: List[EntryMeta], want_rows: List[int],
                        max_context: int) -> torch.Tensor:
-        batch = len(metas)
-        bucket = (max_context + self.GRAPH_CONTEXT_BUCKET - 1) // self.GRAPH_CONTEXT_BUCKET * self.GRAPH_CONTEXT_BUCKET
-        bucket = min(bucket, max(self.max_positions, max_context))
-        key = (batch, bucket)
+        key = self._graph_key(len(metas), max_context)
         rec = self._graphs.get(key)
         if rec is None:
             rec = self._capture(key, entries, metas, want_rows)

@@ -156,8 +156,9 @@ def test_command_line(gpu, model_folders, plain_models, capsys):
 
 
 def test_captured_decode_steps_replay_like_eager_ones(gpu, model_folders, plain_logits):
-    """Decode steps are recorded once per (batch, context bucket) and replayed.  Every replay is checked against
-    the eager step and the plain implementation, with eager prompt portions of other requests in between."""
+    """Decode steps are recorded once per (batch, context bucket), when the shape comes for the fourth time, and
+    replayed from then on.  Every replay is checked against the eager step and the plain implementation, with eager
+    prompt portions of other requests in between."""
     from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
     from pulse_infer_amd.models.factory import load_model
     from test_gpu_model import SPLIT_TOL, close
@@ -184,7 +185,7 @@ def test_captured_decode_steps_replay_like_eager_ones(gpu, model_folders, plain_
 
         feed([("a", 20), ("b", 31)])
         for _ in range(10):
-            feed([("a", 1), ("b", 1)])                   # recorded at the first, replayed nine times
+            feed([("a", 1), ("b", 1)])                   # three eager steps, recorded at the fourth, replayed six times
         feed([("c", 17)])                                 # eager work between replays
         for _ in range(8):
             feed([("a", 1), ("b", 1), ("c", 1)])         # another batch size: another recording
