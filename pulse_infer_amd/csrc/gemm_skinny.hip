@@ -260,6 +260,8 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_kernel(const bf16_
 // NORMED: X is not given; the float32 residual H is, with the row sums of squares that the product before left
 // (`sumsq`, `parts` of them a row) and the RMSNorm weight: x = bfloat16(h / sqrt(mean(h^2) + eps) * w) is formed here,
 // as the norm kernel forms it, and that kernel's launch is saved.
+constexpr int STAGGER_BLOCKS = 64;  // consecutive workgroups that start at the same group of k-steps
+
 struct NormInput {
     const float* h;        // [M, K] float32, row stride ldx
     const float* sumsq;    // [M, parts]
@@ -314,7 +316,15 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
     float rstd = 0.f;
     __shared__ float s_rstd[16];
 
-    for (int ks = step_begin; ks < step_begin + per; ks += UNROLL) {
+    // Workgroups do not all walk K from the same end: every 64 of them start one group of steps later than the 64
+    // before (and wrap around).  With everybody at the same offset of its rows at the same time the memory channels
+    // are loaded unevenly; staggered like this the gate+up product of the 8B shape streams 6% faster (a stagger that
+    // changes with every workgroup, or with every 8, is slower than none).  The order of a workgroup's sums depends on
+    // its place in the grid only, so results stay the same from run to run and for any rows beside.
+    const int groups = per / UNROLL;
+    const int rot = static_cast<int>((blockIdx.x / STAGGER_BLOCKS) % static_cast<unsigned>(groups));
+    for (int gi = 0; gi < groups; ++gi) {
+        const int ks = step_begin + (gi + rot >= groups ? gi + rot - groups : gi + rot) * UNROLL;
         bf16x8 xb[UNROLL], wa[UNROLL][SLABS];
         f32x4 hraw[NORMED ? UNROLL / PACK : 1][2];
         bf16x8 nraw[NORMED ? UNROLL / PACK : 1];
@@ -338,7 +348,7 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
                 }
             }
         }
-        if (NORMED && ks == step_begin) {
+        if (NORMED && gi == 0) {
             // 1 / sqrt(mean(h^2) + eps) of every row from the parts; a wavefront takes rows wave, wave + KW, ..  This
             // stands behind the first group's loads so that its own round trip to memory runs beside theirs.
             for (int m = wave; m < M; m += KW) {
