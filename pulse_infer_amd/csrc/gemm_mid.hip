@@ -28,6 +28,8 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
 
 constexpr int KC_MIN = 128;    // what a share of K must be a multiple of
+constexpr int STAGGER_ROWS = 960;    // consecutive weight rows whose owners start at the same chunk of K ..
+constexpr int STAGGER_CHUNKS = 4;    // .. this many chunks after the owners of the rows before
 
 template <class F, int... Is>
 __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
@@ -77,6 +79,12 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
     const int split = blockIdx.y;
     const int64_t k0 = static_cast<int64_t>(split) * k_len;
     const int chunks = k_len / KC;
+    // Workgroups do not all walk their share of K from the same end: the owners of every 960 weight rows start four
+    // chunks later than the owners of the 960 before (and wrap around), which loads the memory channels more evenly
+    // (gate+up of the 8B shape: 5 to 9% faster).  The order of the sums depends on the weight row and the share only,
+    // not on the workgroup's shape (960 is a multiple of the rows of every shape: 32, 48, 64, 96) or on X.
+    const int rot = static_cast<int>(((n_base / STAGGER_ROWS) * STAGGER_CHUNKS + blockIdx.y) % static_cast<unsigned>(chunks));
+    auto placed = [&](int c) { return c + rot >= chunks ? c + rot - chunks : c + rot; };  // where chunk c of the walk lies
 
     // Weight loads: 16 consecutive lanes fetch two whole 128-byte lines (rows 2kg + r/8 and that + 8, piece r%8);
     // rows beyond N repeat the last row: their products only reach outputs that are never stored.
@@ -110,14 +118,15 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
     auto load_x = [&](int c, bf16x8 (&x)[XP]) {
 #pragma unroll
         for (int i = 0; i < XP; ++i)
-            x[i] = (xsrc[i] && c < chunks) ? *reinterpret_cast<const bf16x8*>(xsrc[i] + static_cast<int64_t>(c) * KC) : zeros8();
+            x[i] = (xsrc[i] && c < chunks) ? *reinterpret_cast<const bf16x8*>(xsrc[i] + static_cast<int64_t>(placed(c)) * KC) : zeros8();
     };
     auto load_w = [&](int c, bf16x8 (&w)[2 * PAIRS]) {
         if (c >= chunks) return;
+        const int64_t at = static_cast<int64_t>(placed(c)) * KC;
 #pragma unroll
         for (int pair = 0; pair < PAIRS; ++pair) {
-            w[2 * pair] = *reinterpret_cast<const bf16x8*>(w0 + static_cast<int64_t>(c) * KC + pair * 64);
-            w[2 * pair + 1] = *reinterpret_cast<const bf16x8*>(w1 + static_cast<int64_t>(c) * KC + pair * 64);
+            w[2 * pair] = *reinterpret_cast<const bf16x8*>(w0 + at + pair * 64);
+            w[2 * pair + 1] = *reinterpret_cast<const bf16x8*>(w1 + at + pair * 64);
         }
     };
     // One chunk (J = its number modulo RING, which names its register sets): X into its stage, loads for later chunks
