@@ -54,6 +54,8 @@ def parse_args(argv: Optional[List[str]] = None) -> argparse.Namespace:
     p.add_argument("--max-batch", type=int, default=8, help="most requests in one step")
     p.add_argument("--max-tokens", type=int, default=None, help="most tokens in one step (the budget)")
     p.add_argument("--chunk", type=int, default=256, help="longest prompt portion in one step")
+    p.add_argument("--rope-pairing", choices=["interleaved", "half"], default=None,
+                   help="channels a rotation pairs: interleaved (2i, 2i+1), as the reference computes, or half (i, i + d/2)")
     p.add_argument("--stats", action="store_true")
     return p.parse_args(argv)
 
@@ -73,13 +75,17 @@ def main(argv: Optional[List[str]] = None) -> int:
     from .sampling.params import SamplingParams
 
     config = load_config(model_dir)
+    overrides = {"rope_pairing": args.rope_pairing} if args.rope_pairing else None
+    if overrides:
+        config.rope_pairing = args.rope_pairing
+        config.validate(model_dir)
     options = dict(max_batch_size=args.max_batch, chunk_size=args.chunk, page_size=args.page_size,
                    num_pages=args.num_pages, max_num_batched_tokens=args.max_tokens, seed=args.seed)
     if args.random_weights:
         init = args.init if args.init == "fan_in" else float(args.init)
         llm = LLM.from_config_random(config, weights_seed=args.seed, init=init, dtype=dtype, device=args.device, **options)
     else:
-        llm = LLM.from_pretrained(model_dir, dtype=dtype, device=args.device, **options)
+        llm = LLM.from_pretrained(model_dir, dtype=dtype, device=args.device, config_overrides=overrides, **options)
 
     prompts: List[List[int]] = [[int(t) for t in s.split(",") if t.strip()] for s in args.prompt_ids]
     if args.prompt_file:

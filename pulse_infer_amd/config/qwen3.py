@@ -42,6 +42,10 @@ class Qwen3Config:
     temperature: float = 0.0
     top_k: int = 0
     top_p: float = 0.0
+    # An option of the engine, not a key of config.json: which channels a rotation pairs.  "interleaved" is
+    # (2i, 2i+1), what the reference computes (src/ops/kernels/cuda/rope_kernel.cu:100-126); "half" is
+    # (i, i + d/2), for checkpoints whose q/k projections were trained under that convention.
+    rope_pairing: str = "interleaved"
     architecture: str = ARCHITECTURE
 
     # ------------------------------------------------------------------ reading
@@ -137,6 +141,8 @@ class Qwen3Config:
             raise ConfigError(f"rms_norm_eps({self.rms_norm_eps}) must not be negative in '{origin}'")
         if not self.rope_theta > 0.0:
             raise ConfigError(f"rope_theta({self.rope_theta}) must be positive in '{origin}'")
+        if self.rope_pairing not in ("interleaved", "half"):
+            raise ConfigError(f"rope_pairing '{self.rope_pairing}' is not one of 'interleaved', 'half' in '{origin}'")
         if self.torch_dtype not in ("bfloat16", "float32", "float16"):
             raise ConfigError(f"torch_dtype '{self.torch_dtype}' is not supported in '{origin}'")
         if self.use_sliding_window:
@@ -201,7 +207,7 @@ class Qwen3Config:
         norm = PartSpec("rmsnorm", {"size": self.hidden_size, "eps": self.rms_norm_eps})
         rope = PartSpec("rope", {
             "theta": self.rope_theta, "rotary_dim": self.head_dim, "head_dim": self.head_dim,
-            "pairing": "interleaved",
+            "pairing": self.rope_pairing,
         })
         layers = []
         for i in range(self.num_hidden_layers):

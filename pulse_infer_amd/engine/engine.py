@@ -146,8 +146,9 @@ class LLM:
             max_num_batched_tokens=max_num_batched_tokens, eos_token_ids=eos, seed=seed)
 
     @classmethod
-    def from_pretrained(cls, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0", **engine_options):
-        config, model = load_model(model_dir, mode=dtype, device=device)
+    def from_pretrained(cls, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0",
+                        config_overrides: Optional[Dict[str, Any]] = None, **engine_options):
+        config, model = load_model(model_dir, mode=dtype, device=device, config_overrides=config_overrides)
         return cls(model, config, **engine_options)
 
     @classmethod

@@ -18,8 +18,17 @@ def build_model(config: Any, source: Any, mode: str = "bfloat16", device: Any = 
 
 
 def load_model(model_dir: str, mode: str = "bfloat16", device: Any = "cuda:0", strict: bool = True,
-               options: Optional[Dict[str, Any]] = None):
-    """config.json chooses the class; every *.safetensors file of the folder supplies the weights."""
+               options: Optional[Dict[str, Any]] = None, config_overrides: Optional[Dict[str, Any]] = None):
+    """config.json chooses the class; every *.safetensors file of the folder supplies the weights.
+
+    ``config_overrides`` sets fields of the configuration that are options of the engine rather than keys of
+    config.json (such as ``rope_pairing``); the configuration is validated again afterwards."""
     config = load_config(model_dir)
+    if config_overrides:
+        for key, value in config_overrides.items():
+            if not hasattr(config, key):
+                raise ValueError(f"the configuration of '{config.architecture}' has no field '{key}'")
+            setattr(config, key, value)
+        config.validate(model_dir)
     return config, build_model(config, SafetensorsSource(model_dir), mode=mode, device=device, strict=strict,
                                options=options)

@@ -139,3 +139,19 @@ def test_registry(tmp_path):
         unregister_architecture("OtherForCausalLM")
     with pytest.raises(ConfigError, match="does not exist"):
         load_config(str(tmp_path / "nowhere"))
+
+
+def test_rope_pairing_is_an_option_of_the_engine():
+    from pulse_infer_amd.config import ConfigError, Qwen3Config
+    from conftest import TINY_A
+
+    cfg = Qwen3Config.from_dict(TINY_A)
+    assert cfg.rope_pairing == "interleaved"   # what the reference computes (rope_kernel.cu:100-126)
+    assert cfg.model_spec().positions["rope"].params["pairing"] == "interleaved"
+    cfg.rope_pairing = "half"
+    cfg.validate()
+    assert cfg.model_spec().positions["rope"].params["pairing"] == "half"
+    assert "rope_pairing" not in cfg.to_dict()
+    cfg.rope_pairing = "pairs"
+    with pytest.raises(ConfigError):
+        cfg.validate()

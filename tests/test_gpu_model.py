@@ -266,3 +266,28 @@ def test_trace_run_program(model_folders, plain_logits, tmp_path, dtype):
             row += len(e["want"])
     for k, parts in got.items():
         close(torch.cat(parts), plain_logits(name, ids[k]), dtype, f"trace_run request {k}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,page", [("A", 4), ("B", 16)])
+def test_half_pairing_option(model_folders, plain_models, name, page, dtype):
+    """``rope_pairing="half"`` (an option of the engine, no key of config.json) rotates (i, i + d/2): whole, then the
+    tail token by token (which in bfloat16 rotates inside the decode attention kernel), against the plain
+    implementation under the same pairing; and it is another function of the same weights than the default."""
+    from plain.qwen3_plain import PlainQwen3
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+
+    cfg = TINY[name][0]
+    ids = token_ids(cfg["vocab_size"], 90, seed=8)
+    plain = PlainQwen3.from_folder(model_folders[name], pairing="half")
+    want = plain.logits(ids)
+    config, model = load_model(model_folders[name], mode=dtype, config_overrides={"rope_pairing": "half"})
+    assert config.rope_pairing == "half"
+    runner = ModelRunner(model, page_size=page, num_pages=256 // page, max_requests=4)
+    close(run_alone(runner, ids, [len(ids)]), want, dtype, "whole, half pairing")
+    close(run_alone(runner, ids, [len(ids) - 32] + [1] * 32), want, dtype, "tail, half pairing")
+    other = plain_models[name].logits(ids)
+    assert float((other - want).abs().max()) > 0.05 * float(want.abs().max())
+    with pytest.raises(ValueError):
+        load_model(model_folders[name], mode=dtype, config_overrides={"no_such_field": 1})
