@@ -855,6 +855,15 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_p
     const int row0 = uniform(a.items[4 * item]);
     const int ntok = uniform(a.items[4 * item + 1]);         // at most NW * CT * per
     const int hi = uniform(a.positions[row0 + ntok - 1]);    // last key of the workgroup
+    // With splits (grid.z; split_size is a multiple of BK, so blocks never straddle two) a workgroup walks the
+    // keys of its split only.  An item all of whose keys lie in the first split is finished here as without
+    // splits; the others leave unnormalised partial results for attn_prefill_reduce_kernel.
+    const bool splits = a.n_splits > 1;
+    const int split = splits ? static_cast<int>(blockIdx.z) : 0;
+    const int split_begin = splits ? split * a.split_size : 0;
+    if (split_begin > hi) return;                            // no key of the item here; the merge does not read this split
+    const int split_last = splits ? min(hi, split_begin + a.split_size - 1) : hi;
+    const bool direct = !splits || hi < a.split_size;
     const int pos_first = uniform(a.positions[row0]);
     const int lo_item = (a.window > 0 && pos_first - a.window + 1 > 0) ? pos_first - a.window + 1 : 0;
     const int* bt = a.block_table + static_cast<int64_t>(uniform(a.items[4 * item + 2])) * a.bt_width;
@@ -1049,10 +1058,14 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_p
         }
     };
 
-    const int first_block = lo_item / BK;
-    const int last_block = hi / BK;
-    fetch(first_block, page_ahead(first_block), 0);
-    int page_next = page_ahead(first_block + 1);
+    const int first_block = max(lo_item, split_begin) / BK;
+    const int last_block = split_last / BK;
+    // (a split that lies below the item's window has no block to walk: nothing is fetched, its columns stay empty)
+    int page_next = 0;
+    if (first_block <= last_block) {
+        fetch(first_block, page_ahead(first_block), 0);
+        page_next = page_ahead(first_block + 1);
+    }
     for (int b = first_block; b <= last_block; ++b) {
         const int stage = (b - first_block) & 1;
         // This block's loads were issued a block ago; nothing else is in flight, so the wait does not depend on a
@@ -1073,7 +1086,7 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_p
         float l = l_part[ct];
         l += __shfl_xor(l, 16, PULSE_WAVE);
         l += __shfl_xor(l, 32, PULSE_WAVE);
-        if (col_ok[ct]) {
+        if (col_ok[ct] && direct) {
             const float inv = l > 0.f ? 1.0f / l : 0.f;
             bf16_t* dst = a.out + static_cast<int64_t>(col_row[ct]) * a.o_stride + static_cast<int64_t>(col_head) * D;
 #pragma unroll
@@ -1084,8 +1097,60 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_p
                                     (static_cast<uint32_t>(f32_to_bf16(acc[ct][dt][3] * inv)) << 16);
                 *reinterpret_cast<u32x2*>(dst + dt * 16 + 4 * kg) = u32x2{w0, w1};
             }
+        } else if (col_ok[ct]) {
+            // the split's share of the column: sums as they are, the maximum in the exponent's units
+            const int64_t slot = (static_cast<int64_t>(col_row[ct]) * a.nq + col_head) * a.n_splits + split;
+            float* dst = a.part_o + slot * D;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f32x4*>(dst + dt * 16 + 4 * kg) = acc[ct][dt];
+            if (kg == 0) {
+                a.part_ml[2 * slot] = m[ct] == -INFINITY ? -INFINITY : m[ct] * c2;
+                a.part_ml[2 * slot + 1] = l;
+            }
         }
     }
+}
+
+// The merge of the prompt-portion kernel's splits: out[row, head, :] = sum_z w_z o_z / sum_z w_z l_z with
+// w_z = exp2(m_z - max m) over the splits that begin at or below the row's position, in the order of the splits.
+// A thread takes four channels of one head; rows of items that were finished in the first split are left alone.
+constexpr int PR_THREADS = 256;
+constexpr int PR_QUADS = D / 4;
+constexpr int PR_HEADS = PR_THREADS / PR_QUADS;
+
+__global__ __launch_bounds__(PR_THREADS) void attn_prefill_reduce_kernel(const float* __restrict__ part_o,
+                                                                        const float* __restrict__ part_ml,
+                                                                        const int* __restrict__ positions,
+                                                                        const int* __restrict__ items, int item_tokens,
+                                                                        bf16_t* __restrict__ out, int64_t o_stride, int nq,
+                                                                        int n_splits, int split_size) {
+    const int item = blockIdx.x / item_tokens;
+    const int tok = blockIdx.x % item_tokens;
+    const int row0 = items[4 * item];
+    const int ntok = items[4 * item + 1];
+    if (tok >= ntok) return;
+    if (positions[row0 + ntok - 1] < split_size) return;   // the item was finished by its only split
+    const int64_t row = row0 + tok;
+    const int head = blockIdx.y * PR_HEADS + threadIdx.x / PR_QUADS;
+    const int quad = threadIdx.x % PR_QUADS;
+    if (head >= nq) return;
+    const int valid = min(n_splits, positions[row] / split_size + 1);
+    const int64_t base = (row * nq + head) * n_splits;
+    float mm = -INFINITY;
+    for (int z = 0; z < valid; ++z) mm = fmaxf(mm, part_ml[2 * (base + z)]);
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    float ll = 0.f;
+    for (int z = 0; z < valid; ++z) {
+        const float mz = part_ml[2 * (base + z)];
+        const float wz = mz == -INFINITY ? 0.f : exp2f(mz - mm);
+        ll += wz * part_ml[2 * (base + z) + 1];
+        // a split below the row's window holds sums of nothing (zeros), never stale memory: it was written
+        acc += *reinterpret_cast<const f32x4*>(part_o + (base + z) * D + 4 * quad) * wz;
+    }
+    const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+    const uint32_t w0 = static_cast<uint32_t>(f32_to_bf16(acc[0] * inv)) | (static_cast<uint32_t>(f32_to_bf16(acc[1] * inv)) << 16);
+    const uint32_t w1 = static_cast<uint32_t>(f32_to_bf16(acc[2] * inv)) | (static_cast<uint32_t>(f32_to_bf16(acc[3] * inv)) << 16);
+    *reinterpret_cast<u32x2*>(out + row * o_stride + static_cast<int64_t>(head) * D + 4 * quad) = u32x2{w0, w1};
 }
 
 #endif  // PULSE_WIDE
@@ -1288,13 +1353,26 @@ extern "C" int pulse_attn_decode(const void* qkv, int64_t qkv_stride, void* out,
                             max_context, part_o, part_ml, &prep, stream);
 }
 
-// Prompt portions: items of up to 4 * pulse_attn_mfma_tokens_per_item(group) tokens of one request, one workgroup each,
-// keys shared through LDS, no split.
+// Keys a split of the prompt-portion kernel must be a multiple of; 0 when this head size's kernel has no splits.
+extern "C" int pulse_attn_prefill_split_keys() { return PULSE_WIDE ? 64 : 0; }
+
+// Prompt portions: items of up to 4 * pulse_attn_prefill_tiles() * pulse_attn_mfma_tokens_per_item(group) tokens of one
+// request, a workgroup each (and per split), keys shared through LDS.  With n_splits > 1 (head sizes for which
+// pulse_attn_prefill_split_keys() > 0) the keys are cut into splits of split_size keys; part_o holds
+// tokens * nq * n_splits * D floats and part_ml tokens * nq * n_splits * 2, as for pulse_attn_mfma.
 extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, int64_t o_stride, const void* kcache,
                                   const void* vcache, const int* positions, const int* block_table, int bt_width,
                                   const int* items, int n_items, int tokens,
                                   int nq, int nkv, int page_size, int num_pages, float scale, int window,
-                                  hipStream_t stream) {
+                                  int split_size, int n_splits, float* part_o, float* part_ml, hipStream_t stream) {
+    PULSE_REQUIRE(n_splits >= 1 && n_splits < 65536, "attn_prefill: bad number of splits %d", n_splits);
+    if (n_splits > 1) {
+        PULSE_REQUIRE(pulse_attn_prefill_split_keys() > 0, "attn_prefill: head size %d has no split variant", D);
+        PULSE_REQUIRE(split_size > 0 && split_size % pulse_attn_prefill_split_keys() == 0,
+                      "attn_prefill: split size %d must be a positive multiple of %d", split_size, pulse_attn_prefill_split_keys());
+        PULSE_REQUIRE(part_o && part_ml && (reinterpret_cast<uintptr_t>(part_o) % 16) == 0,
+                      "attn_prefill: scratch for the split results is missing or not 16-byte aligned");
+    }
     PULSE_REQUIRE(tokens >= 0 && n_items >= 0 && nq > 0 && nkv > 0, "attn_prefill: bad sizes");
     PULSE_REQUIRE(nq % nkv == 0, "attn_prefill: %d query heads are not a multiple of %d kv heads", nq, nkv);
     PULSE_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_prefill: page size %d must be a multiple of 16", page_size);
@@ -1320,10 +1398,18 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
     a.page_size = page_size; a.num_pages = num_pages;
     a.page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
     a.scale_log2e = scale * 1.4426950408889634f;
-    a.window = window; a.split_size = 0; a.n_splits = 1;
+    a.window = window; a.split_size = n_splits > 1 ? split_size : 0; a.n_splits = n_splits;
+    a.part_o = n_splits > 1 ? part_o : nullptr; a.part_ml = n_splits > 1 ? part_ml : nullptr;
 #if PULSE_WIDE
-    hipLaunchKernelGGL((attn_prefill_wide_kernel<WIDE_CT, 4, WIDE_NW>), dim3(n_items, nkv * a.head_chunks),
+    hipLaunchKernelGGL((attn_prefill_wide_kernel<WIDE_CT, 4, WIDE_NW>), dim3(n_items, nkv * a.head_chunks, n_splits),
                        dim3(WIDE_NW * PULSE_WAVE), 0, stream, a, 16 / gp);
+    if (n_splits > 1) {
+        PULSE_LAUNCH_CHECK("attn_prefill");
+        const int item_tokens = WIDE_NW * WIDE_CT * (16 / gp);
+        hipLaunchKernelGGL(attn_prefill_reduce_kernel, dim3(n_items * item_tokens, (nq + PR_HEADS - 1) / PR_HEADS),
+                           dim3(PR_THREADS), 0, stream, part_o, part_ml, positions, items, item_tokens, a.out, o_stride, nq,
+                           n_splits, split_size);
+    }
 #else
     hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_items, nkv * a.head_chunks), dim3(WAVES * PULSE_WAVE), 0, stream, a,
                        16 / gp);

@@ -104,12 +104,72 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
             _i32(window), _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml), _stream())
 
 
+PREFILL_SPLIT_KEYS = 64        # a split of the prompt-portion kernel is a whole number of its 64-key blocks
+PREFILL_SPLIT_HEAD_DIMS = (32, 64, 128)
+PREFILL_MAX_SPLITS = 64
+PREFILL_SCRATCH_BYTES = 512 << 20
+
+
+def choose_prefill_splits(entries: Sequence, portion: int, nkv: int, group: int, d: int, window: int,
+                          target_groups: int = 512, min_blocks: int = 8) -> Tuple[int, int]:
+    """(split_size, n_splits) for the prompt-portion kernel over these (index, entry) pairs.
+
+    A workgroup walks its item's keys block by block, so the longest item sets the kernel's time while the chip
+    waits.  Two cases gain from cutting the keys into splits with workgroups of their own: fewer workgroups than the
+    chip runs at a time (``target_groups``; a short portion over a long context), which get as many splits as fill
+    it; and a full chip whose longest item walks much more than its share of all blocks (the late portions of a
+    whole prompt), which is cut at one and a half shares.  Splits never hold fewer than ``min_blocks`` blocks, and
+    nothing is cut otherwise: the partial results cost a trip through memory and a second launch."""
+    if d not in PREFILL_SPLIT_HEAD_DIMS or window > 0:   # (a window keeps every walk short)
+        return 0, 1
+    total = longest = tokens = items = 0
+    for _, e in entries:
+        tokens += e.count
+        for b in range(0, e.count, portion):
+            blocks = (e.start + min(b + portion, e.count) - 1) // PREFILL_SPLIT_KEYS + 1
+            total += blocks
+            longest = max(longest, blocks)
+            items += 1
+    if items == 0:
+        return 0, 1
+    per_item = nkv * ((group + 15) // 16)
+    groups = items * per_item
+    even = groups < target_groups
+    if even:
+        size = max(min_blocks, (longest * groups + target_groups - 1) // target_groups)
+    else:
+        share = (total * per_item + target_groups - 1) // target_groups
+        if longest * 4 < share * 7:
+            return 0, 1
+        size = max(min_blocks, (share * 3 + 1) // 2)
+    n_splits = (longest + size - 1) // size
+    budget = PREFILL_SCRATCH_BYTES // max(1, tokens * nkv * group * d * 4)
+    n_splits = min(n_splits, PREFILL_MAX_SPLITS, max(1, budget))
+    if n_splits <= 1:
+        return 0, 1
+    if even or n_splits * size < longest:
+        size = (longest + n_splits - 1) // n_splits   # splits of equal length
+    return size * PREFILL_SPLIT_KEYS, (longest + size - 1) // size
+
+
 def attn_prefill(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
                  vcache: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
-                 items: torch.Tensor, scale: float, window: int) -> None:
-    """Attention for prompt portions: items of up to portion_tokens(group, d) tokens, keys shared through LDS."""
-    _gpu("attn_prefill", q, out, kcache, vcache, positions, block_table, items)
+                 items: torch.Tensor, scale: float, window: int, split_size: int = 0, n_splits: int = 1,
+                 part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None) -> None:
+    """Attention for prompt portions: items of up to portion_tokens(group, d) tokens, keys shared through LDS.
+    With ``n_splits > 1`` the keys are walked in splits of ``split_size`` (a multiple of 64) by workgroups of their
+    own and merged by a second kernel; ``part_o`` / ``part_ml`` are float32 scratch of tokens * nq * n_splits * d
+    and * 2 elements."""
+    _gpu("attn_prefill", q, out, kcache, vcache, positions, block_table, items, part_o, part_ml)
     tokens = q.shape[0]
+    if n_splits > 1:
+        _need(d in PREFILL_SPLIT_HEAD_DIMS, f"attn_prefill: head size {d} has no split variant")
+        _need(split_size > 0 and split_size % PREFILL_SPLIT_KEYS == 0,
+              f"attn_prefill: split size {split_size} must be a positive multiple of {PREFILL_SPLIT_KEYS}")
+        need = tokens * nq * n_splits
+        _need(part_o is not None and part_ml is not None and part_o.dtype == torch.float32
+              and part_ml.dtype == torch.float32 and part_o.numel() >= need * d and part_ml.numel() >= need * 2,
+              "attn_prefill: scratch for the split results is too small")
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.stride(1) == 1 and out.stride(1) == 1,
           "attn_prefill: q and out must be bfloat16 matrices with contiguous rows")
     _need(q.shape[1] >= nq * d and out.shape[1] >= nq * d and out.shape[0] == tokens, "attn_prefill: q/out too narrow")
@@ -125,7 +185,8 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, 
     call_in(lib, "pulse_attn_prefill", _ptr(q), _i64(q.stride(0)), _ptr(out), _i64(out.stride(0)), _ptr(kcache),
             _ptr(vcache), _ptr(positions), _ptr(block_table), _i32(block_table.shape[1]),
             _ptr(items), _i32(items.numel() // ITEM_INTS), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages),
-            _f32(scale), _i32(window), _stream())
+            _f32(scale), _i32(window), _i32(split_size if n_splits > 1 else 0), _i32(n_splits),
+            _ptr(part_o if n_splits > 1 else None), _ptr(part_ml if n_splits > 1 else None), _stream())
 
 
 def decode_takes(d: int, rotary_dim: int, pairing: int) -> bool:

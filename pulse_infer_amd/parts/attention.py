@@ -144,8 +144,18 @@ class PagedAttention(Part):
                 max((e.start + e.count for _, e in short), default=0))
         short_items, long_items, short_context = ctx.extras[key]
         if long_items is not None:
+            skey = f"static:attention.portion_splits:{portion}:{window}"
+            if skey not in ctx.extras:
+                ctx.extras[skey] = attention_mfma.choose_prefill_splits(
+                    attention_mfma.split_entries(ctx.entries)[1], portion, self.nkv, group, self.d, window)
+            split_size, n_splits = ctx.extras[skey]
+            part_o = part_ml = None
+            if n_splits > 1:
+                rows = ctx.num_tokens * self.nq * n_splits
+                part_o = ctx.workspace.buffer("attention.portion_part_o", rows, self.d, torch.float32)
+                part_ml = ctx.workspace.buffer("attention.portion_part_ml", rows, 2, torch.float32)
             attention_mfma.attn_prefill(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
-                                        table, long_items, self.scale, window)
+                                        table, long_items, self.scale, window, split_size, n_splits, part_o, part_ml)
         if short_items is not None:
             # a recorded step passes its context bucket as max_context: its splits must cover that
             max_context = ctx.max_context if long_items is None else short_context

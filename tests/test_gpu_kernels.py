@@ -416,8 +416,9 @@ def test_kernels_refuse_what_they_cannot_do(k):
 
 
 # ------------------------------------------------------- matrix-core attention
-def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0):
-    """Requests with contexts `lens`; request 0 brings its last `portion` tokens, the others one token each."""
+def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0, portion_split=0):
+    """Requests with contexts `lens`; request 0 brings its last `portion` tokens, the others one token each.
+    ``portion_split``: request 0's portion goes through the prompt-portion kernel with its keys in splits of that size."""
     from pulse_infer_amd.ops import attention_mfma as M
     dtype = torch.bfloat16
     pages_per = [(n + bs - 1) // bs for n in lens]
@@ -450,7 +451,7 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0):
     q, qref = as_stored(rnd(len(positions), (nq + 2 * nkv) * d, seed=300 + seed), dtype)
     out = torch.zeros(len(positions), nq * d, dtype=dtype, device=DEV)
     max_ctx = max(lens)
-    if split is None or split == "portion":
+    if split is None or split == "portion" or portion_split:
         split_size, n_splits = M.choose_splits(items.numel() // M.ITEM_INTS, nkv, group, max_ctx)
     else:
         split_size, n_splits = split, (max_ctx + split - 1) // split
@@ -459,10 +460,17 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0):
     part_ml = torch.full((rows, 2), float("nan"), device=DEV)
     scale = d ** -0.5
     pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
-    if split == "portion":
+    if split == "portion" or portion_split:
         # request 0's portion through the kernel that shares keys through LDS, the single tokens through the other
         big = torch.tensor(M.build_items(numbered[:1], M.portion_tokens(group, d)), dtype=torch.int32, device=DEV)
-        M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), big, scale, window)
+        if portion_split:
+            n_big = (lens[0] + portion_split - 1) // portion_split
+            big_o = torch.full((len(positions) * nq * n_big, d), float("nan"), device=DEV)
+            big_ml = torch.full((len(positions) * nq * n_big, 2), float("nan"), device=DEV)
+            M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), big, scale, window, portion_split, n_big,
+                           big_o, big_ml)
+        else:
+            M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), big, scale, window)
         if len(entries) > 1:
             small = torch.tensor(M.build_items(numbered[1:], M.tokens_per_item(group)), dtype=torch.int32, device=DEV)
             M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), small, scale, window, split_size,
@@ -495,7 +503,22 @@ def test_attn_mfma(k, case, split):
     _mfma_case(k, split=split, **case)
 
 
-@pytest.mark.parametrize("path", ["decode", "decode_raw", "portion"])
+@pytest.mark.parametrize("case", [
+    dict(nq=32, nkv=8, d=128, bs=16, window=0, lens=[300, 513, 512, 31], portion=37),
+    dict(nq=32, nkv=8, d=128, bs=16, window=0, lens=[700, 20], portion=700),             # a whole prompt: early items finish in split 0
+    dict(nq=8, nkv=2, d=64, bs=32, window=40, lens=[333, 64], portion=150),              # splits that lie below the window
+    dict(nq=2, nkv=2, d=32, bs=16, window=0, lens=[390, 17], portion=129),
+    dict(nq=16, nkv=2, d=128, bs=64, window=0, lens=[257, 100], portion=257),
+    dict(nq=12, nkv=2, d=64, bs=16, window=100, lens=[450], portion=260),                # 6 heads a kv head, a window over several splits
+])
+@pytest.mark.parametrize("size", [64, 128, 192, 1024])
+def test_attn_prefill_with_its_keys_in_splits(k, case, size):
+    """The prompt-portion kernel with the keys cut into splits (a workgroup a split, a second kernel merges): splits of
+    one block, of several, and one that holds everything; the scratch starts as NaN, so nothing unwritten is read."""
+    _mfma_case(k, split=None, portion_split=size, **case)
+
+
+@pytest.mark.parametrize("path", ["decode", "decode_raw", "portion", "portion_splits"])
 def test_attn_mfma_one_far_key_in_a_long_context(k, path):
     """A context of 20,000 keys (scattered pages, many splits) in which one key's score stands out: the output is that
     key's value wherever it lies (the first block, a page's edge, a split's edge, the far end), and not when a window
@@ -507,14 +530,14 @@ def test_attn_mfma_one_far_key_in_a_long_context(k, path):
     pages = torch.randperm(n // bs + 1, generator=torch.Generator().manual_seed(8)).tolist()
     table = torch.tensor([pages], dtype=torch.int32, device=DEV)
     group = nq // nkv
-    rows = 1 if path != "portion" else 40
+    rows = 1 if not path.startswith("portion") else 40
     positions = list(range(n - rows, n))
     pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
 
     class E:
         def __init__(self, first_row, count):
             self.first_row, self.count = first_row, count
-    per = M.tokens_per_item(group) if path != "portion" else M.portion_tokens(group, d)
+    per = M.tokens_per_item(group) if not path.startswith("portion") else M.portion_tokens(group, d)
     items = torch.tensor(M.build_items([(0, E(0, rows))], per), dtype=torch.int32, device=DEV)
     split_size, n_splits = M.choose_splits(1, nkv, group, n)
     assert n_splits > 8
@@ -542,6 +565,10 @@ def test_attn_mfma_one_far_key_in_a_long_context(k, path):
         out = torch.zeros(rows, nq * d, dtype=dtype, device=DEV)
         if path == "portion":
             M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos_t, table, items, 1.0, window)
+        elif path == "portion_splits":
+            assert split_size % 64 == 0
+            M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos_t, table, items, 1.0, window, split_size, n_splits,
+                           part_o, part_ml)
         elif path == "decode":
             M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, table, items, 1.0, window, split_size, n_splits, n,
                         part_o, part_ml)

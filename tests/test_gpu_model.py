@@ -291,3 +291,41 @@ def test_half_pairing_option(model_folders, plain_models, name, page, dtype):
     assert float((other - want).abs().max()) > 0.05 * float(want.abs().max())
     with pytest.raises(ValueError):
         load_model(model_folders[name], mode=dtype, config_overrides={"no_such_field": 1})
+
+
+LONG = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=300, hidden_size=128, intermediate_size=160,
+    num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=64, max_position_embeddings=2048,
+    rms_norm_eps=1e-6, rope_theta=1e4, tie_word_embeddings=True, torch_dtype="bfloat16", attention_bias=False,
+    use_sliding_window=False, hidden_act="silu")
+
+
+def test_long_prompts_walk_their_keys_in_splits(tmp_path):
+    """A prompt of 1,300 tokens whole, and in portions that come late in a long context: few work items with long
+    walks, which the prompt-portion kernel cuts into splits (asserted), against the plain implementation."""
+    from plain.qwen3_plain import PlainQwen3
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.ops import attention_mfma as M
+    from pulse_infer_amd.weights import write_model_folder
+
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    folder = write_model_folder(Qwen3Config.from_dict(LONG), str(tmp_path / "m"), seed=31)
+    ids = token_ids(LONG["vocab_size"], 1300, seed=12)
+    want = PlainQwen3.from_folder(folder).logits(ids)
+
+    class E:
+        def __init__(self, start, count):
+            self.start, self.count = start, count
+    portion = M.portion_tokens(2, 64)
+    for start, count in ((0, 1300), (1000, 300), (1236, 64)):
+        assert M.choose_prefill_splits([(0, E(start, count))], portion, 2, 2, 64, 0)[1] > 1
+    _, model = load_model(folder, mode="bfloat16")
+    runner = ModelRunner(model, page_size=16, num_pages=90, max_requests=2)
+    whole = run_alone(runner, ids, [1300])
+    close(whole, want, "bfloat16", "whole, in splits")
+    portions = run_alone(runner, ids, [1000, 236, 64])
+    close(portions, want, "bfloat16", "late portions, in splits")
+    close(portions, whole, "bfloat16", "late portions against whole", SPLIT_TOL)

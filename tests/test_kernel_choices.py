@@ -1,0 +1,20 @@
+"""Decisions the host takes for the kernels (no GPU needed)."""
+import pytest
+
+
+def test_prefill_splits_are_chosen_for_long_walks():
+    from pulse_infer_amd.ops import attention_mfma as M
+
+    class E:
+        def __init__(self, start, count):
+            self.start, self.count = start, count
+    choose = lambda entries, **kw: M.choose_prefill_splits(list(enumerate(entries)), 32, 8, 4, 128, kw.get("window", 0))
+    assert choose([E(0, 512)]) == (0, 1)                      # short walks: nothing to gain
+    assert choose([E(0, 2048)], window=256) == (0, 1)         # a window keeps them short
+    size, n = choose([E(16384 - 512, 512)])                   # few items over a long context
+    assert n > 1 and size % 64 == 0 and size * n >= 16384 and size * (n - 1) < 16384
+    size, n = choose([E(4032, 64)])
+    assert n >= 4 and size >= 8 * 64
+    size, n = choose([E(0, 2048)])                            # a whole prompt: its late items walk twice their share
+    assert n == 2 and size > 1024 and size * n >= 2048        # cut beyond the middle: most items finish in one split
+    assert M.choose_prefill_splits([(0, E(0, 4096))], 16, 8, 4, 96, 0) == (0, 1)     # no split variant for this head size
