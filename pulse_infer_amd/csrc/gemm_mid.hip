@@ -97,13 +97,18 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
 
     // X pieces (16 bytes) of a chunk that this thread stages: piece p = tid + THREADS i is row p / ROWP, columns
     // 8 (p % ROWP)..; xdst < 0: no such piece
+    // Every load of the walk is issued whatever the thread, the row or the chunk: a load under a condition would keep
+    // the compiler from counting the loads in flight, and it would wait for all of them before every chunk (which
+    // undoes the ring).  So rows beyond M repeat row M - 1 (their products only reach outputs that are never
+    // stored; a thread without a piece to stage fetches from that row too), and chunks beyond the last one fetch
+    // the last one again.
     const bf16_t* xsrc[XP];
     int xdst[XP];
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
         const int p = tid + THREADS * i;
         const int xr = p / ROWP, xc = p % ROWP;
-        xsrc[i] = (xr < M && p < PIECES) ? X + static_cast<int64_t>(xr) * ldx + k0 + xc * 8 : nullptr;
+        xsrc[i] = X + static_cast<int64_t>(min(xr, M - 1)) * ldx + k0 + xc * 8;
         xdst[i] = p < PIECES ? xr * XROW + xc * 8 : -1;
     }
 
@@ -116,13 +121,12 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
     bf16x8 xg[2][XP];
     bf16x8 wr[RING][2 * PAIRS];
     auto load_x = [&](int c, bf16x8 (&x)[XP]) {
+        const int64_t at = static_cast<int64_t>(placed(min(c, chunks - 1))) * KC;
 #pragma unroll
-        for (int i = 0; i < XP; ++i)
-            x[i] = (xsrc[i] && c < chunks) ? *reinterpret_cast<const bf16x8*>(xsrc[i] + static_cast<int64_t>(placed(c)) * KC) : zeros8();
+        for (int i = 0; i < XP; ++i) x[i] = *reinterpret_cast<const bf16x8*>(xsrc[i] + at);
     };
     auto load_w = [&](int c, bf16x8 (&w)[2 * PAIRS]) {
-        if (c >= chunks) return;
-        const int64_t at = static_cast<int64_t>(placed(c)) * KC;
+        const int64_t at = static_cast<int64_t>(placed(min(c, chunks - 1))) * KC;
 #pragma unroll
         for (int pair = 0; pair < PAIRS; ++pair) {
             w[2 * pair] = *reinterpret_cast<const bf16x8*>(w0 + at + pair * 64);
@@ -173,10 +177,12 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
     load_w(0, wr[0]);
     load_x(1, xg[1]);
     static_for<RING - 2>([&](auto J) { load_w(decltype(J)::value + 1, wr[decltype(J)::value + 1]); });
-    for (int c = 0; c < chunks; c += RING)
-        static_for<RING>([&](auto J) {
-            if (c + decltype(J)::value < chunks) body(J, c + decltype(J)::value);
-        });
+    int c = 0;
+    for (; c + RING <= chunks; c += RING)   // whole turns of the ring without a branch inside
+        static_for<RING>([&](auto J) { body(J, c + decltype(J)::value); });
+    static_for<RING - 1>([&](auto J) {
+        if (c + decltype(J)::value < chunks) body(J, c + decltype(J)::value);
+    });
 
     // lane (kg, r) holds features n_base + 16 wave + 4 kg + i of row 16 mt + r
     if (!SWIGLU) {
@@ -255,13 +261,14 @@ void launch_rows(const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, voi
     else launch_mid<NW, 4>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
 }
 
-// 65 to 192 rows: four wavefronts, chunks of 64 k, rows rounded up to 32
+// 65 to 192 rows: four or six wavefronts, chunks of 64 k, rows rounded up to 32
+template <int NW>
 void launch_many_rows(const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
                       int k_len, int splits, int mode, bool swiglu, hipStream_t stream) {
-    if (M <= 96) launch_mid<4, 6, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
-    else if (M <= 128) launch_mid<4, 8, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
-    else if (M <= 160) launch_mid<4, 10, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
-    else launch_mid<4, 12, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+    if (M <= 96) launch_mid<NW, 6, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+    else if (M <= 128) launch_mid<NW, 8, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+    else if (M <= 160) launch_mid<NW, 10, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
+    else launch_mid<NW, 12, 64>(X, ldx, W, ldw, C, ldc, M, N, k_len, splits, mode, swiglu, stream);
 }
 
 }  // namespace
@@ -275,7 +282,7 @@ extern "C" int pulse_gemm_mid_takes(int M, int N, int K, int splits) {
 // products of the shares of K, to be added up by the consumer in split order.  swiglu != 0 (mode 0, splits 1): W holds
 // gate and up rows interleaved in slabs of 16 (gate slab, up slab, ...), N counts both, C is bfloat16 [M, N / 2] =
 // silu(gate) * up.
-// waves: wavefronts (of 16 weight rows) a workgroup, 2, 3, 4 or 6 (4 only above 64 rows); 0 lets the entry point choose.
+// waves: wavefronts (of 16 weight rows) a workgroup, 2, 3, 4 or 6 (4 or 6 above 64 rows); 0 lets the entry point choose.
 extern "C" int pulse_gemm_mid(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
                               int K, int mode, int swiglu, int splits, int waves, hipStream_t stream) {
     PULSE_REQUIRE(pulse_gemm_mid_takes(M, N, K, splits), "gemm_mid: M=%d (1..192) N=%d K=%d in %d shares (multiples of %d)",
@@ -298,8 +305,9 @@ extern "C" int pulse_gemm_mid(const void* X, int64_t ldx, const void* W, int64_t
     if (waves == 0) waves = 4;
     PULSE_REQUIRE(waves == 2 || waves == 3 || waves == 4 || waves == 6, "gemm_mid: 2, 3, 4 or 6 wavefronts a workgroup, got %d", waves);
     PULSE_REQUIRE(!swiglu || waves % 2 == 0, "gemm_mid: SwiGLU needs an even number of wavefronts");
-    PULSE_REQUIRE(M <= 64 || waves == 4, "gemm_mid: more than 64 rows take 4 wavefronts a workgroup, got %d", waves);
-    if (M > 64) launch_many_rows(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
+    PULSE_REQUIRE(M <= 64 || waves == 4 || waves == 6, "gemm_mid: more than 64 rows take 4 or 6 wavefronts a workgroup, got %d", waves);
+    if (M > 64 && waves == 6) launch_many_rows<6>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
+    else if (M > 64) launch_many_rows<4>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
     else if (waves == 2) launch_rows<2>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
     else if (waves == 3) launch_rows<3>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
     else if (waves == 4) launch_rows<4>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);

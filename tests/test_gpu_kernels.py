@@ -845,7 +845,7 @@ def test_gemm_mid(k, m, n, kk):
     w, wref = as_stored(rnd(n, kk, seed=91), torch.bfloat16)
     want = aref @ wref.T
     first = None
-    for waves in ((0, 2, 3, 4, 6) if m <= 64 else (0, 4)):     # more than 64 rows: four wavefronts, chunks of 64
+    for waves in ((0, 2, 3, 4, 6) if m <= 64 else (0, 4, 6)):  # more than 64 rows: four or six wavefronts, chunks of 64
         out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
         k.gemm_mid(a, w, out, waves=waves)
         assert torch.allclose(out.cpu().to(F64), want, atol=3e-2 * math.sqrt(kk / 128), rtol=1e-2), waves
@@ -861,7 +861,7 @@ def test_gemm_mid(k, m, n, kk):
             part = aref[:, s_ * share:(s_ + 1) * share] @ wref[:, s_ * share:(s_ + 1) * share].T
             assert torch.allclose(parts[s_].cpu().to(F64), part, atol=2e-3 * math.sqrt(share), rtol=1e-5), (splits, s_)
         again = torch.empty_like(parts)
-        k.gemm_mid(a, w, again, splits=splits, waves=2 if m <= 64 else 4)
+        k.gemm_mid(a, w, again, splits=splits, waves=2 if m <= 64 else 6)
         assert torch.equal(again, parts)
     if m > 1:                                                # strided rows (a view into a wider buffer)
         wide = torch.zeros(m, kk + 24, dtype=torch.bfloat16, device=DEV)
@@ -879,7 +879,7 @@ def test_gemm_mid_swiglu(k, m, inter, kk):
     up, uref = as_stored(rnd(inter, kk, seed=95, scale=kk ** -0.5), torch.bfloat16)
     mixed = torch.stack([gate.view(-1, 16, kk), up.view(-1, 16, kk)], dim=1).reshape(2 * inter, kk).contiguous()
     want = P.silu(aref @ gref.T) * (aref @ uref.T)
-    for waves in ((0, 2, 4, 6) if m <= 64 else (0, 4)):
+    for waves in ((0, 2, 4, 6) if m <= 64 else (0, 4, 6)):
         out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
         k.gemm_mid(a, mixed, out, swiglu=True, waves=waves)
         assert torch.allclose(out.cpu().to(F64), want, atol=1e-2, rtol=1e-2), waves
@@ -893,7 +893,7 @@ def test_gemm_mid_refuses(k):
     assert not k.gemm_mid_takes(8, 64, 192) and not k.gemm_mid_takes(8, 64, 256, 3) and k.gemm_mid_takes(8, 64, 256, 2)
     with pytest.raises(KernelError, match="not a shape"):
         k.gemm_mid(a, w, torch.zeros(193, 64, dtype=torch.bfloat16, device=DEV))
-    with pytest.raises(KernelError, match="4 wavefronts"):
+    with pytest.raises(KernelError, match="4 or 6 wavefronts"):
         k.gemm_mid(a[:100], w, torch.zeros(100, 64, dtype=torch.bfloat16, device=DEV), waves=2)
     with pytest.raises(KernelError, match="partial sums"):
         k.gemm_mid(a[:8], w, torch.zeros(8, 64, device=DEV), splits=2)
