@@ -210,7 +210,7 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     const int chunk = blockIdx.y % a.head_chunks;   // which 16 heads of the group
     const int split = blockIdx.z;
     const int tid = threadIdx.x;
-    const int wave = tid / PULSE_WAVE;
+    const int wave = uniform(tid / PULSE_WAVE);   // the same in every lane: block numbers and pages become scalar work
     const int lane = tid % PULSE_WAVE;
     const int r = lane % 16;   // operand row / result column
     const int kg = lane / 16;  // contraction group / result row group
@@ -369,17 +369,33 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     float m = -INFINITY;
     float l_part = 0.f;
 
-    // Issue every load of a 32-key block: K rows of the two 16-key tiles (a tile never straddles pages:
-    // page_size % 16 == 0) and V rows in the order {tile0: 4kg.., tile1: 4kg..}.  Nothing is done to the values here.
-    // A page that the table does not hold (-1, or beyond its width) reads page 0: those keys are masked.
-    auto load_block = [&](int b, BlockRegs& x) {
+    // The loads of a 32-key block come in two steps, each issued whatever the block (a load under a condition would
+    // keep the compiler from counting the loads in flight: it would then wait for all of them, the next block's
+    // too, before it touches this block's).  First the pages of the block's two 16-key tiles (a tile never straddles
+    // pages: page_size % 16 == 0) from the block table, an iteration before they are needed; an index beyond the
+    // table reads its last entry, which is not used then.
+    struct BlockPages { int page[2]; };
+    auto load_pages = [&](int b) {
+        BlockPages p;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            int pi, slot0;
+            page_of(b * BLOCK_KEYS + 16 * t, a.page_size, a.page_shift, pi, slot0);
+            p.page[t] = bt[min(pi, a.bt_width - 1)];
+        }
+        return p;
+    };
+    // Then every load of the block: K rows of the two tiles and V rows in the order {tile0: 4kg.., tile1: 4kg..}.
+    // Nothing is done to the values here.  A page that the table does not hold (-1, or beyond its width) reads
+    // page 0: those keys are masked.
+    auto load_block = [&](int b, const BlockPages& pages, BlockRegs& x) {
         const int j0 = b * BLOCK_KEYS;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             const int jt = j0 + 16 * t;
             int pi, slot0;
             page_of(jt, a.page_size, a.page_shift, pi, slot0);
-            int page = pi < a.bt_width ? bt[pi] : 0;
+            int page = pi < a.bt_width ? pages.page[t] : 0;
             page = (page >= 0 && page < a.num_pages) ? page : 0;  // masked keys may sit in pages given back
             const int64_t pg = static_cast<int64_t>(page) * a.nkv + g;
             const bf16_t* krow = a.kc + (pg * a.page_size + slot0 + r) * D;
@@ -459,13 +475,15 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
         }
     };
 
-    // two register sets in turn: the next block's loads are in flight while this block is computed.  Without a window
-    // the first block is known from the split alone: its loads go out before the positions have arrived.
+    // Two register sets in turn: the next block's loads are in flight while this block is computed, and the pages
+    // of the block after that are on their way.  Behind a wavefront's last block the "next" block is the one in hand
+    // once more (its lines are in the cache; nothing uses the result).  Without a window the first block is known
+    // from the split alone: its loads go out before the positions have arrived.
     {
         BlockRegs xa, xb;
         const bool early = a.window == 0;
         int b = split_begin / BLOCK_KEYS + wave;
-        if (early && b <= (split_begin + a.split_size - 1) / BLOCK_KEYS) load_block(b, xa);
+        if (early && b <= (split_begin + a.split_size - 1) / BLOCK_KEYS) load_block(b, load_pages(b), xa);
         load_q();   // behind the keys' pages in the queue: results come back in the order asked for
         if (split_begin > hi) return;                   // nothing here; the merge does not read this split
         split_end = min(split_begin + a.split_size, hi + 1);
@@ -474,18 +492,25 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
         // FUSED: the split that holds the token's position (the last one with keys) has its key to prepare
         const bool own_key = FUSED && a.new_key && hi < split_begin + a.split_size;
         const int own_block = own_key ? hi / BLOCK_KEYS : -1;
+        auto after = [&](int blk) { return blk + WAVES <= last_block ? blk + WAVES : blk; };
+        BlockPages pa = load_pages(after(b)), pb;       // (with a window b moves below; the pages are asked for again)
         if (FUSED) prepare(own_key);
         if (!early) {
             b = first_block + wave;
-            if (b <= last_block) load_block(b, xa);
+            if (b <= last_block) load_block(b, load_pages(b), xa);
+            pa = load_pages(after(b));
         }
         while (b <= last_block) {
-            if (b + WAVES <= last_block) load_block(b + WAVES, xb);
+            int nb = after(b);
+            pb = load_pages(after(nb));
+            load_block(nb, pa, xb);
             if (FUSED && b == own_block) patch(xa);
             compute_block(b, xa);
             b += WAVES;
             if (b > last_block) break;
-            if (b + WAVES <= last_block) load_block(b + WAVES, xa);
+            nb = after(b);
+            pa = load_pages(after(nb));
+            load_block(nb, pb, xa);
             if (FUSED && b == own_block) patch(xb);
             compute_block(b, xb);
             b += WAVES;
