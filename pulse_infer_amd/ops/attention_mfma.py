@@ -60,17 +60,46 @@ def split_entries(entries: Sequence):
     return short, long
 
 
-def choose_splits(num_items: int, nkv: int, group: int, max_context: int, target_groups: int = 512) -> Tuple[int, int]:
-    """(split_size, n_splits): enough workgroups to fill the chip, whole contexts when there are plenty already."""
+CHIP_WORKGROUPS = 256          # compute units: the split kernel's workgroups are counted against them
+SPLIT_OVERHEAD_KEYS = 256      # what a workgroup costs beside its walk (start-up, merge inside it), in keys walked
+MERGE_OVERHEAD_KEYS = 700      # what splitting at all costs (partial results through memory, the second kernel)
+MAX_CHOSEN_SPLITS = 64
+
+
+def choose_splits(num_items: int, nkv: int, group: int, max_context: int) -> Tuple[int, int]:
+    """(split_size, n_splits) for the kernel of decoded tokens and short portions.
+
+    The kernel's time is that of the compute unit with the longest walk: the workgroups that land on it times the
+    keys of a split plus a fixed cost each, and splitting at all costs the partial results' trip through memory and
+    the second kernel.  The number of splits with the least such cost is taken.  Measured at 8 kv heads of 4 query
+    heads, contexts of 4,096: one request is fastest in 32 splits, two in 16, four in 8, eight in 4 (256 workgroups
+    each time; 6 splits at batch 8, which leave half the units two workgroups, are 15% slower); 20 to 32 requests in
+    one (160 to 256 workgroups; two splits are 10 to 25% slower), 40 in 4 and 48 in 2 (a multiple of the units
+    again), 64 in one.  Walks of 2,048 keys and more stream better with two workgroups a unit (16 requests at 4,096:
+    4 splits 61 us, 2 splits 65), so a choice that gives every unit one such walk is cut in two once more."""
     groups = num_items * nkv * ((group + 15) // 16)
     whole = (max_context + BLOCK_KEYS - 1) // BLOCK_KEYS * BLOCK_KEYS
-    if groups * 2 > target_groups:
+    if groups <= 0 or max_context <= 0:
+        return max(whole, BLOCK_KEYS), 1
+
+    def split_size(n: int) -> int:
+        return ((max_context + n - 1) // n + BLOCK_KEYS - 1) // BLOCK_KEYS * BLOCK_KEYS
+
+    best = None
+    for n in range(1, MAX_CHOSEN_SPLITS + 1):
+        size = split_size(n)
+        if n > 1 and (size < 128 or (n - 1) * size >= max_context):
+            continue
+        on_a_unit = (groups * n + CHIP_WORKGROUPS - 1) // CHIP_WORKGROUPS
+        cost = on_a_unit * (size + SPLIT_OVERHEAD_KEYS) + (MERGE_OVERHEAD_KEYS if n > 1 else 0)
+        if best is None or cost < best[0]:
+            best = (cost, n)
+    n = best[1]
+    if n > 1 and split_size(n) >= 2048 and groups * n * 2 in (CHIP_WORKGROUPS, 2 * CHIP_WORKGROUPS):
+        n *= 2
+    if n == 1:
         return whole, 1
-    want = (target_groups + groups - 1) // groups
-    size = (max_context + want - 1) // want
-    size = max(128, (size + BLOCK_KEYS - 1) // BLOCK_KEYS * BLOCK_KEYS)
-    if size >= whole:
-        return whole, 1
+    size = split_size(n)
     return size, (max_context + size - 1) // size
 
 
