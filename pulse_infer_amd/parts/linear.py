@@ -84,6 +84,18 @@ class Linear:
                                      self.out_features, torch.float32).view(splits, rows, self.out_features)
             kernels.gemm_mid(x, self.weight, parts, splits=splits)
             return parts
+        splits = self.library_shares_for(x) if workspace is not None else 0
+        if splits:
+            # Many rows but few output tiles (down: a wide inner dimension, a narrow output): the library's product
+            # leaves most compute units idle (14B shape, 544 rows: 179 us), so it runs as a batch over shares of the
+            # inner dimension (102 us) whose float32 results the next norm adds up in order.
+            rows, share = x.shape[0], self.in_features // splits
+            parts = workspace.buffer(f"linear.parts.{self.out_features}.{self.in_features}", splits * rows,
+                                     self.out_features, torch.float32).view(splits, rows, self.out_features)
+            xa = x.view(rows, splits, share).transpose(0, 1)
+            wb = self.weight.view(self.out_features, splits, share).permute(1, 2, 0)
+            torch.bmm(xa, wb, out_dtype=torch.float32, out=parts)
+            return parts
         if (self.library and x.dtype == torch.bfloat16 and x.shape[0] <= kernels.SKINNY_FAST_ROWS
                 and kernels.gemm_skinny_ok(x, self.weight)):
             if (workspace is not None and x.shape[0] <= ResidualStream.LAZY_MAX_ROWS   # nobody would use them otherwise
@@ -103,6 +115,27 @@ class Linear:
                                  # 48, 6% at 64; at 96 to 192 rows the library takes 22 to 33 us for o and 55 to 90 us
                                  # for down, the shared-out product 16 to 22 and 33 to 47)
     MID_WORKGROUPS = 512         # workgroups wanted of it (64 weight rows times a share of the inner dimension each)
+
+    LIBRARY_SHARES_MIN_K = 8192  # inner dimensions from here on are worth sharing out in the library's product
+    LIBRARY_TILE = 256           # its output tiles are about this large in both directions
+
+    def library_shares_for(self, x: torch.Tensor) -> int:
+        """Into how many shares the library's product of more than 192 rows is cut; 0: not at all.  Measured (8B,
+        14B and 32B shapes of down, 272 to 2,048 rows): 4 shares win up to about 50 output tiles, 2 shares up to
+        about 140 (8B shape at 2,048 rows: 182 -> 157 us, which the wider update costs again in the norm that adds
+        it up, so the rule stops at 100 tiles), none beyond; products with an inner dimension of 4,096 to 8,192 (o)
+        gain 5 us at most."""
+        rows = x.shape[0]
+        if not (self.library and x.dtype == torch.bfloat16 and rows > self.SHARES_ROWS[1]
+                and self.in_features >= self.LIBRARY_SHARES_MIN_K and x.is_contiguous()
+                and self.weight.is_contiguous() and self.out_features % 4 == 0):
+            return 0
+        tile = self.LIBRARY_TILE
+        tiles = ((rows + tile - 1) // tile) * ((self.out_features + tile - 1) // tile)
+        splits = 4 if tiles <= 50 else (2 if tiles <= 100 else 0)
+        while splits > 1 and (self.in_features % splits or (self.in_features // splits) % 64):
+            splits //= 2
+        return splits if splits > 1 else 0
 
     def operands_ok(self, x: torch.Tensor) -> bool:
         """Contiguous, aligned bfloat16 rows of a length the kernels' 16-byte loads take."""

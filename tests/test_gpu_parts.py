@@ -65,6 +65,37 @@ def test_norm_part(gpu, mode):
     assert torch.allclose(out.cpu().to(F64), P.rms_norm(h.cpu().to(F64), w.to(F64), 1e-4), **TOL[mode])
 
 
+@pytest.mark.parametrize("rows,n,splits", [(300, 768, 4), (700, 768, 4), (1800, 2048, 2)])
+def test_linear_adds_into_the_residual_through_shares_of_the_library_product(gpu, rows, n, splits):
+    """Many rows, a wide inner dimension and few output tiles: ``Linear.add_into`` runs the library's product as a
+    batch over shares of the inner dimension and hands back their float32 results, which the norm's kernel (and the
+    plain addition) add to the residual in order."""
+    from pulse_infer_amd.ops import kernels
+    from pulse_infer_amd.parts.base import Workspace
+    from pulse_infer_amd.parts.linear import Linear
+    k = 8192
+    w = rnd(n, k, seed=3, scale=k ** -0.5).to(DEV)
+    x = rnd(rows, k, seed=4).to(DEV)
+    lin = Linear(w, "bfloat16")
+    assert lin.library_shares_for(x) == splits
+    h = torch.randn(rows, n, generator=torch.Generator().manual_seed(5)).to(DEV)
+    parts = lin.add_into(x, h, torch.empty(rows, n, dtype=torch.bfloat16, device=DEV), Workspace(torch.device(DEV)))
+    assert parts.shape == (splits, rows, n) and parts.dtype == torch.float32
+    want = x.double() @ w.double().T
+    assert torch.allclose(parts.double().sum(0), want, atol=2e-3, rtol=2e-3)
+    share = k // splits
+    assert torch.allclose(parts[1].double(), x[:, share:2 * share].double() @ w[:, share:2 * share].double().T,
+                          atol=2e-3, rtol=2e-3)
+    norm_w = torch.ones(n, dtype=torch.bfloat16, device=DEV)
+    out = torch.empty(rows, n, dtype=torch.bfloat16, device=DEV)
+    h2 = h.clone()
+    kernels.add_rmsnorm(h2, parts, norm_w, 1e-6, out)
+    assert torch.allclose(h2.double(), h.double() + want, atol=3e-3, rtol=3e-3)
+    h3 = h.clone()
+    kernels.residual_add(h3, parts)
+    assert torch.equal(h3, h2)
+
+
 @pytest.mark.parametrize("mode", ["float32", "bfloat16"])
 def test_feed_forward_part(gpu, mode):
     from pulse_infer_amd.parts.base import FEED_FORWARDS

@@ -18,3 +18,19 @@ def test_prefill_splits_are_chosen_for_long_walks():
     size, n = choose([E(0, 2048)])                            # a whole prompt: its late items walk twice their share
     assert n == 2 and size > 1024 and size * n >= 2048        # cut beyond the middle: most items finish in one split
     assert M.choose_prefill_splits([(0, E(0, 4096))], 16, 8, 4, 96, 0) == (0, 1)     # no split variant for this head size
+
+
+def test_library_products_share_out_a_wide_inner_dimension():
+    import torch
+    from pulse_infer_amd.parts.linear import Linear
+
+    down = Linear(torch.empty(5120, 17408, dtype=torch.bfloat16), "bfloat16")        # 14B shape
+    rows = lambda m, k=17408: torch.empty(m, k, dtype=torch.bfloat16)
+    assert down.library_shares_for(rows(100)) == 0          # up to 192 rows the package's own product takes it
+    assert down.library_shares_for(rows(272)) == 4
+    assert down.library_shares_for(rows(544)) == 2
+    assert down.library_shares_for(rows(2048)) == 0         # enough output tiles to fill the chip
+    o = Linear(torch.empty(5120, 5120, dtype=torch.bfloat16), "bfloat16")
+    assert o.library_shares_for(rows(544, 5120)) == 0       # a narrow inner dimension: nothing to gain
+    f32 = Linear(torch.empty(64, 8192), "float32")
+    assert f32.library_shares_for(torch.empty(300, 8192)) == 0
