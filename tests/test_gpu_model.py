@@ -329,3 +329,41 @@ def test_long_prompts_walk_their_keys_in_splits(tmp_path):
     portions = run_alone(runner, ids, [1000, 236, 64])
     close(portions, want, "bfloat16", "late portions, in splits")
     close(portions, whole, "bfloat16", "late portions against whole", SPLIT_TOL)
+
+
+WIDE = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=211, hidden_size=128, intermediate_size=8192,
+    num_hidden_layers=2, num_attention_heads=2, num_key_value_heads=1, head_dim=32, max_position_embeddings=512,
+    rms_norm_eps=1e-6, rope_theta=1e4, tie_word_embeddings=False, torch_dtype="bfloat16", attention_bias=False,
+    use_sliding_window=False, hidden_act="silu")
+
+
+def test_a_wide_feed_forward_shares_out_its_down_product(tmp_path):
+    """An intermediate size of 8,192 and prompts of a few hundred tokens: the down product runs as the library's
+    batch over shares of its inner dimension (asserted), and the norms, the last one with gathered rows too, add the
+    shares up; whole, in portions and with a decoded tail, against the plain implementation."""
+    from plain.qwen3_plain import PlainQwen3
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.weights import write_model_folder
+
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    folder = write_model_folder(Qwen3Config.from_dict(WIDE), str(tmp_path / "m"), seed=41)
+    ids = token_ids(WIDE["vocab_size"], 400, seed=13)
+    want = PlainQwen3.from_folder(folder).logits(ids)
+    _, model = load_model(folder, mode="bfloat16")
+    down = model.blocks[0].ffn.down
+    assert down.library_shares_for(torch.empty(400, 8192, dtype=torch.bfloat16, device=model.device)) == 4
+    runner = ModelRunner(model, page_size=16, num_pages=40, max_requests=2)
+    whole = run_alone(runner, ids, [400])
+    close(whole, want, "bfloat16", "whole, down in shares")
+    cut = run_alone(runner, ids, [250, 118] + [1] * 32)
+    close(cut, want, "bfloat16", "portions and a tail, down in shares")
+    # only the last row wanted: the final norm gathers rows of a residual whose last update is still in shares
+    runner.add_request("g")
+    runner.reserve("g", 400)
+    last = runner.step([StepEntry("g", ids, [399, 7])])
+    runner.free_request("g")
+    close(last, want[[399, 7]], "bfloat16", "gathered rows, down in shares")
