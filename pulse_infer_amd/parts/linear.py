@@ -77,12 +77,12 @@ class Linear:
         64 rows, given a workspace: the product's inner dimension is shared out over workgroups and the shares' float32
         results [parts, rows, out] are returned as the update, which the next norm adds up in order.  Otherwise the
         product is written to ``scratch`` and returned for the caller to add."""
-        splits = self.shares_for(x) if workspace is not None else 0
+        splits, waves = self.shares_and_waves_for(x) if workspace is not None else (0, 0)
         if splits:
             rows = x.shape[0]
             parts = workspace.buffer(f"linear.parts.{self.out_features}.{self.in_features}", splits * rows,
                                      self.out_features, torch.float32).view(splits, rows, self.out_features)
-            kernels.gemm_mid(x, self.weight, parts, splits=splits)
+            kernels.gemm_mid(x, self.weight, parts, splits=splits, waves=waves)
             return parts
         splits = self.library_shares_for(x) if workspace is not None else 0
         if splits:
@@ -114,7 +114,6 @@ class Linear:
                                  # workgroups (measured on the 8B shape: a decoding step gains 1% at 17 to 32 rows, 4% at
                                  # 48, 6% at 64; at 96 to 192 rows the library takes 22 to 33 us for o and 55 to 90 us
                                  # for down, the shared-out product 16 to 22 and 33 to 47)
-    MID_WORKGROUPS = 512         # workgroups wanted of it (64 weight rows times a share of the inner dimension each)
 
     LIBRARY_SHARES_MIN_K = 8192  # inner dimensions from here on are worth sharing out in the library's product
     LIBRARY_TILE = 256           # its output tiles are about this large in both directions
@@ -150,16 +149,33 @@ class Linear:
 
     def shares_for(self, x: torch.Tensor) -> int:
         """Into how many shares the inner dimension is cut for an update in parts; 0: not this product."""
+        return self.shares_and_waves_for(x)[0]
+
+    def shares_and_waves_for(self, x: torch.Tensor):
+        """(shares of the inner dimension, wavefronts a workgroup) of the product for 17 to 192 rows whose float32
+        partial results the next norm adds up; (0, 0): not this product.
+
+        The pair with the least estimated time of the fullest compute unit is taken: workgroups on it (all of them
+        over 256 units, rounded up) x weight rows a workgroup x (length of a share + 280, what a workgroup costs
+        beside its walk), plus half a microsecond a share for the norm that adds them up.  Measured at 64 rows: down
+        of the 8B shape 4 shares of 64 rows (256 workgroups) 23.8 us, 8 shares 24.9, 6 shares (384 workgroups, two on
+        half the units) 28.6; down of the 14B shape 4 shares of 96 rows (216 workgroups) 40.9 us, 8 shares of 64 rows
+        (640 workgroups) 46.9."""
         if not (self.library and x.dtype == torch.bfloat16 and self.SHARES_ROWS[0] <= x.shape[0] <= self.SHARES_ROWS[1]
                 and self.operands_ok(x)) or self.out_features % 4:
-            return 0
-        tiles = (self.out_features + 63) // 64
-        best = 0
-        for splits in range(1, 17):
-            # a share of at least 1024: every further part costs the norm that adds them up about 0.5 us
-            if self.in_features % splits or (self.in_features // splits) % 128 or self.in_features // splits < 1024:
-                continue
-            best = splits
-            if tiles * splits >= self.MID_WORKGROUPS:
-                break
-        return best
+            return 0, 0
+        best = None
+        for waves in (4, 6):
+            rows = 16 * waves
+            tiles = (self.out_features + rows - 1) // rows
+            for splits in range(1, 17):
+                if self.in_features % splits or (self.in_features // splits) % 128:
+                    continue
+                share = self.in_features // splits
+                on_a_unit = (tiles * splits + self.MID_UNITS - 1) // self.MID_UNITS
+                cost = on_a_unit * rows * (share + 280) + 8000 * splits
+                if best is None or cost < best[0]:
+                    best = (cost, splits, waves)
+        return (best[1], best[2]) if best else (0, 0)
+
+    MID_UNITS = 256              # compute units
