@@ -82,7 +82,7 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
     // Workgroups do not all walk their share of K from the same end: the owners of every 960 weight rows start four
     // chunks later than the owners of the 960 before (and wrap around), which loads the memory channels more evenly
     // (gate+up of the 8B shape: 5 to 9% faster).  The order of the sums depends on the weight row and the share only,
-    // not on the workgroup's shape (960 is a multiple of the rows of every shape: 32, 48, 64, 96) or on X.
+    // not on the workgroup's shape (960 is a multiple of the rows of every shape: 32, 48, 64, 96, 160) or on X.
     const int rot = static_cast<int>(((n_base / STAGGER_ROWS) * STAGGER_CHUNKS + blockIdx.y) % static_cast<unsigned>(chunks));
     auto placed = [&](int c) { return c + rot >= chunks ? c + rot - chunks : c + rot; };  // where chunk c of the walk lies
 
@@ -282,7 +282,7 @@ extern "C" int pulse_gemm_mid_takes(int M, int N, int K, int splits) {
 // products of the shares of K, to be added up by the consumer in split order.  swiglu != 0 (mode 0, splits 1): W holds
 // gate and up rows interleaved in slabs of 16 (gate slab, up slab, ...), N counts both, C is bfloat16 [M, N / 2] =
 // silu(gate) * up.
-// waves: wavefronts (of 16 weight rows) a workgroup, 2, 3, 4 or 6 (4 or 6 above 64 rows); 0 lets the entry point choose.
+// waves: wavefronts (of 16 weight rows) a workgroup, 2, 3, 4, 6 or 10 (4 or 6 above 64 rows); 0 lets the entry point choose.
 extern "C" int pulse_gemm_mid(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
                               int K, int mode, int swiglu, int splits, int waves, hipStream_t stream) {
     PULSE_REQUIRE(pulse_gemm_mid_takes(M, N, K, splits), "gemm_mid: M=%d (1..192) N=%d K=%d in %d shares (multiples of %d)",
@@ -303,7 +303,9 @@ extern "C" int pulse_gemm_mid(const void* X, int64_t ldx, const void* W, int64_t
     const bf16_t* w = static_cast<const bf16_t*>(W);
     const int k_len = K / splits;
     if (waves == 0) waves = 4;
-    PULSE_REQUIRE(waves == 2 || waves == 3 || waves == 4 || waves == 6, "gemm_mid: 2, 3, 4 or 6 wavefronts a workgroup, got %d", waves);
+    // (16 x waves divides the 960 rows of a stagger group, so the order of a row's sums does not depend on the shape)
+    PULSE_REQUIRE(waves == 2 || waves == 3 || waves == 4 || waves == 6 || waves == 10,
+                  "gemm_mid: 2, 3, 4, 6 or 10 wavefronts a workgroup, got %d", waves);
     PULSE_REQUIRE(!swiglu || waves % 2 == 0, "gemm_mid: SwiGLU needs an even number of wavefronts");
     PULSE_REQUIRE(M <= 64 || waves == 4 || waves == 6, "gemm_mid: more than 64 rows take 4 or 6 wavefronts a workgroup, got %d", waves);
     if (M > 64 && waves == 6) launch_many_rows<6>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
@@ -311,7 +313,8 @@ extern "C" int pulse_gemm_mid(const void* X, int64_t ldx, const void* W, int64_t
     else if (waves == 2) launch_rows<2>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
     else if (waves == 3) launch_rows<3>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
     else if (waves == 4) launch_rows<4>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
-    else launch_rows<6>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
+    else if (waves == 6) launch_rows<6>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
+    else launch_rows<10>(x, ldx, w, ldw, C, ldc, M, N, k_len, splits, mode, swiglu != 0, stream);
     PULSE_LAUNCH_CHECK("gemm_mid");
     return 0;
 }

@@ -44,10 +44,7 @@ class Linear:
             return out
         if swiglu:
             if x.shape[0] > kernels.SKINNY_FAST_ROWS:
-                # Workgroups of 96 weight rows fetch X a third less often than those of 64, which counts once X is
-                # 32 rows and more (gate+up of the 8B shape at 64 rows: 46 us against 52; of the 14B shape at 32
-                # rows: 81 against 85); below that, workgroups of 32 rows spread best over the compute units.
-                kernels.gemm_mid(x, w, out, swiglu=True, waves=2 if x.shape[0] <= 24 else 6)
+                kernels.gemm_mid(x, w, out, swiglu=True, waves=self.swiglu_waves_for(x.shape[0]) or 4)
             else:
                 kernels.gemm_skinny(x, w, out, swiglu=True)
             return out
@@ -145,7 +142,30 @@ class Linear:
 
     def takes_mid(self, x: torch.Tensor) -> bool:
         return (self.library and x.dtype == torch.bfloat16 and self.MID_ROWS[0] <= x.shape[0] <= self.MID_ROWS[1]
-                and self.operands_ok(x))
+                and self.operands_ok(x) and self.swiglu_waves_for(x.shape[0]) > 0)
+
+    def swiglu_waves_for(self, rows: int) -> int:
+        """Wavefronts a workgroup of the product for 17 to 64 rows with SwiGLU inside (no sharing out of the inner
+        dimension there), or 0 where the library's product followed by the SwiGLU kernel is faster.
+
+        The estimate is again the fullest compute unit's: workgroups on it x (weight rows a workgroup + half the
+        rows of X, which every workgroup fetches).  Measured at 32 rows: 8B shape (24,576 weight rows) 96 rows a
+        workgroup 37.9 us (one workgroup a unit), 64 rows 43.6; 14B shape (34,816) 160 rows 68.8 us, 96 rows 80.5
+        (363 workgroups: two on some units); 32B shape (51,200) 64 rows 117 us, the best of all shapes, against
+        the library's 100 + 5: no shape shares 200 rows a unit out evenly, so the library takes that one (the rule:
+        this product's estimate must stay below 1.5 x the weight rows a unit)."""
+        n = self.out_features
+        if n <= 32 * self.MID_UNITS:
+            return 2    # too few weight rows to fill the chip in any shape: the most workgroups
+        best = None
+        for waves in (2, 4, 6, 10):
+            on_a_unit = ((n + 16 * waves - 1) // (16 * waves) + self.MID_UNITS - 1) // self.MID_UNITS
+            cost = on_a_unit * (16 * waves + rows // 2)
+            if best is None or cost < best[0]:
+                best = (cost, waves)
+        if n <= 64 * self.MID_UNITS:
+            return best[1]    # (12,288 weight rows: 64 rows a workgroup 12 to 15 us, the library 15 to 18 + 5)
+        return best[1] if best[0] * self.MID_UNITS < 1.5 * n else 0
 
     def shares_for(self, x: torch.Tensor) -> int:
         """Into how many shares the inner dimension is cut for an update in parts; 0: not this product."""

@@ -34,3 +34,14 @@ def test_library_products_share_out_a_wide_inner_dimension():
     assert o.library_shares_for(rows(544, 5120)) == 0       # a narrow inner dimension: nothing to gain
     f32 = Linear(torch.empty(64, 8192), "float32")
     assert f32.library_shares_for(torch.empty(300, 8192)) == 0
+
+
+def test_gate_up_takes_the_workgroup_shape_that_shares_its_rows_out_evenly():
+    import torch
+    from pulse_infer_amd.parts.linear import Linear
+
+    shape = lambda n, k: Linear(torch.empty(n, k, dtype=torch.bfloat16, device="meta"), "bfloat16")
+    assert shape(24576, 4096).swiglu_waves_for(32) == 6       # 8B: 256 workgroups of 96 rows
+    assert shape(34816, 5120).swiglu_waves_for(32) == 10      # 14B: 218 workgroups of 160 rows
+    assert shape(51200, 5120).swiglu_waves_for(32) == 0       # 32B: no even share; the library's product
+    assert shape(448, 96).swiglu_waves_for(20) == 2           # few rows: the most workgroups
