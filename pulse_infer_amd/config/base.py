@@ -27,12 +27,50 @@ def resolve_model_dir(path: str) -> str:
     return path
 
 
+def strip_json_comments(text: str) -> str:
+    """``text`` without // line comments and /* block comments */ outside strings (a comment becomes a blank)."""
+    out: List[str] = []
+    i, n = 0, len(text)
+    in_string = False
+    while i < n:
+        c = text[i]
+        if in_string:
+            out.append(c)
+            if c == "\\" and i + 1 < n:
+                out.append(text[i + 1])
+                i += 1
+            elif c == '"':
+                in_string = False
+        elif c == '"':
+            in_string = True
+            out.append(c)
+        elif c == "/" and text[i:i + 2] == "//":
+            while i < n and text[i] != "\n":
+                i += 1
+            continue
+        elif c == "/" and text[i:i + 2] == "/*":
+            end = text.find("*/", i + 2)
+            i = n if end < 0 else end + 2
+            out.append(" ")
+            continue
+        else:
+            out.append(c)
+        i += 1
+    return "".join(out)
+
+
 def read_json_file(path: str) -> Dict[str, Any]:
+    """A JSON object from a file; comments are allowed, as in the reference's reader
+    (reference: src/model/qwen3/config.cpp:52 parses with ignore_comments)."""
     if not os.path.exists(path):
         raise ConfigError(f"Config file '{path}' does not exist")
     try:
         with open(path, "r", encoding="utf-8") as fh:
-            data = json.load(fh)
+            text = fh.read()
+        try:
+            data = json.loads(text)
+        except json.JSONDecodeError:
+            data = json.loads(strip_json_comments(text))
     except json.JSONDecodeError as exc:
         raise ConfigError(f"Config file '{path}' is not valid JSON: {exc}") from exc
     if not isinstance(data, dict):

@@ -155,3 +155,17 @@ def test_rope_pairing_is_an_option_of_the_engine():
     cfg.rope_pairing = "pairs"
     with pytest.raises(ConfigError):
         cfg.validate()
+
+
+def test_config_json_may_hold_comments(tmp_path):
+    """The reference parses config.json with comments allowed (src/model/qwen3/config.cpp:52)."""
+    text = json.dumps(TINY_B, indent=1)
+    text = text.replace('"hidden_size"', '// the width\n "hidden_size"', 1)
+    text = text.replace('"vocab_size"', '/* tokens:\n   all of them */ "vocab_size"', 1)
+    text = text.replace('"qwen3",', '"qwen3", // not "/*" a comment inside', 1)
+    (tmp_path / "config.json").write_text(text)
+    cfg = load_config(str(tmp_path))
+    assert cfg.hidden_size == TINY_B["hidden_size"] and cfg.vocab_size == TINY_B["vocab_size"]
+    (tmp_path / "config.json").write_text('{"a": "x // y", /* c */ "b": 1} trailing')
+    with pytest.raises(ConfigError, match="not valid JSON"):
+        load_config(str(tmp_path))
