@@ -367,3 +367,50 @@ def test_a_wide_feed_forward_shares_out_its_down_product(tmp_path):
     last = runner.step([StepEntry("g", ids, [399, 7])])
     runner.free_request("g")
     close(last, want[[399, 7]], "bfloat16", "gathered rows, down in shares")
+
+
+MANY = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=300, hidden_size=256, intermediate_size=512,
+    num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=64, max_position_embeddings=256,
+    rms_norm_eps=1e-6, rope_theta=1e4, tie_word_embeddings=False, torch_dtype="bfloat16", attention_bias=False,
+    use_sliding_window=False, hidden_act="silu")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("requests", [24, 70, 200])
+def test_many_requests_decode_together(tmp_path, requests, dtype):
+    """Steps of 24, 70 and 200 decoded tokens (the products for 17 to 192 rows and the library's beyond, attention
+    over many short contexts of different lengths): every request's logits are those of the plain implementation
+    for its own sequence, whatever stands beside it."""
+    from plain.qwen3_plain import PlainQwen3
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.weights import write_model_folder
+
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    folder = write_model_folder(Qwen3Config.from_dict(MANY), str(tmp_path / "m"), seed=51)
+    plain = PlainQwen3.from_folder(folder)
+    steps = 4
+    lengths = [1 + (7 * i) % 40 for i in range(requests)]
+    ids = [token_ids(MANY["vocab_size"], n + steps, seed=100 + i) for i, n in enumerate(lengths)]
+    _, model = load_model(folder, mode=dtype)
+    runner = ModelRunner(model, page_size=16, num_pages=requests * 4, max_requests=requests)
+    for i in range(0, requests, 8):          # prompts, eight requests a step
+        batch = []
+        for r in range(i, min(i + 8, requests)):
+            runner.add_request(r)
+            runner.reserve(r, lengths[r] + steps)
+            batch.append(StepEntry(r, ids[r][:lengths[r]], []))
+        runner.step(batch)
+    got = []
+    for s in range(steps):                   # then every request's next token in one step
+        got.append(runner.step([StepEntry(r, [ids[r][lengths[r] + s]], [0]) for r in range(requests)]))
+    for r in range(0, requests, max(1, requests // 12)):
+        want = plain.logits(ids[r])[lengths[r]:]
+        mine = torch.stack([g[r] for g in got])
+        close(mine, want, dtype, f"request {r} of {requests}")
+    for r in range(requests):
+        runner.free_request(r)
+    runner.cache.check()
