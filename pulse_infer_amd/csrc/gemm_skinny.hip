@@ -522,7 +522,10 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
     if (mt == 1 && tune != 9 && (t_kw ? true : K % 1024 == 0)) {
         // the streaming kernel: pairs of slabs when there are many (or, from 8 rows of X on, enough of them: a
         // pair shares its loads of X), else single slabs with more wavefronts along K
-        const bool pairs = swiglu || wide || (N >= 6144 && M >= 8);
+        // (also where single slabs would put two workgroups on some compute units and pairs one on each: 5,120
+        // weight rows, o and down of the 14B shape, at 8 rows 16.2 -> 14.7 us and 44.7 -> 36.9 us)
+        auto fullest = [&](int rows) { return ((N + rows - 1) / rows + 255) / 256 * rows; };   // weight rows on the fullest of 256 units
+        const bool pairs = swiglu || wide || (M >= 8 && (N >= 6144 || fullest(16) >= fullest(32)));
         const int slabs = t_slabs ? t_slabs : (pairs ? 2 : 1);
         const int kw = t_kw ? t_kw : ((K % 2048 == 0 && !pairs) ? 8 : 4);
         const int pack = t_pack ? t_pack : pack_for(M);
