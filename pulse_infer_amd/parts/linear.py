@@ -69,11 +69,12 @@ class Linear:
 
     def add_into(self, x: torch.Tensor, residual: torch.Tensor, scratch: torch.Tensor,
                  workspace: Optional[Workspace] = None):
-        """residual += x W^T, in one of four ways.  Few rows: the kernel adds into the residual itself and None is
-        returned, or, given a workspace and a shape the fused kernel takes, the ``RowStats`` of the updated rows.  Up to
-        64 rows, given a workspace: the product's inner dimension is shared out over workgroups and the shares' float32
-        results [parts, rows, out] are returned as the update, which the next norm adds up in order.  Otherwise the
-        product is written to ``scratch`` and returned for the caller to add."""
+        """residual += x W^T, in one of five ways.  Few rows: the kernel adds into the residual itself and None is
+        returned, or, given a workspace and a shape the fused kernel takes, the ``RowStats`` of the updated rows.  17 to
+        192 rows, given a workspace: the product's inner dimension is shared out over workgroups and the shares' float32
+        results [parts, rows, out] are returned as the update, which the next norm adds up in order; more rows of a
+        product with a wide inner dimension and a narrow output: the same through the library's batched product.
+        Otherwise the product is written to ``scratch`` and returned for the caller to add."""
         splits, waves = self.shares_and_waves_for(x) if workspace is not None else (0, 0)
         if splits:
             rows = x.shape[0]
