@@ -38,12 +38,10 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
     return __uint_as_float(static_cast<uint32_t>(v) << 16);
 }
 
-// Round to nearest, ties to even; NaN stays NaN.
+// Round to nearest, ties to even; NaN stays NaN.  (The conversion instruction of gfx950, v_cvt_pk_bf16_f32: one
+// instruction for two values where the rounding written out in integer arithmetic takes six a value.)
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<bf16_t>((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return static_cast<bf16_t>(u >> 16);
+    return __builtin_bit_cast(bf16_t, static_cast<__bf16>(f));
 }
 
 template <typename T> __device__ __forceinline__ float to_f32(T v);
