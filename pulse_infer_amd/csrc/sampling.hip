@@ -41,14 +41,30 @@ struct RowView {
     const uint32_t* banned;  // bit per token, or null
     float penalty;
     int vocab;
+    // (without a branch on what was loaded: the loads of several entries can then be in flight together)
     __device__ __forceinline__ float at(int i) const {
-        if (banned && ((banned[i >> 5] >> (i & 31)) & 1u)) return -INFINITY;
-        float x = logits[i];
-        if (x != x) return -INFINITY;
-        if (seen && ((seen[i >> 5] >> (i & 31)) & 1u)) x -= penalty;
-        return x;
+        const float x = logits[i];
+        const bool out = banned ? ((banned[i >> 5] >> (i & 31)) & 1u) != 0u : false;
+        const bool was = seen ? ((seen[i >> 5] >> (i & 31)) & 1u) != 0u : false;
+        return (out || x != x) ? -INFINITY : (was ? x - penalty : x);
     }
 };
+
+// f(i, value) for i = first, first + step, .. below end, in that order; the values of eight entries are asked for
+// before the first is used (a workgroup alone on its row otherwise waits out a trip to memory for every entry).
+template <typename F>
+__device__ __forceinline__ void sweep(const RowView& row, int first, int end, int step, F f) {
+    constexpr int AHEAD = 8;
+    int i = first;
+    for (; i + (AHEAD - 1) * step < end; i += AHEAD * step) {
+        float x[AHEAD];
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) x[u] = row.at(i + u * step);
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) f(i + u * step, x[u]);
+    }
+    for (; i < end; i += step) f(i, row.at(i));
+}
 
 __device__ float block_sum_f(float v, float* scratch) { return block_sum(v, scratch); }
 
@@ -157,11 +173,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     // largest logit, lowest index among equals; the smallest number too (the histogram's range)
     float best = -INFINITY, lowest = INFINITY;
     int best_i = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-        const float x = row.at(i);
+    sweep(row, threadIdx.x, vocab, SAMPLE_THREADS, [&](int i, float x) {
         if (x > best) { best = x; best_i = i; }
         if (x != -INFINITY) lowest = fminf(lowest, x);
-    }
+    });
     block_argmax(best, best_i, sf, si);
     if (best_i == 0x7fffffff) {  // everything banned or NaN
         if (threadIdx.x == 0) out[r] = -1;
@@ -191,10 +206,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         float whole = 0.f;   // without top-k: the mass of the whole vocabulary, which top_p refers to
         if (!by_k) {
             float mass = 0.f;
-            for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-                const float x = row.at(i);
+            sweep(row, threadIdx.x, vocab, SAMPLE_THREADS, [&](int, float x) {
                 if (x != -INFINITY) mass += expf((x - best) * inv_t);
-            }
+            });
             whole = block_sum_f(mass, sf);
         }
         lowest = -block_max_f(-lowest, sf);
@@ -205,10 +219,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         if (ranged) {
             for (int b = threadIdx.x; b < HIST_BINS; b += SAMPLE_THREADS) hist[b] = 0;
             __syncthreads();
-            for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-                const float x = row.at(i);
+            sweep(row, threadIdx.x, vocab, SAMPLE_THREADS, [&](int, float x) {
                 if (x != -INFINITY) atomicAdd(&hist[bin_of(x)], 1);
-            }
+            });
             __syncthreads();
             // the bin in which the count from the top reaches k: first by wavefronts' shares of the bins, then by bins
             constexpr int SHARE = HIST_BINS / SAMPLE_WAVES;
@@ -229,14 +242,24 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         }
         if (edge >= 0 && listed <= LIST_CAP) {
             int count = 0;
-            for (int base = part_begin; base < part_end; base += PULSE_WAVE) {
-                const int i = base + lane;
-                const float x = i < part_end ? row.at(i) : -INFINITY;
-                const bool in = x != -INFINITY && bin_of(x) <= edge;
-                const unsigned long long mask = __ballot(in);
-                const int at = count + __builtin_popcountll(mask & ((1ull << lane) - 1ull));
-                if (in && at < WAVE_CAP) { region_i[wave][at] = i; region_x[wave][at] = x; }
-                count += __builtin_popcountll(mask);
+            constexpr int AHEAD = 8;   // steps of 64 entries whose values are asked for together
+            for (int base = part_begin; base < part_end; base += AHEAD * PULSE_WAVE) {
+                float xs[AHEAD];
+#pragma unroll
+                for (int u = 0; u < AHEAD; ++u) {
+                    const int i = base + u * PULSE_WAVE + lane;
+                    xs[u] = i < part_end ? row.at(i) : -INFINITY;
+                }
+#pragma unroll
+                for (int u = 0; u < AHEAD; ++u) {
+                    const int i = base + u * PULSE_WAVE + lane;
+                    const float x = xs[u];
+                    const bool in = x != -INFINITY && bin_of(x) <= edge;
+                    const unsigned long long mask = __ballot(in);
+                    const int at = count + __builtin_popcountll(mask & ((1ull << lane) - 1ull));
+                    if (in && at < WAVE_CAP) { region_i[wave][at] = i; region_x[wave][at] = x; }
+                    count += __builtin_popcountll(mask);
+                }
             }
             if (lane == 0) region_n[wave] = count;
             __syncthreads();
@@ -337,34 +360,31 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         for (int bit = 31; bit >= 0; --bit) {
             const uint32_t cand = keep | (1u << bit);
             int count = 0;
-            for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) count += order_key(row.at(i)) >= cand;
+            sweep(row, threadIdx.x, vocab, SAMPLE_THREADS, [&](int, float x) { count += order_key(x) >= cand; });
             if (block_sum_i(count, si) >= k) keep = cand;
         }
     }
-    auto weight = [&](int i) {
-        const float x = row.at(i);
-        return (x != -INFINITY && order_key(x) >= keep) ? expf((x - best) * inv_t) : 0.f;
-    };
+    auto weight_of = [&](float x) { return (x != -INFINITY && order_key(x) >= keep) ? expf((x - best) * inv_t) : 0.f; };
+    auto weight = [&](int i) { return weight_of(row.at(i)); };
     if (use_p) {
         float mass = 0.f;
-        for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) mass += weight(i);
+        sweep(row, threadIdx.x, vocab, SAMPLE_THREADS, [&](int, float x) { mass += weight_of(x); });
         const float want = p * block_sum_f(mass, sf);
         uint32_t thr = 0u;
         for (int bit = 31; bit >= 0; --bit) {
             const uint32_t cand = thr | (1u << bit);
             const uint32_t lim = cand > keep ? cand : keep;
             float part_mass = 0.f;
-            for (int i = threadIdx.x; i < vocab; i += SAMPLE_THREADS) {
-                const float x = row.at(i);
+            sweep(row, threadIdx.x, vocab, SAMPLE_THREADS, [&](int, float x) {
                 if (x != -INFINITY && order_key(x) >= lim) part_mass += expf((x - best) * inv_t);
-            }
+            });
             if (block_sum_f(part_mass, sf) >= want) thr = cand;
         }
         if (thr > keep) keep = thr;
     }
     // the kept mass of every wavefront's part, then the part in which the draw falls is walked by its wavefront
     float mine = 0.f;
-    for (int i = part_begin + lane; i < part_end; i += PULSE_WAVE) mine += weight(i);
+    sweep(row, part_begin + lane, part_end, PULSE_WAVE, [&](int, float x) { mine += weight_of(x); });
 #pragma unroll
     for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) mine += __shfl_xor(mine, off, PULSE_WAVE);
     if (lane == 0) part_sum[wave] = mine;
