@@ -86,7 +86,13 @@ class InferenceRequest:
 
     def get_next_chunk_tokens(self, chunk_size: int = 256) -> List[int]:
         n = self.get_next_chunk_size(chunk_size)
-        return [self.token_at(self.num_computed_tokens + i) for i in range(n)]
+        start, end = self.num_computed_tokens, self.num_computed_tokens + n
+        split = self.prompt_len    # prompt tokens, then generated ones (two slices, not a call a token)
+        if end <= split:
+            return self.prompt_tokens[start:end]
+        if start >= split:
+            return self.generated_tokens[start - split:end - split]
+        return self.prompt_tokens[start:] + self.generated_tokens[:end - split]
 
     def get_next_chunk_positions(self, chunk_size: int = 256) -> List[int]:
         n = self.get_next_chunk_size(chunk_size)

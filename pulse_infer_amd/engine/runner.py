@@ -147,9 +147,9 @@ class ModelRunner:
             if self.cache.reserved(e.request) < start + n:
                 raise StepError(f"request {e.request!r}: pages are reserved for {self.cache.reserved(e.request)} "
                                 f"tokens, the step needs {start + n}")
-            for tok in e.tokens:
-                if not 0 <= int(tok) < vocab:
-                    raise StepError(f"request {e.request!r}: token id {tok} is outside the vocabulary of {vocab}")
+            if min(e.tokens) < 0 or max(e.tokens) >= vocab:
+                bad = next(tok for tok in e.tokens if not 0 <= int(tok) < vocab)
+                raise StepError(f"request {e.request!r}: token id {bad} is outside the vocabulary of {vocab}")
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {e.request!r}: wanted place {w} is outside its {n} tokens")
