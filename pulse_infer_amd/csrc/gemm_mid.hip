@@ -129,8 +129,8 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
         const int64_t at = static_cast<int64_t>(placed(min(c, chunks - 1))) * KC;
 #pragma unroll
         for (int pair = 0; pair < PAIRS; ++pair) {
-            w[2 * pair] = *reinterpret_cast<const bf16x8*>(w0 + at + pair * 64);
-            w[2 * pair + 1] = *reinterpret_cast<const bf16x8*>(w1 + at + pair * 64);
+            w[2 * pair] = __builtin_bit_cast(bf16x8, stream_load16(w0 + at + pair * 64));
+            w[2 * pair + 1] = __builtin_bit_cast(bf16x8, stream_load16(w1 + at + pair * 64));
         }
     };
     // One chunk (J = its number modulo RING, which names its register sets): X into its stage, loads for later chunks

@@ -333,7 +333,7 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
             const int pair_k = ((ks + u) & ~1) * 32;
 #pragma unroll
             for (int s = 0; s < SLABS; ++s)
-                wa[u][s] = *reinterpret_cast<const bf16x8*>(((u & 1) ? w1[s] : w0[s]) + pair_k);
+                wa[u][s] = __builtin_bit_cast(bf16x8, stream_load16(((u & 1) ? w1[s] : w0[s]) + pair_k));
             if (u % PACK == 0) {
                 if (NORMED) {
                     hraw[u / PACK][0] = hraw[u / PACK][1] = f32x4{0.f, 0.f, 0.f, 0.f};
