@@ -385,7 +385,8 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
         }
         return p;
     };
-    // Then every load of the block: K rows of the two tiles and V rows in the order {tile0: 4kg.., tile1: 4kg..}.
+    // Then every load of the block (nontemporal: a step reads a request's keys and values once): K rows of the two
+    // tiles and V rows in the order {tile0: 4kg.., tile1: 4kg..}.
     // Nothing is done to the values here.  A page that the table does not hold (-1, or beyond its width) reads
     // page 0: those keys are masked.
     auto load_block = [&](int b, const BlockPages& pages, BlockRegs& x) {
@@ -402,12 +403,12 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
 #pragma unroll
             for (int ch = 0; ch < NCHUNK; ++ch) {
                 const int off = ch * 32 + kg * 8;
-                x.k[t][ch] = off < D ? *reinterpret_cast<const u32x4*>(krow + off) : u32x4{0u, 0u, 0u, 0u};
+                x.k[t][ch] = off < D ? __builtin_bit_cast(u32x4, stream_load16(krow + off)) : u32x4{0u, 0u, 0u, 0u};
             }
             const bf16_t* vrow = a.vc + pg * D * a.page_size + slot0 + 4 * kg + static_cast<int64_t>(r) * a.page_size;
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt)
-                x.v[t][dt] = *reinterpret_cast<const u32x2*>(vrow + static_cast<int64_t>(dt) * 16 * a.page_size);
+                x.v[t][dt] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(vrow + static_cast<int64_t>(dt) * 16 * a.page_size));
         }
     };
 
