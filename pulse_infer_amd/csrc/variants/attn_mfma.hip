@@ -1182,21 +1182,23 @@ __global__ __launch_bounds__(PR_THREADS) void attn_prefill_reduce_kernel(const f
 #endif  // PULSE_WIDE
 
 // out[row, head, :] = sum_z w_z o_z / sum_z w_z l_z with w_z = exp2(m_z - max m), over the splits that hold keys of
-// the row.  One workgroup per (row, head); the splits' (m, l) pairs go through LDS, and the partial outputs of the
-// first splits are asked for before anything waits, so that the kernel is little more than two trips to memory.
+// the row.  One workgroup per (row, `hpw` heads): its groups of threads are dealt out over the heads, a head's groups
+// over the splits (with few splits a workgroup would otherwise be mostly idle, and the launch eight times as wide).
+// The splits' (m, l) pairs go through LDS, and the partial outputs of the first splits are asked for before anything
+// waits, so that the kernel is little more than two trips to memory.
 constexpr int MAX_SPLITS = 1024;
 
 constexpr int REDUCE_THREADS = 256;
 constexpr int REDUCE_QUADS = D / 4;                              // float4 pieces of a head
-constexpr int REDUCE_GROUPS = REDUCE_THREADS / REDUCE_QUADS;     // groups of threads that share the splits out
+constexpr int REDUCE_GROUPS = REDUCE_THREADS / REDUCE_QUADS;     // groups of threads that share heads and splits out
 
 __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const float* __restrict__ part_o,
                                                                          const float* __restrict__ part_ml,
                                                                          const int* __restrict__ positions,
                                                                          const int* __restrict__ items, int per,
                                                                          bf16_t* __restrict__ out, int64_t o_stride, int nq,
-                                                                         int n_splits, int split_size) {
-    __shared__ float s_w[MAX_SPLITS];
+                                                                         int n_splits, int split_size, int hpw_log2) {
+    __shared__ float s_w[MAX_SPLITS];      // hpw * n_splits <= MAX_SPLITS (hpw > 1 only with few splits)
     __shared__ float s_l[MAX_SPLITS];
     __shared__ f32x4 s_acc[REDUCE_GROUPS][REDUCE_QUADS];
     // only the rows of this launch's items have partial results
@@ -1204,52 +1206,64 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
     const int tok = blockIdx.x % per;
     if (tok >= items[4 * item + 1]) return;
     const int64_t row = items[4 * item] + tok;
-    const int head = blockIdx.y;
+    const int hpw = 1 << hpw_log2;            // heads of this workgroup
+    const int head0 = blockIdx.y * hpw;
     const int valid = min(n_splits, positions[row] / split_size + 1);
-    const int64_t base = (row * nq + head) * n_splits;
-    for (int z = threadIdx.x; z < valid; z += REDUCE_THREADS) {
-        s_w[z] = part_ml[2 * (base + z)];
-        s_l[z] = part_ml[2 * (base + z) + 1];
+    for (int i = threadIdx.x; i < hpw * valid; i += REDUCE_THREADS) {
+        const int hs = i & (hpw - 1), z = i >> hpw_log2;
+        if (head0 + hs < nq) {
+            const int64_t at = (row * nq + head0 + hs) * n_splits + z;
+            s_w[hs * n_splits + z] = part_ml[2 * at];
+            s_l[hs * n_splits + z] = part_ml[2 * at + 1];
+        }
     }
-    // group `grp` of threads takes splits grp, grp + REDUCE_GROUPS, ..; a thread four channels of them.  The partial
-    // outputs are asked for before the weights are known, eight splits of a group at a time.
+    // group `grp` of threads takes head grp % hpw and of its splits sg = grp / hpw, sg + gph, ..; a thread four
+    // channels of them.
+    // The partial outputs are asked for before the weights are known, eight splits of a group at a time.
+    const int gph = REDUCE_GROUPS >> hpw_log2;   // groups a head
     const int quad = threadIdx.x % REDUCE_QUADS;
     const int grp = threadIdx.x / REDUCE_QUADS;
-    const bool works = grp < REDUCE_GROUPS;
+    const int hs = grp & (hpw - 1);
+    const int sg = grp >> hpw_log2;
+    const int head = head0 + hs;
+    const bool works = sg < gph && head < nq;
+    const int64_t base = (row * nq + (works ? head : head0)) * n_splits;
+    const float* my_w = s_w + (works ? hs : 0) * n_splits;
+    const float* my_l = s_l + (works ? hs : 0) * n_splits;
     constexpr int AHEAD = 8;
     f32x4 first[AHEAD];
 #pragma unroll
     for (int i = 0; i < AHEAD; ++i) {
-        const int z = grp + i * REDUCE_GROUPS;
+        const int z = sg + i * gph;
         // a split without keys of the row left nothing behind: what is read there is not used (z < valid below)
         first[i] = (works && z < n_splits) ? *reinterpret_cast<const f32x4*>(part_o + (base + z) * D + 4 * quad)
                                            : f32x4{0.f, 0.f, 0.f, 0.f};
     }
     __syncthreads();
-    float mm = -INFINITY;
-    for (int z = 0; z < valid; ++z) mm = fmaxf(mm, s_w[z]);
-    float ll = 0.f;
-    for (int z = 0; z < valid; ++z) ll += (s_w[z] == -INFINITY ? 0.f : exp2f(s_w[z] - mm)) * s_l[z];
-    const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+    float inv = 0.f;
     if (works) {
+        float mm = -INFINITY;
+        for (int z = 0; z < valid; ++z) mm = fmaxf(mm, my_w[z]);
+        float ll = 0.f;
+        for (int z = 0; z < valid; ++z) ll += (my_w[z] == -INFINITY ? 0.f : exp2f(my_w[z] - mm)) * my_l[z];
+        inv = ll > 0.f ? 1.0f / ll : 0.f;
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < AHEAD; ++i) {
-            const int z = grp + i * REDUCE_GROUPS;
-            if (z < valid) acc += first[i] * (s_w[z] == -INFINITY ? 0.f : exp2f(s_w[z] - mm));
+            const int z = sg + i * gph;
+            if (z < valid) acc += first[i] * (my_w[z] == -INFINITY ? 0.f : exp2f(my_w[z] - mm));
         }
-        for (int z = grp + AHEAD * REDUCE_GROUPS; z < valid; z += REDUCE_GROUPS) {
-            const float wz = s_w[z] == -INFINITY ? 0.f : exp2f(s_w[z] - mm);
+        for (int z = sg + AHEAD * gph; z < valid; z += gph) {
+            const float wz = my_w[z] == -INFINITY ? 0.f : exp2f(my_w[z] - mm);
             acc += *reinterpret_cast<const f32x4*>(part_o + (base + z) * D + 4 * quad) * wz;
         }
         s_acc[grp][quad] = acc;
     }
     __syncthreads();
-    // the groups' sums in a fixed order
-    if (threadIdx.x < REDUCE_QUADS) {
-        f32x4 v = s_acc[0][quad];
-#pragma unroll
-        for (int gi = 1; gi < REDUCE_GROUPS; ++gi) v += s_acc[gi][quad];
+    // a head's groups' sums in a fixed order
+    if (works && sg == 0) {
+        f32x4 v = s_acc[grp][quad];
+        for (int gi = 1; gi < gph; ++gi) v += s_acc[grp + gi * hpw][quad];
         bf16_t* dst = out + row * o_stride + static_cast<int64_t>(head) * D + 4 * quad;
 #pragma unroll
         for (int e = 0; e < 4; ++e) dst[e] = f32_to_bf16(v[e] * inv);
@@ -1321,9 +1335,11 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
     }
     PULSE_LAUNCH_CHECK("attn_mfma");
     if (n_splits > 1) {
-        const int per = 16 / gp;
-        hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(n_items * per, nq), dim3(REDUCE_THREADS), 0, stream, part_o, part_ml,
-                           positions, items, per, a.out, o_stride, nq, n_splits, split_size);
+        const int per = prep ? 1 : 16 / gp;   // tokens an item may hold: decoded tokens come one an item
+        int hpw = 1, hpw_log2 = 0;            // heads a workgroup: as many as leave every split of a head a group of threads
+        while (hpw * 2 * n_splits <= REDUCE_GROUPS && hpw * 2 <= nq) { hpw *= 2; ++hpw_log2; }
+        hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(n_items * per, (nq + hpw - 1) / hpw), dim3(REDUCE_THREADS), 0, stream,
+                           part_o, part_ml, positions, items, per, a.out, o_stride, nq, n_splits, split_size, hpw_log2);
         PULSE_LAUNCH_CHECK("attn_mfma_reduce");
     }
     return 0;

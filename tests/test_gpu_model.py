@@ -377,9 +377,9 @@ MANY = dict(
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("requests", [24, 70, 200])
+@pytest.mark.parametrize("requests", [14, 24, 70, 200])
 def test_many_requests_decode_together(tmp_path, requests, dtype):
-    """Steps of 24, 70 and 200 decoded tokens (the products for 17 to 192 rows and the library's beyond, attention
+    """Steps of 14, 24, 70 and 200 decoded tokens (the products for 13 to 192 rows and the library's beyond, attention
     over many short contexts of different lengths): every request's logits are those of the plain implementation
     for its own sequence, whatever stands beside it."""
     from plain.qwen3_plain import PlainQwen3
