@@ -51,7 +51,7 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--output-tokens", type=int, default=256, help="serving: tokens generated per request")
     p.add_argument("--chunk", type=int, default=512, help="serving: longest prompt portion in a step")
     p.add_argument("--token-budget", type=int, default=None,
-                   help="serving: most tokens a step computes (default: a portion beside one token of every request)")
+                   help="serving: most tokens a step computes (default: four portions)")
     p.add_argument("--temperature", type=float, default=0.7, help="serving: sampling temperature")
     p.add_argument("--prefill-tokens", type=int, default=2048)
     p.add_argument("--page-size", type=int, default=16)
@@ -97,7 +97,7 @@ def serving(args, cfg, model, full_layers: int) -> int:
     pages = args.requests * ((per_request + args.page_size - 1) // args.page_size)
     engine = ContinuousBatchEngine(model, max_batch_size=args.requests, chunk_size=args.chunk, page_size=args.page_size,
                                    num_pages=pages, max_sequences=args.requests,
-                                   max_num_batched_tokens=args.token_budget or args.chunk + args.requests, seed=args.seed)
+                                   max_num_batched_tokens=args.token_budget or 4 * args.chunk, seed=args.seed)
     for i, n in enumerate(lengths):
         prompt = torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
         engine.add_request(prompt, args.output_tokens,
