@@ -116,7 +116,8 @@ def serving(args, cfg, model, full_layers: int) -> int:
         "config": {"model": f"Qwen3-{args.model.upper()} shape, random weights", "global_batch": args.requests,
                    "seq_len": hi + args.output_tokens, "parallelism": "single GPU", "layers": args.layers,
                    "layers_full_model": full_layers, "requests": args.requests, "prompt_min": lo, "prompt_max": hi,
-                   "output_tokens": args.output_tokens, "chunk": args.chunk, "temperature": args.temperature,
+                   "output_tokens": args.output_tokens, "chunk": args.chunk, "token_budget": engine.scheduler.max_num_batched_tokens,
+                   "temperature": args.temperature,
                    "prompt_tokens": sum(lengths), "preemptions": stats.num_preemptions},
         "seconds": round(seconds, 3), "tokens_computed": stats.tokens_computed}))
     return 0
