@@ -232,7 +232,7 @@ __global__ __launch_bounds__(64) void qk_rope_kv_vec_kernel(bf16_t* __restrict__
     if (!on) oa = 0, ob = 4;
 
     // every load before anything waits for one
-    float e[8], wv[8], cs[4], sn[4], vv[8];
+    float e[8], wv[8], cs[4], sn[4];
     if (PAIRING == 0) {
         load8<bf16_t>(x + oa, e);
     } else {
@@ -260,17 +260,15 @@ __global__ __launch_bounds__(64) void qk_rope_kv_vec_kernel(bf16_t* __restrict__
     if (is_k) {
         pos = positions[t];
         entry = token_entry[t];
-        load8<bf16_t>(row + static_cast<int64_t>(a.nq + a.nkv + g) * d + c * 8, vv);
     }
     bool store_kv = false;
-    int64_t kbase = 0, vbase = 0;
+    int64_t kbase = 0;
     if (is_k) {
         const int page = block_table[static_cast<int64_t>(entry) * a.bt_width + pos / a.page_size];
         const int slot = pos % a.page_size;
         store_kv = page >= 0 && page < a.num_pages;
         const int64_t pg = static_cast<int64_t>(page) * a.nkv + g;
         kbase = (pg * a.page_size + slot) * d;
-        vbase = pg * d * a.page_size + slot;
     }
 
     if (!on) {
@@ -307,9 +305,39 @@ __global__ __launch_bounds__(64) void qk_rope_kv_vec_kernel(bf16_t* __restrict__
     } else if (store_kv) {
         *reinterpret_cast<vu2*>(kcache + kbase + oa) = lo;
         *reinterpret_cast<vu2*>(kcache + kbase + ob) = hi;
+    }
+}
+
+// The values of the step's tokens into their pages, whose layout has the slots of a page side by side for every
+// channel: a workgroup takes 16 consecutive tokens of one kv head, a thread one token (tid % 16) and eight channels
+// at a time, so that the 16 lanes of a store write the 16 two-byte slots of one channel, 32 contiguous bytes when
+// the tokens fill a page in order (a thread finds its own token's page and slot: any other arrangement is written
+// just as correctly, only in smaller pieces).  Written from the kernel above, a token at a time, the same bytes
+// took twice as long as everything else that kernel does.
+constexpr int VW_TOKENS = 16;
+constexpr int VW_THREADS = 256;
+
+__global__ __launch_bounds__(VW_THREADS) void v_page_write_kernel(const bf16_t* __restrict__ qkv, bf16_t* __restrict__ vcache,
+                                                                  const int* __restrict__ positions,
+                                                                  const int* __restrict__ token_entry,
+                                                                  const int* __restrict__ block_table, QkRopeArgs a,
+                                                                  int tokens) {
+    const int t = blockIdx.x * VW_TOKENS + threadIdx.x % VW_TOKENS;
+    const int cg = threadIdx.x / VW_TOKENS;
+    const int g = blockIdx.y;
+    if (t >= tokens) return;
+    const int pos = positions[t];
+    const int page = block_table[static_cast<int64_t>(token_entry[t]) * a.bt_width + pos / a.page_size];
+    if (page < 0 || page >= a.num_pages) return;
+    const int slot = pos % a.page_size;
+    const bf16_t* src = qkv + static_cast<int64_t>(t) * a.row_stride + static_cast<int64_t>(a.nq + a.nkv + g) * a.d;
+    bf16_t* dst = vcache + (static_cast<int64_t>(page) * a.nkv + g) * a.d * a.page_size + slot;
+    for (int c0 = cg * 8; c0 < a.d; c0 += 8 * (VW_THREADS / VW_TOKENS)) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(src + c0);
+        const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
         for (int i = 0; i < 8; ++i)
-            vcache[vbase + static_cast<int64_t>(c * 8 + i) * a.page_size] = f32_to_bf16(vv[i]);
+            dst[static_cast<int64_t>(c0 + i) * a.page_size] = static_cast<bf16_t>(words[i / 2] >> (16 * (i % 2)));
     }
 }
 
@@ -376,6 +404,12 @@ extern "C" int pulse_qk_rope_kv(void* qkv, int x_dtype, int64_t row_stride, cons
                                   static_cast<const TW*>(k_w), cos_t, sin_t, static_cast<bf16_t*>(kcache),
                                   static_cast<bf16_t*>(vcache), positions, token_entry, block_table, a));
         PULSE_LAUNCH_CHECK("qk_rope_kv");
+        if (write_kv) {
+            hipLaunchKernelGGL(v_page_write_kernel, dim3((tokens + VW_TOKENS - 1) / VW_TOKENS, nkv), dim3(VW_THREADS), 0, stream,
+                               static_cast<const bf16_t*>(qkv), static_cast<bf16_t*>(vcache), positions, token_entry,
+                               block_table, a, tokens);
+            PULSE_LAUNCH_CHECK("v_page_write");
+        }
         return 0;
     }
     const dim3 grid(tokens, heads);
