@@ -75,8 +75,9 @@ def choose_splits(num_items: int, nkv: int, group: int, max_context: int) -> Tup
     heads, contexts of 4,096: one request is fastest in 32 splits, two in 16, four in 8, eight in 4 (256 workgroups
     each time; 6 splits at batch 8, which leave half the units two workgroups, are 15% slower); 20 to 32 requests in
     one (160 to 256 workgroups; two splits are 10 to 25% slower), 40 in 4 and 48 in 2 (a multiple of the units
-    again), 64 in one.  Walks of 2,048 keys and more stream better with two workgroups a unit (16 requests at 4,096:
-    4 splits 61 us, 2 splits 65), so a choice that gives every unit one such walk is cut in two once more."""
+    again), 64 in one.  Walks of 4,096 keys and more stream better with two workgroups a unit (16 requests at 8,192:
+    4 splits 95.9 us, 2 splits 97.6; at 4,096, walks of 2,048 keys, 2 splits 51.9 us and 4 splits 53.8), so a choice
+    that gives every unit one such walk is cut in two once more."""
     groups = num_items * nkv * ((group + 15) // 16)
     whole = (max_context + BLOCK_KEYS - 1) // BLOCK_KEYS * BLOCK_KEYS
     if groups <= 0 or max_context <= 0:
@@ -95,7 +96,7 @@ def choose_splits(num_items: int, nkv: int, group: int, max_context: int) -> Tup
         if best is None or cost < best[0]:
             best = (cost, n)
     n = best[1]
-    if n > 1 and split_size(n) >= 2048 and groups * n * 2 in (CHIP_WORKGROUPS, 2 * CHIP_WORKGROUPS):
+    if n > 1 and split_size(n) >= 4096 and groups * n * 2 in (CHIP_WORKGROUPS, 2 * CHIP_WORKGROUPS):
         n *= 2
     if n == 1:
         return whole, 1
