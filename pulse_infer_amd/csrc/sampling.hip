@@ -21,8 +21,11 @@
 // uniform number u comes from the host's per-request counter-based generator,
 // so a row's result does not depend on the other rows.
 #include "common.h"
+#include "no_alloc.h"
 
 #include <math.h>
+
+#include <mutex>
 
 namespace {
 
@@ -498,6 +501,54 @@ extern "C" int pulse_argmax(const float* logits, int rows, int vocab, int64_t ro
     PULSE_LAUNCH_CHECK("argmax_chunks");
     hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(PULSE_WAVE), 0, stream, part_val, part_idx, chunks, out);
     PULSE_LAUNCH_CHECK("argmax_merge");
+    return 0;
+}
+
+// The same without a workspace argument: the chunk winners go through an array in the library's device image.
+// In host code the array's name is only a stand-in for the symbol; its address on a device comes from
+// hipGetSymbolAddress, once per device, and that pointer is what the kernels get.
+static __device__ __align__(256) unsigned char argmax_static_scratch[PULSE_ARGMAX_STATIC_ENTRIES * 8];
+
+namespace {
+constexpr int STATIC_MAX_DEVICES = 64;
+void* g_static_scratch[STATIC_MAX_DEVICES] = {};
+std::mutex g_static_lock;
+}  // namespace
+
+extern "C" int pulse_argmax_static(const float* logits, int rows, int vocab, int64_t row_stride, int* out,
+                                   hipStream_t stream) {
+    PULSE_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "argmax_static: bad sizes rows=%d V=%d", rows, vocab);
+    PULSE_REQUIRE(rows < 65536, "argmax_static: at most 65535 rows");
+    PULSE_REQUIRE(logits && out, "argmax_static: null pointer");
+    const int chunks = pulse_argmax_chunks(vocab);
+    PULSE_REQUIRE(static_cast<int64_t>(rows) * chunks <= PULSE_ARGMAX_STATIC_ENTRIES,
+                  "argmax_static: %d rows x %d chunks of the vocabulary exceed the %d entries of the built-in scratch "
+                  "array; use pulse_argmax with a workspace", rows, chunks, PULSE_ARGMAX_STATIC_ENTRIES);
+    if (rows == 0) return 0;
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    PULSE_REQUIRE(err == hipSuccess, "argmax_static: hipGetDevice: %s", hipGetErrorString(err));
+    PULSE_REQUIRE(device >= 0 && device < STATIC_MAX_DEVICES, "argmax_static: device %d is beyond the %d this entry "
+                  "point keeps an address for", device, STATIC_MAX_DEVICES);
+    void* base = nullptr;
+    {
+        std::lock_guard<std::mutex> hold(g_static_lock);
+        if (!g_static_scratch[device]) {   // each GPU holds its own copy of the array at its own address
+            void* found = nullptr;
+            err = hipGetSymbolAddress(&found, HIP_SYMBOL(argmax_static_scratch));
+            PULSE_REQUIRE(err == hipSuccess && found, "argmax_static: hipGetSymbolAddress on device %d: %s", device,
+                          hipGetErrorString(err));
+            g_static_scratch[device] = found;
+        }
+        base = g_static_scratch[device];
+    }
+    float* part_val = static_cast<float*>(base);
+    int* part_idx = reinterpret_cast<int*>(static_cast<unsigned char*>(base) + PULSE_ARGMAX_STATIC_ENTRIES * 4);
+    hipLaunchKernelGGL(argmax_chunks_kernel, dim3(chunks, rows), dim3(ARGMAX_THREADS), 0, stream, logits, vocab,
+                       row_stride, 2048, part_val, part_idx);
+    PULSE_LAUNCH_CHECK("argmax_static chunks");
+    hipLaunchKernelGGL(argmax_merge_kernel, dim3(rows), dim3(PULSE_WAVE), 0, stream, part_val, part_idx, chunks, out);
+    PULSE_LAUNCH_CHECK("argmax_static merge");
     return 0;
 }
 
