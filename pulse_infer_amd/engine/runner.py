@@ -111,6 +111,8 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and model.options.get("decode_graph", True)
         self._graphs: dict = {}
         self._graph_seen: dict = {}
+        self.graph_records = 0      # recordings made so far
+        self.graph_replays = 0      # steps that ran as a replay of a recording
         self.max_positions = model.spec.max_positions
         self.steps = 0
         self.tokens_run = 0
@@ -257,6 +259,7 @@ class ModelRunner:
         if rec is None:
             rec = self._capture(key, entries, metas, want_rows)
             self._graphs[key] = rec
+            self.graph_records += 1
             if len(self._graphs) > self.GRAPH_LIMIT:   # oldest recording out: contexts move on to higher buckets
                 self._graphs.pop(next(iter(self._graphs)))
         rec.wait()
@@ -264,6 +267,7 @@ class ModelRunner:
         rec.dev.copy_(rec.host, non_blocking=True)
         rec.graph.replay()
         rec.mark()
+        self.graph_replays += 1
         return rec.logits.clone()
 
     def _capture(self, key, entries, metas, want_rows) -> "_Captured":

@@ -129,42 +129,49 @@ class PlainQwen3:
         first = c.get("max_window_layers") or 0
         return c.get("sliding_window") if layer >= first else None
 
-    def layer(self, h: torch.Tensor, index: int, positions: List[int]) -> torch.Tensor:
+    def layer(self, h: torch.Tensor, index: int, positions: List[int],
+              rows: Optional[List[int]] = None) -> torch.Tensor:
+        """One layer on the whole sequence.  ``rows``: the layer's output is wanted for these places only; keys and
+        values are still those of every position, queries and everything after them only of the rows."""
         c, w = self.c, self.w
         p = f"model.layers.{index}."
         nq, nkv = c["num_attention_heads"], c["num_key_value_heads"]
         d = c.get("head_dim", c["hidden_size"] // nq)
         eps = c["rms_norm_eps"]
         t = h.shape[0]
+        sel = list(range(t)) if rows is None else list(rows)
+        sel_pos = [positions[i] for i in sel]
         # pre-norm stands before the projections (model.cpp:779)
         a = rms_norm(h, w[p + "input_layernorm.weight"], eps)
-        q = linear(a, w[p + "self_attn.q_proj.weight"]).view(t, nq, d)     # model.cpp:784-813
+        q = linear(a[sel], w[p + "self_attn.q_proj.weight"]).view(len(sel), nq, d)     # model.cpp:784-813
         k = linear(a, w[p + "self_attn.k_proj.weight"]).view(t, nkv, d)
         v = linear(a, w[p + "self_attn.v_proj.weight"]).view(t, nkv, d)
         # per-head norm over d, after projection and before rotation; v untouched (model.cpp:815-838)
         q = rms_norm(q, w[p + "self_attn.q_norm.weight"], eps)
         k = rms_norm(k, w[p + "self_attn.k_norm.weight"], eps)
-        q = rope(q, positions, c["rope_theta"], d, self.pairing)
+        q = rope(q, sel_pos, c["rope_theta"], d, self.pairing)
         k = rope(k, positions, c["rope_theta"], d, self.pairing)
         # keys are indexed by their place in the sequence; positions only enter through the rotation
-        o = causal_attention(q, k, v, 1.0 / math.sqrt(d), self.layer_window(index))  # scale: paged_attention.cu:108
-        h = h + linear(o.reshape(t, nq * d), w[p + "self_attn.o_proj.weight"])               # model.cpp:875-886
+        o = causal_attention(q, k, v, 1.0 / math.sqrt(d), self.layer_window(index), sel)  # scale: paged_attention.cu:108
+        h = h[sel] + linear(o.reshape(len(sel), nq * d), w[p + "self_attn.o_proj.weight"])   # model.cpp:875-886
         m = rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)                       # model.cpp:888
         h = h + gated_mlp(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                           w[p + "mlp.down_proj.weight"])                                    # model.cpp:893-923
         return h
 
-    def hidden(self, ids: List[int]) -> torch.Tensor:
+    def hidden(self, ids: List[int], rows: Optional[List[int]] = None) -> torch.Tensor:
         positions = list(range(len(ids)))
         h = embedding(self.w["model.embed_tokens.weight"], ids)
-        for i in range(self.c["num_hidden_layers"]):
-            h = self.layer(h, i, positions)
+        last = self.c["num_hidden_layers"] - 1
+        for i in range(last + 1):
+            h = self.layer(h, i, positions, rows if i == last else None)
         return h
 
-    def logits(self, ids: List[int]) -> torch.Tensor:
-        """[T, V] logits of every position (model.cpp:1305-1371: final norm, then the head;
-        lm_head.weight if present, else the embedding table when tied)."""
-        h = rms_norm(self.hidden(ids), self.w["model.norm.weight"], self.c["rms_norm_eps"])
+    def logits(self, ids: List[int], rows: Optional[List[int]] = None) -> torch.Tensor:
+        """[T, V] logits of every position, or [len(rows), V] of the places in ``rows`` (the last layer then computes
+        queries for those only)  (model.cpp:1305-1371: final norm, then the head; lm_head.weight if present, else the
+        embedding table when tied)."""
+        h = rms_norm(self.hidden(ids, rows), self.w["model.norm.weight"], self.c["rms_norm_eps"])
         head = self.w.get("lm_head.weight")
         if head is None:
             if not self.c.get("tie_word_embeddings", False):

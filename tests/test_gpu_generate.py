@@ -192,10 +192,53 @@ def test_captured_decode_steps_replay_like_eager_ones(gpu, model_folders, plain_
         feed([("c", 9)])
         for _ in range(12):
             feed([("b", 1), ("a", 1)])                   # the first recording again, entries in another order
-        assert runner.use_graphs == (which == 0) and (len(runner._graphs) == 2) == (which == 0)
+        assert runner.use_graphs == (which == 0) and runner.graph_records == (2 if which == 0 else 0)
     for k in ids:
         want = plain_logits("B", ids[k])
         for (pos_g, row_g), (pos_e, row_e) in zip(got[0][k], got[1][k]):
             assert pos_g == pos_e
             close(row_g[None], want[pos_g][None], "bfloat16", f"captured {k}@{pos_g}")
             close(row_g[None], row_e[None], "bfloat16", f"captured against eager {k}@{pos_g}", SPLIT_TOL)
+
+
+def test_recorded_steps_while_a_window_gives_pages_back_and_after_eviction(gpu, model_folders, plain_logits):
+    """Tiny W (windows of 24 keys on some layers, pages of 16): two requests decode far past window + page while
+    their steps are replayed, so the windowed group gives pages back under a live recording and its table rows hold
+    -1 there.  Only one recording is kept, and the batch alternates between two and one request, so every change
+    evicts the recording and the next step of that shape records again.  Against the plain implementation and the
+    eager steps."""
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from test_gpu_model import SPLIT_TOL, close
+
+    cfg, _ = TINY["W"]
+    _, model = load_model(model_folders["W"], mode="bfloat16")
+    ids = {"a": token_ids(cfg["vocab_size"], 120, seed=71), "b": token_ids(cfg["vocab_size"], 100, seed=72)}
+    start = {"a": 20, "b": 9}
+    outs = []
+    for graphs in (True, False):
+        runner = ModelRunner(model, page_size=16, num_pages=24, max_requests=2, use_graphs=graphs)
+        runner.GRAPH_AFTER_STEPS, runner.GRAPH_LIMIT = 1, 1
+        fed, got = dict(start), {k: [] for k in ids}
+        for k, n in start.items():
+            runner.add_request(k)
+            runner.reserve(k, len(ids[k]))
+            runner.step([StepEntry(k, ids[k][:n], [])])
+        windowed = next(g for g in runner.cache.groups if g.spec.window is not None)
+        for s in range(80):
+            who = ["a", "b"] if (s // 5) % 2 == 0 else ["a"]          # five steps of two, five of one, ...
+            logits = runner.step([StepEntry(k, [ids[k][fed[k]]], [0]) for k in who])
+            for row, k in enumerate(who):
+                got[k].append(logits[row])
+                fed[k] += 1
+        assert -1 in windowed.tables["a"] and -1 in windowed.tables["b"]          # pages were given back on the way
+        if graphs:
+            assert runner.graph_replays == 80 and runner.graph_records == 16      # every change of batch records anew
+        outs.append({k: torch.stack(v) for k, v in got.items()})
+        runner.cache.reset()
+        runner.cache.check()
+    for k in ids:
+        n = outs[0][k].shape[0]
+        want = plain_logits("W", ids[k])[start[k]:start[k] + n]
+        close(outs[0][k], want, "bfloat16", f"recorded under a window, request {k}")
+        close(outs[0][k], outs[1][k], "bfloat16", f"recorded against eager under a window, request {k}", SPLIT_TOL)

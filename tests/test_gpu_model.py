@@ -98,9 +98,9 @@ def test_whole_tail_and_portions(engines, plain_logits, name, page, dtype):
     close(first, want[:3], dtype, f"{name} first tokens")
 
 
-def mixed_trace(vocab, seed):
+def mixed_trace(vocab, seed, sizes=(2, 3, 5, 8, 13, 21)):
     """Six requests, at most four live, over a pool that holds 256 tokens: pages of finished requests are
-    used again by later ones.  Steps mix prompt portions of some with single tokens of others."""
+    used again by later ones.  Steps mix prompt portions of some (of the given sizes) with single tokens of others."""
     rng = np.random.RandomState(seed)
     lengths = {"a": 60, "b": 45, "c": 64, "d": 30, "e": 50, "f": 58}
     ids = {k: token_ids(vocab, n, seed=seed * 10 + i) for i, (k, n) in enumerate(lengths.items())}
@@ -120,7 +120,7 @@ def mixed_trace(vocab, seed):
             if fed[k] >= lengths[k] - 12:
                 n = 1                                                # its last tokens come one by one
             else:
-                n = int(min(left - 12, rng.choice([2, 3, 5, 8, 13, 21])))
+                n = int(min(left - 12, rng.choice(list(sizes))))
                 n = max(n, 1)
             entries.append({"id": k, "tokens": ids[k][fed[k]:fed[k] + n], "want": list(range(n))})
             fed[k] += n
@@ -132,17 +132,12 @@ def mixed_trace(vocab, seed):
     return ids, steps
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name,page", CASES)
-def test_mixed_batches_with_page_reuse(engines, plain_logits, name, page, dtype):
+def run_mixed(runner, steps):
+    """Drive the steps of ``mixed_trace`` through a runner: per request the logits of all its places, the pages it
+    ever held, and the most requests that were live at once."""
     from pulse_infer_amd.engine.runner import StepEntry
 
-    cfg = TINY[name][0]
-    ids, steps = mixed_trace(cfg["vocab_size"], seed=5)
-    runner = engines(name, dtype, page)
-    got = {k: [] for k in ids}
-    pages_seen = {}
-    most_live = 0
+    got, pages_seen, most_live = {}, {}, 0
     for step in steps:
         entries = []
         for e in step["entries"]:
@@ -155,18 +150,32 @@ def test_mixed_batches_with_page_reuse(engines, plain_logits, name, page, dtype)
         logits = runner.step(entries)
         row = 0
         for e in step["entries"]:
-            got[e["id"]].append(logits[row:row + len(e["want"])])
+            got.setdefault(e["id"], []).append(logits[row:row + len(e["want"])])
             row += len(e["want"])
         for k in step["end"]:
             runner.free_request(k)
         runner.cache.check()
+    return {k: torch.cat(parts) for k, parts in got.items()}, pages_seen, most_live
+
+
+def pages_were_used_again(pages_seen):
+    names = list(pages_seen)
+    return any(pages_seen[a] & pages_seen[b] for i, a in enumerate(names) for b in names[i + 1:])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,page", CASES)
+def test_mixed_batches_with_page_reuse(engines, plain_logits, name, page, dtype):
+    cfg = TINY[name][0]
+    ids, steps = mixed_trace(cfg["vocab_size"], seed=5)
+    runner = engines(name, dtype, page)
+    got, pages_seen, most_live = run_mixed(runner, steps)
     assert most_live == 4 and any(len(s["entries"]) >= 3 for s in steps)
     assert any(len(e["tokens"]) > 1 for s in steps for e in s["entries"]) and \
         any(len(e["tokens"]) == 1 and len(s["entries"]) > 1 for s in steps for e in s["entries"])
-    names = list(ids)
-    assert any(pages_seen[a] & pages_seen[b] for i, a in enumerate(names) for b in names[i + 1:]), "no page was used again"
-    for k, parts in got.items():
-        close(torch.cat(parts), plain_logits(name, ids[k]), dtype, f"{name} mixed request {k}")
+    assert pages_were_used_again(pages_seen), "no page was used again"
+    for k, mine in got.items():
+        close(mine, plain_logits(name, ids[k]), dtype, f"{name} mixed request {k}")
 
 
 # The layer sizes of the benchmark's model (Qwen3-8B: 32 query heads over 8 kv heads of 128, hidden 4096, feed-forward
@@ -190,8 +199,8 @@ def layer_shape(tmp_path_factory):
     folder = str(tmp_path_factory.mktemp("layer_shape"))
     write_model_folder(Qwen3Config.from_dict(LAYER_SHAPE), folder, seed=41)
     ids = token_ids(LAYER_SHAPE["vocab_size"], 150, seed=42)
-    want = PlainQwen3.from_folder(folder).logits(ids)
-    return folder, ids, want
+    plain = PlainQwen3.from_folder(folder)
+    return folder, ids, plain.logits(ids), plain
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -199,7 +208,7 @@ def test_benchmark_layer_sizes(layer_shape, dtype):
     from pulse_infer_amd.engine.runner import ModelRunner
     from pulse_infer_amd.models.factory import load_model
 
-    folder, ids, want = layer_shape
+    folder, ids, want, _ = layer_shape
     _, model = load_model(folder, mode=dtype)
     runner = ModelRunner(model, page_size=16, num_pages=24, max_requests=4)
     whole = run_alone(runner, ids, [len(ids)])
@@ -211,7 +220,129 @@ def test_benchmark_layer_sizes(layer_shape, dtype):
     close(portions, want, dtype, "layer sizes, portions")
     close(portions, whole, dtype, "layer sizes, portions against whole", SPLIT_TOL)
     if dtype == "bfloat16":
-        assert len(runner._graphs) >= 1            # the single tokens ran as recorded steps
+        assert runner.graph_replays >= 1           # the single tokens ran as recorded steps
+    del runner, model
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_benchmark_layer_sizes_mixed_with_page_reuse(layer_shape, dtype):
+    """Up to four live requests at the benchmark model's layer sizes over a pool of 256 tokens: steps that hold a
+    portion of 16 tokens and more (the prompt-portion attention kernel) beside single decoded tokens (the split
+    kernel) and steps of 17 to 64 rows (the products for those row counts, the shares of o and down), which no
+    single request alone ever makes."""
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+
+    folder, _, _, plain = layer_shape
+    ids, steps = mixed_trace(LAYER_SHAPE["vocab_size"], seed=4, sizes=(2, 3, 16, 21, 34))
+    rows = [sum(len(e["tokens"]) for e in s["entries"]) for s in steps]
+    assert any(17 <= r <= 64 for r in rows) and any(13 <= r <= 16 for r in rows)
+    assert any(any(len(e["tokens"]) >= 16 for e in s["entries"]) and any(len(e["tokens"]) == 1 for e in s["entries"])
+               for s in steps), "no step holds a portion of 16 tokens beside a single token"
+    assert any(len(s["entries"]) == 4 and all(len(e["tokens"]) == 1 for e in s["entries"]) for s in steps)
+    _, model = load_model(folder, mode=dtype)
+    runner = ModelRunner(model, page_size=16, num_pages=16, max_requests=4)
+    got, pages_seen, most_live = run_mixed(runner, steps)
+    assert most_live == 4 and pages_were_used_again(pages_seen)
+    for k, mine in got.items():
+        close(mine, plain.logits(ids[k]), dtype, f"layer sizes, mixed request {k}")
+    del runner, model
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("batch", [8, 3])
+def test_benchmark_layer_sizes_recorded_decode_steps(layer_shape, batch):
+    """Recorded steps at the benchmark's attention shape (heads of 128 in groups of four, the decode kernel writing
+    keys and values from inside the graph): eight (and three) requests of unequal contexts, from 5 to more than a
+    thousand keys, so that some of the splits chosen for the context bucket are empty for the short ones; the longest
+    walks across a multiple of 1,024 on the way, which takes a new recording with a wider block table.  Every
+    replay against the eager step and the plain implementation."""
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+
+    folder, _, _, plain = layer_shape
+    lengths = [1018, 5, 700, 300, 1000, 64, 513, 17][:batch]
+    steps = 12
+    vocab = LAYER_SHAPE["vocab_size"]
+    ids = [token_ids(vocab, n + steps, seed=300 + i) for i, n in enumerate(lengths)]
+    _, model = load_model(folder, mode="bfloat16")
+    results = []
+    for graphs in (True, False):
+        runner = ModelRunner(model, page_size=16, num_pages=sum((n + steps + 15) // 16 for n in lengths) + 2,
+                             max_requests=batch, use_graphs=graphs)
+        runner.GRAPH_AFTER_STEPS = 1                     # record at once: every single-token step here is a replay
+        for r, n in enumerate(lengths):
+            runner.add_request(r)
+            runner.reserve(r, n + steps)
+            runner.step([StepEntry(r, ids[r][:n], [])])
+        got = [runner.step([StepEntry(r, [ids[r][n + s]], [0]) for r, n in enumerate(lengths)]) for s in range(steps)]
+        results.append(torch.stack(got))                 # [steps, batch, vocab]
+        assert runner.graph_replays == (steps if graphs else 0)
+        assert runner.graph_records == (2 if graphs else 0)      # contexts up to 1,024, then up to 2,048
+        for r in range(batch):
+            runner.free_request(r)
+        runner.cache.check()
+        del runner
+    recorded, eager = results
+    for r, n in enumerate(lengths):
+        want = plain.logits(ids[r], rows=list(range(n, n + steps)))
+        close(recorded[:, r], want, "bfloat16", f"recorded, request {r} ({n} keys)")
+        close(eager[:, r], want, "bfloat16", f"eager, request {r} ({n} keys)")
+        close(recorded[:, r], eager[:, r], "bfloat16", f"recorded against eager, request {r}", SPLIT_TOL)
+    del model
+    torch.cuda.empty_cache()
+
+
+FAR_PAGES = dict(
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=300, hidden_size=512, intermediate_size=768,
+    num_hidden_layers=1, num_attention_heads=16, num_key_value_heads=8, head_dim=128, max_position_embeddings=512,
+    rms_norm_eps=1e-6, rope_theta=1e4, tie_word_embeddings=False, torch_dtype="bfloat16", attention_bias=False,
+    use_sliding_window=False, hidden_act="silu")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_beyond_two_to_the_31_elements(tmp_path, dtype):
+    """A pool of more than 131,072 pages of 8 heads x 16 slots x 128 channels: the low pages are held by idle
+    requests, so that every page of the tested request starts past element 2^31 of the key and value arrays, where
+    an offset computed in 32 bits would wrap (the reference computes them in 64 bits,
+    src/ops/kernels/cuda/paged_attention.cu:96-98).  Whole, the last 32 tokens one by one, and portions of 64 tokens
+    and more, against the plain implementation."""
+    from plain.qwen3_plain import PlainQwen3
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.weights import write_model_folder
+
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    folder = write_model_folder(Qwen3Config.from_dict(FAR_PAGES), str(tmp_path / "m"), seed=61)
+    ids = token_ids(FAR_PAGES["vocab_size"], 230, seed=62)
+    want = PlainQwen3.from_folder(folder).logits(ids)
+    page_elems = 8 * 16 * 128
+    low = (1 << 31) // page_elems                          # pages that start below element 2^31
+    _, model = load_model(folder, mode=dtype)
+    runner = ModelRunner(model, page_size=16, num_pages=low + 24, max_requests=4)
+    for half in ("idle0", "idle1"):                        # they hold every low page and are never stepped
+        runner.add_request(half)
+        runner.reserve(half, low // 2 * 16)
+    assert runner.cache.groups[0].pool.num_free == 24
+
+    def far(rid="r"):
+        table = runner.cache.table(0, rid)
+        assert table and min(table) >= low and min(table) * page_elems >= 1 << 31
+    from pulse_infer_amd.engine.runner import StepEntry
+    for cuts in ([230], [198] + [1] * 32, [100, 64, 66]):
+        runner.add_request("r")
+        outs, p = [], 0
+        for n in cuts:
+            runner.reserve("r", p + n)
+            far()
+            outs.append(runner.step([StepEntry("r", ids[p:p + n], list(range(n)))]))
+            p += n
+        runner.free_request("r")
+        close(torch.cat(outs), want, dtype, f"far pages, cuts {cuts[:3]}")
+    runner.cache.check()
     del runner, model
     torch.cuda.empty_cache()
 

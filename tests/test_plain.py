@@ -207,3 +207,13 @@ def test_greedy_takes_the_lowest_index_among_equals(plain_models):
     out = a.greedy(ids, 3)
     assert len(out) == 3 and out[0] == int(torch.argmax(a.logits(ids)[-1]))
     assert int(torch.argmax(torch.tensor([1.0, 3.0, 3.0]))) == 1
+
+
+def test_logits_of_chosen_rows_are_those_of_the_whole(plain_models):
+    """``logits(ids, rows)`` computes the last layer's queries for the rows only; nothing else may change, with and
+    without windows."""
+    for name in ("B", "W"):
+        model = plain_models[name]
+        ids = token_ids(model.c["vocab_size"], 70, seed=5)
+        rows = [0, 69, 31, 32]
+        assert torch.allclose(model.logits(ids, rows), model.logits(ids)[rows], rtol=0, atol=1e-12)
