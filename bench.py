@@ -6,15 +6,24 @@
 A "step" is one decode step of the whole batch: the step function on one token
 per request, the argmax kernel, and the tokens' way back to the host and into
 the next step.  Weights are random (made on the GPU), token ids are seeded
-synthetic ids, and the cache of the context before the timed steps is filled
-with random keys and values instead of being computed (its content does not
-change the work of a decode step).  Prints one JSON line.
+synthetic ids, and for the fixed-context points the cache of the context before
+the timed steps is filled with random keys and values instead of being computed
+(its content does not change the work of a decode step).  Every point is timed
+three times and the median is reported; ``value`` is the batch over the median
+step time of ``--steps`` steps at contexts ending at ``--context``.  ``trajectory``
+is the workload as stated, end to end: every request a prompt of ``--prefill-tokens``
+tokens and as many greedy tokens, through the scheduler, the step function and
+the sampler.  Bytes and arithmetic of the rooflines come from the model's own
+description (``models/cost.py``), not from formulas of one architecture.
+``--kernels`` prints where one decode step's time goes, entry point by entry
+point.  Prints one JSON line.
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -57,30 +66,58 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
     p.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    p.add_argument("--more-points", action="store_true",
+                   help="further points: batch 8 at contexts of 1,024 / 16,384 / 40,000, batch 16 / 32 / 128 at the "
+                        "context, prompts of 512 and 8,192 tokens")
     p.add_argument("--no-prefill", action="store_true")
+    p.add_argument("--no-trajectory", action="store_true",
+                   help="skip the end-to-end run (prompt + as many greedy tokens per request through the scheduler)")
+    p.add_argument("--trajectory-tokens", type=int, default=None,
+                   help="greedy tokens per request of the end-to-end run (default: --prefill-tokens)")
+    p.add_argument("--runs", type=int, default=3, help="timed runs per point; the median is reported")
+    p.add_argument("--kernels", action="store_true",
+                   help="print where one decode step's time goes by entry point (eager, GPU events) and exit")
     p.add_argument("--seed", type=int, default=0)
     return p.parse_args()
 
 
-def weight_bytes(cfg, element_size: int) -> int:
-    """Bytes of every weight a decode step reads once: all layers and the head."""
-    h, i, d = cfg.hidden_size, cfg.intermediate_size, cfg.head_dim
-    nq, nkv = cfg.num_attention_heads, cfg.num_key_value_heads
-    per_layer = (nq + 2 * nkv) * d * h + h * nq * d + 2 * i * h + h * i + 2 * h + 2 * d
-    return (per_layer * cfg.num_hidden_layers + cfg.vocab_size * h + h) * element_size
+def trajectory(args, cfg, model, batch: int, prompt_tokens: int, new_tokens: int) -> dict:
+    """The stated workload end to end: ``batch`` requests of ``prompt_tokens`` tokens each, ``new_tokens`` greedy
+    tokens each, through scheduler, step function and sampler (prompts in portions of 512 under a budget of 2,048
+    tokens a step).  Returns output tokens a second over the whole run and over its decoding steps alone."""
+    import torch
 
+    from pulse_infer_amd.engine.engine import ContinuousBatchEngine
+    from pulse_infer_amd.sampling.params import SamplingParams
 
-def kv_bytes_per_token(cfg, element_size: int) -> int:
-    return 2 * cfg.num_hidden_layers * cfg.num_key_value_heads * cfg.head_dim * element_size
-
-
-def prefill_flops(cfg, tokens: int) -> float:
-    """Multiply-adds of one prompt of ``tokens`` tokens, times two; logits for the last row only."""
-    h, i, d = cfg.hidden_size, cfg.intermediate_size, cfg.head_dim
-    nq, nkv = cfg.num_attention_heads, cfg.num_key_value_heads
-    linear = (nq + 2 * nkv) * d * h + h * nq * d + 3 * i * h
-    attn = 4 * nq * d * tokens * (tokens + 1) / 2          # QK^T and PV over the causal triangle
-    return cfg.num_hidden_layers * (2.0 * tokens * linear + attn) + 2.0 * cfg.vocab_size * h
+    gen = torch.Generator().manual_seed(args.seed + 17)
+    pages = batch * ((prompt_tokens + new_tokens + args.page_size - 1) // args.page_size + 1)
+    engine = ContinuousBatchEngine(model, max_batch_size=batch, chunk_size=512, page_size=args.page_size,
+                                   num_pages=pages, max_sequences=batch, max_num_batched_tokens=2048, seed=args.seed)
+    for _ in range(batch):
+        engine.add_request(torch.randint(0, cfg.vocab_size, (prompt_tokens,), generator=gen).tolist(), new_tokens,
+                           SamplingParams(ignore_eos=True))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    t_decode, decode_steps = None, 0
+    while engine.scheduler.has_work():
+        if t_decode is None and not any(r.is_prefill for r in engine.scheduler.running + list(engine.scheduler.waiting)):
+            torch.cuda.synchronize()
+            t_decode = time.perf_counter()
+        if engine.step().empty():
+            break
+        decode_steps += t_decode is not None
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    stats = engine.get_stats()
+    total = stats.tokens_generated
+    assert total == batch * new_tokens, (total, batch, new_tokens)
+    decode_s = t1 - (t_decode if t_decode is not None else t0)
+    del engine
+    torch.cuda.empty_cache()
+    return {"value": round(total / (t1 - t0), 2), "decode_value": round(batch * decode_steps / decode_s, 2),
+            "batch": batch, "prompt_tokens": prompt_tokens, "new_tokens": new_tokens, "seconds": round(t1 - t0, 3),
+            "decode_ms_per_step": round(decode_s * 1e3 / max(1, decode_steps), 4), "steps": stats.num_steps}
 
 
 def serving(args, cfg, model, full_layers: int) -> int:
@@ -155,52 +192,79 @@ def main() -> int:
     if args.workload == "serving":
         return serving(args, cfg, model, full_layers)
 
-    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
-    max_batch = max(batches)
-    pages_per_request = (args.context + args.page_size - 1) // args.page_size + 1
-    prefill_pages = (args.prefill_tokens + args.page_size - 1) // args.page_size + 1
-    runner = ModelRunner(model, page_size=args.page_size, num_pages=max(max_batch * pages_per_request, prefill_pages),
-                         max_requests=max_batch + 1)
+    from pulse_infer_amd.models.cost import step_cost
+
+    spec = cfg.model_spec()
+    peak_flops = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+    # (batch, context) of every decode point, prompt lengths of every prefill point
+    decode_points = {} if args.no_points else {"decode_b1": (1, args.context), "decode_b64": (64, args.context)}
+    prefill_points = {}
+    if args.more_points:
+        for ctx in (1024, 16384, 40000):
+            decode_points[f"decode_b8_ctx{ctx}"] = (8, ctx)
+        for b in (16, 32, 128):
+            decode_points[f"decode_b{b}"] = (b, args.context)
+        prefill_points = {"prefill_512": 512, "prefill_8192": 8192}
+    shapes = [(args.batch, args.context)] + list(decode_points.values())
+    max_batch = max(b for b, _ in shapes)
+    page = args.page_size
+    pool = max([b * ((c + page - 1) // page + 1) for b, c in shapes]
+               + [(n + page - 1) // page + 1 for n in [args.prefill_tokens] + list(prefill_points.values())])
+    runner = ModelRunner(model, page_size=page, num_pages=pool, max_requests=max_batch + 1)
     for g in runner.cache.groups:  # a cache that looks computed: random keys and values
         g.keys.normal_(0.0, 1.0)
         g.values.normal_(0.0, 1.0)
     sampler = Sampler(cfg.vocab_size, max_batch + 1, device)
     gen = torch.Generator().manual_seed(args.seed)
 
-    def decode_run(batch: int, steps: int, warmup: int):
-        """Time ``steps`` decode steps of ``batch`` requests whose contexts end at ``args.context``."""
-        start = args.context - (steps + warmup)
+    def decode_run(batch: int, context: int, steps: int, warmup: int, runs: int):
+        """``runs`` timings of ``steps`` decode steps of ``batch`` requests whose contexts end at ``context`` (every run
+        walks the same contexts).  Returns (median seconds a step by the host's clock between two synchronisations,
+        the same by GPU events, every run's host figure)."""
+        start = context - (steps + warmup)
         if start < 1:
-            raise SystemExit(f"--context {args.context} is too short for {steps} + {warmup} steps")
+            raise SystemExit(f"a context of {context} is too short for {steps} + {warmup} steps")
         names = [f"d{batch}_{i}" for i in range(batch)]
-        for n in names:
-            runner.add_request(n)
-            runner.reserve(n, args.context)
-            runner.cache.advance(n, start)          # the context so far counts as computed
-        tokens = torch.randint(0, cfg.vocab_size, (batch,), generator=gen).tolist()
         greedy = [SamplingParams()] * batch
-        slots = [runner.cache.slot_of(n) for n in names]
+        host, events = [], []
+        for _ in range(runs):
+            for n in names:
+                runner.add_request(n)
+                runner.reserve(n, context)
+                runner.cache.advance(n, start)          # the context so far counts as computed
+            tokens = torch.randint(0, cfg.vocab_size, (batch,), generator=gen).tolist()
+            slots = [runner.cache.slot_of(n) for n in names]
 
-        def one_step(toks):
-            logits = runner.step([StepEntry(n, [t], [0]) for n, t in zip(names, toks)])
-            return sampler.sample(logits, greedy, slots, [0] * batch, [0] * batch)
+            def one_step(toks):
+                logits = runner.step([StepEntry(n, [t], [0]) for n, t in zip(names, toks)])
+                return sampler.sample(logits, greedy, slots, [0] * batch, [0] * batch)
 
-        for _ in range(warmup):
-            tokens = one_step(tokens)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            tokens = one_step(tokens)
-        torch.cuda.synchronize()
-        seconds = time.perf_counter() - t0
-        for n in names:
-            runner.free_request(n)
-        return seconds / steps
+            for _ in range(warmup):
+                tokens = one_step(tokens)
+            first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            first.record()
+            for _ in range(steps):
+                tokens = one_step(tokens)
+            last.record()
+            torch.cuda.synchronize()
+            host.append((time.perf_counter() - t0) / steps)
+            events.append(first.elapsed_time(last) * 1e-3 / steps)
+            for n in names:
+                runner.free_request(n)
+        return statistics.median(host), statistics.median(events), host
 
-    def prefill_run(tokens: int, repeats: int = 3):
+    def decode_bytes(batch: int, context: int, steps: int) -> float:
+        """What a decode step of the timed run has to read: every weight once and the live requests' cache, at the
+        run's mean context."""
+        cost = step_cost(spec, [(int(context - steps / 2.0) - 1, 1)] * batch, batch, element, element)
+        return cost.weight_bytes + cost.cache_bytes
+
+    def prefill_run(tokens: int, runs: int):
         ids = torch.randint(0, cfg.vocab_size, (tokens,), generator=gen).tolist()
-        best = None
-        for r in range(repeats + 1):  # the first run warms up
+        times = []
+        for r in range(runs + 1):  # the first run warms up
             runner.add_request("p")
             runner.reserve("p", tokens)
             torch.cuda.synchronize()
@@ -211,14 +275,15 @@ def main() -> int:
             seconds = time.perf_counter() - t0
             runner.free_request("p")
             if r > 0:
-                best = seconds if best is None else min(best, seconds)
-        return best
+                times.append(seconds)
+        return statistics.median(times)
 
-    step_s = decode_run(args.batch, args.steps, args.warmup)
+    if args.kernels:
+        return kernel_table(args, cfg, runner, sampler, gen)
+
+    step_s, step_gpu_s, all_runs = decode_run(args.batch, args.context, args.steps, args.warmup, args.runs)
     value = args.batch / step_s
-    mean_ctx = args.context - args.steps / 2.0
-    step_bytes = weight_bytes(cfg, element) + args.batch * mean_ctx * kv_bytes_per_token(cfg, element)
-    achieved = step_bytes / step_s / 1e9
+    achieved = decode_bytes(args.batch, args.context, args.steps) / step_s / 1e9
     result = {
         "metric": f"qwen3_{args.model}_decode_tokens_per_s_batch{args.batch}", "value": round(value, 2), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4),
@@ -233,22 +298,69 @@ def main() -> int:
             "rms_norm_eps": cfg.rms_norm_eps, "tie_word_embeddings": cfg.tie_word_embeddings,
             "page_size": args.page_size, "prefill_tokens": args.prefill_tokens,
         },
+        "runs": args.runs, "ms_per_step_runs": [round(t * 1e3, 4) for t in all_runs],
+        "ms_per_step_gpu_events": round(step_gpu_s * 1e3, 4),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
     if not args.no_prefill:
-        pf_s = prefill_run(args.prefill_tokens)
-        peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+        pf_s = prefill_run(args.prefill_tokens, args.runs)
+        flops = step_cost(spec, [(0, args.prefill_tokens)], 1, element, element).flops
         result["prefill"] = {"value": round(args.prefill_tokens / pf_s, 1), "tokens": args.prefill_tokens,
-                             "ms": round(pf_s * 1e3, 3),
-                             "frac": round(prefill_flops(cfg, args.prefill_tokens) / pf_s / peak, 4)}
-    if not args.no_points:
-        points = {}
-        for b in (1, 64):
+                             "ms": round(pf_s * 1e3, 3), "frac": round(flops / pf_s / peak_flops, 4)}
+    if decode_points or prefill_points:
+        points, fracs = {}, {}
+        for name, (b, ctx) in decode_points.items():
             steps = max(8, min(args.steps, 32))
-            points[f"decode_b{b}"] = round(b / decode_run(b, steps, min(args.warmup, 4)), 2)
+            t, _, _ = decode_run(b, ctx, steps, min(args.warmup, 4), args.runs)
+            points[name] = round(b / t, 2)
+            fracs[name] = round(decode_bytes(b, ctx, steps) / t / 1e9 / HBM_PEAK_GBS, 4)
+        for name, n in prefill_points.items():
+            t = prefill_run(n, args.runs)
+            points[name] = round(n / t, 1)
+            fracs[name] = round(step_cost(spec, [(0, n)], 1, element, element).flops / t / peak_flops, 4)
         result["points"] = points
+        result["points_frac"] = fracs     # of 8 TB/s for decoding, of the dense matrix-core peak for prompts
+    if not args.no_trajectory:
+        del runner, sampler
+        torch.cuda.empty_cache()
+        new_tokens = args.trajectory_tokens or args.prefill_tokens
+        result["trajectory"] = trajectory(args, cfg, model, args.batch, args.prefill_tokens, new_tokens)
     print(json.dumps(result))
+    return 0
+
+
+def kernel_table(args, cfg, runner, sampler, gen) -> int:
+    """Where the time of one decode step goes, by entry point: every launch of an eager step is bracketed by GPU
+    events (``ops/timing.py``), over a few steps; printed as a table, most expensive first."""
+    import torch
+
+    from pulse_infer_amd.engine.runner import StepEntry
+    from pulse_infer_amd.ops import timing
+    from pulse_infer_amd.sampling.params import SamplingParams
+
+    runner.use_graphs = False
+    batch, context, steps = args.batch, args.context, 6
+    names = [f"k{i}" for i in range(batch)]
+    for n in names:
+        runner.add_request(n)
+        runner.reserve(n, context)
+        runner.cache.advance(n, context - steps - 2)
+    tokens = torch.randint(0, cfg.vocab_size, (batch,), generator=gen).tolist()
+    slots = [runner.cache.slot_of(n) for n in names]
+
+    def one_step(toks):
+        logits = runner.step([StepEntry(n, [t], [0]) for n, t in zip(names, toks)])
+        return sampler.sample(logits, [SamplingParams()] * batch, slots, [0] * batch, [0] * batch)
+
+    for _ in range(2):
+        tokens = one_step(tokens)
+    with timing.record() as table:
+        for _ in range(steps):
+            tokens = one_step(tokens)
+    print(f"# decode step, batch {batch}, contexts ending at {context}, {args.layers} layers, eager launches, "
+          f"mean of {steps} steps")
+    print(table.format(per=steps))
     return 0
 
 

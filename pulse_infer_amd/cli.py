@@ -29,7 +29,7 @@ def find_default_model_path() -> str:
         here = parent
 
 
-def parse_args(argv: Optional[List[str]] = None) -> argparse.Namespace:
+def build_parser() -> argparse.ArgumentParser:
     p = argparse.ArgumentParser(prog="pulse_infer", description=__doc__.split("\n\n")[0])
     p.add_argument("model_dir", nargs="?", default=None, help="folder with config.json and *.safetensors")
     p.add_argument("--model", dest="model_opt", default=None, help="same as the positional model_dir")
@@ -54,15 +54,56 @@ def parse_args(argv: Optional[List[str]] = None) -> argparse.Namespace:
     p.add_argument("--max-batch", type=int, default=8, help="most requests in one step")
     p.add_argument("--max-tokens", type=int, default=None, help="most tokens in one step (the budget)")
     p.add_argument("--chunk", type=int, default=256, help="longest prompt portion in one step")
-    p.add_argument("--rope-pairing", choices=["interleaved", "half"], default=None,
-                   help="channels a rotation pairs: interleaved (2i, 2i+1), as the reference computes, or half (i, i + d/2)")
+    p.add_argument("--set", dest="overrides", action="append", default=[], metavar="FIELD=VALUE",
+                   help="set a field of the model's configuration that is an option of the engine rather than a key of "
+                        "config.json (for Qwen3: rope_pairing=half, the channels a rotation pairs); may be repeated")
+    p.add_argument("--strict", action="store_true", help="a tensor that no part of the model asks for is an error")
     p.add_argument("--stats", action="store_true")
-    return p.parse_args(argv)
+    return p
+
+
+def parse_args(argv: Optional[List[str]] = None) -> argparse.Namespace:
+    """Options of the program, then those that the model's architecture declares (``engine_options`` of its
+    configuration class, e.g. ``--rope-pairing`` for Qwen3): they are known only once config.json has been read."""
+    parser = build_parser()
+    args, rest = parser.parse_known_args(argv)
+    args.model_path = args.model_opt or args.model_dir or find_default_model_path()
+    args.config = None
+    if rest or os.path.isfile(os.path.join(args.model_path, "config.json")):
+        from .config import load_config
+
+        args.config = load_config(args.model_path)
+        extra = argparse.ArgumentParser(prog="pulse_infer", add_help=False, allow_abbrev=False)
+        for field, keywords in args.config.engine_options.items():
+            extra.add_argument("--" + field.replace("_", "-"), dest=field, default=None, **keywords)
+        known, unknown = extra.parse_known_args(rest)
+        if unknown:
+            parser.error(f"unrecognized arguments: {' '.join(unknown)} (options of '{args.config.architecture}': "
+                         f"{', '.join('--' + f.replace('_', '-') for f in args.config.engine_options) or 'none'})")
+        args.architecture_options = {k: v for k, v in vars(known).items() if v is not None}
+    else:
+        args.architecture_options = {}
+    return args
+
+
+def parse_overrides(items: List[str]) -> dict:
+    """``FIELD=VALUE`` pairs; a value is read as JSON where it is JSON (numbers, true, null), else as a string."""
+    out = {}
+    for item in items:
+        key, sep, text = item.partition("=")
+        if not sep or not key.strip():
+            raise SystemExit(f"pulse_infer: --set expects FIELD=VALUE, got '{item}'")
+        try:
+            value = json.loads(text)
+        except json.JSONDecodeError:
+            value = text
+        out[key.strip()] = value
+    return out
 
 
 def main(argv: Optional[List[str]] = None) -> int:
     args = parse_args(argv)
-    model_dir = args.model_opt or args.model_dir or find_default_model_path()
+    model_dir = args.model_path
     dtype = {"bf16": "bfloat16", "f32": "float32"}.get(args.dtype, args.dtype)
 
     import torch
@@ -74,18 +115,17 @@ def main(argv: Optional[List[str]] = None) -> int:
     from .engine.engine import LLM
     from .sampling.params import SamplingParams
 
-    config = load_config(model_dir)
-    overrides = {"rope_pairing": args.rope_pairing} if args.rope_pairing else None
-    if overrides:
-        config.rope_pairing = args.rope_pairing
-        config.validate(model_dir)
+    config = args.config or load_config(model_dir)
+    overrides = dict(parse_overrides(args.overrides), **args.architecture_options)
+    config.apply_overrides(overrides, "the command line")
     options = dict(max_batch_size=args.max_batch, chunk_size=args.chunk, page_size=args.page_size,
                    num_pages=args.num_pages, max_num_batched_tokens=args.max_tokens, seed=args.seed)
     if args.random_weights:
         init = args.init if args.init == "fan_in" else float(args.init)
         llm = LLM.from_config_random(config, weights_seed=args.seed, init=init, dtype=dtype, device=args.device, **options)
     else:
-        llm = LLM.from_pretrained(model_dir, dtype=dtype, device=args.device, config_overrides=overrides, **options)
+        llm = LLM.from_pretrained(model_dir, dtype=dtype, device=args.device, config_overrides=overrides,
+                                  strict=args.strict, **options)
 
     prompts: List[List[int]] = [[int(t) for t in s.split(",") if t.strip()] for s in args.prompt_ids]
     if args.prompt_file:

@@ -1,15 +1,28 @@
-"""Typed reading of a model folder's JSON configuration.
+"""Typed reading of a model folder's JSON configuration, and what the engine asks of a configuration.
 
-A configuration class declares its fields once; ``JsonReader`` fetches each
-key with a type check and produces errors that name the key and the file, in
-the manner of the reference's ``read_required_*`` helpers
-(reference: src/model/qwen3/config.cpp:70-138).
+``JsonReader`` fetches each key with a type check and produces errors that name the
+file, the key and what was found, in the manner of the reference's ``read_required_*``
+helpers (reference: src/model/qwen3/config.cpp:70-138).
+
+``ModelConfig`` is the base of every architecture's configuration class.  The engine,
+the command line and the loaders use nothing of a configuration beyond it:
+
+* fields: ``architecture``, ``vocab_size``, ``eos_token_ids``, and the sampling defaults
+  ``temperature``, ``top_k``, ``top_p``;
+* ``from_dict(data, origin, generation, generation_origin)`` / ``load(folder)``: read and
+  validate; ``to_dict()``: what ``config.json`` of a written model folder holds;
+* ``validate(origin)``; ``apply_overrides({field: value})``: options of the engine that are
+  no keys of config.json (the command line's ``--set field=value``);
+* ``model_spec()``: the architecture as data (a ``ModelSpec``), which the generic model
+  is built from.
+
+An architecture brings a subclass with its own keys and registers it by name.
 """
 from __future__ import annotations
 
 import json
 import os
-from typing import Any, Dict, List, Optional, Sequence
+from typing import Any, Dict, List, Mapping, Optional, Sequence
 
 
 class ConfigError(ValueError):
@@ -63,7 +76,7 @@ def read_json_file(path: str) -> Dict[str, Any]:
     """A JSON object from a file; comments are allowed, as in the reference's reader
     (reference: src/model/qwen3/config.cpp:52 parses with ignore_comments)."""
     if not os.path.exists(path):
-        raise ConfigError(f"Config file '{path}' does not exist")
+        raise ConfigError(f"there is no file '{path}'")
     try:
         with open(path, "r", encoding="utf-8") as fh:
             text = fh.read()
@@ -72,9 +85,9 @@ def read_json_file(path: str) -> Dict[str, Any]:
         except json.JSONDecodeError:
             data = json.loads(strip_json_comments(text))
     except json.JSONDecodeError as exc:
-        raise ConfigError(f"Config file '{path}' is not valid JSON: {exc}") from exc
+        raise ConfigError(f"'{path}' is not valid JSON: {exc}") from exc
     if not isinstance(data, dict):
-        raise ConfigError(f"Config file '{path}' must hold a JSON object")
+        raise ConfigError(f"'{path}' must hold a JSON object, found {type(data).__name__}")
     return data
 
 
@@ -86,7 +99,9 @@ class JsonReader:
         self.origin = origin
 
     def _fail(self, kind: str, key: str) -> ConfigError:
-        return ConfigError(f"Missing or invalid {kind} key '{key}' in '{self.origin}'")
+        if self.data.get(key) is None:
+            return ConfigError(f"'{self.origin}': key '{key}' ({kind}) is required and missing")
+        return ConfigError(f"'{self.origin}': key '{key}' must be {kind}, found {self.data[key]!r}")
 
     def has(self, key: str) -> bool:
         return key in self.data and self.data[key] is not None
@@ -98,42 +113,42 @@ class JsonReader:
         value = self.data.get(key, None)
         if value is None:
             if default is _MISSING:
-                raise self._fail("integer", key)
+                raise self._fail("an integer", key)
             return default
         if isinstance(value, bool) or not isinstance(value, int):
             if isinstance(value, float) and value.is_integer():
                 return int(value)
-            raise self._fail("integer", key)
+            raise self._fail("an integer", key)
         return int(value)
 
     def number(self, key: str, default: Any = _MISSING) -> float:
         value = self.data.get(key, None)
         if value is None:
             if default is _MISSING:
-                raise self._fail("number", key)
+                raise self._fail("a number", key)
             return default
         if isinstance(value, bool) or not isinstance(value, (int, float)):
-            raise self._fail("number", key)
+            raise self._fail("a number", key)
         return float(value)
 
     def boolean(self, key: str, default: Any = _MISSING) -> bool:
         value = self.data.get(key, None)
         if value is None:
             if default is _MISSING:
-                raise self._fail("boolean", key)
+                raise self._fail("true or false", key)
             return default
         if not isinstance(value, bool):
-            raise self._fail("boolean", key)
+            raise self._fail("true or false", key)
         return value
 
     def string(self, key: str, default: Any = _MISSING) -> str:
         value = self.data.get(key, None)
         if value is None:
             if default is _MISSING:
-                raise self._fail("string", key)
+                raise self._fail("a string", key)
             return default
         if not isinstance(value, str):
-            raise self._fail("string", key)
+            raise self._fail("a string", key)
         return value
 
     def int_or_int_list(self, key: str) -> List[int]:
@@ -146,7 +161,7 @@ class JsonReader:
             return [int(value)]
         if isinstance(value, list) and all(isinstance(v, int) and not isinstance(v, bool) for v in value):
             return [int(v) for v in value]
-        raise ConfigError(f"Invalid int list key '{key}' in '{self.origin}'")
+        raise self._fail("an integer or a list of integers", key)
 
     def string_list(self, key: str) -> Optional[List[str]]:
         value = self.data.get(key, None)
@@ -154,17 +169,94 @@ class JsonReader:
             return None
         if isinstance(value, list) and all(isinstance(v, str) for v in value):
             return list(value)
-        raise self._fail("string list", key)
+        raise self._fail("a list of strings", key)
 
 
 def require_positive(origin: str, **named: int) -> None:
     bad = [name for name, value in named.items() if value <= 0]
     if bad:
-        raise ConfigError(f"Invalid model dimensions in '{origin}': {', '.join(bad)} must be positive")
+        raise ConfigError(f"'{origin}': these sizes must be positive: " + ", ".join(f"{name} = {named[name]}" for name in bad))
 
 
 def architecture_name(data: Dict[str, Any], origin: str) -> str:
     archs = data.get("architectures")
     if not isinstance(archs, Sequence) or isinstance(archs, str) or len(archs) == 0 or not isinstance(archs[0], str):
-        raise ConfigError(f"Missing or invalid string list key 'architectures' in '{origin}'")
+        raise ConfigError(f"'{origin}': key 'architectures' must be a list that starts with the model's class name")
     return archs[0]
+
+
+class ModelConfig:
+    """Base of an architecture's configuration (see the module's text for what the engine uses of it).
+
+    Subclasses are dataclasses with their own fields, among them ``vocab_size``, and set ``architecture``.  The
+    sampling defaults and the end-of-sequence ids have defaults here, so an architecture that has no use for
+    generation_config.json need not mention them."""
+
+    architecture: str = ""
+    # Fields that are options of the engine rather than keys of config.json, by field name: each becomes an option
+    # of the command line (``--field-name``) with these argparse keywords (choices, type, help).  Every field can
+    # also be set with ``--set field=value``.
+    engine_options: Dict[str, Dict[str, Any]] = {}
+    eos_token_ids: Sequence[int] = ()
+    temperature: float = 0.0
+    top_k: int = 0
+    top_p: float = 0.0
+
+    # ------------------------------------------------------------------ reading
+    @classmethod
+    def from_dict(cls, data: Dict[str, Any], origin: str = "<dict>", generation: Optional[Dict[str, Any]] = None,
+                  generation_origin: str = "<dict>") -> "ModelConfig":
+        raise NotImplementedError(f"{cls.__name__} must read its own keys in from_dict")
+
+    @classmethod
+    def load(cls, path: str) -> "ModelConfig":
+        """config.json of the folder, and generation_config.json beside it if there is one."""
+        model_dir = resolve_model_dir(path)
+        config_path = os.path.join(model_dir, "config.json")
+        data = read_json_file(config_path)
+        gen_path = os.path.join(model_dir, "generation_config.json")
+        generation = read_json_file(gen_path) if os.path.exists(gen_path) else None
+        return cls.from_dict(data, config_path, generation, gen_path)
+
+    def read_generation_defaults(self, generation: Optional[Dict[str, Any]], origin: str = "<dict>") -> None:
+        """Sampling defaults and end-of-sequence ids from generation_config.json; its ids replace config.json's
+        (reference: src/model/qwen3/config.cpp:333-365)."""
+        if generation is None:
+            return
+        g = JsonReader(generation, origin)
+        eos = g.int_or_int_list("eos_token_id")
+        if eos:
+            self.eos_token_ids = eos
+        self.temperature = g.number("temperature", self.temperature)
+        self.top_k = g.integer("top_k", self.top_k)
+        self.top_p = g.number("top_p", self.top_p)
+
+    # --------------------------------------------------------------- validation
+    def validate(self, origin: str = "<config>") -> None:
+        """Raise ``ConfigError`` for values the architecture cannot run with."""
+
+    def apply_overrides(self, overrides: Optional[Mapping[str, Any]], origin: str = "<overrides>") -> None:
+        """Set fields by name (options of the engine rather than keys of config.json) and validate again.  A name
+        the configuration does not have, or a value of another type than the field's, is refused."""
+        if not overrides:
+            return
+        for key, value in overrides.items():
+            if key.startswith("_") or key == "engine_options" or not hasattr(self, key) or callable(getattr(self, key)):
+                fields = sorted(k for k in vars(self) if not k.startswith("_"))
+                raise ConfigError(f"the configuration of '{self.architecture}' has no field '{key}' "
+                                  f"(it has: {', '.join(fields)})")
+            current = getattr(self, key)
+            if isinstance(current, float) and isinstance(value, int) and not isinstance(value, bool):
+                value = float(value)
+            if current is not None and value is not None and type(current) is not type(value):
+                raise ConfigError(f"field '{key}' of '{self.architecture}' is {type(current).__name__}, "
+                                  f"got {type(value).__name__} {value!r}")
+            setattr(self, key, value)
+        self.validate(origin)
+
+    # ------------------------------------------------------------------ writing
+    def to_dict(self) -> Dict[str, Any]:
+        raise NotImplementedError(f"{type(self).__name__} must say what its config.json holds in to_dict")
+
+    def model_spec(self) -> Any:
+        raise NotImplementedError(f"{type(self).__name__} must describe its model in model_spec")

@@ -9,18 +9,17 @@ formula for.  The sliding-window keys choose a window per layer.
 """
 from __future__ import annotations
 
-import os
 from dataclasses import dataclass, field
 from typing import Any, Dict, List, Optional
 
-from .base import ConfigError, JsonReader, read_json_file, require_positive, resolve_model_dir
+from .base import ConfigError, JsonReader, ModelConfig, require_positive
 from ..models.spec import LayerSpec, ModelSpec, PartSpec, RunSpec
 
 ARCHITECTURE = "Qwen3ForCausalLM"
 
 
 @dataclass
-class Qwen3Config:
+class Qwen3Config(ModelConfig):
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -48,6 +47,10 @@ class Qwen3Config:
     rope_pairing: str = "interleaved"
     architecture: str = ARCHITECTURE
 
+    engine_options = {"rope_pairing": {
+        "choices": ["interleaved", "half"],
+        "help": "channels a rotation pairs: interleaved (2i, 2i+1), as the reference computes, or half (i, i + d/2)"}}
+
     # ------------------------------------------------------------------ reading
     @classmethod
     def from_dict(cls, data: Dict[str, Any], origin: str = "<dict>",
@@ -57,21 +60,20 @@ class Qwen3Config:
         num_heads = r.integer("num_attention_heads")
         hidden = r.integer("hidden_size")
         rope_theta = cls._read_rope_theta(r)
-        dtype = r.string("torch_dtype", None)
-        if dtype is None:
-            dtype = r.string("dtype", "bfloat16")
+        # required, as the reference requires it (config.cpp:250); newer checkpoints spell the key "dtype"
+        dtype = r.string("dtype") if r.has("dtype") and not r.has("torch_dtype") else r.string("torch_dtype")
         cfg = cls(
             vocab_size=r.integer("vocab_size"),
             hidden_size=hidden,
             intermediate_size=r.integer("intermediate_size"),
             num_hidden_layers=r.integer("num_hidden_layers"),
             num_attention_heads=num_heads,
-            num_key_value_heads=r.integer("num_key_value_heads", num_heads),
-            head_dim=r.integer("head_dim", hidden // num_heads if num_heads > 0 else 0),
+            num_key_value_heads=r.integer("num_key_value_heads"),
+            head_dim=r.integer("head_dim"),
             max_position_embeddings=r.integer("max_position_embeddings"),
             rms_norm_eps=r.number("rms_norm_eps"),
             rope_theta=rope_theta,
-            tie_word_embeddings=r.boolean("tie_word_embeddings", False),
+            tie_word_embeddings=r.boolean("tie_word_embeddings"),
             torch_dtype=dtype,
             eos_token_ids=r.int_or_int_list("eos_token_id"),
             use_sliding_window=r.boolean("use_sliding_window", False),
@@ -89,14 +91,7 @@ class Qwen3Config:
         if scaling is not None and not (isinstance(scaling, dict) and scaling.get("rope_type", scaling.get("type")) == "default"):
             raise ConfigError(f"'rope_scaling' other than null is not supported (in '{origin}')")
 
-        if generation is not None:
-            g = JsonReader(generation, generation_origin)
-            eos = g.int_or_int_list("eos_token_id")
-            if eos:
-                cfg.eos_token_ids = eos
-            cfg.temperature = g.number("temperature", cfg.temperature)
-            cfg.top_k = g.integer("top_k", cfg.top_k)
-            cfg.top_p = g.number("top_p", cfg.top_p)
+        cfg.read_generation_defaults(generation, generation_origin)
         cfg.validate(origin)
         return cfg
 
@@ -112,15 +107,6 @@ class Qwen3Config:
             return float(params["rope_theta"])
         return r.number("rope_theta")  # raises the named error
 
-    @classmethod
-    def load(cls, path: str) -> "Qwen3Config":
-        model_dir = resolve_model_dir(path)
-        config_path = os.path.join(model_dir, "config.json")
-        data = read_json_file(config_path)
-        gen_path = os.path.join(model_dir, "generation_config.json")
-        generation = read_json_file(gen_path) if os.path.exists(gen_path) else None
-        return cls.from_dict(data, config_path, generation, gen_path)
-
     # --------------------------------------------------------------- validation
     def validate(self, origin: str = "<config>") -> None:
         """Reference checks (src/model/qwen3/config.cpp:209-227) plus the ones the kernels need."""
@@ -133,8 +119,9 @@ class Qwen3Config:
         )
         if self.num_attention_heads % self.num_key_value_heads != 0:
             raise ConfigError(
-                f"num_attention_heads({self.num_attention_heads}) is not divisible by "
-                f"num_key_value_heads({self.num_key_value_heads}) in '{origin}'")
+                f"'{origin}': {self.num_attention_heads} attention heads cannot be shared out evenly over "
+                f"{self.num_key_value_heads} key/value heads (num_attention_heads must be a multiple of "
+                f"num_key_value_heads)")
         if self.head_dim % 2 != 0:
             raise ConfigError(f"head_dim({self.head_dim}) must be even for rotary pairs in '{origin}'")
         if not self.rms_norm_eps >= 0.0:
@@ -230,7 +217,8 @@ class Qwen3Config:
                 "prefix": "mlp",
             })
             block = PartSpec("prenorm", {"mixer_norm": "input_layernorm", "ffn_norm": "post_attention_layernorm"})
-            layers.append(LayerSpec(prefix=f"model.layers.{i}", mixer=mixer, ffn=ffn, norm=norm, block=block))
+            layers.append(LayerSpec(prefix=f"model.layers.{i}", mixer=mixer, ffn=ffn,
+                                    norms={"mixer_norm": norm, "ffn_norm": norm}, block=block))
         spec = ModelSpec(
             architecture=self.architecture,
             vocab_size=self.vocab_size,

@@ -16,6 +16,7 @@ typedef uint16_t bf16_t;  // raw bfloat16 bits
 // pulse_last_error().  Arguments are checked on the host before any launch.
 extern "C" const char* pulse_last_error();
 void pulse_set_error(const char* fmt, ...);
+int pulse_compute_units();  // of the current device, asked once
 
 #define PULSE_REQUIRE(cond, ...)            \
     do {                                    \

@@ -7,8 +7,9 @@
 
 // ------------------------------------------------------------------ embedding
 // out[t, :] = table[ids[t], :] widened to float32 (the residual stream).
-// Ids are checked on the host; a bad id here still reads nothing out of range
-// and raises *bad_id so that the caller can fail.
+// Ids are checked on the host; a bad id here still reads nothing out of range:
+// its row becomes NaN, which every later product carries into that token's logits
+// (no token is then chosen for it), and *bad_id is raised for a caller that asks.
 // (reference: src/ops/kernels/cuda/embedding_kernel.cu:7-28 leaves zeros silently)
 template <typename TW>
 __global__ void embed_gather_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
@@ -17,7 +18,7 @@ __global__ void embed_gather_kernel(const int* __restrict__ ids, const TW* __res
     const int id = ids[t];
     float* dst = out + static_cast<int64_t>(t) * hidden;
     if (id < 0 || id >= vocab) {
-        for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = 0.f;
+        for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = __builtin_nanf("");
         if (threadIdx.x == 0) *bad_id = 1;
         return;
     }

@@ -508,7 +508,8 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
     const int parts_out = (N + 15) / 16;
     const bf16_t* w = static_cast<const bf16_t*>(W);
     const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-    const bool wide = N >= 16384;  // enough slabs that pairs of them still fill the chip
+    const int units = pulse_compute_units();
+    const bool wide = N >= 64 * units;  // enough slabs that pairs of them still give every compute unit two workgroups
     // tune (tests and measurements): decimal digits S K P, S slabs (1, 2), K wavefronts (4, 8), P = 1 + log2 of the
     // k-steps a load of X serves (1..4), all for the streaming kernel; 9 asks for the general kernel.
     int t_slabs = 0, t_kw = 0, t_pack = 0;
@@ -524,8 +525,9 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
         // pair shares its loads of X), else single slabs with more wavefronts along K
         // (also where single slabs would put two workgroups on some compute units and pairs one on each: 5,120
         // weight rows, o and down of the 14B shape, at 8 rows 16.2 -> 14.7 us and 44.7 -> 36.9 us)
-        auto fullest = [&](int rows) { return ((N + rows - 1) / rows + 255) / 256 * rows; };   // weight rows on the fullest of 256 units
-        const bool pairs = swiglu || wide || (M >= 8 && (N >= 6144 || fullest(16) >= fullest(32)));
+        auto fullest = [&](int rows) { return ((N + rows - 1) / rows + units - 1) / units * rows; };   // weight rows on the fullest unit
+        // (from 8 rows on, pairs also where they still reach three quarters of the units: N / 32 >= 3 units / 4)
+        const bool pairs = swiglu || wide || (M >= 8 && (N >= 24 * units || fullest(16) >= fullest(32)));
         const int slabs = t_slabs ? t_slabs : (pairs ? 2 : 1);
         const int kw = t_kw ? t_kw : ((K % 2048 == 0 && !pairs) ? 8 : 4);
         const int pack = t_pack ? t_pack : pack_for(M);

@@ -97,14 +97,14 @@ class ContinuousBatchEngine:
         while self.scheduler.has_work():
             if print_progress and step % 10 == 0:
                 s = self.scheduler.get_stats()
-                print(f"Continuous batch step {step} running={s.num_running} waiting={s.num_waiting} "
-                      f"finished={s.num_finished}", file=sys.stderr, flush=True)
+                print(f"[pulse_infer_amd] step {step}: {s.num_running} requests running, {s.num_waiting} waiting, "
+                      f"{s.num_finished} finished", file=sys.stderr, flush=True)
             if self.step().empty():
                 break
             step += 1
         if print_progress:
             s = self.scheduler.get_stats()
-            print(f"Continuous batch complete steps={step} total_requests={s.total_requests}", file=sys.stderr,
+            print(f"[pulse_infer_amd] all {s.total_requests} requests finished after {step} steps", file=sys.stderr,
                   flush=True)
 
     # ----------------------------------------------------------------- results
@@ -147,8 +147,10 @@ class LLM:
 
     @classmethod
     def from_pretrained(cls, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0",
-                        config_overrides: Optional[Dict[str, Any]] = None, **engine_options):
-        config, model = load_model(model_dir, mode=dtype, device=device, config_overrides=config_overrides)
+                        config_overrides: Optional[Dict[str, Any]] = None, strict: bool = False, **engine_options):
+        """``strict``: a tensor in the folder that no part of the model asks for is an error (else a warning)."""
+        config, model = load_model(model_dir, mode=dtype, device=device, config_overrides=config_overrides,
+                                   strict=strict)
         return cls(model, config, **engine_options)
 
     @classmethod

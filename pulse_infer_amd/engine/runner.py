@@ -108,7 +108,10 @@ class ModelRunner:
             else:
                 self.views.append(None)
         self._staging = _Staging(self.device)
-        self.use_graphs = bool(use_graphs) and model.options.get("decode_graph", True)
+        # a step is recorded only if every part it runs says that it records cleanly (Part.records_cleanly)
+        clean = all(getattr(model.blocks[run.layer], "records_cleanly", lambda: False)() for run in order) and all(
+            getattr(p, "records_cleanly", False) for p in getattr(model, "positions", {}).values())
+        self.use_graphs = bool(use_graphs) and model.options.get("decode_graph", True) and clean
         self._graphs: dict = {}
         self._graph_seen: dict = {}
         self.graph_records = 0      # recordings made so far
@@ -234,8 +237,6 @@ class ModelRunner:
     def _graph_ok(self, entries: Sequence[StepEntry], metas: List[EntryMeta]) -> bool:
         if not self.use_graphs or self.model.mode != "bfloat16" or len(metas) > self.GRAPH_MAX_BATCH:
             return False
-        if self.cache.state_runs:   # parts with per-request state may run host code of their own
-            return False
         return all(m.count == 1 for m in metas) and all(list(e.want) == [0] for e in entries)
 
     def _graph_key(self, batch: int, max_context: int):
@@ -257,11 +258,14 @@ class ModelRunner:
         key = self._graph_key(len(metas), max_context)
         rec = self._graphs.get(key)
         if rec is None:
-            rec = self._capture(key, entries, metas, want_rows)
+            # The step that meets a new shape runs eagerly (over the recording's own buffers, which sizes them) and is
+            # recorded afterwards without being run again: a part with state of its own must see every step once.
+            rec, logits = self._capture(key, entries, metas, want_rows)
             self._graphs[key] = rec
             self.graph_records += 1
             if len(self._graphs) > self.GRAPH_LIMIT:   # oldest recording out: contexts move on to higher buckets
                 self._graphs.pop(next(iter(self._graphs)))
+            return logits
         rec.wait()
         self._fill(rec.host_np, rec.offsets, entries, metas, want_rows, rec.widths)
         rec.dev.copy_(rec.host, non_blocking=True)
@@ -270,7 +274,7 @@ class ModelRunner:
         self.graph_replays += 1
         return rec.logits.clone()
 
-    def _capture(self, key, entries, metas, want_rows) -> "_Captured":
+    def _capture(self, key, entries, metas, want_rows):
         from ..parts.base import Workspace
 
         batch, bucket = key
@@ -284,8 +288,8 @@ class ModelRunner:
         ctx = self._context(dev, offsets, metas, batch, widths, workspace, bucket)
         self._fill(rec.host_np, offsets, entries, metas, want_rows, widths)
         dev.copy_(host, non_blocking=True)
-        # an eager run first: it sizes the workspace and lets parts build what depends only on the step's shape
-        self.model.forward(ctx, self.views)
+        # the step itself, eagerly: it sizes the workspace and lets parts build what depends only on the step's shape
+        logits = self.model.forward(ctx, self.views)
         torch.cuda.synchronize()
         ctx.extras = {k: v for k, v in ctx.extras.items() if k.startswith("static:")}
         graph = torch.cuda.CUDAGraph()
@@ -294,4 +298,5 @@ class ModelRunner:
         rec.graph = graph
         rec.workspace = workspace
         rec.context = ctx
-        return rec
+        rec.mark()
+        return rec, logits

@@ -8,7 +8,7 @@ from ..weights.store import SafetensorsSource
 from .causal_lm import CausalLM
 
 
-def build_model(config: Any, source: Any, mode: str = "bfloat16", device: Any = "cuda:0", strict: bool = True,
+def build_model(config: Any, source: Any, mode: str = "bfloat16", device: Any = "cuda:0", strict: bool = False,
                 options: Optional[Dict[str, Any]] = None):
     """The model that ``config``'s architecture registered, with weights from ``source``."""
     entry = lookup_architecture(config.architecture)
@@ -17,18 +17,14 @@ def build_model(config: Any, source: Any, mode: str = "bfloat16", device: Any = 
     return CausalLM(config.model_spec(), source, mode=mode, device=device, strict=strict, options=options)
 
 
-def load_model(model_dir: str, mode: str = "bfloat16", device: Any = "cuda:0", strict: bool = True,
+def load_model(model_dir: str, mode: str = "bfloat16", device: Any = "cuda:0", strict: bool = False,
                options: Optional[Dict[str, Any]] = None, config_overrides: Optional[Dict[str, Any]] = None):
     """config.json chooses the class; every *.safetensors file of the folder supplies the weights.
 
     ``config_overrides`` sets fields of the configuration that are options of the engine rather than keys of
-    config.json (such as ``rope_pairing``); the configuration is validated again afterwards."""
+    config.json (such as Qwen3's ``rope_pairing``); the configuration is validated again afterwards.  ``strict``:
+    a tensor in the folder that no part of the model asked for is an error instead of a warning."""
     config = load_config(model_dir)
-    if config_overrides:
-        for key, value in config_overrides.items():
-            if not hasattr(config, key):
-                raise ValueError(f"the configuration of '{config.architecture}' has no field '{key}'")
-            setattr(config, key, value)
-        config.validate(model_dir)
+    config.apply_overrides(config_overrides, model_dir)
     return config, build_model(config, SafetensorsSource(model_dir), mode=mode, device=device, strict=strict,
                                options=options)

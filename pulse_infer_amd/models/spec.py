@@ -10,7 +10,7 @@ describes; configuration classes produce it, ``CausalLM`` consumes it.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass, field, replace
 from typing import Any, Dict, List, Optional
 
 
@@ -27,14 +27,32 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One decoder layer: which parts it is made of and where its weights are."""
+    """One decoder layer: which parts it is made of and where its weights are.
+
+    ``norms`` names a norm for every place the block arrangement has one ("mixer_norm" and "ffn_norm" for the
+    pre-norm block; another arrangement may name more): each is a ``PartSpec`` of its own, so the norms of a layer
+    may differ in kind and in constants.  The block's parameters say under which tensor prefix each of them loads.
+    """
 
     prefix: str
     mixer: PartSpec
     ffn: PartSpec
-    norm: PartSpec
+    norms: Dict[str, PartSpec]
     block: PartSpec = field(default_factory=lambda: PartSpec("prenorm", {"mixer_norm": "input_layernorm",
                                                                          "ffn_norm": "post_attention_layernorm"}))
+
+    def norm(self, place: str) -> PartSpec:
+        try:
+            return self.norms[place]
+        except KeyError:
+            raise KeyError(f"layer '{self.prefix}' names no norm for '{place}' (it has {sorted(self.norms)})") from None
+
+    def with_parts(self, **changes: Any) -> "LayerSpec":
+        """A copy with some of its fields replaced."""
+        return replace(self, **changes)
+
+    def __hash__(self) -> int:
+        return hash((self.prefix, self.mixer, self.ffn, tuple(sorted(self.norms.items())), self.block))
 
 
 @dataclass(frozen=True)

@@ -6,6 +6,7 @@ from typing import List, Optional, Sequence, Tuple
 
 import torch
 
+from .device import compute_units
 from .kernels import _check_cache, _f32, _gpu, _i32, _i64, _int_vec, _need, _ptr, _stream
 from .library import call_in, load_variant
 
@@ -60,7 +61,6 @@ def split_entries(entries: Sequence):
     return short, long
 
 
-CHIP_WORKGROUPS = 256          # compute units: the split kernel's workgroups are counted against them
 SPLIT_OVERHEAD_KEYS = 256      # what a workgroup costs beside its walk (start-up, merge inside it), in keys walked
 MERGE_OVERHEAD_KEYS = 700      # what splitting at all costs (partial results through memory, the second kernel)
 MAX_CHOSEN_SPLITS = 64
@@ -78,6 +78,7 @@ def choose_splits(num_items: int, nkv: int, group: int, max_context: int) -> Tup
     again), 64 in one.  Walks of 4,096 keys and more stream better with two workgroups a unit (16 requests at 8,192:
     4 splits 95.9 us, 2 splits 97.6; at 4,096, walks of 2,048 keys, 2 splits 51.9 us and 4 splits 53.8), so a choice
     that gives every unit one such walk is cut in two once more."""
+    units = compute_units()        # the split kernel's workgroups are counted against them
     groups = num_items * nkv * ((group + 15) // 16)
     whole = (max_context + BLOCK_KEYS - 1) // BLOCK_KEYS * BLOCK_KEYS
     if groups <= 0 or max_context <= 0:
@@ -91,12 +92,12 @@ def choose_splits(num_items: int, nkv: int, group: int, max_context: int) -> Tup
         size = split_size(n)
         if n > 1 and (size < 128 or (n - 1) * size >= max_context):
             continue
-        on_a_unit = (groups * n + CHIP_WORKGROUPS - 1) // CHIP_WORKGROUPS
+        on_a_unit = (groups * n + units - 1) // units
         cost = on_a_unit * (size + SPLIT_OVERHEAD_KEYS) + (MERGE_OVERHEAD_KEYS if n > 1 else 0)
         if best is None or cost < best[0]:
             best = (cost, n)
     n = best[1]
-    if n > 1 and split_size(n) >= 4096 and groups * n * 2 in (CHIP_WORKGROUPS, 2 * CHIP_WORKGROUPS):
+    if n > 1 and split_size(n) >= 4096 and groups * n * 2 in (units, 2 * units):
         n *= 2
     if n == 1:
         return whole, 1
@@ -141,17 +142,19 @@ PREFILL_SCRATCH_BYTES = 512 << 20
 
 
 def choose_prefill_splits(entries: Sequence, portion: int, nkv: int, group: int, d: int, window: int,
-                          target_groups: int = 512, min_blocks: int = 8) -> Tuple[int, int]:
+                          target_groups: Optional[int] = None, min_blocks: int = 8) -> Tuple[int, int]:
     """(split_size, n_splits) for the prompt-portion kernel over these (index, entry) pairs.
 
     A workgroup walks its item's keys block by block, so the longest item sets the kernel's time while the chip
     waits.  Two cases gain from cutting the keys into splits with workgroups of their own: fewer workgroups than the
-    chip runs at a time (``target_groups``; a short portion over a long context), which get as many splits as fill
+    chip runs at a time (``target_groups``, two a compute unit unless given; a short portion over a long context), which get as many splits as fill
     it; and a full chip whose longest item walks much more than its share of all blocks (the late portions of a
     whole prompt), which is cut at one and a half shares.  Splits never hold fewer than ``min_blocks`` blocks, and
     nothing is cut otherwise: the partial results cost a trip through memory and a second launch."""
     if d not in PREFILL_SPLIT_HEAD_DIMS or window > 0:   # (a window keeps every walk short)
         return 0, 1
+    if target_groups is None:
+        target_groups = 2 * compute_units()
     total = longest = tokens = items = 0
     for _, e in entries:
         tokens += e.count

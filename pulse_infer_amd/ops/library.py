@@ -11,6 +11,7 @@ import threading
 from typing import Optional
 
 from ..csrc import build as _build
+from . import timing
 
 
 class KernelLibraryError(RuntimeError):
@@ -72,19 +73,23 @@ def load_variant(source: str, defines: dict) -> ctypes.CDLL:
         return lib
 
 
-def call_in(lib: ctypes.CDLL, name: str, *args) -> None:
+def _invoke(lib: ctypes.CDLL, name: str, args) -> None:
     fn = getattr(lib, name)
     fn.restype = ctypes.c_int
     code = fn(*args)
     if code != 0:
         raise KernelError(f"{name}: {lib.pulse_last_error().decode(errors='replace')}")
+
+
+def call_in(lib: ctypes.CDLL, name: str, *args) -> None:
+    """Call an entry point of ``lib``; a non-zero return becomes a ``KernelError`` with the library's message."""
+    if timing._active is not None:
+        with timing.region(name):
+            _invoke(lib, name, args)
+        return
+    _invoke(lib, name, args)
 
 
 def call(name: str, *args) -> None:
-    """Call an entry point; a non-zero return becomes a ``KernelError`` with the library's message."""
-    lib = load()
-    fn = getattr(lib, name)
-    fn.restype = ctypes.c_int
-    code = fn(*args)
-    if code != 0:
-        raise KernelError(f"{name}: {lib.pulse_last_error().decode(errors='replace')}")
+    """The same for the core library."""
+    call_in(load(), name, *args)

@@ -21,7 +21,7 @@ import torch
 from ..cache.manager import PagedKVSpec
 from ..ops import attention_mfma, kernels
 from ..weights.store import TensorSpec
-from .base import MIXERS, BuildContext, LazyNorm, PagedCacheView, Part, StepContext
+from .base import MIXERS, BuildContext, LazyNorm, PagedCacheView, Part, StepContext, StepCost
 from .linear import Linear
 
 
@@ -40,6 +40,21 @@ class PagedAttention(Part):
             specs["q_norm.weight"] = TensorSpec((d,), kind="norm")
             specs["k_norm.weight"] = TensorSpec((d,), kind="norm")
         return specs
+
+    @classmethod
+    def step_cost(cls, params: Dict[str, Any], entries, weight_bytes: int, cache_bytes: int) -> StepCost:
+        """The projections, plus scores and weighted values over the keys each token sees (2 x 2 x heads x head size
+        a key), plus the keys and values of every request's visible context read once."""
+        cost = super().step_cost(params, entries, weight_bytes, cache_bytes)
+        nq, nkv, d, window = params["num_heads"], params["num_kv_heads"], params["head_dim"], params.get("window")
+        for start, count in entries:
+            seen = 0
+            for p in range(start, start + count):
+                seen += min(p + 1, window) if window else p + 1
+            cost.flops += 4.0 * nq * d * seen
+            context = start + count
+            cost.cache_bytes += 2.0 * nkv * d * cache_bytes * (min(context, window + count - 1) if window else context)
+        return cost
 
     def __init__(self, params: Dict[str, Any], prefix: str, build: BuildContext):
         self.hidden = int(params["hidden_size"])
@@ -73,6 +88,7 @@ class PagedAttention(Part):
 
     accepts_residual = True
     accepts_lazy_input = True   # the first product may compute the norm before it by itself
+    records_cleanly = True      # positions, tables and work lists are read on the device
 
     def forward(self, x, ctx: StepContext, cache: PagedCacheView, residual: Optional[torch.Tensor] = None):
         tokens = x.shape[0]
@@ -144,7 +160,7 @@ class PagedAttention(Part):
                 max((e.start + e.count for _, e in short), default=0))
         short_items, long_items, short_context = ctx.extras[key]
         if long_items is not None:
-            skey = f"static:attention.portion_splits:{portion}:{window}"
+            skey = f"static:attention.portion_splits:{portion}:{window}:{self.nkv}:{group}:{self.d}"
             if skey not in ctx.extras:
                 ctx.extras[skey] = attention_mfma.choose_prefill_splits(
                     attention_mfma.split_entries(ctx.entries)[1], portion, self.nkv, group, self.d, window)

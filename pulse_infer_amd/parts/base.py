@@ -244,14 +244,51 @@ class ResidualStream:
         self.pending = delta
 
 
+@dataclass
+class StepCost:
+    """What a step costs a part: arithmetic, the weights it has to read (once a step, whatever the rows), and what
+    it reads of its cache."""
+
+    flops: float = 0.0
+    weight_bytes: float = 0.0
+    cache_bytes: float = 0.0
+
+    def __add__(self, other: "StepCost") -> "StepCost":
+        return StepCost(self.flops + other.flops, self.weight_bytes + other.weight_bytes,
+                        self.cache_bytes + other.cache_bytes)
+
+
 class Part:
-    """Base of all parts: declares the tensors it loads."""
+    """Base of all parts: declares the tensors it loads and what a step costs it."""
 
     kind = "?"
+    # A step that runs this part may be recorded as a graph and replayed only if the part says so: its forward
+    # must then issue the same launches whatever the step's values are (request slots, positions and tables read
+    # on the device from the step's arrays, no host decision on them, no synchronisation, no library call that
+    # clears memory).  Parts that do not say so keep a model's steps eager.
+    records_cleanly = False
 
     @classmethod
     def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
         return {}
+
+    @classmethod
+    def step_cost(cls, params: Dict[str, Any], entries: List[Tuple[int, int]], weight_bytes: int,
+                  cache_bytes: int) -> StepCost:
+        """The cost of one step of ``entries`` ((tokens already cached, tokens in this step) per request), with
+        ``weight_bytes`` / ``cache_bytes`` a stored element.  Unless a part knows better: every tensor is read once
+        and every matrix is multiplied with every row.  Parts with a cache add what they read of it and the
+        arithmetic over it; a part that reads only some of its tensors (chosen experts) overrides the whole."""
+        rows = sum(count for _, count in entries)
+        cost = StepCost()
+        for spec in cls.weight_specs(params).values():
+            n = 1
+            for dim in spec.shape:
+                n *= dim
+            cost.weight_bytes += n * weight_bytes
+            if len(spec.shape) == 2 and spec.kind == "linear":
+                cost.flops += 2.0 * rows * n
+        return cost
 
 
 def joined(prefix: str, name: str) -> str:

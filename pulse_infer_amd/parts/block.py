@@ -15,14 +15,16 @@ from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BuildContext, Part, Resi
 
 @BLOCKS.register("prenorm")
 class PreNormBlock(Part):
+    NORM_PLACES = ("mixer_norm", "ffn_norm")   # the norms this arrangement has; a layer names a spec for each
+
     @classmethod
     def layer_weight_specs(cls, layer: LayerSpec) -> Dict[str, TensorSpec]:
         """All tensors of one layer, by full name."""
         p = layer.block.params
         out: Dict[str, TensorSpec] = {}
-        norm_cls = NORMS.get(layer.norm.kind)
-        for which in ("mixer_norm", "ffn_norm"):
-            for name, spec in norm_cls.weight_specs(layer.norm.params).items():
+        for which in cls.NORM_PLACES:
+            norm = layer.norm(which)
+            for name, spec in NORMS.get(norm.kind).weight_specs(norm.params).items():
                 out[joined(joined(layer.prefix, p[which]), name)] = spec
         for part, registry in ((layer.mixer, MIXERS), (layer.ffn, FEED_FORWARDS)):
             sub = joined(layer.prefix, part.params.get("prefix", ""))
@@ -32,18 +34,24 @@ class PreNormBlock(Part):
 
     def __init__(self, layer: LayerSpec, build: BuildContext):
         p = layer.block.params
-        norm_cls = NORMS.get(layer.norm.kind)
-        self.mixer_norm = norm_cls(layer.norm.params, joined(layer.prefix, p["mixer_norm"]), build)
-        self.ffn_norm = norm_cls(layer.norm.params, joined(layer.prefix, p["ffn_norm"]), build)
+        made = {}
+        for which in self.NORM_PLACES:
+            norm = layer.norm(which)
+            made[which] = NORMS.get(norm.kind)(norm.params, joined(layer.prefix, p[which]), build)
+        self.mixer_norm, self.ffn_norm = made["mixer_norm"], made["ffn_norm"]
         self.mixer = MIXERS.get(layer.mixer.kind)(layer.mixer.params,
                                                   joined(layer.prefix, layer.mixer.params.get("prefix", "")), build)
         self.ffn = FEED_FORWARDS.get(layer.ffn.kind)(layer.ffn.params,
                                                      joined(layer.prefix, layer.ffn.params.get("prefix", "")), build)
-        self.hidden = int(layer.norm.params["size"])
         self.act_dtype = build.act_dtype
 
     def cache_spec(self) -> Optional[Any]:
         return self.mixer.cache_spec()
+
+    def records_cleanly(self) -> bool:
+        """Whether a step of this block may be recorded as a graph and replayed: every part of it says so."""
+        return all(getattr(part, "records_cleanly", False)
+                   for part in (self.mixer, self.ffn, self.mixer_norm, self.ffn_norm))
 
     def _input(self, stream: ResidualStream, norm: Any, part: Any, ctx: StepContext) -> Any:
         """norm(h) for ``part``: left to the part's first product where that is possible, else computed here."""
@@ -51,7 +59,7 @@ class PreNormBlock(Part):
             lazy = stream.lazy(norm)
             if lazy is not None:
                 return lazy
-        x = ctx.workspace.buffer("block.normed", ctx.num_tokens, self.hidden, self.act_dtype)
+        x = ctx.workspace.buffer("block.normed", ctx.num_tokens, stream.h.shape[1], self.act_dtype)
         return stream.normed(norm, x)
 
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: Any) -> None:

@@ -30,8 +30,17 @@ class TokenEmbedding(Part):
         self.bad_id = torch.zeros(1, dtype=torch.int32, device=build.device)
 
     def forward(self, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """The step function checks ids on the host before it runs.  A caller that comes another way and brings an
+        id outside the table gets a row of NaN, which reaches that token's logits (no token is chosen from them),
+        never a silent row of zeros; ``saw_bad_id`` tells, at the price of a synchronisation."""
         kernels.embed_gather(ids, self.table, out, self.bad_id)
         return out
+
+    def saw_bad_id(self, clear: bool = True) -> bool:
+        seen = bool(self.bad_id.item())
+        if seen and clear:
+            self.bad_id.zero_()
+        return seen
 
 
 class OutputHead(Part):

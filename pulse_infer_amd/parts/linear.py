@@ -16,7 +16,8 @@ from typing import Optional
 
 import torch
 
-from ..ops import kernels
+from ..ops import kernels, timing
+from ..ops.device import compute_units
 from .base import LazyNorm, ResidualStream, RowStats, Workspace
 
 
@@ -54,11 +55,13 @@ class Linear:
                 kernels.gemm_skinny(x, w, out)
                 return out
             if out.dtype == torch.bfloat16:
-                torch.matmul(x, w.t(), out=out)
+                with timing.region("library matmul"):
+                    torch.matmul(x, w.t(), out=out)
                 return out
             if out.dtype == torch.float32 and out.is_contiguous():
                 # float32 results of many rows (logits): the library's product with a float32 output
-                torch.mm(x, w.t(), out_dtype=torch.float32, out=out)
+                with timing.region("library matmul (float32 out)"):
+                    torch.mm(x, w.t(), out_dtype=torch.float32, out=out)
                 return out
             if w.shape[1] % 8 == 0:  # otherwise the few-rows kernel, 64 rows at a time
                 for r0 in range(0, x.shape[0], kernels.SKINNY_MAX_ROWS):
@@ -92,7 +95,8 @@ class Linear:
                                      self.out_features, torch.float32).view(splits, rows, self.out_features)
             xa = x.view(rows, splits, share).transpose(0, 1)
             wb = self.weight.view(self.out_features, splits, share).permute(1, 2, 0)
-            torch.bmm(xa, wb, out_dtype=torch.float32, out=parts)
+            with timing.region("library batched matmul"):
+                torch.bmm(xa, wb, out_dtype=torch.float32, out=parts)
             return parts
         if (self.library and x.dtype == torch.bfloat16 and x.shape[0] <= kernels.SKINNY_FAST_ROWS
                 and kernels.gemm_skinny_ok(x, self.weight)):
@@ -158,17 +162,18 @@ class Linear:
         the library's 100 + 5: no shape shares 200 rows a unit out evenly, so the library takes that one (the rule:
         this product's estimate must stay below 1.5 x the weight rows a unit)."""
         n = self.out_features
-        if n <= 32 * self.MID_UNITS:
+        units = compute_units()
+        if n <= 32 * units:
             return 2    # too few weight rows to fill the chip in any shape: the most workgroups
         best = None
         for waves in (2, 4, 6, 10):
-            on_a_unit = ((n + 16 * waves - 1) // (16 * waves) + self.MID_UNITS - 1) // self.MID_UNITS
+            on_a_unit = ((n + 16 * waves - 1) // (16 * waves) + units - 1) // units
             cost = on_a_unit * (16 * waves + rows // 2)
             if best is None or cost < best[0]:
                 best = (cost, waves)
-        if n <= 64 * self.MID_UNITS:
+        if n <= 64 * units:
             return best[1]    # (12,288 weight rows: 64 rows a workgroup 12 to 15 us, the library 15 to 18 + 5)
-        return best[1] if best[0] * self.MID_UNITS < 1.5 * n else 0
+        return best[1] if best[0] * units < 1.5 * n else 0
 
     def shares_for(self, x: torch.Tensor) -> int:
         """Into how many shares the inner dimension is cut for an update in parts; 0: not this product."""
@@ -179,7 +184,7 @@ class Linear:
         partial results the next norm adds up; (0, 0): not this product.
 
         The pair with the least estimated time of the fullest compute unit is taken: workgroups on it (all of them
-        over 256 units, rounded up) x weight rows a workgroup x (length of a share + 280, what a workgroup costs
+        over the compute units, rounded up) x weight rows a workgroup x (length of a share + 280, what a workgroup costs
         beside its walk), plus half a microsecond a share for the norm that adds them up.  Measured at 64 rows: down
         of the 8B shape 4 shares of 64 rows (256 workgroups) 23.8 us, 8 shares 24.9, 6 shares (384 workgroups, two on
         half the units) 28.6; down of the 14B shape 4 shares of 96 rows (216 workgroups) 40.9 us, 8 shares of 64 rows
@@ -188,6 +193,7 @@ class Linear:
                 and self.operands_ok(x)) or self.out_features % 4:
             return 0, 0
         best = None
+        units = compute_units()
         for waves in (4, 6):
             rows = 16 * waves
             tiles = (self.out_features + rows - 1) // rows
@@ -195,10 +201,9 @@ class Linear:
                 if self.in_features % splits or (self.in_features // splits) % 128:
                     continue
                 share = self.in_features // splits
-                on_a_unit = (tiles * splits + self.MID_UNITS - 1) // self.MID_UNITS
+                on_a_unit = (tiles * splits + units - 1) // units
                 cost = on_a_unit * rows * (share + 280) + 8000 * splits
                 if best is None or cost < best[0]:
                     best = (cost, splits, waves)
         return (best[1], best[2]) if best else (0, 0)
 
-    MID_UNITS = 256              # compute units

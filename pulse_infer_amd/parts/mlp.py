@@ -51,6 +51,7 @@ class GatedMLP(Part):
 
     accepts_residual = True
     accepts_lazy_input = True   # the first product may compute the norm before it by itself
+    records_cleanly = True
 
     def forward(self, x, ctx: StepContext, residual: Optional[torch.Tensor] = None):
         tokens = x.shape[0]

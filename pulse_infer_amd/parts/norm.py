@@ -22,6 +22,7 @@ class RMSNorm(Part):
         self.eps = float(params["eps"])
         self.weight = build.loader.get(f"{prefix}.weight")
 
+    records_cleanly = True
     takes_parts = True   # delta may be [parts, T, H] float32: the kernel adds the parts in order
 
     def apply(self, h: torch.Tensor, delta: Optional[torch.Tensor], out: torch.Tensor,

@@ -29,6 +29,8 @@ class RotationTables:
 
 @POSITIONS.register("rope")
 class RotaryEmbedding(Part):
+    records_cleanly = True
+
     def __init__(self, params: Dict[str, Any], build: BuildContext):
         self.theta = float(params["theta"])
         self.rotary_dim = int(params["rotary_dim"])
@@ -57,6 +59,8 @@ class RotaryEmbedding(Part):
 @POSITIONS.register("none")
 class NoPositionEncoding(Part):
     """Attention that learns order from the causal mask alone."""
+
+    records_cleanly = True
 
     def __init__(self, params: Dict[str, Any], build: BuildContext):
         pass

@@ -8,8 +8,10 @@ from conftest import TINY_A, TINY_B, TINY_W
 from pulse_infer_amd.config import (ConfigError, Qwen3Config, config_from_dict, load_config, lookup_architecture,
                                     register_architecture, registered_architectures, unregister_architecture)
 
+# the keys the reference requires (src/model/qwen3/config.cpp:250-325), torch_dtype apart (a string, tested below)
 REQUIRED = ["head_dim", "hidden_size", "intermediate_size", "max_position_embeddings", "num_attention_heads",
-            "num_hidden_layers", "rms_norm_eps", "rope_theta", "vocab_size"]
+            "num_hidden_layers", "num_key_value_heads", "rms_norm_eps", "rope_theta", "tie_word_embeddings",
+            "vocab_size"]
 
 
 def test_reads_every_size_from_the_keys():
@@ -19,7 +21,7 @@ def test_reads_every_size_from_the_keys():
         assert getattr(a, key) != getattr(b, key), f"the tiny configurations should differ in {key}"
 
 
-@pytest.mark.parametrize("key", [k for k in REQUIRED if k != "head_dim"])
+@pytest.mark.parametrize("key", REQUIRED + ["torch_dtype"])
 def test_missing_required_key_is_named(key):
     data = dict(TINY_A)
     del data[key]
@@ -40,9 +42,9 @@ def test_head_dim_is_free_of_hidden_size():
 
 
 def test_validation():
-    with pytest.raises(ConfigError, match="not divisible"):
+    with pytest.raises(ConfigError, match="shared out evenly"):
         Qwen3Config.from_dict(dict(TINY_A, num_attention_heads=5))
-    with pytest.raises(ConfigError, match="Invalid model dimensions"):
+    with pytest.raises(ConfigError, match="sizes must be positive"):
         Qwen3Config.from_dict(dict(TINY_A, vocab_size=0))
     with pytest.raises(ConfigError, match="even"):
         Qwen3Config.from_dict(dict(TINY_A, head_dim=15))
@@ -137,7 +139,7 @@ def test_registry(tmp_path):
         assert isinstance(load_config(str(tmp_path)), Other)
     finally:
         unregister_architecture("OtherForCausalLM")
-    with pytest.raises(ConfigError, match="does not exist"):
+    with pytest.raises(ConfigError, match="there is no file"):
         load_config(str(tmp_path / "nowhere"))
 
 

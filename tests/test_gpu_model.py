@@ -271,14 +271,14 @@ def test_benchmark_layer_sizes_recorded_decode_steps(layer_shape, batch):
     for graphs in (True, False):
         runner = ModelRunner(model, page_size=16, num_pages=sum((n + steps + 15) // 16 for n in lengths) + 2,
                              max_requests=batch, use_graphs=graphs)
-        runner.GRAPH_AFTER_STEPS = 1                     # record at once: every single-token step here is a replay
+        runner.GRAPH_AFTER_STEPS = 1                     # record at once: all other single-token steps are replays
         for r, n in enumerate(lengths):
             runner.add_request(r)
             runner.reserve(r, n + steps)
             runner.step([StepEntry(r, ids[r][:n], [])])
         got = [runner.step([StepEntry(r, [ids[r][n + s]], [0]) for r, n in enumerate(lengths)]) for s in range(steps)]
         results.append(torch.stack(got))                 # [steps, batch, vocab]
-        assert runner.graph_replays == (steps if graphs else 0)
+        assert runner.graph_replays == (steps - 2 if graphs else 0)
         assert runner.graph_records == (2 if graphs else 0)      # contexts up to 1,024, then up to 2,048
         for r in range(batch):
             runner.free_request(r)

@@ -168,18 +168,29 @@ def test_attention_part(gpu, mode, variant):
 
 
 # ----------------------------------------------------------------- toy parts
+TOY = dict(architectures=["ToyForCausalLM"], vocab=211, width=96, depth=4, heads=6, kv_heads=2, head_width=32, inner=160,
+           most_positions=256, eps=2e-6, theta=3e4, decay=0.5)
+
+
 def register_toys():
-    """A mixer with state of its own (a decayed running sum per request), a position encoding that adds
-    nothing, and an architecture that uses them beside ordinary attention layers."""
+    """An architecture of its own: a configuration class with keys of its own (it derives from the engine's
+    ``ModelConfig`` only), a mixer with state of its own (a decayed running sum per request) in its odd layers,
+    whose feed-forward norm is of another kind than the layer's other norm (a toy norm that centres the row first),
+    beside ordinary attention layers."""
+    from dataclasses import dataclass
     from pulse_infer_amd.cache import StateSpec
-    from pulse_infer_amd.config import Qwen3Config, register_architecture
+    from pulse_infer_amd.config import ConfigError, JsonReader, ModelConfig, register_architecture
     from pulse_infer_amd.models.spec import LayerSpec, ModelSpec, PartSpec, RunSpec
-    from pulse_infer_amd.parts.base import MIXERS, Part
+    from pulse_infer_amd.ops import kernels
+    from pulse_infer_amd.parts.base import MIXERS, NORMS, Part
     from pulse_infer_amd.weights import TensorSpec
 
     @MIXERS.register("toy_running_sum", replace=True)
     class RunningSum(Part):
-        """state <- decay * state + x_t, output_t = state W^T; the state lives in the request's slot."""
+        """state <- decay * state + x_t, output_t = state W^T; the state lives in the request's slot.  A step of single
+        tokens reads slots and starts from the step's device arrays only, so it records cleanly."""
+
+        records_cleanly = True
 
         @classmethod
         def weight_specs(cls, params):
@@ -195,6 +206,14 @@ def register_toys():
 
         def forward(self, x, ctx, cache):
             out = torch.empty(x.shape[0], self.hidden, dtype=torch.float32, device=x.device)
+            if ctx.max_count == 1:                     # one token a request: no host value decides anything
+                slots = ctx.entry_slot.long()
+                old = cache.state.index_select(0, slots)
+                old = torch.where((ctx.entry_start == 0).unsqueeze(1), torch.zeros_like(old), old)
+                new = old * self.decay + x.float()
+                cache.state.index_copy_(0, slots, new)
+                kernels.gemm_f32(new, self.weight, out)
+                return out.to(self.act)
             for e in ctx.entries:
                 state = cache.state[e.slot]
                 if e.start == 0:
@@ -204,25 +223,123 @@ def register_toys():
                     out[row] = state @ self.weight.t()
             return out.to(self.act)
 
-    class ToyConfig(Qwen3Config):
+    @NORMS.register("toy_centered", replace=True)
+    class CenteredNorm(Part):
+        """y = (x - mean) / sqrt(var + eps) * w over the row, x = h + delta."""
+
+        records_cleanly = True
+
+        @classmethod
+        def weight_specs(cls, params):
+            return {"weight": TensorSpec((params["size"],), kind="norm")}
+
+        def __init__(self, params, prefix, build):
+            self.eps = params["eps"]
+            self.weight = build.loader.get(f"{prefix}.weight").float()
+
+        def apply(self, h, delta, out, rows=None):
+            if delta is not None and rows is None:
+                h.add_(delta.float())
+            x = h if delta is None or rows is None else h + delta.float()
+            if rows is not None:
+                x = x.index_select(0, rows.long())
+            x = x - x.mean(dim=-1, keepdim=True)
+            out.copy_(x * torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + self.eps) * self.weight)
+            return out
+
+    @dataclass
+    class ToyConfig(ModelConfig):
+        vocab_size: int
+        width: int
+        depth: int
+        heads: int
+        kv_heads: int
+        head_width: int
+        inner: int
+        most_positions: int
+        eps: float
+        theta: float
+        decay: float
+        odd_norm: str = "toy_centered"      # an option of the engine: which norm stands before an odd layer's feed-forward
+        architecture: str = "ToyForCausalLM"
+
+        engine_options = {"odd_norm": {"choices": ["toy_centered", "rmsnorm"], "help": "norm before an odd layer's feed-forward"}}
+
+        @classmethod
+        def from_dict(cls, data, origin="<dict>", generation=None, generation_origin="<dict>"):
+            r = JsonReader(data, origin)
+            cfg = cls(vocab_size=r.integer("vocab"), width=r.integer("width"), depth=r.integer("depth"),
+                      heads=r.integer("heads"), kv_heads=r.integer("kv_heads"), head_width=r.integer("head_width"),
+                      inner=r.integer("inner"), most_positions=r.integer("most_positions"), eps=r.number("eps"),
+                      theta=r.number("theta"), decay=r.number("decay"))
+            cfg.read_generation_defaults(generation, generation_origin)
+            cfg.validate(origin)
+            return cfg
+
+        def validate(self, origin="<config>"):
+            if not 0.0 < self.decay < 1.0:
+                raise ConfigError(f"'{origin}': decay must lie between 0 and 1, got {self.decay}")
+            if self.odd_norm not in ("toy_centered", "rmsnorm"):
+                raise ConfigError(f"'{origin}': odd_norm '{self.odd_norm}' is unknown")
+
+        def to_dict(self):
+            return dict(architectures=[self.architecture], vocab=self.vocab_size, width=self.width, depth=self.depth,
+                        heads=self.heads, kv_heads=self.kv_heads, head_width=self.head_width, inner=self.inner,
+                        most_positions=self.most_positions, eps=self.eps, theta=self.theta, decay=self.decay)
+
         def model_spec(self):
-            base = super().model_spec()
+            rms = PartSpec("rmsnorm", {"size": self.width, "eps": self.eps})
+            odd = PartSpec(self.odd_norm, {"size": self.width, "eps": self.eps})
+            ffn = PartSpec("gated_mlp", {"hidden_size": self.width, "intermediate_size": self.inner, "prefix": "mlp"})
             layers = []
-            for i, layer in enumerate(base.layers):
+            for i in range(self.depth):
                 if i % 2 == 1:
-                    mixer = PartSpec("toy_running_sum", {"hidden_size": self.hidden_size, "decay": 0.5, "prefix": "toy"})
-                    layer = LayerSpec(layer.prefix, mixer, layer.ffn, layer.norm, layer.block)
-                layers.append(layer)
-            base.layers = layers
-            base.architecture = "ToyForCausalLM"
-            return base
+                    mixer = PartSpec("toy_running_sum", {"hidden_size": self.width, "decay": self.decay, "prefix": "toy"})
+                    norms = {"mixer_norm": rms, "ffn_norm": odd}
+                else:
+                    mixer = PartSpec("attention", {
+                        "hidden_size": self.width, "num_heads": self.heads, "num_kv_heads": self.kv_heads,
+                        "head_dim": self.head_width, "qk_norm": True, "qk_norm_eps": self.eps,
+                        "scale": self.head_width ** -0.5, "window": None, "position": "rope", "prefix": "self_attn"})
+                    norms = {"mixer_norm": rms, "ffn_norm": rms}
+                layers.append(LayerSpec(f"model.layers.{i}", mixer, ffn, norms))
+            return ModelSpec(
+                architecture=self.architecture, vocab_size=self.vocab_size, hidden_size=self.width,
+                max_positions=self.most_positions,
+                embedding=PartSpec("embedding", {"vocab_size": self.vocab_size, "hidden_size": self.width,
+                                                 "name": "model.embed_tokens.weight"}),
+                layers=layers, order=[RunSpec(i) for i in range(self.depth)], final_norm=rms,
+                head=PartSpec("lm_head", {"vocab_size": self.vocab_size, "hidden_size": self.width, "name": "lm_head.weight",
+                                          "tied": False, "tied_to": "model.embed_tokens.weight"}),
+                positions={"rope": PartSpec("rope", {"theta": self.theta, "rotary_dim": self.head_width,
+                                                     "head_dim": self.head_width, "pairing": "interleaved"})})
 
     register_architecture("ToyForCausalLM", ToyConfig, replace=True)
     return ToyConfig
 
 
-def plain_toy_logits(plain, ids, decay):
-    """The toy model with plain functions: odd layers use the running sum in place of attention."""
+def unregister_toys():
+    from pulse_infer_amd.config import unregister_architecture
+    from pulse_infer_amd.parts.base import MIXERS, NORMS
+
+    unregister_architecture("ToyForCausalLM")
+    MIXERS.unregister("toy_running_sum")
+    NORMS.unregister("toy_centered")
+
+
+def toy_plain(folder):
+    """The plain decoder over the toy's tensors (its attention layers are ordinary ones): the toy's keys under the
+    names the plain implementation reads."""
+    from safetensors.torch import load_file
+    c = dict(num_attention_heads=TOY["heads"], num_key_value_heads=TOY["kv_heads"], head_dim=TOY["head_width"],
+             hidden_size=TOY["width"], rms_norm_eps=TOY["eps"], rope_theta=TOY["theta"], num_hidden_layers=TOY["depth"],
+             vocab_size=TOY["vocab"])
+    return P.PlainQwen3(c, load_file(f"{folder}/model.safetensors"))
+
+
+def plain_toy_logits(plain, ids, odd_norm="toy_centered"):
+    """The toy model with plain functions: odd layers use the running sum in place of attention, and centre the row
+    in the norm before their feed-forward."""
     c, w = plain.c, plain.w
     h = P.embedding(w["model.embed_tokens.weight"], ids)
     pos = list(range(len(ids)))
@@ -234,34 +351,44 @@ def plain_toy_logits(plain, ids, decay):
         a = P.rms_norm(h, w[p + "input_layernorm.weight"], c["rms_norm_eps"])
         state, rows = torch.zeros(h.shape[1], dtype=F64), []
         for t in range(len(ids)):
-            state = decay * state + a[t]
+            state = TOY["decay"] * state + a[t]
             rows.append(state @ w[p + "toy.mix.weight"].T)
         h = h + torch.stack(rows)
-        m = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], c["rms_norm_eps"])
+        if odd_norm == "toy_centered":
+            x = h - h.mean(dim=-1, keepdim=True)
+            m = x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + c["rms_norm_eps"]) * w[p + "post_attention_layernorm.weight"]
+        else:
+            m = P.rms_norm(h, w[p + "post_attention_layernorm.weight"], c["rms_norm_eps"])
         h = h + P.gated_mlp(m, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
     return P.linear(P.rms_norm(h, w["model.norm.weight"], c["rms_norm_eps"]), w["lm_head.weight"])
 
 
+def plain_toy_greedy(plain, prompt, steps, odd_norm="toy_centered"):
+    ids, out = list(prompt), []
+    for _ in range(steps):
+        out.append(int(torch.argmax(plain_toy_logits(plain, ids, odd_norm)[-1])))
+        ids.append(out[-1])
+    return out
+
+
 def test_a_toy_mixer_with_state_is_registered_built_and_stepped(gpu, tmp_path):
-    from conftest import TINY_B
+    from pulse_infer_amd.config import load_config
     from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
     from pulse_infer_amd.models.factory import load_model
     from pulse_infer_amd.weights import write_model_folder
-    from pulse_infer_amd.config import unregister_architecture
-    from pulse_infer_amd.parts.base import MIXERS
     from test_gpu_model import close
 
     toy_config = register_toys()
     try:
-        cfg = toy_config.from_dict(dict(TINY_B, architectures=["ToyForCausalLM"], num_hidden_layers=4))
-        cfg.architecture = "ToyForCausalLM"
-        folder = write_model_folder(cfg, str(tmp_path / "toy"), seed=21)
-        plain = P.PlainQwen3.from_folder(folder)
-        _, model = load_model(folder, mode="float32")
+        folder = write_model_folder(toy_config.from_dict(TOY), str(tmp_path / "toy"), seed=21)
+        plain = toy_plain(folder)
+        config, model = load_model(folder, mode="float32")
+        assert type(config) is toy_config and type(load_config(folder)) is toy_config
         assert type(model.blocks[1].mixer).__name__ == "RunningSum"
+        assert type(model.blocks[1].ffn_norm).__name__ == "CenteredNorm" and type(model.blocks[1].mixer_norm).__name__ == "RMSNorm"
         runner = ModelRunner(model, page_size=16, num_pages=16, max_requests=2)
         assert len(runner.cache.groups) == 1 and sorted(runner.cache.state_runs) == [1, 3]
-        ids = {k: token_ids(cfg.vocab_size, n, seed=60 + n) for k, n in (("a", 40), ("b", 23), ("c", 31))}
+        ids = {k: token_ids(config.vocab_size, n, seed=60 + n) for k, n in (("a", 40), ("b", 23), ("c", 31))}
         got = {k: [] for k in ids}
         # a and b interleaved (portions beside single tokens); c afterwards in b's slot, whose state must not leak
         plan = [[("a", 7), ("b", 2)], [("a", 1), ("b", 9)], [("b", 1)], [("a", 20), ("b", 11)], [("a", 12)],
@@ -284,10 +411,100 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(gpu, tmp_path):
                 if fed[k] == len(ids[k]) and runner.cache.has_request(k):
                     runner.free_request(k)
         for k in ids:
-            close(torch.cat(got[k]), plain_toy_logits(plain, ids[k], 0.5), "float32", f"toy request {k}")
+            close(torch.cat(got[k]), plain_toy_logits(plain, ids[k]), "float32", f"toy request {k}")
     finally:
-        unregister_architecture("ToyForCausalLM")
-        MIXERS.unregister("toy_running_sum")
+        unregister_toys()
+
+
+def test_a_toy_architecture_runs_through_the_entry_points(gpu, tmp_path, capsys):
+    """The toy's own configuration class (no Qwen3 field in it) through ``LLM.from_pretrained`` / ``generate`` and
+    through the command line, including the option its class declares and ``--set``; greedy tokens against the
+    plain formulas."""
+    import json
+    from pulse_infer_amd import LLM, cli
+    from pulse_infer_amd.config import ConfigError
+    from pulse_infer_amd.weights import write_model_folder
+
+    toy_config = register_toys()
+    try:
+        folder = write_model_folder(toy_config.from_dict(TOY), str(tmp_path / "toy"), seed=23)
+        plain = toy_plain(folder)
+        prompts = [token_ids(TOY["vocab"], n, seed=30 + n) for n in (9, 21)]
+        llm = LLM.from_pretrained(folder, dtype="float32", max_batch_size=2, chunk_size=8, page_size=16, num_pages=16)
+        assert llm.generate(prompts, max_new_tokens=5, ignore_eos=True) == [plain_toy_greedy(plain, p, 5) for p in prompts]
+        common = [folder, "--dtype", "f32", "--prompt-ids", ",".join(map(str, prompts[0])), "--max-new-tokens", "4",
+                  "--num-pages", "16", "--ignore-eos"]
+        assert cli.main(common) == 0
+        assert json.loads(capsys.readouterr().out.splitlines()[0])["output_ids"] == plain_toy_greedy(plain, prompts[0], 4)
+        for how in (["--odd-norm", "rmsnorm"], ["--set", "odd_norm=rmsnorm"]):
+            assert cli.main(common + how) == 0
+            assert json.loads(capsys.readouterr().out.splitlines()[0])["output_ids"] == \
+                plain_toy_greedy(plain, prompts[0], 4, "rmsnorm")
+        with pytest.raises(ConfigError, match="no field 'rope_pairing'"):
+            cli.main(common + ["--set", "rope_pairing=half"])
+        with pytest.raises(SystemExit):
+            cli.main(common + ["--rope-pairing", "half"])            # an option of another architecture
+    finally:
+        unregister_toys()
+
+
+def test_a_toy_mixer_that_records_cleanly_is_replayed(gpu, tmp_path):
+    """bfloat16: the toy says that its parts record cleanly, so steps of single tokens run as replays of a recording
+    although the model has per-request state: every replay against the eager step, with eager prompt portions of
+    another request in between, a request that restarts in a used slot, and the plain formulas."""
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.weights import write_model_folder
+    from test_gpu_model import SPLIT_TOL, close
+
+    toy_config = register_toys()
+    try:
+        folder = write_model_folder(toy_config.from_dict(TOY), str(tmp_path / "toy"), seed=25)
+        plain = toy_plain(folder)
+        _, model = load_model(folder, mode="bfloat16")
+        ids = {k: token_ids(TOY["vocab"], n, seed=40 + n) for k, n in (("a", 46), ("b", 37), ("c", 25))}
+        outs = []
+        for graphs in (True, False):
+            runner = ModelRunner(model, page_size=16, num_pages=16, max_requests=2, use_graphs=graphs)
+            runner.GRAPH_AFTER_STEPS = 1
+            assert runner.use_graphs == graphs
+            fed, got = {k: 0 for k in ids}, {k: [] for k in ids}
+
+            def feed(pairs):
+                entries = []
+                for k, n in pairs:
+                    if not runner.cache.has_request(k):
+                        runner.add_request(k)
+                    runner.reserve(k, fed[k] + n)
+                    entries.append(StepEntry(k, ids[k][fed[k]:fed[k] + n], list(range(n))))
+                    fed[k] += n
+                logits = runner.step(entries)
+                row = 0
+                for k, n in pairs:
+                    got[k].append(logits[row:row + n])
+                    row += n
+
+            feed([("a", 18), ("b", 5)])
+            for _ in range(8):
+                feed([("a", 1), ("b", 1)])
+            feed([("b", 9)])                               # eager work between the replays
+            for _ in range(15):
+                feed([("b", 1), ("a", 1)])
+            feed([("a", 1)])                               # a step of one request: its shape is recorded here ..
+            runner.free_request("b")
+            feed([("c", 1)])                               # .. and replayed here, where c starts in the slot b left
+            for _ in range(3):
+                feed([("a", 1), ("c", 1)])
+            feed([("c", 20)])
+            assert runner.graph_replays == (7 + 15 + 1 + 3 if graphs else 0) and runner.graph_records == (2 if graphs else 0)
+            outs.append({k: torch.cat(v) for k, v in got.items()})
+            del runner
+        for k in ids:
+            want = plain_toy_logits(plain, ids[k])[:outs[0][k].shape[0]]
+            close(outs[0][k], want, "bfloat16", f"recorded toy, request {k}")
+            close(outs[0][k], outs[1][k], "bfloat16", f"recorded toy against eager, request {k}", SPLIT_TOL)
+    finally:
+        unregister_toys()
 
 
 def test_order_may_name_a_layer_twice_and_share_a_cache(gpu, tmp_path):
@@ -414,7 +631,7 @@ def register_routed_toys():
                     mixer = PartSpec("attention", dict(mixer.params, position="bands"))
                 else:
                     ffn = PartSpec("toy_routed", dict(ROUTED, hidden_size=self.hidden_size, prefix="moe"))
-                layers.append(LayerSpec(layer.prefix, mixer, ffn, layer.norm, layer.block))
+                layers.append(layer.with_parts(mixer=mixer, ffn=ffn))
             base.layers = layers
             base.architecture = "RoutedToyForCausalLM"
             return base

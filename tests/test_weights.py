@@ -95,10 +95,38 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes():
     for needle in ("somewhere", "missing tensors (2)", "model.norm.weight", "unexpected tensors (1)", "inv_freq",
                    "wrong shapes (2)", "expected [192, 96], found [5, 7]", "expected [32], found [33]"):
         assert needle in text, needle
-    # non-strict loading tolerates the unexpected tensor but nothing else
-    with pytest.raises(WeightError) as lenient:
-        check(DictSource(tensors), expected, strict=False)
-    assert lenient.value.unexpected == [] and len(lenient.value.missing) == 2
+
+
+def test_tensors_that_no_part_asked_for():
+    """Alone they do not fail a load (a warning counts them) unless strict is set; when the load fails anyway the
+    error names them, strict or not."""
+    cfg = Qwen3Config.from_dict(TINY_B)
+    expected = expected_tensors(cfg.model_spec())
+    tensors = {n: torch.zeros(s.shape, dtype=torch.bfloat16) for n, s in expected.items()}
+    tensors["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)
+    tensors["extra.bias"] = torch.zeros(3)
+    assert check(DictSource(tensors), expected) == ["extra.bias", "model.layers.0.self_attn.rotary_emb.inv_freq"]
+    with pytest.warns(UserWarning, match="2 tensors .* belong to no part"):
+        loader = WeightLoader(DictSource(tensors, "folder"), expected, "bfloat16", "cpu")
+    assert loader.ignored == ["extra.bias", "model.layers.0.self_attn.rotary_emb.inv_freq"]
+    with pytest.raises(WeightError, match=r"unexpected tensors \(2\)") as strict:
+        check(DictSource(tensors), expected, strict=True)
+    assert not strict.value.missing and not strict.value.wrong_shape
+    del tensors["model.norm.weight"]
+    with pytest.raises(WeightError) as err:
+        check(DictSource(tensors), expected)
+    assert err.value.missing == ["model.norm.weight"] and len(err.value.unexpected) == 2
+
+
+def test_float16_is_not_rounded_to_bfloat16_silently():
+    expected = {"w": TensorSpec((2, 2)), "v": TensorSpec((2, 2)), "n": TensorSpec((2,), kind="norm")}
+    big = torch.tensor([[1.0009765625, 2.0], [3.0, 4.0]], dtype=torch.float16)    # 1 + 2^-10: no bfloat16 value
+    src = DictSource({"w": big, "v": torch.ones(2, 2, dtype=torch.bfloat16), "n": torch.ones(2)}, "half")
+    with pytest.raises(WeightError, match="would round") as err:
+        WeightLoader(src, expected, "bfloat16", "cpu")
+    assert err.value.narrowed == [("w", "float16")] and "w (float16)" in str(err.value)
+    wide = WeightLoader(src, expected, "float32", "cpu").get("w")                 # the 32-bit run widens it exactly
+    assert wide.dtype == torch.float32 and wide[0, 0].item() == 1.0009765625
 
 
 def test_tied_head_is_optional_untied_head_is_required():
@@ -113,7 +141,9 @@ def test_tied_head_is_optional_untied_head_is_required():
 
 def test_storage_types():
     assert storage_dtype(torch.bfloat16, "bfloat16") == torch.bfloat16
-    assert storage_dtype(torch.float16, "bfloat16") == torch.bfloat16
+    with pytest.raises(ValueError, match="rounding"):
+        storage_dtype(torch.float16, "bfloat16")
+    assert storage_dtype(torch.float16, "float32") == torch.float32
     assert storage_dtype(torch.float32, "bfloat16") == torch.float32   # a tensor stored in 32-bit stays so
     assert storage_dtype(torch.int64, "bfloat16") == torch.int32       # integer tables
     assert storage_dtype(torch.bfloat16, "float32") == torch.float32
