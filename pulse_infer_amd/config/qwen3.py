@@ -4,8 +4,11 @@ Required keys are the ones the reference requires
 (reference: src/model/qwen3/config.cpp:250-325); optional sampling defaults
 come from generation_config.json (reference: src/model/qwen3/config.cpp:333-365).
 Keys the reference never reads (``attention_bias``, ``hidden_act``,
-``rope_scaling``) are read here only to refuse values this engine has no
-formula for.  The sliding-window keys choose a window per layer.
+``rope_scaling``, ``use_sliding_window``, ``layer_types``) are read here only to
+refuse values that the reference has no formula for: it attends to all keys in
+every layer, whatever those keys say.  Attention windows are a parameter of the
+attention part and an option of the engine (``layer_windows``), not something
+config.json can ask for.
 """
 from __future__ import annotations
 
@@ -33,10 +36,9 @@ class Qwen3Config(ModelConfig):
     tie_word_embeddings: bool = False
     torch_dtype: str = "bfloat16"
     eos_token_ids: List[int] = field(default_factory=list)
-    use_sliding_window: bool = False
+    # read back and written out unchanged (the reference never reads them); only "no window" is accepted
     sliding_window: Optional[int] = None
     max_window_layers: Optional[int] = None
-    layer_types: Optional[List[str]] = None
     # sampling defaults (generation_config.json)
     temperature: float = 0.0
     top_k: int = 0
@@ -45,11 +47,19 @@ class Qwen3Config(ModelConfig):
     # (2i, 2i+1), what the reference computes (src/ops/kernels/cuda/rope_kernel.cu:100-126); "half" is
     # (i, i + d/2), for checkpoints whose q/k projections were trained under that convention.
     rope_pairing: str = "interleaved"
+    # Another option of the engine: an attention window per layer (None or 0: all keys; w: the last w keys, the
+    # token's own included).  Layers with a window form a cache group of their own whose pages are given back once
+    # the window has passed them.  The reference has no windows, so no key of config.json sets this.
+    layer_windows: Optional[List[Optional[int]]] = None
     architecture: str = ARCHITECTURE
 
-    engine_options = {"rope_pairing": {
-        "choices": ["interleaved", "half"],
-        "help": "channels a rotation pairs: interleaved (2i, 2i+1), as the reference computes, or half (i, i + d/2)"}}
+    engine_options = {
+        "rope_pairing": {
+            "choices": ["interleaved", "half"],
+            "help": "channels a rotation pairs: interleaved (2i, 2i+1), as the reference computes, or half (i, i + d/2)"},
+        "layer_windows": {
+            "type": lambda text: [int(w) or None for w in text.split(",")],
+            "help": "an attention window per layer, comma separated, 0 for all keys (the reference has none)"}}
 
     # ------------------------------------------------------------------ reading
     @classmethod
@@ -76,10 +86,8 @@ class Qwen3Config(ModelConfig):
             tie_word_embeddings=r.boolean("tie_word_embeddings"),
             torch_dtype=dtype,
             eos_token_ids=r.int_or_int_list("eos_token_id"),
-            use_sliding_window=r.boolean("use_sliding_window", False),
             sliding_window=r.integer("sliding_window", None),
             max_window_layers=r.integer("max_window_layers", None),
-            layer_types=r.string_list("layer_types"),
         )
         # values this engine has no formula for
         if r.boolean("attention_bias", False):
@@ -87,6 +95,13 @@ class Qwen3Config(ModelConfig):
         act = r.string("hidden_act", "silu")
         if act != "silu":
             raise ConfigError(f"'hidden_act': '{act}' is not supported, only 'silu' (in '{origin}')")
+        if r.boolean("use_sliding_window", False):
+            raise ConfigError(f"'{origin}': 'use_sliding_window': true is not supported: the reference attends to all "
+                              f"keys in every layer; windows are an option of the engine (layer_windows)")
+        kinds = r.string_list("layer_types")
+        if kinds is not None and any(kind != "full_attention" for kind in kinds):
+            other = sorted(set(kinds) - {"full_attention"})
+            raise ConfigError(f"'{origin}': 'layer_types' other than 'full_attention' are not supported ({', '.join(other)})")
         scaling = r.raw("rope_scaling")
         if scaling is not None and not (isinstance(scaling, dict) and scaling.get("rope_type", scaling.get("type")) == "default"):
             raise ConfigError(f"'rope_scaling' other than null is not supported (in '{origin}')")
@@ -132,18 +147,14 @@ class Qwen3Config(ModelConfig):
             raise ConfigError(f"rope_pairing '{self.rope_pairing}' is not one of 'interleaved', 'half' in '{origin}'")
         if self.torch_dtype not in ("bfloat16", "float32", "float16"):
             raise ConfigError(f"torch_dtype '{self.torch_dtype}' is not supported in '{origin}'")
-        if self.use_sliding_window:
-            if self.sliding_window is None or self.sliding_window <= 0:
-                raise ConfigError(f"use_sliding_window needs a positive 'sliding_window' in '{origin}'")
-        if self.layer_types is not None:
-            if len(self.layer_types) != self.num_hidden_layers:
-                raise ConfigError(
-                    f"layer_types has {len(self.layer_types)} entries for {self.num_hidden_layers} layers in '{origin}'")
-            for kind in self.layer_types:
-                if kind not in ("full_attention", "sliding_attention"):
-                    raise ConfigError(f"layer type '{kind}' is not supported in '{origin}'")
-            if "sliding_attention" in self.layer_types and (self.sliding_window is None or self.sliding_window <= 0):
-                raise ConfigError(f"sliding_attention layers need a positive 'sliding_window' in '{origin}'")
+        if self.layer_windows is not None:
+            if len(self.layer_windows) != self.num_hidden_layers:
+                raise ConfigError(f"layer_windows has {len(self.layer_windows)} entries for {self.num_hidden_layers} "
+                                  f"layers in '{origin}'")
+            for w in self.layer_windows:
+                if w is not None and (isinstance(w, bool) or not isinstance(w, int) or w < 0):
+                    raise ConfigError(f"layer_windows holds {w!r}; a window is a positive number of keys, or "
+                                      f"null / 0 for all keys (in '{origin}')")
 
     # ------------------------------------------------------------------ writing
     def to_dict(self) -> Dict[str, Any]:
@@ -165,29 +176,20 @@ class Qwen3Config(ModelConfig):
             "torch_dtype": self.torch_dtype,
             "hidden_act": "silu",
             "attention_bias": False,
-            "use_sliding_window": self.use_sliding_window,
+            "use_sliding_window": False,
             "sliding_window": self.sliding_window,
             "max_window_layers": self.max_window_layers,
         }
-        if self.layer_types is not None:
-            out["layer_types"] = list(self.layer_types)
         if self.eos_token_ids:
             out["eos_token_id"] = self.eos_token_ids[0] if len(self.eos_token_ids) == 1 else list(self.eos_token_ids)
         return out
 
     # --------------------------------------------------------- layers from keys
     def layer_window(self, layer: int) -> Optional[int]:
-        """The attention window of one layer, or None for all keys.
-
-        ``layer_types`` decides where given; else, with ``use_sliding_window``,
-        the first ``max_window_layers`` layers see all keys and the rest a window.
-        """
-        if self.layer_types is not None:
-            return self.sliding_window if self.layer_types[layer] == "sliding_attention" else None
-        if not self.use_sliding_window:
+        """The attention window of one layer, or None for all keys (``layer_windows``, an option of the engine)."""
+        if self.layer_windows is None:
             return None
-        first_windowed = self.max_window_layers if self.max_window_layers is not None else 0
-        return self.sliding_window if layer >= first_windowed else None
+        return self.layer_windows[layer] or None
 
     def model_spec(self) -> ModelSpec:
         """The decoder as data (reference order of operations: src/model/qwen3/model.cpp:750-926)."""

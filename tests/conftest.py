@@ -29,13 +29,16 @@ TINY_B = dict(
     num_hidden_layers=3, num_attention_heads=6, num_key_value_heads=1, head_dim=32, max_position_embeddings=256,
     rms_norm_eps=1e-5, rope_theta=1e6, tie_word_embeddings=False, torch_dtype="bfloat16", attention_bias=False,
     use_sliding_window=False, hidden_act="silu")
-# a third one with windows on some layers and yet other sizes (head_dim 48 is no power of two)
+# a third one with yet other sizes (head_dim 48 is no power of two), run with attention windows on some layers: an
+# option of the engine (the reference has no windows, so config.json cannot ask for them), given as overrides
 TINY_W = dict(
     architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=331, hidden_size=80, intermediate_size=176,
     num_hidden_layers=4, num_attention_heads=6, num_key_value_heads=3, head_dim=48, max_position_embeddings=512,
     rms_norm_eps=3e-6, rope_theta=5e4, tie_word_embeddings=False, torch_dtype="bfloat16", attention_bias=False,
-    use_sliding_window=True, sliding_window=24, max_window_layers=2, hidden_act="silu")
+    use_sliding_window=False, hidden_act="silu")
+WINDOW_W = 24
 TINY = {"A": (TINY_A, 4), "B": (TINY_B, 16), "W": (TINY_W, 8)}  # config, cache page size used with it
+OVERRIDES = {"A": None, "B": None, "W": {"layer_windows": [None, None, WINDOW_W, WINDOW_W]}}   # options of the engine
 
 
 @pytest.fixture(scope="session")
@@ -60,7 +63,8 @@ def token_ids(vocab: int, count: int, seed: int):
 def plain_models(model_folders):
     from plain.qwen3_plain import PlainQwen3
 
-    return {name: PlainQwen3.from_folder(folder) for name, folder in model_folders.items()}
+    return {name: PlainQwen3.from_folder(folder, windows=(OVERRIDES[name] or {}).get("layer_windows"))
+            for name, folder in model_folders.items()}
 
 
 class _PlainLogits:

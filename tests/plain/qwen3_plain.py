@@ -102,13 +102,18 @@ def gated_mlp(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down:
 class PlainQwen3:
     """The whole decoder on whole sequences (src/model/qwen3/model.cpp:750-926 per layer, :1283-1371 around)."""
 
-    def __init__(self, config: Dict, weights: Dict[str, torch.Tensor], pairing: str = "interleaved"):
+    def __init__(self, config: Dict, weights: Dict[str, torch.Tensor], pairing: str = "interleaved",
+                 windows: Optional[List[Optional[int]]] = None):
+        """``windows``: an attention window per layer (None: all keys).  The reference has no windows; they are a
+        parameter of ``causal_attention`` here and an option of the engine there."""
         self.c = config
         self.w = {k: v.to(DT) for k, v in weights.items()}
         self.pairing = pairing
+        self.windows = windows
 
     @classmethod
-    def from_folder(cls, folder: str, pairing: str = "interleaved") -> "PlainQwen3":
+    def from_folder(cls, folder: str, pairing: str = "interleaved",
+                    windows: Optional[List[Optional[int]]] = None) -> "PlainQwen3":
         from safetensors.torch import load_file
 
         with open(os.path.join(folder, "config.json")) as fh:
@@ -117,17 +122,10 @@ class PlainQwen3:
         for name in sorted(os.listdir(folder)):
             if name.endswith(".safetensors"):
                 weights.update(load_file(os.path.join(folder, name)))
-        return cls(config, weights, pairing)
+        return cls(config, weights, pairing, windows)
 
     def layer_window(self, layer: int) -> Optional[int]:
-        c = self.c
-        types = c.get("layer_types")
-        if types is not None:
-            return c.get("sliding_window") if types[layer] == "sliding_attention" else None
-        if not c.get("use_sliding_window", False):
-            return None
-        first = c.get("max_window_layers") or 0
-        return c.get("sliding_window") if layer >= first else None
+        return self.windows[layer] if self.windows is not None else None
 
     def layer(self, h: torch.Tensor, index: int, positions: List[int],
               rows: Optional[List[int]] = None) -> torch.Tensor:

@@ -51,8 +51,12 @@ def test_validation():
     for key, value in (("attention_bias", True), ("hidden_act", "gelu"), ("rope_scaling", {"rope_type": "yarn"})):
         with pytest.raises(ConfigError, match=key):
             Qwen3Config.from_dict(dict(TINY_A, **{key: value}))
-    with pytest.raises(ConfigError, match="sliding_window"):
-        Qwen3Config.from_dict(dict(TINY_A, use_sliding_window=True))
+    # the reference attends to all keys whatever config.json says: window keys are refused, not interpreted
+    with pytest.raises(ConfigError, match="use_sliding_window"):
+        Qwen3Config.from_dict(dict(TINY_A, use_sliding_window=True, sliding_window=24, max_window_layers=1))
+    with pytest.raises(ConfigError, match="layer_types"):
+        Qwen3Config.from_dict(dict(TINY_A, layer_types=["full_attention", "sliding_attention"]))
+    Qwen3Config.from_dict(dict(TINY_A, layer_types=["full_attention"] * 2, sliding_window=4096, max_window_layers=2))
 
 
 def test_eos_int_or_list_and_generation_override(tmp_path):
@@ -89,15 +93,20 @@ def test_qwen3_0_6b_values(tmp_path):
     assert all(cfg.layer_window(i) is None for i in range(28))
 
 
-def test_windows_per_layer():
+def test_windows_per_layer_are_an_option_of_the_engine():
+    from conftest import OVERRIDES
     cfg = Qwen3Config.from_dict(TINY_W)
+    assert all(cfg.layer_window(i) is None for i in range(4))
+    cfg.apply_overrides(OVERRIDES["W"])
     assert [cfg.layer_window(i) for i in range(4)] == [None, None, 24, 24]
-    spec = cfg.model_spec()
-    assert [l.mixer.params["window"] for l in spec.layers] == [None, None, 24, 24]
-    typed = Qwen3Config.from_dict(dict(TINY_W, layer_types=["sliding_attention", "full_attention"] * 2))
-    assert [typed.layer_window(i) for i in range(4)] == [24, None, 24, None]
-    with pytest.raises(ConfigError, match="layer_types"):
-        Qwen3Config.from_dict(dict(TINY_W, layer_types=["full_attention"]))
+    assert [l.mixer.params["window"] for l in cfg.model_spec().layers] == [None, None, 24, 24]
+    assert "layer_windows" not in cfg.to_dict()                   # no key of config.json
+    cfg.apply_overrides({"layer_windows": [8, 0, None, 3]})
+    assert [cfg.layer_window(i) for i in range(4)] == [8, None, None, 3]
+    for bad in ([24], [None, None, -1, 24], [None, None, "24", 24], [None, None, True, 24]):
+        with pytest.raises(ConfigError, match="layer_windows"):
+            Qwen3Config.from_dict(TINY_W).apply_overrides({"layer_windows": bad})
+    assert Qwen3Config.engine_options["layer_windows"]["type"]("0,0,24,24") == [None, None, 24, 24]
 
 
 def test_model_spec_carries_no_size_of_its_own():

@@ -5,7 +5,7 @@ import json
 import pytest
 import torch
 
-from conftest import TINY, token_ids
+from conftest import OVERRIDES, TINY, WINDOW_W, token_ids
 
 pytestmark = pytest.mark.gpu
 
@@ -16,23 +16,23 @@ def gpu():
         pytest.skip("no GPU visible")
 
 
-def make_llm(folder, dtype="float32", **options):
+def make_llm(folder, dtype="float32", name=None, **options):
     from pulse_infer_amd import LLM
-    return LLM.from_pretrained(folder, dtype=dtype, **options)
+    return LLM.from_pretrained(folder, dtype=dtype, config_overrides=OVERRIDES.get(name), **options)
 
 
 @pytest.mark.parametrize("name", ["A", "B", "W"])
 def test_greedy_generation_matches_the_plain_implementation(gpu, model_folders, plain_models, name):
     cfg, page = TINY[name]
     prompts = [token_ids(cfg["vocab_size"], n, seed=20 + n) for n in (5, 11, 17)]
-    llm = make_llm(model_folders[name], "float32", max_batch_size=3, chunk_size=8, page_size=page, num_pages=64)
+    llm = make_llm(model_folders[name], "float32", name, max_batch_size=3, chunk_size=8, page_size=page, num_pages=64)
     got = llm.generate(prompts, max_new_tokens=8, ignore_eos=True)
     for prompt, out in zip(prompts, got):
         assert out == plain_models[name].greedy(prompt, 8)
     llm.engine.runner.cache.check()
     assert not llm.engine.runner.cache.requests                       # everything was given back
     # bfloat16: the same tokens wherever the plain top-two margin is clear of bfloat16's error
-    llm16 = make_llm(model_folders[name], "bfloat16", max_batch_size=3, chunk_size=8, page_size=page, num_pages=64)
+    llm16 = make_llm(model_folders[name], "bfloat16", name, max_batch_size=3, chunk_size=8, page_size=page, num_pages=64)
     for prompt, out in zip(prompts, llm16.generate(prompts, max_new_tokens=8, ignore_eos=True)):
         ids = list(prompt)
         for tok in out:
@@ -53,7 +53,7 @@ def test_long_decoding_token_by_token(gpu, model_folders, plain_logits, dtype):
     for name in ("B", "W"):
         cfg, page = TINY[name]
         ids = token_ids(cfg["vocab_size"], 240, seed=33)
-        _, model = load_model(model_folders[name], mode=dtype)
+        _, model = load_model(model_folders[name], mode=dtype, config_overrides=OVERRIDES[name])
         runner = ModelRunner(model, page_size=page, num_pages=256 // page, max_requests=2)
         runner.add_request("r")
         rows = []
@@ -62,7 +62,7 @@ def test_long_decoding_token_by_token(gpu, model_folders, plain_logits, dtype):
             rows.append(runner.step([StepEntry("r", [tok], [0])]))
         if name == "W":
             held = [p for p in runner.cache.table(1, "r") if p >= 0]
-            assert len(held) <= cfg["sliding_window"] // page + 2      # the window's pages only
+            assert len(held) <= WINDOW_W // page + 2      # the window's pages only
         runner.free_request("r")
         close(torch.cat(rows), plain_logits(name, ids), dtype, f"{name} long decoding")
 
@@ -212,7 +212,7 @@ def test_recorded_steps_while_a_window_gives_pages_back_and_after_eviction(gpu, 
     from test_gpu_model import SPLIT_TOL, close
 
     cfg, _ = TINY["W"]
-    _, model = load_model(model_folders["W"], mode="bfloat16")
+    _, model = load_model(model_folders["W"], mode="bfloat16", config_overrides=OVERRIDES["W"])
     ids = {"a": token_ids(cfg["vocab_size"], 120, seed=71), "b": token_ids(cfg["vocab_size"], 100, seed=72)}
     start = {"a": 20, "b": 9}
     outs = []

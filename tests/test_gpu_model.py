@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from conftest import ROOT, TINY, token_ids
+from conftest import OVERRIDES, ROOT, TINY, token_ids
 
 pytestmark = pytest.mark.gpu
 
@@ -43,7 +43,7 @@ def engines(model_folders):
         page = page or TINY[name][1]
         key = (name, dtype, page)
         if key not in made:
-            _, model = load_model(model_folders[name], mode=dtype)
+            _, model = load_model(model_folders[name], mode=dtype, config_overrides=OVERRIDES[name])
             made[key] = ModelRunner(model, page_size=page, num_pages=tokens // page, max_requests=4)
         return made[key]
 

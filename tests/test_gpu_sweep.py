@@ -17,6 +17,7 @@ pytestmark = pytest.mark.gpu
 
 
 def random_config(rng, hidden_choices, max_positions=1024):
+    """(config.json's keys, options of the engine): windows on the later layers of some configurations are the latter."""
     d = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
     nkv = rng.choice([1, 2, 3, 4])
     group = rng.choice([1, 2, 3, 4, 5, 7, 8])
@@ -26,10 +27,12 @@ def random_config(rng, hidden_choices, max_positions=1024):
                num_hidden_layers=rng.choice([1, 2, 3]), num_attention_heads=nkv * group, num_key_value_heads=nkv,
                head_dim=d, max_position_embeddings=max_positions, rms_norm_eps=rng.choice([1e-6, 1e-5]),
                rope_theta=rng.choice([1e4, 1e6]), tie_word_embeddings=rng.random() < 0.5, torch_dtype="bfloat16",
-               attention_bias=False, hidden_act="silu", use_sliding_window=window is not None)
+               attention_bias=False, hidden_act="silu", use_sliding_window=False)
+    options = None
     if window is not None:
-        cfg.update(sliding_window=window, max_window_layers=rng.choice([0, 1]))
-    return cfg
+        first = rng.choice([0, 1])
+        options = {"layer_windows": [window if i >= first else None for i in range(cfg["num_hidden_layers"])]}
+    return cfg, options
 
 
 @pytest.mark.parametrize("seed", range(8))
@@ -42,14 +45,15 @@ def test_random_configurations_whole_tail_and_portions(tmp_path, seed):
     from pulse_infer_amd.weights import write_model_folder
 
     rng = random.Random(1000 + seed)
-    cfg = random_config(rng, [128, 256, 384, 1024])
+    cfg, options = random_config(rng, [128, 256, 384, 1024])
+    windows = (options or {}).get("layer_windows")
     page, length = rng.choice([16, 32, 64]), rng.choice([90, 200, 333])
     folder = write_model_folder(Qwen3Config.from_dict(cfg), str(tmp_path / "m"), seed=seed)
     ids = token_ids(cfg["vocab_size"], length, seed=seed)
-    want = PlainQwen3.from_folder(folder).logits(ids)
-    what = f"{cfg} page {page} length {length}"
+    want = PlainQwen3.from_folder(folder, windows=windows).logits(ids)
+    what = f"{cfg} {options} page {page} length {length}"
     for dtype in ("float32", "bfloat16"):
-        _, model = load_model(folder, mode=dtype)
+        _, model = load_model(folder, mode=dtype, config_overrides=options)
         runner = ModelRunner(model, page_size=page, num_pages=(length + page - 1) // page + 2, max_requests=2)
         whole = run_alone(runner, ids, [length])
         close(whole, want, dtype, f"whole: {what}")
@@ -82,16 +86,17 @@ def test_random_configurations_continuous_batching_and_preemption(tmp_path, seed
     from pulse_infer_amd.weights import write_model_folder
 
     rng = random.Random(2000 + seed)
-    cfg = random_config(rng, [128, 256], max_positions=512)
+    cfg, options = random_config(rng, [128, 256], max_positions=512)
+    windows = (options or {}).get("layer_windows")
     page = rng.choice([16, 32])
     folder = write_model_folder(Qwen3Config.from_dict(cfg), str(tmp_path / "m"), seed=50 + seed)
     prompts = [token_ids(cfg["vocab_size"], rng.choice([1, 5, 18, 40, 77]), seed=seed * 10 + i)
                for i in range(rng.choice([3, 5, 7]))]
     new = rng.choice([8, 20])
-    make = lambda **kw: LLM.from_pretrained(folder, dtype="float32", page_size=page, **kw)
+    make = lambda **kw: LLM.from_pretrained(folder, dtype="float32", page_size=page, config_overrides=options, **kw)
     alone = [make(max_batch_size=1, chunk_size=256, num_pages=64).generate([p], max_new_tokens=new, ignore_eos=True)[0]
              for p in prompts]
-    plain = PlainQwen3.from_folder(folder)
+    plain = PlainQwen3.from_folder(folder, windows=windows)
     assert alone[:2] == [plain.greedy(p, new) for p in prompts[:2]]
     roomy = make(max_batch_size=4, chunk_size=rng.choice([8, 16, 50]), num_pages=64,
                  max_num_batched_tokens=rng.choice([24, 64]))
@@ -115,14 +120,15 @@ def test_random_configurations_mixed_batches_with_page_reuse(tmp_path, seed):
     from test_gpu_model import mixed_trace
 
     rng = random.Random(3000 + seed)
-    cfg = random_config(rng, [128, 256, 1024])
+    cfg, options = random_config(rng, [128, 256, 1024])
+    windows = (options or {}).get("layer_windows")
     page = rng.choice([16, 32, 64])
     folder = write_model_folder(Qwen3Config.from_dict(cfg), str(tmp_path / "m"), seed=70 + seed)
-    plain = PlainQwen3.from_folder(folder)
+    plain = PlainQwen3.from_folder(folder, windows=windows)
     ids, steps = mixed_trace(cfg["vocab_size"], seed=20 + seed)
     want = {k: plain.logits(v) for k, v in ids.items()}
     for dtype in ("float32", "bfloat16"):
-        _, model = load_model(folder, mode=dtype)
+        _, model = load_model(folder, mode=dtype, config_overrides=options)
         runner = ModelRunner(model, page_size=page, num_pages=256 // page, max_requests=4)
         got = {k: [] for k in ids}
         for step in steps:
@@ -141,6 +147,6 @@ def test_random_configurations_mixed_batches_with_page_reuse(tmp_path, seed):
                 runner.free_request(k)
             runner.cache.check()
         for k, parts in got.items():
-            close(torch.cat(parts), want[k], dtype, f"mixed request {k}: {cfg} page {page}")
+            close(torch.cat(parts), want[k], dtype, f"mixed request {k}: {cfg} {options} page {page}")
         del runner, model
     torch.cuda.empty_cache()
