@@ -41,9 +41,12 @@ constexpr int WAVES = 4;
 constexpr int BLOCK_KEYS = 32;
 // Column tiles a wavefront takes in the prompt-portion kernel: two while the accumulators of both fit the registers.
 #define PULSE_WIDE (PULSE_HEAD_DIM == 32 || PULSE_HEAD_DIM == 64 || PULSE_HEAD_DIM == 128)
-constexpr int PREFILL_TILES = PULSE_WIDE ? 2 : 1;
+#ifndef PULSE_WIDE_CT
+#define PULSE_WIDE_CT 2
+#endif
 constexpr int WIDE_NW = 4;   // wavefronts of the wide prompt-portion kernel
-constexpr int WIDE_CT = 2;   // column tiles each takes
+constexpr int WIDE_CT = PULSE_WIDE_CT;   // column tiles each takes
+constexpr int PREFILL_TILES = PULSE_WIDE ? WIDE_CT : 1;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -857,8 +860,13 @@ __device__ __forceinline__ void load_to_lds(const void* from, uint32_t lds_base)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_base), "v"(from) : "memory", "m0");
 }
 
+#if PULSE_WIDE_CT > 2
+#define PULSE_WIDE_WAVES_PER_EU __attribute__((amdgpu_waves_per_eu(1, 1)))
+#else
+#define PULSE_WIDE_WAVES_PER_EU PULSE_ATTN_WAVES_PER_EU
+#endif
 template <int CT, int KT, int NW>
-__global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_prefill_wide_kernel(MfmaArgs a, int per) {
+__global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_prefill_wide_kernel(MfmaArgs a, int per) {
     using Shape = WideShape<CT, KT, NW>;
     constexpr int BK = Shape::BK;
     static_assert(KT % 2 == 0, "the second product takes pairs of key tiles");
@@ -963,17 +971,23 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_p
     auto page_ahead = [&](int b) {
         int pi, slot0;
         page_of(b * BK + 16 * wave, a.page_size, a.page_shift, pi, slot0);
-        // volatile: the load stays here, a block ahead of its use (the compiler would move it next to the use and
-        // wait for it there); it is said to be uniform only where it is used, not to wait here either
-        return *static_cast<const volatile int*>(bt + min(pi, a.bt_width - 1));
+        // A scalar load written here, so that it stays where it is, a block ahead of its use, and is waited for
+        // with the scalar counter (page_landed) where it is used.  As a vector load it would share the counter of the
+        // copies into LDS, and the compiler, which does not see those, would wait for all of them with it: the
+        // next block's copy would have to land before this block is computed.
+        const int* entry = bt + min(pi, a.bt_width - 1);
+        int page;
+        asm volatile("s_load_dword %0, %1, 0x0" : "=s"(page) : "s"(entry) : "memory");
+        return page;
     };
+    auto page_landed = [&](int& page) { asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(page) : : "memory"); };
     const int64_t page_elems = static_cast<int64_t>(a.nkv) * a.page_size * D;  // of K and of V alike
     const int head_elems = g * a.page_size * D;
     auto fetch = [&](int b, int page_read, int stage) {
         const int jt = b * BK + 16 * wave;
         int pi, slot0;
         page_of(jt, a.page_size, a.page_shift, pi, slot0);
-        int page = (jt <= hi && pi < a.bt_width) ? uniform(page_read) : 0;
+        int page = (jt <= hi && pi < a.bt_width) ? page_read : 0;
         page = (page >= 0 && page < a.num_pages) ? page : 0;
         const int64_t base = page * page_elems + head_elems;
         const bf16_t* kfrom = a.kc + base + slot0 * D;
@@ -1015,19 +1029,25 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_p
         float alpha[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
-            // The mask without a branch: key j0 + 16 t + 4 kg + i is seen when 16 t + i lies in [lim_lo, lim_hi]
-            // (a compare with a constant and a select a score; a branch a score costs a lone wavefront more).
-            const int lim_hi = col_ok[ct] ? pos_c[ct] - j0 - 4 * kg : -1;
-            const int lim_lo = lo_c[ct] - j0 - 4 * kg;
+            // Most blocks lie wholly below a tile's diagonal and inside its window: every column of the tile sees
+            // every key, and nothing is masked (columns that stand for no token or head have q = 0 and are never
+            // written).  Only a tile whose first token does not see the block's last key, or one of whose windows
+            // starts inside the block, takes the mask: key j0 + 16 t + 4 kg + i is seen when 16 t + i lies in
+            // [lim_lo, lim_hi] (two compares and a select a score, on a branch that is the same for the wavefront).
+            if (j0 + BK - 1 > t_pos0[ct] || j0 < t_hi_lo[ct] || !t_any[ct]) {
+                const int lim_hi = col_ok[ct] ? pos_c[ct] - j0 - 4 * kg : -1;
+                const int lim_lo = lo_c[ct] - j0 - 4 * kg;
+#pragma unroll
+                for (int t = 0; t < KT; ++t)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        s[ct][t][i] = (16 * t + i <= lim_hi && 16 * t + i >= lim_lo) ? s[ct][t][i] : -INFINITY;
+            }
             float mx = -INFINITY;
 #pragma unroll
             for (int t = 0; t < KT; ++t)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float v = (16 * t + i <= lim_hi && 16 * t + i >= lim_lo) ? s[ct][t][i] : -INFINITY;
-                    s[ct][t][i] = v;
-                    mx = fmaxf(mx, v);
-                }
+                for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[ct][t][i]);
             mx = fmaxf(mx, __shfl_xor(mx, 16, PULSE_WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, PULSE_WAVE));
             const float m_new = fmaxf(m[ct], mx);
@@ -1055,27 +1075,14 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_p
 #pragma unroll
                 for (int dt = 0; dt < NDT; ++dt) acc[ct][dt] = acc[ct][dt] * alpha[ct];
         }
-        // stale values under keys outside [lo_item, hi] are cleared (see the split kernel)
-        const bool edge = (j0 + BK - 1 > hi) || (j0 < lo_item);
+        // (values under keys outside [lo_item, hi] have been cleared in LDS by clear_stale before this block is computed)
 #pragma unroll
         for (int ks = 0; ks < KT / 2; ++ks) {
-            uint32_t keep[2][2] = {{0xffffffffu, 0xffffffffu}, {0xffffffffu, 0xffffffffu}};
-            if (edge) {
-#pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int h2 = 0; h2 < 2; ++h2) {
-                        const int j = j0 + 16 * (2 * ks + t) + 4 * kg + 2 * h2;
-                        keep[t][h2] = ((j <= hi && j >= lo_item) ? 0x0000ffffu : 0u) |
-                                      ((j + 1 <= hi && j + 1 >= lo_item) ? 0xffff0000u : 0u);
-                    }
-            }
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt) {
                 const u32x2 v0 = *reinterpret_cast<const u32x2*>(&s_v[(2 * ks) * D * 16 + dt * 256 + v_at]);
                 const u32x2 v1 = *reinterpret_cast<const u32x2*>(&s_v[(2 * ks + 1) * D * 16 + dt * 256 + v_at]);
-                u32x4 words = {v0[0], v0[1], v1[0], v1[1]};
-                if (edge) words = u32x4{v0[0] & keep[0][0], v0[1] & keep[0][1], v1[0] & keep[1][0], v1[1] & keep[1][1]};
+                const u32x4 words = {v0[0], v0[1], v1[0], v1[1]};
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct)
                     acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, words), pb[ct][ks],
@@ -1083,13 +1090,34 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_p
             }
         }
     };
+    // Stale values under keys that no column of the item may see (beyond its last position, below its window) must
+    // not reach the sums, not even as 0 * (inf or nan).  Only the item's last block and the block its window starts
+    // in hold such keys, which the whole workgroup knows from the block's number: there the value tiles are cleared
+    // in LDS, a 16-byte piece (8 keys of a channel) a thread, before anybody reads them.
+    auto clear_stale = [&](int b, int stage) {
+        bf16_t* s_v = s_kv + stage * Shape::STAGE + Shape::STAGE_K;
+#pragma unroll
+        for (int t = 0; t < KT; ++t)
+            for (int piece = tid; piece < 2 * D; piece += NW * PULSE_WAVE) {
+                const int j = b * BK + 16 * t + 8 * ((piece / 16) % 2);    // the piece's first key
+                u32x4 mask;
+#pragma unroll
+                for (int w = 0; w < 4; ++w)
+                    mask[w] = ((j + 2 * w <= hi && j + 2 * w >= lo_item) ? 0x0000ffffu : 0u) |
+                              ((j + 2 * w + 1 <= hi && j + 2 * w + 1 >= lo_item) ? 0xffff0000u : 0u);
+                u32x4* at = reinterpret_cast<u32x4*>(s_v + t * D * 16 + piece * 8);
+                *at = *at & mask;
+            }
+    };
 
     const int first_block = max(lo_item, split_begin) / BK;
     const int last_block = split_last / BK;
     // (a split that lies below the item's window has no block to walk: nothing is fetched, its columns stay empty)
     int page_next = 0;
     if (first_block <= last_block) {
-        fetch(first_block, page_ahead(first_block), 0);
+        int page_first = page_ahead(first_block);
+        page_landed(page_first);
+        fetch(first_block, page_first, 0);
         page_next = page_ahead(first_block + 1);
     }
     for (int b = first_block; b <= last_block; ++b) {
@@ -1099,10 +1127,15 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void attn_p
         asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
         __syncthreads();  // every wavefront's part of this block has landed
         if (b < last_block) {
+            page_landed(page_next);
             fetch(b + 1, page_next, stage ^ 1);  // that stage was read a block ago; the barrier that ended that block released it
             page_next = page_ahead(b + 2);       // used an iteration later
         }
         // a wavefront skips blocks that none of its columns sees (above its diagonal, below its window)
+        if (b * BK + BK - 1 > hi || b * BK < lo_item) {   // the same for the whole workgroup
+            clear_stale(b, stage);
+            __syncthreads();
+        }
         if (w_hi >= 0 && b * BK <= w_hi && b * BK + BK - 1 >= w_lo) compute(b, stage);
         __syncthreads();  // everybody has read this block
     }
