@@ -1005,24 +1005,49 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
     const int v_at = ((kg >> 1) * 16 + r) * 8 + (kg & 1) * 4;
 
     const float c2 = a.scale_log2e;
+    constexpr float LAZY_BITS = 8.f;
+    const float lazy = LAZY_BITS / c2;   // in the raw scores' units
     auto compute = [&](int b, int stage) {
         const int j0 = b * BK;
         const bf16_t* s_k = s_kv + stage * Shape::STAGE;
         const bf16_t* s_v = s_k + Shape::STAGE_K;
+        // Operand reads run AHEAD steps in front of the products that use them, in an order that is fixed here (the
+        // scheduling fences keep the compiler from regrouping them into bursts that are each waited for in full): a
+        // read's latency is then covered by the products of the steps before it, not added to them.
+        constexpr int AHEAD = 4;
         f32x4 s[CT][KT];
+        {
+            constexpr int STEPS = KT * NCHUNK;
+            auto k_read = [&](int i) {
+                const int t = i / NCHUNK, ch = i % NCHUNK;
+                return ch * 32 + kg * 8 < D ? *reinterpret_cast<const bf16x8*>(&s_k[16 * t * D + k_at[ch]]) : zero8();
+            };
+            bf16x8 ak[STEPS];
 #pragma unroll
-        for (int t = 0; t < KT; ++t) {
+            for (int i = 0; i < AHEAD && i < STEPS; ++i) ak[i] = k_read(i);
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) s[ct][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ch = 0; ch < NCHUNK; ++ch) {
-                const int off = ch * 32 + kg * 8;
-                const bf16x8 ak = off < D ? *reinterpret_cast<const bf16x8*>(&s_k[16 * t * D + k_at[ch]]) : zero8();
+            for (int i = 0; i < STEPS; ++i) {
+                const int t = i / NCHUNK, ch = i % NCHUNK;
+                if (i + AHEAD < STEPS) ak[i + AHEAD] = k_read(i + AHEAD);
 #pragma unroll
                 for (int ct = 0; ct < CT; ++ct)
-                    s[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak, bq[ct][ch], s[ct][t], 0, 0, 0);
+                    s[ct][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak[i], bq[ct][ch],
+                                                                       ch == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[ct][t], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
+        // the first value operands are asked for before the weights are computed, the rest as the products go
+        constexpr int V_STEPS = (KT / 2) * NDT;
+        auto v_read = [&](int i) {
+            const int ks = i / NDT, dt = i % NDT;
+            const u32x2 v0 = *reinterpret_cast<const u32x2*>(&s_v[(2 * ks) * D * 16 + dt * 256 + v_at]);
+            const u32x2 v1 = *reinterpret_cast<const u32x2*>(&s_v[(2 * ks + 1) * D * 16 + dt * 256 + v_at]);
+            return u32x4{v0[0], v0[1], v1[0], v1[1]};
+        };
+        u32x4 vw[V_STEPS];
+#pragma unroll
+        for (int i = 0; i < AHEAD && i < V_STEPS; ++i) vw[i] = v_read(i);
+        __builtin_amdgcn_sched_barrier(0);
         // the maximum is tracked on the raw scores (the scale is positive); p = exp2((s - m) * scale * log2 e)
         bf16x8 pb[CT][KT / 2];
         bool moved = false;
@@ -1050,7 +1075,12 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
                 for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[ct][t][i]);
             mx = fmaxf(mx, __shfl_xor(mx, 16, PULSE_WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, PULSE_WAVE));
-            const float m_new = fmaxf(m[ct], mx);
+            // The reference point of the exponents follows the maximum only when that has grown by more than
+            // 2^LAZY_BITS in the weights' units: until then weights may exceed 1 (by at most that factor, which float32
+            // sums and bfloat16 weights hold with the same relative precision), and the accumulators, which are most of
+            // a wavefront's registers, are rescaled in few blocks instead of nearly all.  The result is the same
+            // quotient of sums.
+            const float m_new = mx > m[ct] + lazy ? mx : m[ct];
             const bool dead = m_new == -INFINITY;  // no key of this column so far
             alpha[ct] = dead ? 1.f : __builtin_amdgcn_exp2f((m[ct] - m_new) * c2);
             const float shift = dead ? 0.f : -m_new * c2;
@@ -1076,18 +1106,16 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
                 for (int dt = 0; dt < NDT; ++dt) acc[ct][dt] = acc[ct][dt] * alpha[ct];
         }
         // (values under keys outside [lo_item, hi] have been cleared in LDS by clear_stale before this block is computed)
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int ks = 0; ks < KT / 2; ++ks) {
+        for (int i = 0; i < V_STEPS; ++i) {
+            const int ks = i / NDT, dt = i % NDT;
+            if (i + AHEAD < V_STEPS) vw[i + AHEAD] = v_read(i + AHEAD);
 #pragma unroll
-            for (int dt = 0; dt < NDT; ++dt) {
-                const u32x2 v0 = *reinterpret_cast<const u32x2*>(&s_v[(2 * ks) * D * 16 + dt * 256 + v_at]);
-                const u32x2 v1 = *reinterpret_cast<const u32x2*>(&s_v[(2 * ks + 1) * D * 16 + dt * 256 + v_at]);
-                const u32x4 words = {v0[0], v0[1], v1[0], v1[1]};
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct)
-                    acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, words), pb[ct][ks],
-                                                                          acc[ct][dt], 0, 0, 0);
-            }
+            for (int ct = 0; ct < CT; ++ct)
+                acc[ct][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vw[i]), pb[ct][ks],
+                                                                      acc[ct][dt], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
     // Stale values under keys that no column of the item may see (beyond its last position, below its window) must
