@@ -835,8 +835,8 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
 //
 // LDS holds 16-byte pieces without padding; which piece a lane fetches is chosen so that the matrix-core operand
 // reads are free of bank conflicts:
-//   K: piece c of key j (P = D / 8 pieces a key) sits at slot j * P + (c + rot(j)) % P, rot(j) = (j * P / 16) % P, so
-//      the 16 keys that 16 consecutive lanes read for one c lie in 16 different 16-byte bank groups;
+//   K: piece c of key j (P = D / 8 pieces a key) sits at slot j * P + (c + piece_rot(j)) % P, so that the key rows
+//      which eight neighbouring lanes read for one c lie in eight different 16-byte places of an LDS cycle;
 //   V: a tile of 16 keys is D channel rows of 32 bytes; the piece (channel ch, half h) sits at slot
 //      (ch / 16) * 32 + h * 16 + ch % 16, so the 16 channel rows of one half are 256 contiguous bytes.
 // Needs D in {32, 64, 128} (P a power of two, whole 1 KB chunks a tile).
@@ -844,6 +844,13 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
 // The loads are written in assembly: the compiler knows nothing of them (it would wait for every one before any LDS
 // read), so the waits for them are written here too.  Its own vector loads inside the loop (the block table) only
 // ever make it wait longer, never shorter: the counter runs in issue order.
+// Where piece c of key row j sits inside the row in LDS: at (c + piece_rot(j)) % P.  The eight key rows that eight
+// neighbouring lanes read together are j0 .. j0 + 3 and j0 + 8 .. j0 + 11 (j0 a multiple of 4); the rotation sends
+// them to eight different 16-byte places of the 128 bytes that LDS serves in a cycle.
+__device__ __forceinline__ constexpr int piece_rot(int j, int P) {
+    return P >= 8 ? ((j & 3) | (((j >> 3) & 1) << 2)) : (((j >> 1) & 1) | (((j >> 3) & 1) << 1));
+}
+
 template <int CT, int KT, int NW>
 struct WideShape {
     static constexpr int BK = KT * 16;                    // keys a block
@@ -961,7 +968,7 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
     for (int i = 0; i < Shape::TILE_CHUNKS; ++i) {
         const int slot = 64 * i + lane;         // within the tile's 16 * P slots
         const int key = slot / P, pos = slot % P;
-        const int c8 = (pos - (key * P / 16) % P + P) % P;
+        const int c8 = (pos - piece_rot(key, P) + P) % P;
         k_from[i] = key * D + c8 * 8;
         const int blk = slot / 32, half = (slot / 16) % 2, chr = slot % 16;
         v_from[i] = (blk * 16 + chr) * a.page_size + half * 8;
@@ -998,11 +1005,19 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
 #pragma unroll
         for (int i = 0; i < Shape::TILE_CHUNKS; ++i) load_to_lds(vfrom + v_from[i], to + Shape::STAGE_K * 2 + i * 1024);
     };
-    // operand reads: K piece 4 ch + kg of key 16 t + r, V words of channel row 16 dt + r
-    int k_at[NCHUNK];
+    // Operand reads.  Row r of score tile t is not key 16 t + r but key 32 (t / 2) + 8 (r / 4) + 4 (t % 2) + r % 4 of
+    // the block: the four rows that lane group kg gets back of tiles 2 ks and 2 ks + 1 are then the eight
+    // consecutive keys 32 ks + 8 kg .. + 7, whose values for one channel are one 16-byte piece of the value tile,
+    // read whole by one lane (eight lanes a cycle read eight neighbouring pieces: no bank is asked twice; as two
+    // 8-byte halves of pieces 16 bytes apart every read took two turns).
+    int k_at[2][NCHUNK];
 #pragma unroll
-    for (int ch = 0; ch < NCHUNK; ++ch) k_at[ch] = (r * P + (4 * ch + kg + (r * P / 16) % P) % P) * 8;
-    const int v_at = ((kg >> 1) * 16 + r) * 8 + (kg & 1) * 4;
+    for (int par = 0; par < 2; ++par) {
+        const int row = 4 * par + 8 * (r / 4) + r % 4;
+#pragma unroll
+        for (int ch = 0; ch < NCHUNK; ++ch) k_at[par][ch] = (row * P + (4 * ch + kg + piece_rot(row, P)) % P) * 8;
+    }
+    const int v_at = (kg >> 1) * D * 16 + ((kg & 1) * 16 + r) * 8;
 
     const float c2 = a.scale_log2e;
     constexpr float LAZY_BITS = 8.f;
@@ -1020,7 +1035,7 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
             constexpr int STEPS = KT * NCHUNK;
             auto k_read = [&](int i) {
                 const int t = i / NCHUNK, ch = i % NCHUNK;
-                return ch * 32 + kg * 8 < D ? *reinterpret_cast<const bf16x8*>(&s_k[16 * t * D + k_at[ch]]) : zero8();
+                return ch * 32 + kg * 8 < D ? *reinterpret_cast<const bf16x8*>(&s_k[32 * (t / 2) * D + k_at[t % 2][ch]]) : zero8();
             };
             bf16x8 ak[STEPS];
 #pragma unroll
@@ -1040,9 +1055,7 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
         constexpr int V_STEPS = (KT / 2) * NDT;
         auto v_read = [&](int i) {
             const int ks = i / NDT, dt = i % NDT;
-            const u32x2 v0 = *reinterpret_cast<const u32x2*>(&s_v[(2 * ks) * D * 16 + dt * 256 + v_at]);
-            const u32x2 v1 = *reinterpret_cast<const u32x2*>(&s_v[(2 * ks + 1) * D * 16 + dt * 256 + v_at]);
-            return u32x4{v0[0], v0[1], v1[0], v1[1]};
+            return *reinterpret_cast<const u32x4*>(&s_v[(2 * ks) * D * 16 + dt * 256 + v_at]);
         };
         u32x4 vw[V_STEPS];
 #pragma unroll
@@ -1057,16 +1070,18 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
             // Most blocks lie wholly below a tile's diagonal and inside its window: every column of the tile sees
             // every key, and nothing is masked (columns that stand for no token or head have q = 0 and are never
             // written).  Only a tile whose first token does not see the block's last key, or one of whose windows
-            // starts inside the block, takes the mask: key j0 + 16 t + 4 kg + i is seen when 16 t + i lies in
+            // starts inside the block, takes the mask: score i of tile t belongs to key j0 + 32 (t / 2) + 4 (t % 2) + 8 kg + i,
+            // which is seen when 32 (t / 2) + 4 (t % 2) + i lies in
             // [lim_lo, lim_hi] (two compares and a select a score, on a branch that is the same for the wavefront).
             if (j0 + BK - 1 > t_pos0[ct] || j0 < t_hi_lo[ct] || !t_any[ct]) {
-                const int lim_hi = col_ok[ct] ? pos_c[ct] - j0 - 4 * kg : -1;
-                const int lim_lo = lo_c[ct] - j0 - 4 * kg;
+                const int lim_hi = col_ok[ct] ? pos_c[ct] - j0 - 8 * kg : -1;
+                const int lim_lo = lo_c[ct] - j0 - 8 * kg;
 #pragma unroll
                 for (int t = 0; t < KT; ++t)
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
-                        s[ct][t][i] = (16 * t + i <= lim_hi && 16 * t + i >= lim_lo) ? s[ct][t][i] : -INFINITY;
+                        s[ct][t][i] = (32 * (t / 2) + 4 * (t % 2) + i <= lim_hi && 32 * (t / 2) + 4 * (t % 2) + i >= lim_lo)
+                                          ? s[ct][t][i] : -INFINITY;
             }
             float mx = -INFINITY;
 #pragma unroll
