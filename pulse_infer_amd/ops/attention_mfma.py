@@ -146,42 +146,37 @@ def choose_prefill_splits(entries: Sequence, portion: int, nkv: int, group: int,
     """(split_size, n_splits) for the prompt-portion kernel over these (index, entry) pairs.
 
     A workgroup walks its item's keys block by block, so the longest item sets the kernel's time while the chip
-    waits.  Two cases gain from cutting the keys into splits with workgroups of their own: fewer workgroups than the
-    chip runs at a time (``target_groups``, two a compute unit unless given; a short portion over a long context), which get as many splits as fill
-    it; and a full chip whose longest item walks much more than its share of all blocks (the late portions of a
-    whole prompt), which is cut at one and a half shares.  Splits never hold fewer than ``min_blocks`` blocks, and
-    nothing is cut otherwise: the partial results cost a trip through memory and a second launch."""
+    waits.  Cutting the keys into splits with workgroups of their own pays when there are fewer workgroups than the
+    chip runs at a time (``target_groups``, two a compute unit unless given; a short portion over a long context):
+    they get as many splits as fill it.  Splits never hold fewer than ``min_blocks`` blocks, and nothing is cut
+    otherwise: the partial results cost a trip through memory and a second launch.  (A full chip whose latest items
+    walk much more than their share, the late portions of a whole prompt, was cut too while a block took a
+    workgroup 2.7 us; at 1.8 us the detour costs what it saves: 2,048 tokens 64.7 us whole, 67.4 cut at 1,664 keys,
+    88 at 1,024.)"""
     if d not in PREFILL_SPLIT_HEAD_DIMS or window > 0:   # (a window keeps every walk short)
         return 0, 1
     if target_groups is None:
         target_groups = 2 * compute_units()
-    total = longest = tokens = items = 0
+    longest = tokens = items = 0
     for _, e in entries:
         tokens += e.count
         for b in range(0, e.count, portion):
             blocks = (e.start + min(b + portion, e.count) - 1) // PREFILL_SPLIT_KEYS + 1
-            total += blocks
             longest = max(longest, blocks)
             items += 1
     if items == 0:
         return 0, 1
     per_item = nkv * ((group + 15) // 16)
     groups = items * per_item
-    even = groups < target_groups
-    if even:
-        size = max(min_blocks, (longest * groups + target_groups - 1) // target_groups)
-    else:
-        share = (total * per_item + target_groups - 1) // target_groups
-        if longest * 4 < share * 7:
-            return 0, 1
-        size = max(min_blocks, (share * 3 + 1) // 2)
+    if groups >= target_groups:
+        return 0, 1
+    size = max(min_blocks, (longest * groups + target_groups - 1) // target_groups)
     n_splits = (longest + size - 1) // size
     budget = PREFILL_SCRATCH_BYTES // max(1, tokens * nkv * group * d * 4)
     n_splits = min(n_splits, PREFILL_MAX_SPLITS, max(1, budget))
     if n_splits <= 1:
         return 0, 1
-    if even or n_splits * size < longest:
-        size = (longest + n_splits - 1) // n_splits   # splits of equal length
+    size = (longest + n_splits - 1) // n_splits   # splits of equal length
     return size * PREFILL_SPLIT_KEYS, (longest + size - 1) // size
 
 

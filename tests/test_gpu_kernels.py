@@ -519,6 +519,42 @@ def test_attn_prefill_with_its_keys_in_splits(k, case, size):
     _mfma_case(k, split=None, portion_split=size, **case)
 
 
+@pytest.mark.parametrize("n", [2048, 8192])
+def test_attn_prefill_at_the_benchmark_shape(k, n):
+    """A whole prompt of 2,048 (and 8,192) tokens at 32 query heads over 8 kv heads of 128 (every workgroup of the chip busy, items
+    of every length, one diagonal block each): rows at the edges of items, of key blocks and of pages against the
+    plain formula.  (The profile of this kernel is taken from this test.)"""
+    from pulse_infer_amd.ops import attention_mfma as M
+    nq, nkv, d, bs = 32, 8, 128, 16
+    dtype = torch.bfloat16
+    pages = n // bs
+    perm = torch.randperm(pages + 3, generator=torch.Generator().manual_seed(9)).tolist()[:pages]
+    kc, vc = _cache(pages + 3, nkv, bs, d, dtype)
+    kc.normal_()
+    vc.normal_()
+    ks, kref = as_stored(rnd(n, nkv, d, seed=501), dtype)
+    vs, vref = as_stored(rnd(n, nkv, d, seed=502), dtype)
+    _fill_cache(kc, vc, ks, vs, perm, bs)
+    q, qref = as_stored(rnd(n, nq * d, seed=503), dtype)
+    out = torch.zeros(n, nq * d, dtype=dtype, device=DEV)
+    table = torch.tensor([perm], dtype=torch.int32, device=DEV)
+
+    class E:
+        def __init__(self, first_row, count):
+            self.first_row, self.count, self.start = first_row, count, 0
+    entries = [(0, E(0, n))]
+    portion = M.portion_tokens(nq // nkv, d)
+    items = torch.tensor(M.build_items(entries, portion), dtype=torch.int32, device=DEV)
+    assert M.choose_prefill_splits(entries, portion, nkv, nq // nkv, d, 0) == (0, 1)      # a full chip is not cut
+    pos = torch.arange(n, dtype=torch.int32, device=DEV)
+    for _ in range(3):
+        M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos, table, items, d ** -0.5, 0)
+    got = out.cpu().to(F64).reshape(n, nq, d)
+    for t in (0, 1, 15, 16, 31, 32, 33, 63, 64, 65, 127, 128, 1000, 1023, 1024, 1055, 1056, 2015, 2016, 2046, 2047, n - 33, n - 32, n - 1):
+        want = P.causal_attention(qref[t:t + 1].reshape(1, nq, d), kref[:t + 1], vref[:t + 1], d ** -0.5, None, [t])
+        assert torch.allclose(got[t], want[0], atol=2e-2, rtol=2e-2), (t, float((got[t] - want[0]).abs().max()))
+
+
 @pytest.mark.parametrize("path", ["decode", "decode_raw", "portion", "portion_splits"])
 def test_attn_mfma_one_far_key_in_a_long_context(k, path):
     """A context of 20,000 keys (scattered pages, many splits) in which one key's score stands out: the output is that
