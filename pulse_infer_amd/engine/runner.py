@@ -114,6 +114,7 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and model.options.get("decode_graph", True) and clean
         self._graphs: dict = {}
         self._graph_seen: dict = {}
+        self._graph_refused: set = set()   # shapes whose step holds a library call: no library call is ever recorded
         self.graph_records = 0      # recordings made so far
         self.graph_replays = 0      # steps that ran as a replay of a recording
         self.max_positions = model.spec.max_positions
@@ -229,7 +230,8 @@ class ModelRunner:
     # A step of single tokens (one per request, each wanting its logits) has the same launches every time,
     # so it is recorded once per (batch, context bucket) as a HIP graph over buffers of its own and replayed:
     # the host then only copies the step's integers and starts the graph.
-    GRAPH_MAX_BATCH = 16        # up to here every product is this package's own kernel (no library call is recorded)
+    GRAPH_MAX_BATCH = 64        # up to here every product can be this package's own kernel; a shape whose step does
+                                # call the vendor library (seen when it is first run for recording) stays eager
     GRAPH_CONTEXT_BUCKET = 1024
     GRAPH_LIMIT = 64            # recordings kept
     GRAPH_AFTER_STEPS = 4       # a (batch, context bucket) is recorded when it comes for this many-th time
@@ -249,6 +251,8 @@ class ModelRunner:
         key = self._graph_key(batch, max_context)
         if key in self._graphs:
             return True
+        if key in self._graph_refused:
+            return False
         seen = self._graph_seen.get(key, 0) + 1
         self._graph_seen[key] = seen
         return seen >= self.GRAPH_AFTER_STEPS
@@ -261,6 +265,9 @@ class ModelRunner:
             # The step that meets a new shape runs eagerly (over the recording's own buffers, which sizes them) and is
             # recorded afterwards without being run again: a part with state of its own must see every step once.
             rec, logits = self._capture(key, entries, metas, want_rows)
+            if rec is None:
+                self._graph_refused.add(key)
+                return logits
             self._graphs[key] = rec
             self.graph_records += 1
             if len(self._graphs) > self.GRAPH_LIMIT:   # oldest recording out: contexts move on to higher buckets
@@ -289,8 +296,13 @@ class ModelRunner:
         self._fill(rec.host_np, offsets, entries, metas, want_rows, widths)
         dev.copy_(host, non_blocking=True)
         # the step itself, eagerly: it sizes the workspace and lets parts build what depends only on the step's shape
+        from ..parts import linear
+
+        library_before = linear.library_calls
         logits = self.model.forward(ctx, self.views)
         torch.cuda.synchronize()
+        if linear.library_calls != library_before:
+            return None, logits   # the step went through the vendor library somewhere: it is not recorded
         ctx.extras = {k: v for k, v in ctx.extras.items() if k.startswith("static:")}
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):

@@ -21,6 +21,9 @@ from ..ops.device import compute_units
 from .base import LazyNorm, ResidualStream, RowStats, Workspace
 
 
+library_calls = 0   # products that went to the vendor library so far (a step that made none can be recorded as a graph)
+
+
 class Linear:
     def __init__(self, weight: torch.Tensor, mode: str):
         if weight.dim() != 2:
@@ -36,9 +39,12 @@ class Linear:
         return (self.library and kernels.gemm_skinny_fusable(x.shape[0], n, self.in_features)
                 and x.h.stride(1) == 1 and self.weight.stride(1) == 1)
 
-    def forward(self, x, out: torch.Tensor, rows: Optional[int] = None, swiglu: bool = False) -> torch.Tensor:
+    def forward(self, x, out: torch.Tensor, rows: Optional[int] = None, swiglu: bool = False,
+                own: bool = True) -> torch.Tensor:
         """``out`` [M, out_features] receives the product; its storage type is bfloat16 or float32.  ``x`` may be a
-        ``LazyNorm`` that ``takes_lazy`` accepted.  ``swiglu``: few rows of a slab-interleaved gate/up weight only."""
+        ``LazyNorm`` that ``takes_lazy`` accepted.  ``swiglu``: few rows of a slab-interleaved gate/up weight only.
+        ``own=False``: 17 to 64 rows go to the library although this package has a product for them (a caller that
+        measured the library faster for its shape)."""
         w = self.weight if rows is None else self.weight[:rows]
         if isinstance(x, LazyNorm):
             kernels.gemm_skinny(None, w, out, swiglu=swiglu, norm=(x.h, x.sumsq, x.weight, x.eps))
@@ -54,6 +60,17 @@ class Linear:
             if few and kernels.gemm_skinny_ok(x, w):
                 kernels.gemm_skinny(x, w, out)
                 return out
+            if own and self.takes_own_rows(x, w, out):
+                # 17 to 64 rows: X through LDS, 16 weight rows a wavefront.  A float32 result (logits) is the "parts"
+                # output with one share; many weight rows take wide workgroups, few take narrow ones so that there
+                # are enough of them (measured: logits of a 152K vocabulary 212 to 237 us against the library's 276 to
+                # 281; 6,144 rows of qkv 17 to 21 us against 15 to 18, which a step without a library call, recorded
+                # and replayed as a whole, makes up several times over).
+                waves = 10 if w.shape[0] >= 64 * compute_units() else 2
+                kernels.gemm_mid(x, w, out.view(1, *out.shape) if out.dtype == torch.float32 else out, waves=waves)
+                return out
+            global library_calls
+            library_calls += 1
             if out.dtype == torch.bfloat16:
                 with timing.region("library matmul"):
                     torch.matmul(x, w.t(), out=out)
@@ -95,6 +112,8 @@ class Linear:
                                      self.out_features, torch.float32).view(splits, rows, self.out_features)
             xa = x.view(rows, splits, share).transpose(0, 1)
             wb = self.weight.view(self.out_features, splits, share).permute(1, 2, 0)
+            global library_calls
+            library_calls += 1
             with timing.region("library batched matmul"):
                 torch.bmm(xa, wb, out_dtype=torch.float32, out=parts)
             return parts
@@ -146,6 +165,17 @@ class Linear:
         return (x.dim() == 2 and x.shape[1] % 8 == 0 and x.stride(1) == 1 and w.stride(1) == 1
                 and (x.shape[0] <= 1 or x.stride(0) % 8 == 0) and (w.shape[0] <= 1 or w.stride(0) % 8 == 0)
                 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+    def takes_own_rows(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
+        """Whether a plain product of this many rows (bfloat16 or float32 result) runs as this package's product for
+        17 to 64 rows instead of the library's."""
+        rows = x.shape[0]
+        if not (self.MID_ROWS[0] <= rows <= self.MID_ROWS[1] and self.operands_ok(x) and w.stride(1) == 1
+                and kernels.gemm_mid_takes(rows, w.shape[0], w.shape[1])):
+            return False
+        if out.dtype == torch.float32:
+            return out.is_contiguous() and out.data_ptr() % 16 == 0 and w.shape[0] % 4 == 0
+        return out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.stride(0) % 4 == 0 and out.data_ptr() % 16 == 0
 
     def takes_mid(self, x: torch.Tensor) -> bool:
         return (self.library and x.dtype == torch.bfloat16 and self.MID_ROWS[0] <= x.shape[0] <= self.MID_ROWS[1]

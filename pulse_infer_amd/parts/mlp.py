@@ -68,7 +68,7 @@ class GatedMLP(Part):
             self.gate_up.forward(x, z, swiglu=True)   # 17 to 64 rows: X shared through LDS, SwiGLU in the epilogue
         else:
             gu = ws.buffer("mlp.gate_up", tokens, 2 * self.inter, self.act_dtype)
-            self.gate_up.forward(x, gu)
+            self.gate_up.forward(x, gu, own=False)   # (the shapes that come here at 17 to 64 rows are those the library wins)
             kernels.swiglu(gu, z, slab=self.slab)
         out = ws.buffer("mlp.out", tokens, self.hidden, self.act_dtype)
         if residual is not None:

@@ -182,7 +182,7 @@ def test_mixed_batches_with_page_reuse(engines, plain_logits, name, page, dtype)
 # 12288) with two layers and a small vocabulary: the sizes at which the serving kernels run (the streaming product with
 # K = 4096 and 12288, 128-wide heads in groups of four), against the plain implementation.
 LAYER_SHAPE = dict(
-    architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=1031, hidden_size=4096, intermediate_size=12288,
+    architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=1032, hidden_size=4096, intermediate_size=12288,
     num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128, max_position_embeddings=4096,
     rms_norm_eps=1e-6, rope_theta=1e6, tie_word_embeddings=False, torch_dtype="bfloat16", attention_bias=False,
     use_sliding_window=False, hidden_act="silu")
@@ -251,18 +251,19 @@ def test_benchmark_layer_sizes_mixed_with_page_reuse(layer_shape, dtype):
     torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("batch", [8, 3])
+@pytest.mark.parametrize("batch", [8, 3, 24, 40])
 def test_benchmark_layer_sizes_recorded_decode_steps(layer_shape, batch):
     """Recorded steps at the benchmark's attention shape (heads of 128 in groups of four, the decode kernel writing
     keys and values from inside the graph): eight (and three) requests of unequal contexts, from 5 to more than a
     thousand keys, so that some of the splits chosen for the context bucket are empty for the short ones; the longest
-    walks across a multiple of 1,024 on the way, which takes a new recording with a wider block table.  Every
-    replay against the eager step and the plain implementation."""
+    walks across a multiple of 1,024 on the way, which takes a new recording with a wider block table.  With 24 and 40
+    requests the step's products are those for 17 to 64 rows (qkv and the logits among them: no library call, or the
+    step would not be recorded).  Every replay against the eager step and the plain implementation."""
     from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
     from pulse_infer_amd.models.factory import load_model
 
     folder, _, _, plain = layer_shape
-    lengths = [1018, 5, 700, 300, 1000, 64, 513, 17][:batch]
+    lengths = ([1018, 5, 700, 300, 1000, 64, 513, 17] + [20 + (7 * i) % 31 for i in range(32)])[:batch]
     steps = 12
     vocab = LAYER_SHAPE["vocab_size"]
     ids = [token_ids(vocab, n + steps, seed=300 + i) for i, n in enumerate(lengths)]
