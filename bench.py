@@ -52,9 +52,11 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--context", type=int, default=4096, help="context length the timed decode steps end at")
     p.add_argument("--model", choices=sorted(SHAPES), default="8b", help="layer sizes: Qwen3-8B (the default), 14B or 32B")
     p.add_argument("--layers", type=int, default=None, help="fewer layers than the model has, if memory or time needs it")
-    p.add_argument("--workload", choices=["decode", "serving"], default="decode",
+    p.add_argument("--workload", choices=["decode", "serving", "long-prompt"], default="decode",
                    help="decode: fixed batch at a fixed context; serving: continuous batching of requests with "
-                        "seeded prompt lengths, chunked prefill mixed with decoding")
+                        "seeded prompt lengths, chunked prefill mixed with decoding; long-prompt: one prompt of "
+                        "--prompt-tokens tokens in portions of --chunk tokens")
+    p.add_argument("--prompt-tokens", type=int, default=16384, help="long-prompt: length of the prompt")
     p.add_argument("--requests", type=int, default=32, help="serving: number of requests")
     p.add_argument("--prompt-range", type=int, nargs=2, default=[128, 2048], help="serving: prompt lengths drawn from [lo, hi]")
     p.add_argument("--output-tokens", type=int, default=256, help="serving: tokens generated per request")
@@ -160,6 +162,47 @@ def serving(args, cfg, model, full_layers: int) -> int:
     return 0
 
 
+def long_prompt(args, cfg, model, full_layers: int) -> int:
+    """One prompt of ``--prompt-tokens`` tokens computed in portions of ``--chunk`` tokens (every portion attends to
+    all the keys before it: few workgroups with long walks, the split prompt-portion kernel's case)."""
+    import torch
+
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.cost import step_cost
+
+    tokens, chunk, page = args.prompt_tokens, args.chunk, args.page_size
+    runner = ModelRunner(model, page_size=page, num_pages=(tokens + page - 1) // page + 1, max_requests=2)
+    ids = torch.randint(0, cfg.vocab_size, (tokens,), generator=torch.Generator().manual_seed(args.seed)).tolist()
+    element = 2 if args.dtype == "bfloat16" else 4
+    spec = cfg.model_spec()
+    flops = sum(step_cost(spec, [(p, min(chunk, tokens - p))], 0, element, element).flops for p in range(0, tokens, chunk))
+    times = []
+    for r in range(args.runs + 1):          # the first run warms up
+        runner.add_request("p")
+        runner.reserve("p", tokens)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for p in range(0, tokens, chunk):
+            part = ids[p:p + chunk]
+            runner.step([StepEntry("p", part, [len(part) - 1] if p + chunk >= tokens else [])])
+        torch.cuda.synchronize()
+        if r > 0:
+            times.append(time.perf_counter() - t0)
+        runner.free_request("p")
+    seconds = statistics.median(times)
+    peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+    steps = (tokens + chunk - 1) // chunk
+    print(json.dumps({
+        "metric": f"qwen3_{args.model}_long_prompt_tokens_per_s", "value": round(tokens / seconds, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": steps, "ms_per_step": round(seconds * 1e3 / steps, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {"model": f"Qwen3-{args.model.upper()} shape, random weights", "global_batch": 1, "seq_len": tokens,
+                   "parallelism": "single GPU", "layers": args.layers, "layers_full_model": full_layers, "chunk": chunk},
+        "runs": args.runs, "seconds": round(seconds, 4), "frac_of_peak": round(flops / seconds / peak, 4)}))
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -191,6 +234,8 @@ def main() -> int:
 
     if args.workload == "serving":
         return serving(args, cfg, model, full_layers)
+    if args.workload == "long-prompt":
+        return long_prompt(args, cfg, model, full_layers)
 
     from pulse_infer_amd.models.cost import step_cost
 
