@@ -38,7 +38,7 @@ class StepEntry:
 class _Staging:
     """Pinned host buffers for a step's integer metadata, used in turn."""
 
-    def __init__(self, device: torch.device, depth: int = 2):
+    def __init__(self, device: torch.device, depth: int = 4):
         self.device = device
         self.host: List[Optional[torch.Tensor]] = [None] * depth
         self.events: List[Optional[torch.cuda.Event]] = [None] * depth
@@ -197,7 +197,8 @@ class ModelRunner:
             entry_start=part[3], entry_count=part[4], entry_first_row=part[5], entry_slot=part[6],
             block_tables={gi: part[8 + gi].view(batch, w) for gi, w in enumerate(widths)},
             want_rows=part[7], num_wanted=wanted, workspace=workspace,
-            max_count=max(m.count for m in metas), max_context=max_context)
+            max_count=max(m.count for m in metas), max_context=max_context,
+            upload=lambda values: self._staging.upload(np.asarray(values, dtype=np.int32)))
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         self._check(entries)

@@ -241,11 +241,13 @@ def gemm_skinny(a: Optional[torch.Tensor], w: torch.Tensor, out: torch.Tensor, a
     if norm is not None:
         call("pulse_gemm_skinny_fused", _ptr(None), _i64(ldx), _ptr(w), _i64(w.stride(0) if n > 1 else k), _ptr(out),
              _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0),
-             _i32(tune), _ptr(h), _ptr(sumsq), _i32(sumsq.shape[1]), _ptr(nweight), _f32(eps), _ptr(sumsq_out), _stream())
+             _i32(tune), _ptr(h), _ptr(sumsq), _i32(sumsq.shape[1]), _ptr(nweight), _f32(eps), _ptr(sumsq_out), _stream(),
+             label=f"N={n} K={k}")
     else:
         call("pulse_gemm_skinny_fused", _ptr(a), _i64(ldx), _ptr(w), _i64(w.stride(0) if n > 1 else k), _ptr(out),
              _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0),
-             _i32(tune), _ptr(None), _ptr(None), _i32(0), _ptr(None), _f32(0.0), _ptr(sumsq_out), _stream())
+             _i32(tune), _ptr(None), _ptr(None), _i32(0), _ptr(None), _f32(0.0), _ptr(sumsq_out), _stream(),
+             label=f"N={n} K={k}")
 
 
 MID_MAX_ROWS = 192
@@ -281,7 +283,7 @@ def gemm_mid(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool =
         mode, ldc = 0, (out.stride(0) if m > 1 else cols)
     call("pulse_gemm_mid", _ptr(a), _i64(a.stride(0) if m > 1 else k), _ptr(w), _i64(w.stride(0) if n > 1 else k),
          _ptr(out), _i64(ldc), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0), _i32(splits), _i32(waves),
-         _stream())
+         _stream(), label=f"N={n} K={k}")
 
 
 def _check_cache(what: str, kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, d: int):

@@ -81,15 +81,16 @@ def _invoke(lib: ctypes.CDLL, name: str, args) -> None:
         raise KernelError(f"{name}: {lib.pulse_last_error().decode(errors='replace')}")
 
 
-def call_in(lib: ctypes.CDLL, name: str, *args) -> None:
-    """Call an entry point of ``lib``; a non-zero return becomes a ``KernelError`` with the library's message."""
+def call_in(lib: ctypes.CDLL, name: str, *args, label: str = "") -> None:
+    """Call an entry point of ``lib``; a non-zero return becomes a ``KernelError`` with the library's message.
+    ``label`` (a shape, say) is added to the name under which a timing table lists the call."""
     if timing._active is not None:
-        with timing.region(name):
+        with timing.region(f"{name} {label}" if label else name):
             _invoke(lib, name, args)
         return
     _invoke(lib, name, args)
 
 
-def call(name: str, *args) -> None:
+def call(name: str, *args, label: str = "") -> None:
     """The same for the core library."""
-    call_in(load(), name, *args)
+    call_in(load(), name, *args, label=label)

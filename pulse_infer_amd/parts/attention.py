@@ -153,7 +153,7 @@ class PagedAttention(Part):
         key = f"static:attention.items:{per}:{portion}"
         if key not in ctx.extras:  # depends only on the step's shape; the same lists serve every layer
             short, long = attention_mfma.split_entries(ctx.entries)
-            dev = lambda flat: torch.tensor(flat, dtype=torch.int32, device=q.device) if flat else None
+            dev = lambda flat: ctx.to_device(flat) if flat else None
             ctx.extras[key] = (
                 dev(attention_mfma.build_items(short, per)),
                 dev(attention_mfma.build_items(long, portion)),

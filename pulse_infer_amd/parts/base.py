@@ -153,6 +153,14 @@ class StepContext:
     max_count: int = 1           # most tokens of one entry
     max_context: int = 1         # longest context (start + count) of an entry
     extras: Dict[str, Any] = field(default_factory=dict)  # per-step products of position encodings etc.
+    upload: Optional[Callable[[List[int]], torch.Tensor]] = None   # integers of a part's own to the device, through the
+                                                                   # step function's pinned staging (no synchronous copy)
+
+    def to_device(self, values: List[int]) -> torch.Tensor:
+        """An int32 device vector of ``values`` (work lists that a part builds from the step's entries)."""
+        if self.upload is not None:
+            return self.upload(values)
+        return torch.tensor(values, dtype=torch.int32, device=self.token_ids.device)
 
     def position_product(self, name: str, encodings: Dict[str, Any]) -> Any:
         """What position encoding ``name`` prepared for this step (prepared on first use)."""
