@@ -63,10 +63,14 @@ __device__ __forceinline__ int row_shift_left(int v, int n) {
 
 // Sum of the wavefronts' partial tiles, in wavefront order, and the store.  With `sumsq` (adding into a float32
 // matrix only) every slab also leaves the sum of squares of its 16 new values of each row, sumsq[row * parts + slab
-// number]: what a following RMSNorm needs of the row, so that the product after it can normalise by itself.
+// number]: what a following RMSNorm needs of the row, so that the product after it can normalise by itself; `copy`
+// takes the new values once more, rounded to bfloat16 (that product's input).  `row_scale` (one factor for each of
+// at most 16 rows) multiplies the sums before anything else is done with them.
 template <int SLABS, int MT, int KW, bool SWIGLU>
 __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void* __restrict__ C, int64_t ldc, int M, int N,
-                                         int n_base, int mode, int tid, float* __restrict__ sumsq = nullptr, int parts = 0) {
+                                         int n_base, int mode, int tid, float* __restrict__ sumsq = nullptr, int parts = 0,
+                                         const float* row_scale = nullptr, bf16_t* __restrict__ copy = nullptr,
+                                         int64_t ldcopy = 0) {
     constexpr int TILES = SLABS * MT;
     constexpr int THREADS = KW * PULSE_WAVE;
     if (!SWIGLU) {
@@ -77,6 +81,7 @@ __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void*
             float v = 0.f;
 #pragma unroll
             for (int w = 0; w < KW; ++w) v += red[w][tile][n_in][m_in];
+            if (row_scale) v *= row_scale[m_in];
             const int m = (tile % MT) * 16 + m_in;
             const int n = n_base + (tile / MT) * 16 + n_in;
             float updated = 0.f;
@@ -87,6 +92,7 @@ __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void*
                 else {
                     updated = static_cast<float*>(C)[at] + v;
                     static_cast<float*>(C)[at] = updated;
+                    if (copy) copy[static_cast<int64_t>(m) * ldcopy + n] = f32_to_bf16(updated);
                 }
             }
             if (sumsq) {  // the 16 lanes of a row of lanes hold the 16 columns of one row of the tile
@@ -111,6 +117,10 @@ __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void*
             for (int w = 0; w < KW; ++w) {
                 g += red[w][(2 * pair) * MT + mt][n_in][m_in];
                 u += red[w][(2 * pair + 1) * MT + mt][n_in][m_in];
+            }
+            if (row_scale) {
+                g *= row_scale[m_in];
+                u *= row_scale[m_in];
             }
             const int m = mt * 16 + m_in;
             const int n = n_base / 2 + pair * 16 + n_in;
@@ -257,25 +267,28 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_kernel(const bf16_
 //
 // Both only change which lane fetches what; every product and the order of the sums are those of the kernel above.
 //
-// NORMED: X is not given; the float32 residual H is, with the row sums of squares that the product before left
-// (`sumsq`, `parts` of them a row) and the RMSNorm weight: x = bfloat16(h / sqrt(mean(h^2) + eps) * w) is formed here,
-// as the norm kernel forms it, and that kernel's launch is saved.
+// SCALED: X is a matrix whose rows have not been normalised yet (a bfloat16 copy of the residual); the row sums of
+// squares that the product before left come with it (`sumsq`, `parts` of them a row), and every row of the result is
+// multiplied by 1 / sqrt(mean(x^2) + eps) in the epilogue, where it costs nothing: x W^T scaled by rows is (x scaled
+// by rows) W^T.  A weight of the norm has to be part of W already (W' = W diag(w)).  That saves the norm kernel's
+// launch.  (Forming the normalised x in this kernel's loop from the float32 residual was measured too: every k-step
+// then reads float32 values and a weight of the norm, and from 8 rows on that costs what the launch saves.)
 constexpr int STAGGER_BLOCKS = 64;  // consecutive workgroups that start at the same group of k-steps
 
-struct NormInput {
-    const float* h;        // [M, K] float32, row stride ldx
-    const float* sumsq;    // [M, parts]
-    const bf16_t* weight;  // [K]
+struct RowScale {
+    const float* sumsq;  // [M, parts]
     int parts;
     float eps;
 };
 
-template <int SLABS, int KW, int PACK, bool SWIGLU, bool NORMED>
+template <int SLABS, int KW, int PACK, bool SWIGLU, bool SCALED>
 __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(const bf16_t* __restrict__ X, int64_t ldx,
                                                                              const bf16_t* __restrict__ W, int64_t ldw,
                                                                              void* __restrict__ C, int64_t ldc, int M,
-                                                                             int N, int K, int mode, NormInput norm,
-                                                                             float* __restrict__ sumsq_out, int parts_out) {
+                                                                             int N, int K, int mode, RowScale scale,
+                                                                             float* __restrict__ sumsq_out, int parts_out,
+                                                                             bf16_t* __restrict__ copy_out, int64_t ldcopy) {
+    constexpr int THREADS = KW * PULSE_WAVE;
     static_assert(PACK == 1 || PACK == 2 || PACK == 4 || PACK == 8, "PACK k-steps a load of X");
     static_assert(UNROLL % 2 == 0 && UNROLL % PACK == 0, "groups hold whole pairs and whole packs");
     constexpr int MP = 16 / PACK;  // rows of X a pack has room for
@@ -310,10 +323,7 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
     const int xr = r % MP;
     const bool xok = xr < M;
     const int x_at = (r / MP) * 32 + kg * 8;
-    const bf16_t* xrow = NORMED ? nullptr : X + static_cast<int64_t>(xok ? xr : 0) * ldx + x_at;
-    const float* hrow = NORMED ? norm.h + static_cast<int64_t>(xok ? xr : 0) * ldx + x_at : nullptr;
-    const bf16_t* nrow = NORMED ? norm.weight + x_at : nullptr;
-    float rstd = 0.f;
+    const bf16_t* xrow = X + static_cast<int64_t>(xok ? xr : 0) * ldx + x_at;
     __shared__ float s_rstd[16];
 
     // Workgroups do not all walk K from the same end: every 64 of them start one group of steps later than the 64
@@ -323,11 +333,25 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
     // its place in the grid only, so results stay the same from run to run and for any rows beside.
     const int groups = per / UNROLL;
     const int rot = static_cast<int>((blockIdx.x / STAGGER_BLOCKS) % static_cast<unsigned>(groups));
+
+    // SCALED: 1 / sqrt(mean(x^2) + eps) of every row from the parts of its sum of squares, all rows at once:
+    // THREADS / 16 threads a row, each with four 16-byte loads in flight first of all, so that one round trip to
+    // memory brings rows of up to THREADS parts (any number of parts is taken; no multiple of four: one by one).
+    constexpr int TPR = THREADS / 16;
+    const int srow = tid / TPR, sl = tid % TPR;
+    const bool sok = SCALED && srow < M;
+    const float* src = SCALED ? scale.sumsq + static_cast<int64_t>(sok ? srow : 0) * scale.parts : nullptr;
+    const int quads = (SCALED && (scale.parts & 3) == 0) ? scale.parts / 4 : 0;
+    f32x4 first_parts[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        first_parts[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (sok && j * TPR + sl < quads) first_parts[j] = *reinterpret_cast<const f32x4*>(src + 4 * (j * TPR + sl));
+    }
+
     for (int gi = 0; gi < groups; ++gi) {
         const int ks = step_begin + (gi + rot >= groups ? gi + rot - groups : gi + rot) * UNROLL;
         bf16x8 xb[UNROLL], wa[UNROLL][SLABS];
-        f32x4 hraw[NORMED ? UNROLL / PACK : 1][2];
-        bf16x8 nraw[NORMED ? UNROLL / PACK : 1];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int pair_k = ((ks + u) & ~1) * 32;
@@ -335,30 +359,34 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
             for (int s = 0; s < SLABS; ++s)
                 wa[u][s] = __builtin_bit_cast(bf16x8, stream_load16(((u & 1) ? w1[s] : w0[s]) + pair_k));
             if (u % PACK == 0) {
-                if (NORMED) {
-                    hraw[u / PACK][0] = hraw[u / PACK][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-                    if (xok) {
-                        hraw[u / PACK][0] = *reinterpret_cast<const f32x4*>(hrow + (ks + u) * 32);
-                        hraw[u / PACK][1] = *reinterpret_cast<const f32x4*>(hrow + (ks + u) * 32 + 4);
-                    }
-                    nraw[u / PACK] = *reinterpret_cast<const bf16x8*>(nrow + (ks + u) * 32);
-                } else {
-                    xb[u] = zeros8();
-                    if (xok) xb[u] = *reinterpret_cast<const bf16x8*>(xrow + (ks + u) * 32);
-                }
+                xb[u] = zeros8();
+                if (xok) xb[u] = *reinterpret_cast<const bf16x8*>(xrow + (ks + u) * 32);
             }
         }
-        if (NORMED && gi == 0) {
-            // 1 / sqrt(mean(h^2) + eps) of every row from the parts; a wavefront takes rows wave, wave + KW, ..  This
-            // stands behind the first group's loads so that its own round trip to memory runs beside theirs.
-            for (int m = wave; m < M; m += KW) {
-                float sum = 0.f;
-                for (int p = lane; p < norm.parts; p += PULSE_WAVE) sum += norm.sumsq[static_cast<int64_t>(m) * norm.parts + p];
-                sum = wave_sum(sum);
-                if (lane == 0) s_rstd[m] = 1.0f / sqrtf(sum / static_cast<float>(K) + norm.eps);
+        if (SCALED && gi == 0) {
+            // the parts' loads went out before this group's; adding them up here keeps their round trip to memory
+            // beside the weights'.  The factors are read in the epilogue, behind the barrier that it needs anyway.
+            float sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) sum += (first_parts[j][0] + first_parts[j][1]) + (first_parts[j][2] + first_parts[j][3]);
+            if (quads > 0) {
+                for (int q0 = 4 * TPR; q0 < quads; q0 += 4 * TPR) {  // rows of more than 16 * TPR parts
+                    f32x4 v[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int q = q0 + j * TPR + sl;
+                        v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+                        if (sok && q < quads) v[j] = *reinterpret_cast<const f32x4*>(src + 4 * q);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) sum += (v[j][0] + v[j][1]) + (v[j][2] + v[j][3]);
+                }
+            } else {
+                for (int p = sl; sok && p < scale.parts; p += TPR) sum += src[p];
             }
-            __syncthreads();
-            rstd = xok ? s_rstd[xr] : 0.f;
+#pragma unroll
+            for (int off = TPR / 2; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, TPR);
+            if (sl == 0 && sok) s_rstd[srow] = 1.0f / sqrtf(sum / static_cast<float>(K) + scale.eps);
         }
         // every load of the group is on its way; now the lane exchanges
 #pragma unroll
@@ -379,18 +407,6 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
                 }
                 wa[u][s] = __builtin_bit_cast(bf16x8, a0);
                 wa[u + 1][s] = __builtin_bit_cast(bf16x8, a1);
-            }
-        }
-        if (NORMED) {
-#pragma unroll
-            for (int u = 0; u < UNROLL; u += PACK) {
-                bf16x8 x;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float hv = hraw[u / PACK][e / 4][e % 4];
-                    x[e] = (__bf16)(hv * rstd * static_cast<float>(nraw[u / PACK][e]));  // as the norm kernel: (h * inv) * w, one rounding
-                }
-                xb[u] = x;
             }
         }
         if (PACK > 1) {
@@ -417,7 +433,8 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
 #pragma unroll
         for (int i = 0; i < 4; ++i) red[wave][s][4 * kg + i][r] = acc[s][i];
     __syncthreads();
-    epilogue<SLABS, 1, KW, SWIGLU>(red, C, ldc, M, N, n_base, mode, tid, sumsq_out, parts_out);
+    epilogue<SLABS, 1, KW, SWIGLU>(red, C, ldc, M, N, n_base, mode, tid, sumsq_out, parts_out,
+                                   SCALED ? s_rstd : nullptr, copy_out, ldcopy);
 }
 
 template <int SLABS, int MT, int KW, bool SWIGLU>
@@ -438,23 +455,23 @@ void launch(bool xlds, const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ld
 
 template <int SLABS, int KW, bool SWIGLU>
 void launch_stream(int pack, const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
-                   int K, int mode, const NormInput& norm, float* sumsq_out, int parts_out, hipStream_t stream) {
+                   int K, int mode, const RowScale& scale, float* sumsq_out, int parts_out, bf16_t* copy_out, int64_t ldcopy,
+                   hipStream_t stream) {
     const dim3 grid((N + SLABS * 16 - 1) / (SLABS * 16)), block(KW * PULSE_WAVE);
     const size_t red_bytes = sizeof(float) * KW * SLABS * 16 * 17;
-#define PULSE_STREAM(P, NORMED)                                                                                          \
-    hipLaunchKernelGGL((gemm_skinny_stream_kernel<SLABS, KW, P, SWIGLU, NORMED>), grid, block, red_bytes, stream, X, ldx, \
-                       W, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out)
-    if (norm.h) {
-        if (pack == 8) PULSE_STREAM(8, true);
-        else if (pack == 4) PULSE_STREAM(4, true);
-        else if (pack == 2) PULSE_STREAM(2, true);
-        else PULSE_STREAM(1, true);
-    } else {
-        if (pack == 8) PULSE_STREAM(8, false);
-        else if (pack == 4) PULSE_STREAM(4, false);
-        else if (pack == 2) PULSE_STREAM(2, false);
-        else PULSE_STREAM(1, false);
-    }
+#define PULSE_STREAM(P, SCALED)                                                                                          \
+    hipLaunchKernelGGL((gemm_skinny_stream_kernel<SLABS, KW, P, SWIGLU, SCALED>), grid, block, red_bytes, stream, X, ldx, \
+                       W, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy_out, ldcopy)
+#define PULSE_STREAM_PACKS(SCALED)                    \
+    do {                                              \
+        if (pack == 8) PULSE_STREAM(8, SCALED);       \
+        else if (pack == 4) PULSE_STREAM(4, SCALED);  \
+        else if (pack == 2) PULSE_STREAM(2, SCALED);  \
+        else PULSE_STREAM(1, SCALED);                 \
+    } while (0)
+    if (scale.sumsq) PULSE_STREAM_PACKS(true);
+    else PULSE_STREAM_PACKS(false);
+#undef PULSE_STREAM_PACKS
 #undef PULSE_STREAM
 }
 
@@ -466,31 +483,30 @@ int pack_for(int M) { return M <= 2 ? 8 : (M <= 4 ? 4 : (M <= 8 ? 2 : 1)); }
 // mode: 0 store bfloat16, 1 store float32, 2 add into float32.  swiglu != 0: W holds gate and up rows interleaved in
 // slabs of 16 (gate slab, up slab, ...), N counts both, C is bfloat16 [M, N / 2] = silu(gate) * up.  tune: 0 lets the
 // entry point choose the kernel.
-// The same with the two fusions of the streaming kernel (M <= 16, K a multiple of 1024), each optional:
-//   norm_h != null: X is not read; x = bfloat16(norm_h / sqrt(mean(norm_h^2) + eps) * norm_w) is formed in the kernel
-//     from the float32 matrix norm_h [M, K] (row stride ldx), its row sums of squares norm_sumsq [M, norm_parts] (any
-//     split of the row into parts) and the bfloat16 weight norm_w [K];
+// The same with the fusions of the streaming kernel (M <= 16, K a multiple of 1024), each optional:
+//   scale_sumsq != null: row m of the product is multiplied by 1 / sqrt(sum(scale_sumsq[m, :]) / K + eps) before it is
+//     stored (or goes through SwiGLU): the RMSNorm of X's rows, applied behind the product, from the rows' sums of
+//     squares [M, scale_parts] (any split of a row into parts); a weight of that norm has to be folded into W beforehand;
 //   sumsq_out != null (mode 2 only): besides adding into C, leave sumsq_out[row * parts + slab] = sum of squares of the
-//     new values of C[row, 16 slab .. 16 slab + 15], parts = ceil(N / 16).
+//     new values of C[row, 16 slab .. 16 slab + 15], parts = ceil(N / 16);
+//   copy_out != null (mode 2 only): the new values of C once more as bfloat16, row stride ldcopy.
 // pulse_gemm_skinny_fusable says whether the streaming kernel takes a shape.
 extern "C" int pulse_gemm_skinny_fusable(int M, int N, int K) { return M >= 1 && M <= 16 && N > 0 && K > 0 && K % 1024 == 0; }
 
 extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
-                                       int N, int K, int mode, int swiglu, int tune, const float* norm_h,
-                                       const float* norm_sumsq, int norm_parts, const void* norm_w, float norm_eps,
-                                       float* sumsq_out, hipStream_t stream) {
-    const bool fused = norm_h != nullptr || sumsq_out != nullptr;
+                                       int N, int K, int mode, int swiglu, int tune, const float* scale_sumsq,
+                                       int scale_parts, float scale_eps, float* sumsq_out, void* copy_out,
+                                       int64_t ldcopy, hipStream_t stream) {
+    const bool fused = scale_sumsq != nullptr || sumsq_out != nullptr || copy_out != nullptr;
     if (fused) {
         PULSE_REQUIRE(pulse_gemm_skinny_fusable(M, N, K) && tune != 9, "gemm_skinny: M=%d N=%d K=%d cannot take the fused kernel", M, N, K);
         PULSE_REQUIRE(sumsq_out == nullptr || (mode == OUT_ADD_F32 && !swiglu), "gemm_skinny: row sums of squares come with adding into float32 only");
-        PULSE_REQUIRE(norm_h == nullptr || (norm_sumsq && norm_w && norm_parts > 0 && ldx % 4 == 0 && ldx >= K &&
-                                            (reinterpret_cast<uintptr_t>(norm_h) % 16) == 0 &&
-                                            (reinterpret_cast<uintptr_t>(norm_w) % 16) == 0),
-                      "gemm_skinny: the norm's inputs are missing or misaligned");
+        PULSE_REQUIRE(copy_out == nullptr || (mode == OUT_ADD_F32 && !swiglu && ldcopy >= N), "gemm_skinny: the bfloat16 copy comes with adding into float32 only");
+        PULSE_REQUIRE(scale_sumsq == nullptr || (scale_parts > 0 && (reinterpret_cast<uintptr_t>(scale_sumsq) % 16) == 0),
+                      "gemm_skinny: the row sums of squares need their number of parts and 16-byte alignment");
     }
-    if (norm_h) X = norm_h;  // only for the checks below: a non-null, aligned pointer with a fitting stride
     PULSE_REQUIRE(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: sizes M=%d (at most 64) N=%d K=%d", M, N, K);
-    PULSE_REQUIRE(K % 8 == 0 && (norm_h || ldx % 8 == 0) && ldw % 8 == 0 && ldx >= K && ldw >= K,
+    PULSE_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldx >= K && ldw >= K,
                   "gemm_skinny: K and the row strides must be multiples of 8 (16-byte loads)");
     PULSE_REQUIRE((reinterpret_cast<uintptr_t>(X) % 16) == 0 && (reinterpret_cast<uintptr_t>(W) % 16) == 0,
                   "gemm_skinny: operands must be 16-byte aligned");
@@ -503,9 +519,10 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
         PULSE_REQUIRE(ldc >= N, "gemm_skinny: output row stride too small");
     }
     if (M == 0) return 0;
-    const bf16_t* x = norm_h ? nullptr : static_cast<const bf16_t*>(X);
-    NormInput norm{norm_h, norm_sumsq, static_cast<const bf16_t*>(norm_w), norm_parts, norm_eps};
+    const bf16_t* x = static_cast<const bf16_t*>(X);
+    RowScale scale{scale_sumsq, scale_parts, scale_eps};
     const int parts_out = (N + 15) / 16;
+    bf16_t* copy = static_cast<bf16_t*>(copy_out);
     const bf16_t* w = static_cast<const bf16_t*>(W);
     const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
     const int units = pulse_compute_units();
@@ -532,14 +549,14 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
         const int kw = t_kw ? t_kw : ((K % 2048 == 0 && !pairs) ? 8 : 4);
         const int pack = t_pack ? t_pack : pack_for(M);
         if (swiglu) {
-            if (kw == 8) launch_stream<2, 8, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
-            else launch_stream<2, 4, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
+            if (kw == 8) launch_stream<2, 8, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
+            else launch_stream<2, 4, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
         } else if (slabs == 2) {
-            if (kw == 8) launch_stream<2, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
-            else launch_stream<2, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
+            if (kw == 8) launch_stream<2, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
+            else launch_stream<2, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
         } else {
-            if (kw == 8) launch_stream<1, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
-            else launch_stream<1, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, norm, sumsq_out, parts_out, stream);
+            if (kw == 8) launch_stream<1, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
+            else launch_stream<1, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
         }
         PULSE_LAUNCH_CHECK("gemm_skinny");
         return 0;
@@ -565,6 +582,6 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
 
 extern "C" int pulse_gemm_skinny(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
                                  int N, int K, int mode, int swiglu, int tune, hipStream_t stream) {
-    return pulse_gemm_skinny_fused(X, ldx, W, ldw, C, ldc, M, N, K, mode, swiglu, tune, nullptr, nullptr, 0, nullptr, 0.f,
-                                   nullptr, stream);
+    return pulse_gemm_skinny_fused(X, ldx, W, ldw, C, ldc, M, N, K, mode, swiglu, tune, nullptr, 0, 0.f, nullptr, nullptr, 0,
+                                   stream);
 }

@@ -187,38 +187,28 @@ def gemm_skinny_fusable(m: int, n: int, k: int) -> bool:
     return 1 <= m <= SKINNY_FAST_ROWS and n > 0 and k > 0 and k % 1024 == 0   # as pulse_gemm_skinny_fusable
 
 
-def gemm_skinny(a: Optional[torch.Tensor], w: torch.Tensor, out: torch.Tensor, add: bool = False, swiglu: bool = False,
-                tune: int = 0, norm: Optional[tuple] = None, sumsq_out: Optional[torch.Tensor] = None) -> None:
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool = False, swiglu: bool = False,
+                tune: int = 0, sumsq_out: Optional[torch.Tensor] = None, row_scale: Optional[tuple] = None,
+                copy_out: Optional[torch.Tensor] = None) -> None:
     """out = a @ w^T for at most 64 rows of bfloat16, float32 accumulation on the matrix cores.
 
     ``out`` bfloat16 or float32 is stored; with ``add`` (float32 only) the product is added to it.  With
     ``swiglu`` the weight holds gate and up rows in alternating slabs of 16 and out is silu(gate) * up.
     ``tune`` picks a kernel variant by hand (tests and measurements); 0 lets the library choose.
 
-    Two fusions for shapes that ``gemm_skinny_fusable`` accepts.  ``norm = (h, sumsq, weight, eps)`` instead of
-    ``a``: the input is RMSNorm(h) * weight, formed inside the kernel from the float32 matrix ``h`` and the sums of
-    squares of its rows, given in parts ``sumsq`` [M, parts].  ``sumsq_out`` [M, ceil(N / 16)] with ``add``: the
-    kernel also leaves the sums of squares of the rows of the updated ``out``, 16 columns a part.
+    Fusions for shapes that ``gemm_skinny_fusable`` accepts.  ``row_scale = (sumsq, eps)``: row m of the product is
+    multiplied by 1 / sqrt(sum(sumsq[m]) / K + eps) before it is stored or goes through SwiGLU, which is the product
+    of the RMS-normalised rows of ``a`` when ``sumsq`` [M, parts] holds the sums of squares of those rows in parts (a
+    weight of that norm has to be part of ``w``).  ``sumsq_out`` [M, ceil(N / 16)] with ``add``: the kernel also
+    leaves the sums of squares of the rows of the updated ``out``, 16 columns a part; ``copy_out`` [M, N] bfloat16
+    with ``add``: the updated ``out`` once more, rounded.
     """
-    if norm is not None:
-        h, sumsq, nweight, eps = norm
-        _gpu("gemm_skinny", h, sumsq, nweight, w, out, sumsq_out)
-        _need(a is None, "gemm_skinny: give either the input or what it is the norm of")
-        _need(h.dtype == torch.float32 and h.dim() == 2 and h.stride(1) == 1 and w.dim() == 2 and h.shape[1] == w.shape[1],
-              "gemm_skinny: the norm's input must be a float32 matrix with the weight's inner size")
-        m, k = h.shape
-        _need(sumsq.dtype == torch.float32 and sumsq.dim() == 2 and sumsq.shape[0] >= m and sumsq.is_contiguous(),
-              "gemm_skinny: the row sums of squares must be a contiguous float32 [M, parts]")
-        _need(nweight.dtype == torch.bfloat16 and nweight.numel() == k and nweight.is_contiguous(),
-              "gemm_skinny: the fused norm takes a bfloat16 weight of the inner size")
-        _need(w.dtype == torch.bfloat16 and w.stride(1) == 1 and w.data_ptr() % 16 == 0, "gemm_skinny: bad weight")
-        ldx = h.stride(0) if m > 1 else k
-    else:
-        _gpu("gemm_skinny", a, w, out, sumsq_out)
-        _need(gemm_skinny_ok(a, w), "gemm_skinny: needs bfloat16 operands with at most 64 rows, K a multiple of 8, "
-              "contiguous 16-byte aligned rows")
-        m, k = a.shape
-        ldx = a.stride(0) if m > 1 else k
+    scale_sumsq, scale_eps = row_scale if row_scale is not None else (None, 0.0)
+    _gpu("gemm_skinny", a, w, out, sumsq_out, copy_out, scale_sumsq)
+    _need(gemm_skinny_ok(a, w), "gemm_skinny: needs bfloat16 operands with at most 64 rows, K a multiple of 8, "
+          "contiguous 16-byte aligned rows")
+    m, k = a.shape
+    ldx = a.stride(0) if m > 1 else k
     n, k2 = w.shape
     _need(k == k2, f"gemm_skinny: inner sizes differ: a is [{m}, {k}], w is [{n}, {k2}]")
     cols = n // 2 if swiglu else n
@@ -232,22 +222,26 @@ def gemm_skinny(a: Optional[torch.Tensor], w: torch.Tensor, out: torch.Tensor, a
     if swiglu:
         _need(m <= SKINNY_SWIGLU_MAX_ROWS and n % 32 == 0 and out.dtype == torch.bfloat16,
               "gemm_skinny: the SwiGLU epilogue needs at most 32 rows, N a multiple of 32 and bfloat16 output")
-    if norm is not None or sumsq_out is not None:
+    if sumsq_out is not None or row_scale is not None or copy_out is not None:
         _need(gemm_skinny_fusable(m, n, k), f"gemm_skinny: M={m} N={n} K={k} cannot take the fused kernel")
     if sumsq_out is not None:
         _need(add and sumsq_out.dtype == torch.float32 and sumsq_out.is_contiguous() and sumsq_out.dim() == 2
               and sumsq_out.shape[0] >= m and sumsq_out.shape[1] == (n + 15) // 16,
               "gemm_skinny: sumsq_out must be a contiguous float32 [M, ceil(N / 16)] and comes with add")
-    if norm is not None:
-        call("pulse_gemm_skinny_fused", _ptr(None), _i64(ldx), _ptr(w), _i64(w.stride(0) if n > 1 else k), _ptr(out),
-             _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0),
-             _i32(tune), _ptr(h), _ptr(sumsq), _i32(sumsq.shape[1]), _ptr(nweight), _f32(eps), _ptr(sumsq_out), _stream(),
-             label=f"N={n} K={k}")
-    else:
-        call("pulse_gemm_skinny_fused", _ptr(a), _i64(ldx), _ptr(w), _i64(w.stride(0) if n > 1 else k), _ptr(out),
-             _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0),
-             _i32(tune), _ptr(None), _ptr(None), _i32(0), _ptr(None), _f32(0.0), _ptr(sumsq_out), _stream(),
-             label=f"N={n} K={k}")
+    if copy_out is not None:
+        _need(add and copy_out.dtype == torch.bfloat16 and tuple(copy_out.shape) == (m, n) and copy_out.stride(1) == 1,
+              f"gemm_skinny: copy_out must be bfloat16 [{m}, {n}] and comes with add")
+    ldcopy = 0 if copy_out is None else (copy_out.stride(0) if m > 1 else n)
+    scale_parts = 0
+    if scale_sumsq is not None:
+        _need(scale_sumsq.dtype == torch.float32 and scale_sumsq.dim() == 2 and scale_sumsq.shape[0] >= m
+              and scale_sumsq.is_contiguous() and scale_sumsq.shape[1] > 0 and scale_sumsq.data_ptr() % 16 == 0,
+              "gemm_skinny: the row sums of squares must be a contiguous, 16-byte aligned float32 [M, parts]")
+        scale_parts = scale_sumsq.shape[1]
+    call("pulse_gemm_skinny_fused", _ptr(a), _i64(ldx), _ptr(w), _i64(w.stride(0) if n > 1 else k), _ptr(out),
+         _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0),
+         _i32(tune), _ptr(scale_sumsq), _i32(scale_parts), _f32(scale_eps), _ptr(sumsq_out), _ptr(copy_out),
+         _i64(ldcopy), _stream(), label=f"N={n} K={k}")
 
 
 MID_MAX_ROWS = 192

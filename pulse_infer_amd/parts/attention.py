@@ -87,8 +87,12 @@ class PagedAttention(Part):
         return PagedKVSpec(self.nkv, self.d, int(self.window) if self.window is not None else None)
 
     accepts_residual = True
-    accepts_lazy_input = True   # the first product may compute the norm before it by itself
+    accepts_lazy_input = True   # the first product may take rows that are not normalised yet and scale its result
     records_cleanly = True      # positions, tables and work lists are read on the device
+
+    def fold_input_weight(self, scale: torch.Tensor) -> bool:
+        """Column factors of the input (the weight of the norm before) go into the q, k and v weights."""
+        return self.qkv.fold_input_weight(scale)
 
     def forward(self, x, ctx: StepContext, cache: PagedCacheView, residual: Optional[torch.Tensor] = None):
         tokens = x.shape[0]

@@ -173,25 +173,30 @@ class StepContext:
 @dataclass
 class RowStats:
     """What a part that added into the residual itself knows about the new rows: their sums of squares, in parts
-    (``sumsq`` [rows, parts] float32).  A norm that only needs that of a row can then be left to its consumer."""
+    (``sumsq`` [rows, parts] float32), and the rows themselves once more, rounded to the activations' type
+    (``rounded`` [rows, H]).  A norm that only divides a row by a figure of its own can then be left to its consumer."""
 
     sumsq: torch.Tensor
+    rounded: Optional[torch.Tensor] = None
 
 
 @dataclass
 class LazyNorm:
-    """A normalised input that has not been computed: norm(h) * weight, for a consumer whose first product can form
-    it by itself (``accepts_lazy_input``).  ``materialize`` computes it the ordinary way."""
+    """A normalised input that has not been computed: the rows of ``x`` (the residual ``h``, rounded) each divided by
+    sqrt(mean of its squares + eps), the mean taken from the sums of squares in ``sumsq`` [rows, parts].  A consumer
+    whose first product is linear (``accepts_lazy_input``) multiplies the rows of that product's result instead, which
+    is the same and costs nothing.  The norm has no weight of its own then: the consumer's first product holds it
+    (``fold_input_weight``).  ``materialize`` computes the input the ordinary way."""
 
-    h: torch.Tensor
+    x: torch.Tensor
     sumsq: torch.Tensor
-    weight: torch.Tensor
     eps: float
+    h: torch.Tensor
     norm: Any
 
     @property
     def shape(self):
-        return self.h.shape
+        return self.x.shape
 
     def materialize(self, out: torch.Tensor) -> torch.Tensor:
         return self.norm.apply(self.h, None, out)
@@ -203,11 +208,6 @@ class ResidualStream:
     Adding is deferred so that it happens inside the next norm's kernel.  A part that added its result itself may
     hand back ``RowStats`` of the new ``h``; they stay valid until ``h`` changes again.
     """
-
-    # Up to here a consumer that forms the norm itself is faster than the norm's kernel followed by it (measured on a
-    # decoding step: 5% at 1 row, 0.3% at 6; at 8 rows the norm's kernel wins by 2.5%: every k-step of the product
-    # reads the float32 residual then).
-    LAZY_MAX_ROWS = 6
 
     def __init__(self, h: torch.Tensor):
         self.h = h
@@ -232,8 +232,6 @@ class ResidualStream:
         """The norm of the current ``h`` as something a consumer can compute itself, if the norm allows that and the
         rows' statistics are at hand."""
         if self.pending is not None or self.stats is None or not hasattr(norm, "lazy"):
-            return None
-        if self.h.shape[0] > self.LAZY_MAX_ROWS:
             return None
         return norm.lazy(self.h, self.stats)
 

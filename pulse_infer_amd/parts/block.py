@@ -44,6 +44,13 @@ class PreNormBlock(Part):
         self.ffn = FEED_FORWARDS.get(layer.ffn.kind)(layer.ffn.params,
                                                      joined(layer.prefix, layer.ffn.params.get("prefix", "")), build)
         self.act_dtype = build.act_dtype
+        # A norm that scales columns and a part whose first product is linear: the product's weight takes the norm's
+        # over (W diag(w)), and what is left of the norm, a division of each row, can move behind that product.
+        for norm, part in ((self.mixer_norm, self.mixer), (self.ffn_norm, self.ffn)):
+            if hasattr(norm, "foldable_weight") and hasattr(part, "fold_input_weight"):
+                weight = norm.foldable_weight()
+                if weight is not None and part.fold_input_weight(weight):
+                    norm.weight_folded()
 
     def cache_spec(self) -> Optional[Any]:
         return self.mixer.cache_spec()

@@ -18,7 +18,7 @@ import torch
 
 from ..ops import kernels, timing
 from ..ops.device import compute_units
-from .base import LazyNorm, ResidualStream, RowStats, Workspace
+from .base import LazyNorm, RowStats, Workspace
 
 
 library_calls = 0   # products that went to the vendor library so far (a step that made none can be recorded as a graph)
@@ -33,11 +33,24 @@ class Linear:
         self.mode = mode
         self.library = mode == "bfloat16" and weight.dtype == torch.bfloat16
 
+    def fold_input_weight(self, scale: torch.Tensor) -> bool:
+        """W <- W diag(scale), rounded once: a factor of every input column (the weight of the norm before) becomes
+        part of this product.  Only bfloat16 products on the matrix cores do that; False otherwise."""
+        if not self.library or scale.numel() != self.in_features:
+            return False
+        folded = torch.empty_like(self.weight)
+        factor = scale.to(torch.float32).view(1, -1)
+        step = max(1, (1 << 26) // self.in_features)   # a quarter of a gigabyte of float32 at a time
+        for r0 in range(0, self.out_features, step):
+            folded[r0:r0 + step] = (self.weight[r0:r0 + step].to(torch.float32) * factor).to(self.weight.dtype)
+        self.weight = folded
+        return True
+
     def takes_lazy(self, x: LazyNorm, rows: Optional[int] = None) -> bool:
-        """Whether the product can form this not yet computed input by itself."""
+        """Whether the product can take rows that have not been normalised yet and scale its result instead."""
         n = self.out_features if rows is None else rows
         return (self.library and kernels.gemm_skinny_fusable(x.shape[0], n, self.in_features)
-                and x.h.stride(1) == 1 and self.weight.stride(1) == 1)
+                and x.x.dtype == torch.bfloat16 and kernels.gemm_skinny_ok(x.x, self.weight))
 
     def forward(self, x, out: torch.Tensor, rows: Optional[int] = None, swiglu: bool = False,
                 own: bool = True) -> torch.Tensor:
@@ -47,7 +60,7 @@ class Linear:
         measured the library faster for its shape)."""
         w = self.weight if rows is None else self.weight[:rows]
         if isinstance(x, LazyNorm):
-            kernels.gemm_skinny(None, w, out, swiglu=swiglu, norm=(x.h, x.sumsq, x.weight, x.eps))
+            kernels.gemm_skinny(x.x, w, out, swiglu=swiglu, row_scale=(x.sumsq, x.eps))
             return out
         if swiglu:
             if x.shape[0] > kernels.SKINNY_FAST_ROWS:
@@ -90,7 +103,8 @@ class Linear:
     def add_into(self, x: torch.Tensor, residual: torch.Tensor, scratch: torch.Tensor,
                  workspace: Optional[Workspace] = None):
         """residual += x W^T, in one of five ways.  Few rows: the kernel adds into the residual itself and None is
-        returned, or, given a workspace and a shape the fused kernel takes, the ``RowStats`` of the updated rows.  13 to
+        returned, or, given a workspace and a shape the fused kernel takes, the ``RowStats`` of the updated rows (their
+        sums of squares and a rounded copy, with which the next product can do without a norm kernel before it).  13 to
         192 rows, given a workspace: the product's inner dimension is shared out over workgroups and the shares' float32
         results [parts, rows, out] are returned as the update, which the next norm adds up in order; more rows of a
         product with a wide inner dimension and a narrow output: the same through the library's batched product.
@@ -119,12 +133,14 @@ class Linear:
             return parts
         if (self.library and x.dtype == torch.bfloat16 and x.shape[0] <= kernels.SKINNY_FAST_ROWS
                 and kernels.gemm_skinny_ok(x, self.weight)):
-            if (workspace is not None and x.shape[0] <= ResidualStream.LAZY_MAX_ROWS   # nobody would use them otherwise
+            if (workspace is not None
                     and kernels.gemm_skinny_fusable(x.shape[0], self.out_features, self.in_features)):
                 sums = workspace.buffer(f"linear.sumsq.{self.out_features}", x.shape[0], (self.out_features + 15) // 16,
                                         torch.float32)
-                kernels.gemm_skinny(x, self.weight, residual, add=True, sumsq_out=sums)
-                return RowStats(sums)
+                rounded = workspace.buffer(f"linear.rounded.{self.out_features}", x.shape[0], self.out_features,
+                                           torch.bfloat16)
+                kernels.gemm_skinny(x, self.weight, residual, add=True, sumsq_out=sums, copy_out=rounded)
+                return RowStats(sums, rounded)
             kernels.gemm_skinny(x, self.weight, residual, add=True)
             return None
         return self.forward(x, scratch)

@@ -50,8 +50,12 @@ class GatedMLP(Part):
         self.act_dtype = build.act_dtype
 
     accepts_residual = True
-    accepts_lazy_input = True   # the first product may compute the norm before it by itself
+    accepts_lazy_input = True   # the first product may take rows that are not normalised yet and scale its result
     records_cleanly = True
+
+    def fold_input_weight(self, scale: torch.Tensor) -> bool:
+        """Column factors of the input (the weight of the norm before) go into the gate+up weight."""
+        return self.gate_up.fold_input_weight(scale)
 
     def forward(self, x, ctx: StepContext, residual: Optional[torch.Tensor] = None):
         tokens = x.shape[0]

@@ -805,39 +805,53 @@ def test_gemm_skinny_streaming_variants(k, m, n, kk):
 
 @pytest.mark.parametrize("m", [1, 3, 8, 13, 16])
 @pytest.mark.parametrize("n,kk,swiglu", [(48, 1024, False), (4096 + 32, 2048, False), (96, 3072, True)])
-def test_gemm_skinny_fused_norm_and_row_sums(k, m, n, kk, swiglu):
-    """The product that normalises its input itself, from the float32 residual and the row sums of squares that the
-    product before it left, against the norm kernel followed by the plain product; and those row sums themselves."""
+def test_gemm_skinny_rounded_copy_and_rows_scaled_behind_the_product(k, m, n, kk, swiglu):
+    """The norm moved behind the product: the product that adds into the residual leaves the new rows once more in
+    bfloat16 with their sums of squares, and the next product, given those, multiplies row m of its result by
+    1 / sqrt(mean(x_m^2) + eps) before it stores it or applies SwiGLU.  Against the formula in float64."""
     eps = 3e-6
-    h = (rnd(m, kk, seed=80) * 3).to(DEV)
-    nw, _ = as_stored(1 + 0.1 * rnd(kk, seed=81), torch.bfloat16)
-    w, wref = as_stored(rnd(n, kk, seed=82, scale=kk ** -0.5), torch.bfloat16)
-    # 1. adding into the residual leaves the sums of squares of the new rows, 16 columns a part
-    a, aref = as_stored(rnd(m, 2048, seed=83), torch.bfloat16)
-    wo, woref = as_stored(rnd(kk, 2048, seed=84, scale=2048 ** -0.5), torch.bfloat16)
+    h = (rnd(m, kk, seed=90) * 3).to(DEV)
+    a, _ = as_stored(rnd(m, 2048, seed=91), torch.bfloat16)
+    wo, _ = as_stored(rnd(kk, 2048, seed=92, scale=2048 ** -0.5), torch.bfloat16)
+    w, wref = as_stored(rnd(n, kk, seed=93, scale=kk ** -0.5), torch.bfloat16)
     sums = torch.full((m, kk // 16), float("nan"), device=DEV)
+    rounded = torch.full((m + 1, kk), float("nan"), dtype=torch.bfloat16, device=DEV)
     plain = h.clone()
     k.gemm_skinny(a, wo, plain, add=True)
-    k.gemm_skinny(a, wo, h, add=True, sumsq_out=sums)
+    k.gemm_skinny(a, wo, h, add=True, sumsq_out=sums, copy_out=rounded[:m])
     assert torch.equal(h, plain)
+    assert torch.equal(rounded[:m], h.to(torch.bfloat16))
+    assert bool(torch.isnan(rounded[m]).all())        # nothing beyond the rows
     want_sums = (h.cpu().to(F64) ** 2).view(m, kk // 16, 16).sum(-1)
-    assert torch.allclose(sums.cpu().to(F64), want_sums, rtol=1e-5, atol=1e-6)
-    # 2. the product of the normalised residual
-    x = torch.empty(m, kk, dtype=torch.bfloat16, device=DEV)
-    k.add_rmsnorm(h, None, nw, eps, x)
-    cols = n // 2 if swiglu else n
-    want = torch.empty(m, cols, dtype=torch.bfloat16, device=DEV)
-    k.gemm_skinny(x, w, want, swiglu=swiglu)
-    got = torch.full_like(want, float("nan"))
-    k.gemm_skinny(None, w, got, swiglu=swiglu, norm=(h, sums, nw, eps))
-    # the same formula; the norm's 1 / sqrt comes from sums taken in another order, which may move a bfloat16 input
-    # by one unit in the last place
-    scale = float(want.float().abs().max())
-    assert float((got.float() - want.float()).abs().max()) <= 2e-2 * scale
-    assert float((got.float() - want.float()).abs().mean()) <= 2e-3 * scale
+    assert torch.allclose(sums.cpu().to(F64), want_sums, rtol=1e-5, atol=1e-6)      # 16 columns a part
+    # the mean comes from the float32 rows, the product from their rounded copy
+    inv = 1.0 / torch.sqrt((h.cpu().to(F64) ** 2).mean(-1, keepdim=True) + eps)
+    y = (rounded[:m].cpu().to(F64) @ wref.to(F64).t()) * inv
+    if swiglu:
+        g = y.view(m, -1, 2, 16)[:, :, 0].reshape(m, -1)
+        u = y.view(m, -1, 2, 16)[:, :, 1].reshape(m, -1)
+        want = g / (1 + torch.exp(-g)) * u
+        got = torch.full((m, n // 2), float("nan"), dtype=torch.bfloat16, device=DEV)
+        k.gemm_skinny(rounded[:m], w, got, swiglu=True, row_scale=(sums, eps))
+        err = (got.cpu().to(F64) - want).abs()
+        assert bool((err <= 2.0 ** -8 * want.abs() + 1e-5 * math.sqrt(kk)).all())   # one rounding to bfloat16
+    else:
+        got = torch.full((m, n), float("nan"), device=DEV)
+        k.gemm_skinny(rounded[:m], w, got, row_scale=(sums, eps))
+        assert torch.allclose(got.cpu().to(F64), y, atol=1e-5 * math.sqrt(kk), rtol=1e-5)
+        # no scale: the plain product, which the factor 1 / rms tells apart
+        bare = torch.empty_like(got)
+        k.gemm_skinny(rounded[:m], w, bare)
+        assert torch.allclose(bare.cpu().to(F64), y / inv, atol=1e-5 * math.sqrt(kk), rtol=1e-5)
     from pulse_infer_amd.ops import KernelError
     with pytest.raises(KernelError, match="fused"):
-        k.gemm_skinny(None, w[:, :512].contiguous(), got, swiglu=swiglu, norm=(h[:, :512].contiguous(), sums, nw[:512].contiguous(), eps))
+        k.gemm_skinny(rounded[:m, :512].contiguous(), w[:, :512].contiguous(), got, swiglu=swiglu, row_scale=(sums, eps))
+    # sums of squares in another split of the row (parts that are no multiple of four) give the same
+    odd = torch.zeros(m, 7, device=DEV)
+    odd[:, 2] = sums.sum(-1)
+    again = torch.full_like(got, float("nan"))
+    k.gemm_skinny(rounded[:m], w, again, swiglu=swiglu, row_scale=(odd, eps))
+    assert float((again.float() - got.float()).abs().max()) <= 2.0 ** -7 * float(got.float().abs().max())
 
 
 @pytest.mark.parametrize("m", [1, 8, 20, 32])
