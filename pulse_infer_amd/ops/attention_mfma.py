@@ -138,7 +138,8 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
 PREFILL_SPLIT_KEYS = 64        # a split of the prompt-portion kernel is a whole number of its 64-key blocks
 PREFILL_SPLIT_HEAD_DIMS = (32, 64, 128)
 PREFILL_MAX_SPLITS = 64
-PREFILL_SCRATCH_BYTES = 512 << 20
+PREFILL_SCRATCH_BYTES = 1 << 30
+TAIL_SPLIT_MIN_BLOCKS = 64     # walks from here on (4,096 keys) are worth a cut at three quarters on a full chip
 
 
 def choose_prefill_splits(entries: Sequence, portion: int, nkv: int, group: int, d: int, window: int,
@@ -149,30 +150,40 @@ def choose_prefill_splits(entries: Sequence, portion: int, nkv: int, group: int,
     waits.  Cutting the keys into splits with workgroups of their own pays when there are fewer workgroups than the
     chip runs at a time (``target_groups``, two a compute unit unless given; a short portion over a long context):
     they get as many splits as fill it.  Splits never hold fewer than ``min_blocks`` blocks, and nothing is cut
-    otherwise: the partial results cost a trip through memory and a second launch.  (A full chip whose latest items
-    walk much more than their share, the late portions of a whole prompt, was cut too while a block took a
-    workgroup 2.7 us; at 1.8 us the detour costs what it saves: 2,048 tokens 64.7 us whole, 67.4 cut at 1,664 keys,
-    88 at 1,024.)"""
+    otherwise, but for the tail of a long whole prompt (below): the partial results cost a trip through memory and a
+    second launch (2,048 tokens: 64.7 us whole, 67.4 cut at 1,664 keys, 88 at 1,024)."""
     if d not in PREFILL_SPLIT_HEAD_DIMS or window > 0:   # (a window keeps every walk short)
         return 0, 1
     if target_groups is None:
         target_groups = 2 * compute_units()
     longest = tokens = items = 0
+    walks = []
     for _, e in entries:
         tokens += e.count
         for b in range(0, e.count, portion):
             blocks = (e.start + min(b + portion, e.count) - 1) // PREFILL_SPLIT_KEYS + 1
             longest = max(longest, blocks)
+            walks.append(blocks)
             items += 1
     if items == 0:
         return 0, 1
     per_item = nkv * ((group + 15) // 16)
     groups = items * per_item
+    budget = PREFILL_SCRATCH_BYTES // max(1, tokens * nkv * group * d * 4)
     if groups >= target_groups:
+        # A full chip.  What is left to gain is the end of the kernel, when the few items with the longest walks run
+        # on while most units are idle: a whole prompt, whose walks grow from one block to all of them.  From 4,096
+        # keys on, cutting at three quarters of the longest walk gives that last quarter of the items a short
+        # second split (measured, one prompt: 4,096 tokens 228 -> 207 us, 8,192 677 -> 636, 16,384 2,439 -> 2,328;
+        # cuts at 5/8 to 7/8 are within 2% of each other; at 2,048 tokens nothing is gained).  Items that all walk
+        # about as far (portions deep inside a context) would all pay for the detour and are left whole.
+        cut = 3 * longest // 4
+        late = sum(1 for w in walks if w > cut)
+        if longest >= TAIL_SPLIT_MIN_BLOCKS and budget >= 2 and 10 * late <= 3 * items:
+            return cut * PREFILL_SPLIT_KEYS, 2
         return 0, 1
     size = max(min_blocks, (longest * groups + target_groups - 1) // target_groups)
     n_splits = (longest + size - 1) // size
-    budget = PREFILL_SCRATCH_BYTES // max(1, tokens * nkv * group * d * 4)
     n_splits = min(n_splits, PREFILL_MAX_SPLITS, max(1, budget))
     if n_splits <= 1:
         return 0, 1

@@ -254,7 +254,7 @@ def gemm_mid_takes(m: int, n: int, k: int, splits: int = 1) -> bool:
 
 def gemm_mid(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False, splits: int = 1,
              waves: int = 0) -> None:
-    """a @ w^T for up to 192 rows of bfloat16 with X shared through LDS (the regime of 13 to 192 rows).
+    """a @ w^T for up to 192 rows of bfloat16 with X shared through LDS (the regime of 17 to 192 rows).
 
     ``out`` bfloat16 [M, N]: the product (``splits`` must be 1); with ``swiglu`` the weight holds gate and up rows in
     alternating slabs of 16 and out [M, N / 2] is silu(gate) * up.  ``out`` float32 [splits, M, N]: the partial

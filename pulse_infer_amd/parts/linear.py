@@ -104,7 +104,7 @@ class Linear:
                  workspace: Optional[Workspace] = None):
         """residual += x W^T, in one of five ways.  Few rows: the kernel adds into the residual itself and None is
         returned, or, given a workspace and a shape the fused kernel takes, the ``RowStats`` of the updated rows (their
-        sums of squares and a rounded copy, with which the next product can do without a norm kernel before it).  13 to
+        sums of squares and a rounded copy, with which the next product can do without a norm kernel before it).  17 to
         192 rows, given a workspace: the product's inner dimension is shared out over workgroups and the shares' float32
         results [parts, rows, out] are returned as the update, which the next norm adds up in order; more rows of a
         product with a wide inner dimension and a narrow output: the same through the library's batched product.
@@ -147,12 +147,12 @@ class Linear:
 
     MID_ROWS = (17, 64)          # where the product with X shared through LDS and SwiGLU inside beats the library's
                                  # product followed by the SwiGLU kernel
-    SHARES_ROWS = (13, 192)      # where a product that adds into the residual has its inner dimension shared out over
-                                 # workgroups (measured on the 8B shape: a decoding step gains nothing at 9 to 12 rows over
-                                 # the few-rows kernel, 1% at 14, 2% at 16 (o and down: 18.8 us with 16 rows against 14.1
-                                 # with 8 in the few-rows kernel, 15.4 with 48 here), 1% at 17 to 32 rows, 4% at
+    SHARES_ROWS = (17, 192)      # where a product that adds into the residual has its inner dimension shared out over
+                                 # workgroups (measured on the 8B shape: 1% of a decoding step at 17 to 32 rows, 4% at
                                  # 48, 6% at 64; at 96 to 192 rows the library takes 22 to 33 us for o and 55 to 90 us
-                                 # for down, the shared-out product 16 to 22 and 33 to 47)
+                                 # for down, the shared-out product 16 to 22 and 33 to 47.  Up to 16 rows the few-rows
+                                 # kernel stands: it leaves what the next product needs to do without a norm kernel,
+                                 # and a step of 13 rows is 3% faster with it, one of 16 rows as fast)
 
     LIBRARY_SHARES_MIN_K = 8192  # inner dimensions from here on are worth sharing out in the library's product
     LIBRARY_TILE = 256           # its output tiles are about this large in both directions
@@ -226,7 +226,7 @@ class Linear:
         return self.shares_and_waves_for(x)[0]
 
     def shares_and_waves_for(self, x: torch.Tensor):
-        """(shares of the inner dimension, wavefronts a workgroup) of the product for 13 to 192 rows whose float32
+        """(shares of the inner dimension, wavefronts a workgroup) of the product for 17 to 192 rows whose float32
         partial results the next norm adds up; (0, 0): not this product.
 
         The pair with the least estimated time of the fullest compute unit is taken: workgroups on it (all of them

@@ -545,12 +545,17 @@ def test_attn_prefill_at_the_benchmark_shape(k, n):
     entries = [(0, E(0, n))]
     portion = M.portion_tokens(nq // nkv, d)
     items = torch.tensor(M.build_items(entries, portion), dtype=torch.int32, device=DEV)
-    assert M.choose_prefill_splits(entries, portion, nkv, nq // nkv, d, 0) == (0, 1)      # a full chip is not cut
+    # a full chip is not cut, but for the last quarter of the walks of a long prompt, which get a second split
+    split_size, n_splits = M.choose_prefill_splits(entries, portion, nkv, nq // nkv, d, 0)
+    assert (split_size, n_splits) == ((0, 1) if n < 4096 else (3 * n // 4, 2))
+    part_o = torch.full((n * nq * n_splits, d), float("nan"), device=DEV) if n_splits > 1 else None
+    part_ml = torch.full((n * nq * n_splits, 2), float("nan"), device=DEV) if n_splits > 1 else None
     pos = torch.arange(n, dtype=torch.int32, device=DEV)
     for _ in range(3):
-        M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos, table, items, d ** -0.5, 0)
+        M.attn_prefill(q, out, nq, nkv, d, kc, vc, pos, table, items, d ** -0.5, 0, split_size, n_splits, part_o, part_ml)
     got = out.cpu().to(F64).reshape(n, nq, d)
-    for t in (0, 1, 15, 16, 31, 32, 33, 63, 64, 65, 127, 128, 1000, 1023, 1024, 1055, 1056, 2015, 2016, 2046, 2047, n - 33, n - 32, n - 1):
+    for t in (0, 1, 15, 16, 31, 32, 33, 63, 64, 65, 127, 128, 1000, 1023, 1024, 1055, 1056, 2015, 2016, 2046, 2047,
+              3 * n // 4 - 33, 3 * n // 4 - 1, 3 * n // 4, 3 * n // 4 + 1, 3 * n // 4 + 63, 3 * n // 4 + 64, n - 33, n - 32, n - 1):
         want = P.causal_attention(qref[t:t + 1].reshape(1, nq, d), kref[:t + 1], vref[:t + 1], d ** -0.5, None, [t])
         assert torch.allclose(got[t], want[0], atol=2e-2, rtol=2e-2), (t, float((got[t] - want[0]).abs().max()))
 

@@ -221,6 +221,12 @@ def test_benchmark_layer_sizes(layer_shape, dtype):
     close(portions, whole, dtype, "layer sizes, portions against whole", SPLIT_TOL)
     if dtype == "bfloat16":
         assert runner.graph_replays >= 1           # the single tokens ran as recorded steps
+    # bfloat16: the norms' weights live in the products behind them (and the single tokens above ran without norm
+    # kernels between the layers' products); float32 keeps them where the checkpoint has them
+    for block in model.blocks:
+        for norm in (block.mixer_norm, block.ffn_norm):
+            assert norm.folded == (dtype == "bfloat16")
+            assert bool((norm.weight == 1).all()) == norm.folded
     del runner, model
     torch.cuda.empty_cache()
 
@@ -511,7 +517,7 @@ MANY = dict(
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("requests", [14, 24, 70, 200])
 def test_many_requests_decode_together(tmp_path, requests, dtype):
-    """Steps of 14, 24, 70 and 200 decoded tokens (the products for 13 to 192 rows and the library's beyond, attention
+    """Steps of 14, 24, 70 and 200 decoded tokens (the products for up to 16 and for 17 to 192 rows and the library's beyond, attention
     over many short contexts of different lengths): every request's logits are those of the plain implementation
     for its own sequence, whatever stands beside it."""
     from plain.qwen3_plain import PlainQwen3

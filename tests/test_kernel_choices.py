@@ -54,6 +54,12 @@ def test_prefill_splits_are_chosen_for_long_walks(units):
         assert size * n >= longest and size * (n - 1) < longest + M.PREFILL_SPLIT_KEYS
         assert n <= M.PREFILL_MAX_SPLITS and tokens * 8 * 4 * 128 * 4 * n <= M.PREFILL_SCRATCH_BYTES
     assert choose([E(16384 - 64, 64)])[1] > 1                 # few items over a long context are cut
+    # a full chip: only the tail of a long whole prompt is cut, at three quarters of its longest walk
+    if 2048 // 32 * 8 >= 2 * units:
+        assert choose([E(0, 2048)]) == (0, 1)
+        assert choose([E(0, 8192)]) == (6144, 2)
+        assert choose([E(0, 4096), E(0, 8192)]) == (6144, 2)
+        assert choose([E(8192 - 512, 512)] * 8) == (0, 1)     # every item walks as far: nothing to gain
 
 
 def test_library_products_share_out_a_wide_inner_dimension(units):
