@@ -82,6 +82,10 @@ struct MfmaArgs {
     int window;
     int split_size;  // multiple of 32
     int n_splits;
+    // The longest context of the step as it is now, or null.  The launch (and a recording of it) is made for contexts
+    // up to n_splits * split_size; with this the kernel of decoded tokens cuts the keys that are there into n_splits
+    // even splits instead (see live_split_size), so that no split stands empty while another walks its full length.
+    const int* live_context;
     // Only for the kernel that prepares q and the step's own key itself (decoded tokens): then q points at the raw
     // projection output [T, (nq + 2 nkv) D] (q heads, k heads, v heads), as the kernel of qk_rope_kv.hip takes it.
     const bf16_t* q_w;     // per-head RMSNorm weights [D], or null for no norm
@@ -93,6 +97,13 @@ struct MfmaArgs {
     int pairing;           // 0: (2i, 2i+1)   1: (i, i + rotary_dim / 2), rotary_dim a multiple of 64
     int new_key;           // 1: the token's key and value are prepared, used and written to their page here
 };
+
+// The split size for a step whose longest context is `live` (at most n_splits * split_size, what the launch was made
+// for): the keys cut evenly into the launch's number of splits, in whole 32-key blocks, never more than split_size.
+__device__ __forceinline__ int live_split_size(int live, int n_splits, int split_size) {
+    const int even = ((max(live, 1) + n_splits - 1) / n_splits + 31) / 32 * 32;
+    return min(split_size, even);
+}
 
 // A value that is the same in every lane of the wavefront, said so to the compiler: what depends on it becomes
 // scalar work and uniform branches.
@@ -208,10 +219,17 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     __shared__ float s_l[WAVES][16];
     __shared__ float s_o[WAVES][D][17];
 
-    const int item = blockIdx.x;
-    const int g = blockIdx.y / a.head_chunks;       // kv head
-    const int chunk = blockIdx.y % a.head_chunks;   // which 16 heads of the group
-    const int split = blockIdx.z;
+    // Workgroups that follow each other in the grid go to different XCDs, each with its own L2 and its own share of
+    // the way to memory (about an eighth of the chip's rate), and inside an XCD to different compute units, each of
+    // which reads at about 32 GB/s at most in this kernel.  So the kv heads of an item follow each other, then its
+    // splits, then the items: a request with a long context among short ones is then read through every XCD and by
+    // as many compute units as it has workgroups.
+    const int heads = a.nkv * a.head_chunks;
+    const int hy = blockIdx.x % heads;
+    const int split = (blockIdx.x / heads) % a.n_splits;
+    const int item = blockIdx.x / heads / a.n_splits;
+    const int g = hy / a.head_chunks;       // kv head
+    const int chunk = hy % a.head_chunks;   // which 16 heads of the group
     const int tid = threadIdx.x;
     const int wave = uniform(tid / PULSE_WAVE);   // the same in every lane: block numbers and pages become scalar work
     const int lane = tid % PULSE_WAVE;
@@ -225,7 +243,9 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     const int ntok = a.items[4 * item + 1];
     const int* bt = a.block_table + static_cast<int64_t>(a.items[4 * item + 2]) * a.bt_width;
     const int hi = a.positions[row0 + ntok - 1];    // last key any column of the item may see
-    const int split_begin = split * a.split_size;
+    const int split_size = (a.live_context && a.n_splits > 1)
+                               ? live_split_size(uniform(*a.live_context), a.n_splits, a.split_size) : a.split_size;
+    const int split_begin = split * split_size;
     int split_end = 0;                              // set once hi has arrived
 
     // this lane's column: a token of the item and a head of the group
@@ -487,14 +507,14 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
         BlockRegs xa, xb;
         const bool early = a.window == 0;
         int b = split_begin / BLOCK_KEYS + wave;
-        if (early && b <= (split_begin + a.split_size - 1) / BLOCK_KEYS) load_block(b, load_pages(b), xa);
+        if (early && b <= (split_begin + split_size - 1) / BLOCK_KEYS) load_block(b, load_pages(b), xa);
         load_q();   // behind the keys' pages in the queue: results come back in the order asked for
         if (split_begin > hi) return;                   // nothing here; the merge does not read this split
-        split_end = min(split_begin + a.split_size, hi + 1);
+        split_end = min(split_begin + split_size, hi + 1);
         const int first_block = max(split_begin, lo_item) / BLOCK_KEYS;
         const int last_block = (split_end - 1) / BLOCK_KEYS;
         // FUSED: the split that holds the token's position (the last one with keys) has its key to prepare
-        const bool own_key = FUSED && a.new_key && hi < split_begin + a.split_size;
+        const bool own_key = FUSED && a.new_key && hi < split_begin + split_size;
         const int own_block = own_key ? hi / BLOCK_KEYS : -1;
         auto after = [&](int blk) { return blk + WAVES <= last_block ? blk + WAVES : blk; };
         BlockPages pa = load_pages(after(b)), pb;       // (with a window b moves below; the pages are asked for again)
@@ -1273,7 +1293,9 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
                                                                          const int* __restrict__ positions,
                                                                          const int* __restrict__ items, int per,
                                                                          bf16_t* __restrict__ out, int64_t o_stride, int nq,
-                                                                         int n_splits, int split_size, int hpw_log2) {
+                                                                         int n_splits, int static_split_size, int hpw_log2,
+                                                                         const int* __restrict__ live_context) {
+    const int split_size = live_context ? live_split_size(*live_context, n_splits, static_split_size) : static_split_size;
     __shared__ float s_w[MAX_SPLITS];      // hpw * n_splits <= MAX_SPLITS (hpw > 1 only with few splits)
     __shared__ float s_l[MAX_SPLITS];
     __shared__ f32x4 s_acc[REDUCE_GROUPS][REDUCE_QUADS];
@@ -1365,7 +1387,7 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
                      const void* vcache, const int* positions, const int* block_table, int bt_width, const int* items,
                      int n_items, int tokens, int nq, int nkv, int page_size, int num_pages, float scale, int window,
                      int split_size, int n_splits, int max_context, float* part_o, float* part_ml,
-                     const Preparation* prep, hipStream_t stream) {
+                     const Preparation* prep, const int* live_context, hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && n_items >= 0 && nq > 0 && nkv > 0, "attn_mfma: bad sizes");
     PULSE_REQUIRE(nq % nkv == 0, "attn_mfma: %d query heads are not a multiple of %d kv heads", nq, nkv);
     PULSE_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_mfma: page size %d must be a multiple of 16", page_size);
@@ -1381,7 +1403,7 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
     PULSE_REQUIRE(n_splits == 1 || (part_o && part_ml && (reinterpret_cast<uintptr_t>(part_o) % 16) == 0),
                   "attn_mfma: scratch is missing or not 16-byte aligned");
     PULSE_REQUIRE(n_splits <= MAX_SPLITS, "attn_mfma: at most %d splits, got %d", MAX_SPLITS, n_splits);
-    PULSE_REQUIRE(n_splits < 65536 && static_cast<int64_t>(nkv) * ((nq / nkv + 15) / 16) < 65536, "attn_mfma: grid too large");
+    PULSE_REQUIRE(n_splits < 65536 && static_cast<int64_t>(n_items) * nkv * ((nq / nkv + 15) / 16) * n_splits < (int64_t{1} << 31), "attn_mfma: grid too large");
     PULSE_REQUIRE(q && out && kcache && vcache && positions && block_table && items, "attn_mfma: null pointer");
     if (tokens == 0 || n_items == 0) return 0;
     const int group = nq / nkv;
@@ -1398,15 +1420,16 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
     a.page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
     a.scale_log2e = scale * 1.4426950408889634f;
     a.window = window; a.split_size = split_size; a.n_splits = n_splits;
+    a.live_context = n_splits > 1 ? live_context : nullptr;
     a.q_w = a.k_w = nullptr; a.cos_t = a.sin_t = nullptr; a.eps = 0.f; a.rotary_dim = 0; a.pairing = 0; a.new_key = 0;
     if (prep) {
         a.q_w = static_cast<const bf16_t*>(prep->q_w); a.k_w = static_cast<const bf16_t*>(prep->k_w);
         a.cos_t = prep->cos_t; a.sin_t = prep->sin_t; a.eps = prep->eps; a.rotary_dim = prep->rotary_dim;
         a.pairing = prep->pairing; a.new_key = prep->new_key;
-        hipLaunchKernelGGL(attn_mfma_kernel<true>, dim3(n_items, nkv * a.head_chunks, n_splits), dim3(WAVES * PULSE_WAVE),
+        hipLaunchKernelGGL(attn_mfma_kernel<true>, dim3(n_items * nkv * a.head_chunks * n_splits), dim3(WAVES * PULSE_WAVE),
                            0, stream, a);
     } else {
-        hipLaunchKernelGGL(attn_mfma_kernel<false>, dim3(n_items, nkv * a.head_chunks, n_splits), dim3(WAVES * PULSE_WAVE),
+        hipLaunchKernelGGL(attn_mfma_kernel<false>, dim3(n_items * nkv * a.head_chunks * n_splits), dim3(WAVES * PULSE_WAVE),
                            0, stream, a);
     }
     PULSE_LAUNCH_CHECK("attn_mfma");
@@ -1415,7 +1438,8 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
         int hpw = 1, hpw_log2 = 0;            // heads a workgroup: as many as leave every split of a head a group of threads
         while (hpw * 2 * n_splits <= REDUCE_GROUPS && hpw * 2 <= nq) { hpw *= 2; ++hpw_log2; }
         hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(n_items * per, (nq + hpw - 1) / hpw), dim3(REDUCE_THREADS), 0, stream,
-                           part_o, part_ml, positions, items, per, a.out, o_stride, nq, n_splits, split_size, hpw_log2);
+                           part_o, part_ml, positions, items, per, a.out, o_stride, nq, n_splits, split_size, hpw_log2,
+                           a.live_context);
         PULSE_LAUNCH_CHECK("attn_mfma_reduce");
     }
     return 0;
@@ -1424,14 +1448,18 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
 }  // namespace
 
 // Scratch needed for `tokens` rows cut into `n_splits`: tokens * nq * n_splits * D floats of part_o, * 2 of part_ml.
+// live_context (device, or null): the longest context (last position + 1) among ALL items of this call as the step
+// has it; split_size and n_splits say what the launch is made for (max_context), and with live_context the kernel cuts
+// the keys that are there evenly into the same number of splits.  A value below an item's context loses keys.
 extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_stride, const void* kcache,
                                const void* vcache, const int* positions, const int* block_table, int bt_width,
                                const int* items, int n_items, int tokens, int nq,
                                int nkv, int page_size, int num_pages, float scale, int window, int split_size,
-                               int n_splits, int max_context, float* part_o, float* part_ml, hipStream_t stream) {
+                               int n_splits, int max_context, float* part_o, float* part_ml, const int* live_context,
+                               hipStream_t stream) {
     return launch_attn_mfma(q, q_stride, out, o_stride, kcache, vcache, positions, block_table, bt_width, items, n_items,
                             tokens, nq, nkv, page_size, num_pages, scale, window, split_size, n_splits, max_context,
-                            part_o, part_ml, nullptr, stream);
+                            part_o, part_ml, nullptr, live_context, stream);
 }
 
 // Whether pulse_attn_decode takes a rotation: whole 8-element slices, and for pairs (i, i + rotary_dim / 2) a
@@ -1454,7 +1482,7 @@ extern "C" int pulse_attn_decode(const void* qkv, int64_t qkv_stride, void* out,
                                  int num_pages, float scale, int window, int split_size, int n_splits, int max_context,
                                  float* part_o, float* part_ml, const void* q_w, const void* k_w, float eps,
                                  const float* cos_t, const float* sin_t, int rotary_dim, int pairing, int new_key,
-                                 hipStream_t stream) {
+                                 const int* live_context, hipStream_t stream) {
     PULSE_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode: cos and sin come together");
     if (!cos_t) rotary_dim = 0;
     PULSE_REQUIRE(pulse_attn_decode_takes(rotary_dim, pairing), "attn_decode: rotation of %d channels with pairing %d is not "
@@ -1468,7 +1496,7 @@ extern "C" int pulse_attn_decode(const void* qkv, int64_t qkv_stride, void* out,
     Preparation prep{q_w, k_w, cos_t, sin_t, eps, rotary_dim, pairing, new_key ? 1 : 0};
     return launch_attn_mfma(qkv, qkv_stride, out, o_stride, kcache, vcache, positions, block_table, bt_width, items,
                             n_items, tokens, nq, nkv, page_size, num_pages, scale, window, split_size, n_splits,
-                            max_context, part_o, part_ml, &prep, stream);
+                            max_context, part_o, part_ml, &prep, live_context, stream);
 }
 
 // Keys a split of the prompt-portion kernel must be a multiple of; 0 when this head size's kernel has no splits.
@@ -1517,6 +1545,7 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
     a.page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
     a.scale_log2e = scale * 1.4426950408889634f;
     a.window = window; a.split_size = n_splits > 1 ? split_size : 0; a.n_splits = n_splits;
+    a.live_context = nullptr;
     a.part_o = n_splits > 1 ? part_o : nullptr; a.part_ml = n_splits > 1 ? part_ml : nullptr;
 #if PULSE_WIDE
     hipLaunchKernelGGL((attn_prefill_wide_kernel<WIDE_CT, 4, WIDE_NW>), dim3(n_items, nkv * a.head_chunks, n_splits),

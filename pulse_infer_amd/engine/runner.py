@@ -162,8 +162,8 @@ class ModelRunner:
 
     def _layout(self, total: int, batch: int, wanted: int, widths: Sequence[int]) -> np.ndarray:
         """Offsets of the step's integer arrays in one flat buffer:
-        [ids | positions | token_entry | start | count | first_row | slot | want | tables...]"""
-        sizes = [total, total, total, batch, batch, batch + 1, batch, wanted] + [batch * w for w in widths]
+        [ids | positions | token_entry | start | count | first_row | slot | want | tables... | longest context]"""
+        sizes = [total, total, total, batch, batch, batch + 1, batch, wanted] + [batch * w for w in widths] + [1]
         return np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
 
     def _fill(self, flat: np.ndarray, offsets: np.ndarray, entries: Sequence[StepEntry], metas: List[EntryMeta],
@@ -187,6 +187,7 @@ class ModelRunner:
                 pages = cache.table(gi, m.request)[:w]
                 table[i, :len(pages)] = pages
             flat[offsets[8 + gi]:offsets[9 + gi]] = table.reshape(-1)
+        flat[offsets[8 + len(widths)]] = max(m.start + m.count for m in metas)
 
     def _context(self, dev: torch.Tensor, offsets: np.ndarray, metas: List[EntryMeta], wanted: int,
                  widths: Sequence[int], workspace, max_context: int) -> StepContext:
@@ -197,7 +198,7 @@ class ModelRunner:
             entry_start=part[3], entry_count=part[4], entry_first_row=part[5], entry_slot=part[6],
             block_tables={gi: part[8 + gi].view(batch, w) for gi, w in enumerate(widths)},
             want_rows=part[7], num_wanted=wanted, workspace=workspace,
-            max_count=max(m.count for m in metas), max_context=max_context,
+            max_count=max(m.count for m in metas), max_context=max_context, live_context=part[8 + len(widths)],
             upload=lambda values: self._staging.upload(np.asarray(values, dtype=np.int32)))
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:

@@ -108,8 +108,13 @@ def choose_splits(num_items: int, nkv: int, group: int, max_context: int) -> Tup
 def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
               vcache: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
               items: torch.Tensor, scale: float, window: int, split_size: int, n_splits: int, max_context: int,
-              part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor]) -> None:
-    _gpu("attn_mfma", q, out, kcache, vcache, positions, block_table, items, part_o, part_ml)
+              part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor],
+              live_context: Optional[torch.Tensor] = None) -> None:
+    """Attention of decoded tokens and short portions.  ``split_size`` x ``n_splits`` is what the launch is made for
+    (contexts up to ``max_context``); ``live_context`` (one int32 on the device: the longest context among the step's
+    entries as it is now) lets the kernel cut the keys that are there evenly into the same number of splits."""
+    _gpu("attn_mfma", q, out, kcache, vcache, positions, block_table, items, part_o, part_ml, live_context)
+    _live(live_context)
     tokens = q.shape[0]
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.stride(1) == 1 and out.stride(1) == 1,
           "attn_mfma: q and out must be bfloat16 matrices with contiguous rows")
@@ -132,7 +137,14 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
     call_in(lib, "pulse_attn_mfma", _ptr(q), _i64(q.stride(0)), _ptr(out), _i64(out.stride(0)), _ptr(kcache),
             _ptr(vcache), _ptr(positions), _ptr(block_table), _i32(block_table.shape[1]),
             _ptr(items), _i32(n_items), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages), _f32(scale),
-            _i32(window), _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml), _stream())
+            _i32(window), _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml),
+            _ptr(live_context), _stream())
+
+
+def _live(live_context: Optional[torch.Tensor]) -> None:
+    _need(live_context is None or (live_context.dtype == torch.int32 and live_context.numel() >= 1
+                                   and live_context.is_contiguous()),
+          "the live context must be an int32 value on the device")
 
 
 PREFILL_SPLIT_KEYS = 64        # a split of the prompt-portion kernel is a whole number of its 64-key blocks
@@ -239,11 +251,13 @@ def attn_decode(qkv: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int,
                 scale: float, window: int, split_size: int, n_splits: int, max_context: int,
                 part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor], q_w: Optional[torch.Tensor],
                 k_w: Optional[torch.Tensor], eps: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
-                rotary_dim: int, pairing: int, new_key: bool) -> None:
+                rotary_dim: int, pairing: int, new_key: bool, live_context: Optional[torch.Tensor] = None) -> None:
     """Attention for decoded tokens from the raw projection output ``qkv`` [tokens, (nq + 2 nkv) d]: per-head norm
     and rotation of q and of the token's own key happen inside the kernel; with ``new_key`` key and value are also
-    written to the token's page.  Every item must hold one token."""
-    _gpu("attn_decode", qkv, out, kcache, vcache, positions, block_table, items, part_o, part_ml, q_w, k_w, cos, sin)
+    written to the token's page.  Every item must hold one token.  ``live_context``: as for ``attn_mfma``."""
+    _gpu("attn_decode", qkv, out, kcache, vcache, positions, block_table, items, part_o, part_ml, q_w, k_w, cos, sin,
+         live_context)
+    _live(live_context)
     tokens = qkv.shape[0]
     _need(qkv.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and qkv.stride(1) == 1 and out.stride(1) == 1,
           "attn_decode: qkv and out must be bfloat16 matrices with contiguous rows")
@@ -277,4 +291,4 @@ def attn_decode(qkv: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int,
             _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages), _f32(scale), _i32(window),
             _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml), _ptr(q_w), _ptr(k_w),
             _f32(eps), _ptr(cos), _ptr(sin), _i32(rotary_dim if cos is not None else 0), _i32(pairing),
-            _i32(1 if new_key else 0), _stream())
+            _i32(1 if new_key else 0), _ptr(live_context), _stream())

@@ -193,8 +193,8 @@ class PagedAttention(Part):
                     self.scale, window, split_size, n_splits, max_context, part_o, part_ml, self.q_w, self.k_w,
                     self.eps, tables.cos if tables is not None else None, tables.sin if tables is not None else None,
                     tables.rotary_dim if tables is not None else 0, tables.pairing if tables is not None else 0,
-                    new_key=write)
+                    new_key=write, live_context=ctx.live_context)
                 return
             attention_mfma.attn_mfma(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
                                      table, short_items, self.scale, window, split_size, n_splits,
-                                     max_context, part_o, part_ml)
+                                     max_context, part_o, part_ml, live_context=ctx.live_context)

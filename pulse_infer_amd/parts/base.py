@@ -151,7 +151,10 @@ class StepContext:
     num_wanted: int
     workspace: Workspace
     max_count: int = 1           # most tokens of one entry
-    max_context: int = 1         # longest context (start + count) of an entry
+    max_context: int = 1         # longest context (start + count) of an entry that the step's launches must cover
+                                 # (of a recorded step: the most its replays may bring)
+    live_context: Optional[torch.Tensor] = None   # int32 [1] on the device: the longest context as it is in this
+                                                  # step (at most max_context), for kernels that shape their work by it
     extras: Dict[str, Any] = field(default_factory=dict)  # per-step products of position encodings etc.
     upload: Optional[Callable[[List[int]], torch.Tensor]] = None   # integers of a part's own to the device, through the
                                                                    # step function's pinned staging (no synchronous copy)

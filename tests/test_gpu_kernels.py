@@ -417,9 +417,11 @@ def test_kernels_refuse_what_they_cannot_do(k):
 
 
 # ------------------------------------------------------- matrix-core attention
-def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0, portion_split=0):
+def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0, portion_split=0, made_for=None):
     """Requests with contexts `lens`; request 0 brings its last `portion` tokens, the others one token each.
-    ``portion_split``: request 0's portion goes through the prompt-portion kernel with its keys in splits of that size."""
+    ``portion_split``: request 0's portion goes through the prompt-portion kernel with its keys in splits of that size.
+    ``made_for = (context, splits)``: the launch is made for contexts up to that (as a recorded step's is for its
+    bucket) and is told the longest context there is through ``live_context``."""
     from pulse_infer_amd.ops import attention_mfma as M
     dtype = torch.bfloat16
     pages_per = [(n + bs - 1) // bs for n in lens]
@@ -452,6 +454,11 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0, portion_
     q, qref = as_stored(rnd(len(positions), (nq + 2 * nkv) * d, seed=300 + seed), dtype)
     out = torch.zeros(len(positions), nq * d, dtype=dtype, device=DEV)
     max_ctx = max(lens)
+    live = None
+    if made_for is not None:
+        max_ctx, n = made_for
+        split = ((max_ctx + n - 1) // n + 31) // 32 * 32
+        live = torch.tensor([max(lens)], dtype=torch.int32, device=DEV)
     if split is None or split == "portion" or portion_split:
         split_size, n_splits = M.choose_splits(items.numel() // M.ITEM_INTS, nkv, group, max_ctx)
     else:
@@ -478,7 +485,7 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0, portion_
                         n_splits, max_ctx, part_o, part_ml)
     else:
         M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), items, scale, window, split_size,
-                    n_splits, max_ctx, part_o, part_ml)
+                    n_splits, max_ctx, part_o, part_ml, live_context=live)
     got = out.cpu().to(F64).reshape(-1, nq, d)
     for t, (p, e) in enumerate(zip(positions, entry)):
         kref, vref = refs[e]
@@ -502,6 +509,18 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0, portion_
 @pytest.mark.parametrize("split", [None, 32, 128, "portion"])
 def test_attn_mfma(k, case, split):
     _mfma_case(k, split=split, **case)
+
+
+@pytest.mark.parametrize("case", [
+    dict(nq=32, nkv=8, d=128, bs=16, window=0, lens=[300, 513, 512, 31], portion=3),
+    dict(nq=6, nkv=3, d=48, bs=32, window=24, lens=[170, 90, 24, 25], portion=1),
+    dict(nq=8, nkv=2, d=64, bs=16, window=0, lens=[5, 1, 2], portion=1),                 # far fewer keys than splits of a block
+])
+@pytest.mark.parametrize("made_for", [(1024, 4), (4096, 7), (520, 2), (2048, 64)])
+def test_attn_mfma_made_for_longer_contexts_than_the_step_has(k, case, made_for):
+    """A launch shaped for a context bucket (its number of splits, its scratch) that is told the longest context of the
+    step: the kernel and the merge cut the keys that are there into even splits, and both must agree on where."""
+    _mfma_case(k, split=None, made_for=made_for, **case)
 
 
 @pytest.mark.parametrize("case", [
@@ -648,12 +667,14 @@ def test_attn_mfma_refuses_other_sizes(k):
     dict(nq=16, nkv=1, d=224, rot=224, pairing="interleaved", norm=True, bs=16, window=100, lens=[260, 130]),
     dict(nq=40, nkv=2, d=64, rot=32, pairing="interleaved", norm=True, bs=64, window=0, lens=[200, 77, 64]),  # 20 heads a kv head: two chunks
 ])
-@pytest.mark.parametrize("split", [None, 32, 128])
+@pytest.mark.parametrize("split", [None, 32, 128, "bucket"])
 @pytest.mark.parametrize("new_key", [True, False])
 def test_attn_decode_from_raw(k, case, split, new_key):
     """Decoded tokens straight from the raw projection output: per-head norm, rotation, the token's own key and
     value (used from registers, written to the page) inside the attention kernel, against the plain formulas and
-    against what the separate preparation kernel writes.  With new_key False the pages already hold the token."""
+    against what the separate preparation kernel writes.  With new_key False the pages already hold the token.
+    "bucket": the launch is made for contexts of up to 2,048 in five splits, as a recorded step's is, and told the
+    longest context there is: the split that holds a token's position, whose workgroup writes its key, moves with it."""
     from pulse_infer_amd.ops import attention_mfma as M
     nq, nkv, d, rot, bs, window, lens = (case[x] for x in ("nq", "nkv", "d", "rot", "bs", "window", "lens"))
     pairing = 0 if case["pairing"] == "interleaved" else 1
@@ -704,8 +725,13 @@ def test_attn_decode_from_raw(k, case, split, new_key):
     items = torch.tensor(M.build_items(list(enumerate(E(i, 1) for i in range(n))), M.tokens_per_item(group)),
                          dtype=torch.int32, device=DEV)
     max_ctx = max(lens)
+    live = None
     if split is None:
         split_size, n_splits = M.choose_splits(n, nkv, group, max_ctx)
+    elif split == "bucket":
+        live = torch.tensor([max_ctx], dtype=torch.int32, device=DEV)
+        max_ctx, n_splits = 2048, 5
+        split_size = 416
     else:
         split_size, n_splits = split, (max_ctx + split - 1) // split
     part_o = torch.full((n * nq * n_splits, d), float("nan"), device=DEV)
@@ -714,7 +740,7 @@ def test_attn_decode_from_raw(k, case, split, new_key):
     pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
     raw = qkv.clone()
     M.attn_decode(qkv, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), items, scale, window, split_size, n_splits,
-                  max_ctx, part_o, part_ml, qw, kw, eps, cos, sin, rot, pairing, new_key)
+                  max_ctx, part_o, part_ml, qw, kw, eps, cos, sin, rot, pairing, new_key, live_context=live)
     assert torch.equal(qkv, raw)                   # the projection output stays raw
     got = out.cpu().to(F64).reshape(n, nq, d)
     for t, p in enumerate(positions):
