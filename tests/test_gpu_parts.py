@@ -115,6 +115,52 @@ def test_feed_forward_part(gpu, mode):
 
 
 @pytest.mark.parametrize("mode", ["float32", "bfloat16"])
+@pytest.mark.parametrize("rows", [1, 7, 16, 20])
+def test_a_norm_hands_its_weight_to_the_product_behind_it(gpu, mode, rows):
+    """The protocol that takes the norm kernels out of a decoding step, on a feed-forward with a width the fused
+    product takes: the feed-forward folds the norm's weight into its first product (bfloat16 only), the norm then
+    only divides, and given the rows' sums of squares and their rounded copy (what the product before leaves) the
+    feed-forward takes rows that were never normalised.  The norm's weights are far from 1 and differ by column,
+    so that a weight applied twice, not at all or to the wrong operand shows."""
+    from pulse_infer_amd.ops import kernels
+    from pulse_infer_amd.parts.base import FEED_FORWARDS, NORMS, ResidualStream, RowStats
+    hidden, inter, eps = 1024, 96, 1e-5
+    nw = (torch.linspace(0.25, 4.0, hidden) * torch.tensor([1.0, -1.0]).repeat(hidden // 2)).to(torch.bfloat16)
+    ws = {"m.gate_proj.weight": rnd(inter, hidden, seed=3, scale=hidden ** -0.5),
+          "m.up_proj.weight": rnd(inter, hidden, seed=4, scale=hidden ** -0.5),
+          "m.down_proj.weight": rnd(hidden, inter, seed=5, scale=inter ** -0.5), "n.weight": nw}
+    build = build_ctx(ws, mode)
+    mlp = FEED_FORWARDS.get("gated_mlp")({"hidden_size": hidden, "intermediate_size": inter, "activation": "silu"}, "m", build)
+    norm = NORMS.get("rmsnorm")({"size": hidden, "eps": eps}, "n", build)
+    took = mlp.fold_input_weight(norm.foldable_weight())
+    assert took == (mode == "bfloat16")
+    if took:
+        norm.weight_folded()
+        assert norm.foldable_weight() is None              # it can be given away once
+    h = (torch.randn(rows, hidden, generator=torch.Generator().manual_seed(6)) * 3).to(DEV)
+    want = P.gated_mlp(P.rms_norm(h.cpu().to(F64), nw.to(F64), eps),
+                       *(ws[f"m.{n}_proj.weight"].to(F64) for n in ("gate", "up", "down")))
+    ctx = step_ctx(build, list(range(rows)), [0] * rows, [[0]])
+    # 1. through the norm's own kernel (what prompt portions do): the weight is applied exactly once either way
+    x = torch.empty(rows, hidden, dtype=build.act_dtype, device=DEV)
+    norm.apply(h, None, x)
+    out = mlp.forward(x, ctx)
+    scale = float(want.abs().max())
+    assert float((out.cpu().to(F64) - want).abs().max()) <= (3e-5 if mode == "float32" else 3e-2) * scale
+    # 2. as a decoding step does it: the rows as the product before left them, normalised behind the first product
+    stream = ResidualStream(h)
+    sums = (h.double() ** 2).view(rows, hidden // 16, 16).sum(-1).float().contiguous()
+    stream.push(RowStats(sums, h.to(torch.bfloat16)))
+    lazy = stream.lazy(norm)
+    if mode == "float32" or rows > kernels.SKINNY_FAST_ROWS:
+        assert lazy is None or not mlp.gate_up.takes_lazy(lazy)     # the norm's kernel it is
+        return
+    assert lazy is not None and mlp.gate_up.takes_lazy(lazy)
+    out = mlp.forward(lazy, ctx)
+    assert float((out.cpu().to(F64) - want).abs().max()) <= 3e-2 * scale
+
+
+@pytest.mark.parametrize("mode", ["float32", "bfloat16"])
 @pytest.mark.parametrize("variant", ["qwen", "half_partial_window", "no_position_no_norm"])
 def test_attention_part(gpu, mode, variant):
     """The mixer alone over a cache it fills in two steps (a portion, then another portion and a single token
