@@ -9,7 +9,9 @@ What the reference leaves out is decided here:
 * **token budget** — a step computes at most ``max_num_batched_tokens`` tokens:
   decoding requests come first with one token each, what is left goes to
   prefilling requests in order of arrival, each at most ``chunk_size`` tokens,
-  cut anywhere.
+  cut anywhere; if budget is left when every one of them has its portion, the
+  portions are extended in the same order (a lone long prompt runs in steps
+  of the whole budget).
 * **pages** — every portion is reserved in the cache before the step; a request
   is admitted only if its first portion fits.  When a running request cannot
   get the page it needs, the most recently admitted running request is
@@ -239,6 +241,23 @@ class ContinuousBatchScheduler:
                                                    count == request.num_pending_tokens))
             budget -= count
 
+        # 4. what is left of the budget (fewer requests in their prompts than it has room for) extends this step's
+        #    prompt portions, in their order: a lone long prompt then runs in steps of the whole budget, whose
+        #    matrix products are far more efficient than those of a chunk's rows
+        for i, portion in enumerate(batch.portions):
+            if budget <= 0:
+                break
+            request, have = portion.request, len(portion.tokens)
+            more = min(request.num_pending_tokens - have, budget)
+            if more <= 0:
+                continue
+            count = self._largest_fitting(request, have + more)
+            if count <= have:
+                continue
+            self._reserve(request, request.num_computed_tokens + count)
+            batch.portions[i] = ScheduledPortion(request, request.get_next_chunk_tokens(count),
+                                                 request.num_computed_tokens, count == request.num_pending_tokens)
+            budget -= count - have
 
     def update_after_step(self, finished_ids: Sequence[int]) -> None:
         """Take finished requests out of the running list and give their cache back

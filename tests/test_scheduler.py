@@ -135,12 +135,52 @@ def test_preemption_of_the_newest_when_a_decode_needs_a_page():
     c.check()
     _finish_step(s, b2, finished=[a])
     b3 = s.schedule_next_batch()
-    # b runs again from its first token: prompt and the token it had generated, then sampling goes on
-    assert [(p.request.request_id, p.tokens, p.samples) for p in b3.portions] == [(b, list(range(8)), False)]
+    # b runs again from its first token: prompt and the token it had generated (a portion of the chunk's 8 tokens,
+    # extended by the ninth since the step's budget has room), then sampling goes on
+    assert [(p.request.request_id, p.tokens, p.samples) for p in b3.portions] == [(b, list(range(8)) + [7], True)]
     _finish_step(s, b3)
+    s.get_request(b).add_sampled_token(9, [])
     b4 = s.schedule_next_batch()
-    assert [(p.tokens, p.start, p.samples) for p in b4.portions] == [([7], 8, True)]
+    assert [(p.tokens, p.start, p.samples) for p in b4.portions] == [([9], 9, True)]
     c.check()
+
+
+def test_budget_that_is_left_extends_the_portions_in_order():
+    """Every prefilling request gets its portion of at most a chunk first; what the budget still holds then goes to
+    the same portions in their order, as far as tokens, pages and budget reach."""
+    c = _cache(pages=64)
+    s = ContinuousBatchScheduler(4, 4, chunk_size=8, max_num_batched_tokens=40, cache=c, max_positions=256)
+    a = s.add_request(list(range(100)), 2)
+    b1 = s.schedule_next_batch()
+    assert [(p.request.request_id, len(p.tokens), p.start, p.samples) for p in b1.portions] == [(a, 40, 0, False)]
+    _finish_step(s, b1)
+    b = s.add_request(list(range(30)), 2)
+    d = s.add_request(list(range(5)), 2)
+    b2 = s.schedule_next_batch()
+    # a chunk each for a and b, all of d; the 19 left go to a
+    assert [(p.request.request_id, len(p.tokens), p.start, p.samples) for p in b2.portions] == \
+        [(a, 8 + 19, 40, False), (b, 8, 0, False), (d, 5, 0, True)]
+    assert b2.num_tokens() == 40 and b2.portions[0].tokens == list(range(40, 67))
+    _finish_step(s, b2)
+    s.get_request(d).add_sampled_token(1, [])
+    b3 = s.schedule_next_batch()
+    # d decodes first; a and b a chunk each; 23 left: a takes 23 of the 25 tokens it still has
+    assert [(p.request.request_id, len(p.tokens), p.start) for p in b3.portions] == [(d, 1, 5), (a, 31, 67), (b, 8, 8)]
+    _finish_step(s, b3)
+    s.get_request(d).add_sampled_token(1, [])
+    s.update_after_step([d])
+    b4 = s.schedule_next_batch()
+    # a ends its prompt with 2 tokens (sampled); what is left extends b to the end of its prompt (14 tokens)
+    assert [(p.request.request_id, len(p.tokens), p.samples) for p in b4.portions] == [(a, 2, True), (b, 14, True)]
+    c.check()
+    # pages decide too: an extension is cut where the pool ends, and nobody is preempted for it
+    c2 = _cache(pages=5)          # 20 tokens
+    s2 = ContinuousBatchScheduler(4, 4, chunk_size=4, max_num_batched_tokens=64, cache=c2, max_positions=256)
+    x = s2.add_request(list(range(19)), 1)
+    y = s2.add_request(list(range(3)), 1)
+    b5 = s2.schedule_next_batch()
+    assert [(p.request.request_id, len(p.tokens)) for p in b5.portions] == [(x, 16), (y, 3)] and not b5.preempted
+    c2.check()
 
 
 def test_what_can_never_fit_is_refused():
