@@ -13,6 +13,7 @@ returns logits for every token.)
 """
 from __future__ import annotations
 
+import gc
 from dataclasses import dataclass, field
 from typing import Any, Hashable, List, Optional, Sequence
 
@@ -59,6 +60,10 @@ class _Staging:
             self.events[i] = torch.cuda.Event()
         self.events[i].record()
         return dev
+
+    def upload_values(self, values) -> torch.Tensor:
+        """``upload`` of a list of integers (what a part's work list is)."""
+        return self.upload(np.asarray(values, dtype=np.int32))
 
 
 @dataclass
@@ -199,7 +204,9 @@ class ModelRunner:
             block_tables={gi: part[8 + gi].view(batch, w) for gi, w in enumerate(widths)},
             want_rows=part[7], num_wanted=wanted, workspace=workspace,
             max_count=max(m.count for m in metas), max_context=max_context, live_context=part[8 + len(widths)],
-            upload=lambda values: self._staging.upload(np.asarray(values, dtype=np.int32)))
+            upload=self._staging.upload_values)   # (the staging's method, not a closure over the step function: a
+                                                   # recording keeps its context, and would keep the step function
+                                                   # that holds it alive in a circle that only the collector ends)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         self._check(entries)
@@ -307,8 +314,19 @@ class ModelRunner:
             return None, logits   # the step went through the vendor library somewhere: it is not recorded
         ctx.extras = {k: v for k, v in ctx.extras.items() if k.startswith("static:")}
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            rec.logits = self.model.forward(ctx, self.views)
+        # No graph may be destroyed while a stream records (the runtime refuses it, and an error in a destructor ends
+        # the process).  Python's collector runs whenever it likes, also in the middle of the recording, and what it
+        # finds may hold graphs (another step function that was dropped, a caller's own): so it runs now and rests
+        # while the stream records.
+        collecting = gc.isenabled()
+        gc.collect()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                rec.logits = self.model.forward(ctx, self.views)
+        finally:
+            if collecting:
+                gc.enable()
         rec.graph = graph
         rec.workspace = workspace
         rec.context = ctx

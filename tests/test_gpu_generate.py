@@ -201,6 +201,46 @@ def test_captured_decode_steps_replay_like_eager_ones(gpu, model_folders, plain_
             close(row_g[None], row_e[None], "bfloat16", f"captured against eager {k}@{pos_g}", SPLIT_TOL)
 
 
+def test_the_collector_rests_while_a_step_is_recorded(gpu, model_folders):
+    """No graph may be destroyed while a stream records, and Python's collector, which may find dropped recordings (of
+    a step function that is no longer used, of the caller), runs whenever it likes: the step function lets it run
+    before it records and keeps it off meanwhile.  A dropped step function itself goes at once: nothing points back at it
+    in a circle."""
+    import gc
+    import weakref
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+
+    cfg, page = TINY["B"]
+    _, model = load_model(model_folders["B"], mode="bfloat16")
+    ids = token_ids(cfg["vocab_size"], 40, seed=5)
+    seen = []
+    forward = model.forward
+
+    def watched(ctx, views):
+        seen.append((torch.cuda.is_current_stream_capturing(), gc.isenabled()))
+        return forward(ctx, views)
+
+    model.forward = watched
+    try:
+        runner = ModelRunner(model, page_size=16, num_pages=8, max_requests=2)
+        runner.GRAPH_AFTER_STEPS = 1
+        runner.add_request("a")
+        runner.reserve("a", 40)
+        runner.step([StepEntry("a", ids[:30], [29])])
+        for t in range(30, 34):
+            runner.step([StepEntry("a", ids[t:t + 1], [0])])
+    finally:
+        model.forward = forward
+    assert runner.graph_records == 1 and runner.graph_replays == 3
+    assert (True, False) in seen                      # it was recorded, with the collector off
+    assert all(on for capturing, on in seen if not capturing) and not any(on for capturing, on in seen if capturing)
+    assert gc.isenabled()
+    gone = weakref.ref(runner)
+    del runner
+    assert gone() is None                             # no circle: the recordings went with it, not at the collector's whim
+
+
 def test_recorded_steps_while_a_window_gives_pages_back_and_after_eviction(gpu, model_folders, plain_logits):
     """Tiny W (windows of 24 keys on some layers, pages of 16): two requests decode far past window + page while
     their steps are replayed, so the windowed group gives pages back under a live recording and its table rows hold
