@@ -150,3 +150,82 @@ def test_random_configurations_mixed_batches_with_page_reuse(tmp_path, seed):
             close(torch.cat(parts), want[k], dtype, f"mixed request {k}: {cfg} {options} page {page}")
         del runner, model
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_traces_with_recorded_steps_over_small_context_buckets(tmp_path, seed):
+    """Random traces, random configurations (widths whose decoding steps run without norm kernels among them): up to
+    six live requests, prompt portions of random sizes beside decoded tokens, requests left out of steps, and long
+    runs of steps of decoded tokens only, which are recorded at once and replayed, over context buckets so small that
+    the requests walk through many of them (another recording, another number of splits each time, every replay told
+    its own longest context); few pages, so that they are used again.  Every wanted row against the plain
+    implementation, in bfloat16 (recorded) and in 32-bit (eager)."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.weights import write_model_folder
+
+    rng = random.Random(4000 + seed)
+    cfg, options = random_config(rng, [256, 1024, 1024, 2048], max_positions=2048)
+    cfg["num_hidden_layers"] = min(cfg["num_hidden_layers"], 2)
+    if options:
+        options = {"layer_windows": options["layer_windows"][:cfg["num_hidden_layers"]]}
+        if not any(options["layer_windows"]):
+            options = None
+    windows = (options or {}).get("layer_windows")
+    page = rng.choice([16, 32])
+    folder = write_model_folder(Qwen3Config.from_dict(cfg), str(tmp_path / "m"), seed=80 + seed)
+    plain = PlainQwen3.from_folder(folder, windows=windows)
+    lengths = [rng.choice([3, 20, 70, 150, 300]) + rng.randint(0, 30) for _ in range(rng.randint(2, 6))]
+    ids = {r: token_ids(cfg["vocab_size"], n, seed=seed * 10 + r) for r, n in enumerate(lengths)}
+    want = {r: plain.logits(ids[r]) for r in ids}
+    for dtype in ("bfloat16", "float32"):
+        trace = random.Random(5000 + seed)            # the same trace for both
+        _, model = load_model(folder, mode=dtype, config_overrides=options)
+        runner = ModelRunner(model, page_size=page, num_pages=sum((n + page - 1) // page for n in lengths) + 1,
+                             max_requests=len(lengths))
+        runner.GRAPH_AFTER_STEPS = 1
+        runner.GRAPH_CONTEXT_BUCKET = trace.choice([64, 256])
+        fed = {r: 0 for r in ids}
+        live, got = set(), {r: [] for r in ids}
+        prompt_end = {r: trace.randint(1, lengths[r]) for r in ids}      # up to here in portions, then token by token
+        while any(fed[r] < lengths[r] for r in ids):
+            todo = [r for r in ids if fed[r] < lengths[r]]
+            decode_only = trace.random() < 0.6
+            entries, rows = [], []
+            for r in todo:
+                if trace.random() < 0.2 and len(todo) > 1:
+                    continue                                              # left out of this step
+                if fed[r] >= prompt_end[r] or (decode_only and fed[r] > 0):
+                    n = 1
+                elif decode_only:
+                    continue
+                else:
+                    n = min(trace.choice([2, 5, 16, 17, 40, 64, 130]), prompt_end[r] - fed[r])
+                if r not in live:
+                    runner.add_request(r)
+                    live.add(r)
+                runner.reserve(r, fed[r] + n)
+                wanted = [n - 1] if n == 1 or trace.random() < 0.7 else [0, n - 1]
+                entries.append(StepEntry(r, ids[r][fed[r]:fed[r] + n], wanted))
+                rows += [(r, fed[r] + w) for w in wanted]
+                fed[r] += n
+            if not entries:
+                continue
+            for (r, pos), row in zip(rows, runner.step(entries)):
+                got[r].append((pos, row))
+            for r in list(live):
+                if fed[r] >= lengths[r]:
+                    runner.free_request(r)
+                    live.discard(r)
+            runner.cache.check()
+        if dtype == "bfloat16":
+            assert runner.graph_records >= 2 and runner.graph_replays >= 10
+        for r, pairs in got.items():
+            mine = torch.stack([row for _, row in pairs])
+            ref = torch.stack([want[r][pos] for pos, _ in pairs])
+            close(mine, ref, dtype, f"request {r} of {lengths}: {cfg} {options} page {page}")
+        del runner, model
+    torch.cuda.empty_cache()
