@@ -35,8 +35,11 @@ class Linear:
 
     def fold_input_weight(self, scale: torch.Tensor) -> bool:
         """W <- W diag(scale), rounded once: a factor of every input column (the weight of the norm before) becomes
-        part of this product.  Only bfloat16 products on the matrix cores do that; False otherwise."""
-        if not self.library or scale.numel() != self.in_features:
+        part of this product.  Only bfloat16 products of a width for which the product exists that scales its rows
+        (``takes_lazy``) do that: the folded weight is rounded once more than the weight and the normalised input
+        each are, which is paid for only where it saves the norm's kernel.  False otherwise."""
+        if (not self.library or scale.numel() != self.in_features
+                or not kernels.gemm_skinny_fusable(1, self.out_features, self.in_features)):
             return False
         folded = torch.empty_like(self.weight)
         factor = scale.to(torch.float32).view(1, -1)

@@ -134,6 +134,13 @@ def test_a_norm_hands_its_weight_to_the_product_behind_it(gpu, mode, rows):
     norm = NORMS.get("rmsnorm")({"size": hidden, "eps": eps}, "n", build)
     took = mlp.fold_input_weight(norm.foldable_weight())
     assert took == (mode == "bfloat16")
+    # a width for which no product scales its rows keeps the norm's weight in the norm: folding rounds once more
+    # and would buy nothing there
+    narrow = {"m.gate_proj.weight": rnd(96, 72, seed=3), "m.up_proj.weight": rnd(96, 72, seed=4),
+              "m.down_proj.weight": rnd(72, 96, seed=5)}
+    small = FEED_FORWARDS.get("gated_mlp")({"hidden_size": 72, "intermediate_size": 96, "activation": "silu"}, "m",
+                                           build_ctx(narrow, mode))
+    assert not small.fold_input_weight(torch.ones(72, dtype=torch.bfloat16, device=DEV))
     if took:
         norm.weight_folded()
         assert norm.foldable_weight() is None              # it can be given away once
