@@ -64,13 +64,14 @@ __device__ __forceinline__ int row_shift_left(int v, int n) {
 // Sum of the wavefronts' partial tiles, in wavefront order, and the store.  With `sumsq` (adding into a float32
 // matrix only) every slab also leaves the sum of squares of its 16 new values of each row, sumsq[row * parts + slab
 // number]: what a following RMSNorm needs of the row, so that the product after it can normalise by itself; `copy`
-// takes the new values once more, rounded to bfloat16 (that product's input).  `row_scale` (one factor for each of
-// at most 16 rows) multiplies the sums before anything else is done with them.
+// takes the new values once more, each multiplied by its column's `copy_scale` (that norm's weight; null: 1) and
+// rounded to bfloat16 (that product's input).  `row_scale` (one factor for each of at most 16 rows) multiplies the
+// sums before anything else is done with them.
 template <int SLABS, int MT, int KW, bool SWIGLU>
 __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void* __restrict__ C, int64_t ldc, int M, int N,
                                          int n_base, int mode, int tid, float* __restrict__ sumsq = nullptr, int parts = 0,
                                          const float* row_scale = nullptr, bf16_t* __restrict__ copy = nullptr,
-                                         int64_t ldcopy = 0) {
+                                         int64_t ldcopy = 0, const bf16_t* __restrict__ copy_scale = nullptr) {
     constexpr int TILES = SLABS * MT;
     constexpr int THREADS = KW * PULSE_WAVE;
     if (!SWIGLU) {
@@ -92,7 +93,9 @@ __device__ __forceinline__ void epilogue(float (*red)[SLABS * MT][16][17], void*
                 else {
                     updated = static_cast<float*>(C)[at] + v;
                     static_cast<float*>(C)[at] = updated;
-                    if (copy) copy[static_cast<int64_t>(m) * ldcopy + n] = f32_to_bf16(updated);
+                    if (copy)
+                        copy[static_cast<int64_t>(m) * ldcopy + n] =
+                            f32_to_bf16(copy_scale ? updated * bf16_to_f32(copy_scale[n]) : updated);
                 }
             }
             if (sumsq) {  // the 16 lanes of a row of lanes hold the 16 columns of one row of the tile
@@ -267,11 +270,11 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_kernel(const bf16_
 //
 // Both only change which lane fetches what; every product and the order of the sums are those of the kernel above.
 //
-// SCALED: X is a matrix whose rows have not been normalised yet (a bfloat16 copy of the residual); the row sums of
-// squares that the product before left come with it (`sumsq`, `parts` of them a row), and every row of the result is
-// multiplied by 1 / sqrt(mean(x^2) + eps) in the epilogue, where it costs nothing: x W^T scaled by rows is (x scaled
-// by rows) W^T.  A weight of the norm has to be part of W already (W' = W diag(w)).  That saves the norm kernel's
-// launch.  (Forming the normalised x in this kernel's loop from the float32 residual was measured too: every k-step
+// SCALED: X is a matrix whose rows have not been normalised yet (a bfloat16 copy of the residual, already multiplied
+// by the norm's weight, column by column); the sums of squares of the residual's rows that the product before left
+// come with it (`sumsq`, `parts` of them a row), and every row of the result is multiplied by 1 / sqrt(mean + eps)
+// in the epilogue, where it costs nothing: x W^T scaled by rows is (x scaled by rows) W^T.  That saves the norm
+// kernel's launch.  (Forming the normalised x in this kernel's loop from the float32 residual was measured too: every k-step
 // then reads float32 values and a weight of the norm, and from 8 rows on that costs what the launch saves.)
 constexpr int STAGGER_BLOCKS = 64;  // consecutive workgroups that start at the same group of k-steps
 
@@ -287,7 +290,8 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
                                                                              void* __restrict__ C, int64_t ldc, int M,
                                                                              int N, int K, int mode, RowScale scale,
                                                                              float* __restrict__ sumsq_out, int parts_out,
-                                                                             bf16_t* __restrict__ copy_out, int64_t ldcopy) {
+                                                                             bf16_t* __restrict__ copy_out, int64_t ldcopy,
+                                                                             const bf16_t* __restrict__ copy_scale) {
     constexpr int THREADS = KW * PULSE_WAVE;
     static_assert(PACK == 1 || PACK == 2 || PACK == 4 || PACK == 8, "PACK k-steps a load of X");
     static_assert(UNROLL % 2 == 0 && UNROLL % PACK == 0, "groups hold whole pairs and whole packs");
@@ -434,7 +438,7 @@ __global__ __launch_bounds__(KW* PULSE_WAVE) void gemm_skinny_stream_kernel(cons
         for (int i = 0; i < 4; ++i) red[wave][s][4 * kg + i][r] = acc[s][i];
     __syncthreads();
     epilogue<SLABS, 1, KW, SWIGLU>(red, C, ldc, M, N, n_base, mode, tid, sumsq_out, parts_out,
-                                   SCALED ? s_rstd : nullptr, copy_out, ldcopy);
+                                   SCALED ? s_rstd : nullptr, copy_out, ldcopy, copy_scale);
 }
 
 template <int SLABS, int MT, int KW, bool SWIGLU>
@@ -456,12 +460,12 @@ void launch(bool xlds, const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ld
 template <int SLABS, int KW, bool SWIGLU>
 void launch_stream(int pack, const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
                    int K, int mode, const RowScale& scale, float* sumsq_out, int parts_out, bf16_t* copy_out, int64_t ldcopy,
-                   hipStream_t stream) {
+                   const bf16_t* copy_scale, hipStream_t stream) {
     const dim3 grid((N + SLABS * 16 - 1) / (SLABS * 16)), block(KW * PULSE_WAVE);
     const size_t red_bytes = sizeof(float) * KW * SLABS * 16 * 17;
 #define PULSE_STREAM(P, SCALED)                                                                                          \
     hipLaunchKernelGGL((gemm_skinny_stream_kernel<SLABS, KW, P, SWIGLU, SCALED>), grid, block, red_bytes, stream, X, ldx, \
-                       W, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy_out, ldcopy)
+                       W, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy_out, ldcopy, copy_scale)
 #define PULSE_STREAM_PACKS(SCALED)                    \
     do {                                              \
         if (pack == 8) PULSE_STREAM(8, SCALED);       \
@@ -485,18 +489,20 @@ int pack_for(int M) { return M <= 2 ? 8 : (M <= 4 ? 4 : (M <= 8 ? 2 : 1)); }
 // entry point choose the kernel.
 // The same with the fusions of the streaming kernel (M <= 16, K a multiple of 1024), each optional:
 //   scale_sumsq != null: row m of the product is multiplied by 1 / sqrt(sum(scale_sumsq[m, :]) / K + eps) before it is
-//     stored (or goes through SwiGLU): the RMSNorm of X's rows, applied behind the product, from the rows' sums of
-//     squares [M, scale_parts] (any split of a row into parts); a weight of that norm has to be folded into W beforehand;
+//     stored (or goes through SwiGLU): the division of an RMSNorm, applied behind the product, from the sums of
+//     squares [M, scale_parts] of the rows that were normed (any split of a row into parts); the norm's weight has to
+//     be part of X already (see copy_scale);
 //   sumsq_out != null (mode 2 only): besides adding into C, leave sumsq_out[row * parts + slab] = sum of squares of the
 //     new values of C[row, 16 slab .. 16 slab + 15], parts = ceil(N / 16);
-//   copy_out != null (mode 2 only): the new values of C once more as bfloat16, row stride ldcopy.
+//   copy_out != null (mode 2 only): the new values of C once more as bfloat16, row stride ldcopy, each multiplied by
+//     copy_scale[column] first (bfloat16 [N], the weight of the norm that reads C next; null: as they are).
 // pulse_gemm_skinny_fusable says whether the streaming kernel takes a shape.
 extern "C" int pulse_gemm_skinny_fusable(int M, int N, int K) { return M >= 1 && M <= 16 && N > 0 && K > 0 && K % 1024 == 0; }
 
 extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
                                        int N, int K, int mode, int swiglu, int tune, const float* scale_sumsq,
                                        int scale_parts, float scale_eps, float* sumsq_out, void* copy_out,
-                                       int64_t ldcopy, hipStream_t stream) {
+                                       int64_t ldcopy, const void* copy_scale, hipStream_t stream) {
     const bool fused = scale_sumsq != nullptr || sumsq_out != nullptr || copy_out != nullptr;
     if (fused) {
         PULSE_REQUIRE(pulse_gemm_skinny_fusable(M, N, K) && tune != 9, "gemm_skinny: M=%d N=%d K=%d cannot take the fused kernel", M, N, K);
@@ -523,6 +529,7 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
     RowScale scale{scale_sumsq, scale_parts, scale_eps};
     const int parts_out = (N + 15) / 16;
     bf16_t* copy = static_cast<bf16_t*>(copy_out);
+    const bf16_t* cscale = copy ? static_cast<const bf16_t*>(copy_scale) : nullptr;
     const bf16_t* w = static_cast<const bf16_t*>(W);
     const int mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
     const int units = pulse_compute_units();
@@ -549,14 +556,14 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
         const int kw = t_kw ? t_kw : ((K % 2048 == 0 && !pairs) ? 8 : 4);
         const int pack = t_pack ? t_pack : pack_for(M);
         if (swiglu) {
-            if (kw == 8) launch_stream<2, 8, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
-            else launch_stream<2, 4, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
+            if (kw == 8) launch_stream<2, 8, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
+            else launch_stream<2, 4, true>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
         } else if (slabs == 2) {
-            if (kw == 8) launch_stream<2, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
-            else launch_stream<2, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
+            if (kw == 8) launch_stream<2, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
+            else launch_stream<2, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
         } else {
-            if (kw == 8) launch_stream<1, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
-            else launch_stream<1, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, stream);
+            if (kw == 8) launch_stream<1, 8, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
+            else launch_stream<1, 4, false>(pack, x, ldx, w, ldw, C, ldc, M, N, K, mode, scale, sumsq_out, parts_out, copy, ldcopy, cscale, stream);
         }
         PULSE_LAUNCH_CHECK("gemm_skinny");
         return 0;
@@ -583,5 +590,5 @@ extern "C" int pulse_gemm_skinny_fused(const void* X, int64_t ldx, const void* W
 extern "C" int pulse_gemm_skinny(const void* X, int64_t ldx, const void* W, int64_t ldw, void* C, int64_t ldc, int M,
                                  int N, int K, int mode, int swiglu, int tune, hipStream_t stream) {
     return pulse_gemm_skinny_fused(X, ldx, W, ldw, C, ldc, M, N, K, mode, swiglu, tune, nullptr, 0, 0.f, nullptr, nullptr, 0,
-                                   stream);
+                                   nullptr, stream);
 }

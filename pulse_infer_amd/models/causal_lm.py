@@ -76,7 +76,12 @@ class CausalLM:
         h = ws.buffer("model.residual", ctx.num_tokens, self.hidden_size, torch.float32)
         self.embedding.forward(ctx.token_ids, h)
         stream = ResidualStream(h)
-        for index, run in enumerate(self.spec.order):
+        order = self.spec.order
+        for index, run in enumerate(order):
+            # who reads the residual once this block is through: the block behind it (the final norm after the last
+            # one gathers the wanted rows and stays a kernel of its own)
+            follower = self.blocks[order[index + 1].layer] if index + 1 < len(order) else None
+            stream.after_block = follower.entry_norm() if hasattr(follower, "entry_norm") else None
             self.blocks[run.layer].forward(stream, ctx, cache_views[index])
         logits = torch.empty((ctx.num_wanted, self.vocab_size), dtype=torch.float32, device=self.device)
         if ctx.num_wanted == 0:

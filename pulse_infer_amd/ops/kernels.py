@@ -189,7 +189,7 @@ def gemm_skinny_fusable(m: int, n: int, k: int) -> bool:
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool = False, swiglu: bool = False,
                 tune: int = 0, sumsq_out: Optional[torch.Tensor] = None, row_scale: Optional[tuple] = None,
-                copy_out: Optional[torch.Tensor] = None) -> None:
+                copy_out: Optional[torch.Tensor] = None, copy_scale: Optional[torch.Tensor] = None) -> None:
     """out = a @ w^T for at most 64 rows of bfloat16, float32 accumulation on the matrix cores.
 
     ``out`` bfloat16 or float32 is stored; with ``add`` (float32 only) the product is added to it.  With
@@ -197,14 +197,15 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool =
     ``tune`` picks a kernel variant by hand (tests and measurements); 0 lets the library choose.
 
     Fusions for shapes that ``gemm_skinny_fusable`` accepts.  ``row_scale = (sumsq, eps)``: row m of the product is
-    multiplied by 1 / sqrt(sum(sumsq[m]) / K + eps) before it is stored or goes through SwiGLU, which is the product
-    of the RMS-normalised rows of ``a`` when ``sumsq`` [M, parts] holds the sums of squares of those rows in parts (a
-    weight of that norm has to be part of ``w``).  ``sumsq_out`` [M, ceil(N / 16)] with ``add``: the kernel also
-    leaves the sums of squares of the rows of the updated ``out``, 16 columns a part; ``copy_out`` [M, N] bfloat16
-    with ``add``: the updated ``out`` once more, rounded.
+    multiplied by 1 / sqrt(sum(sumsq[m]) / K + eps) before it is stored or goes through SwiGLU: the division of an
+    RMSNorm moved behind the product, ``sumsq`` [M, parts] being the sums of squares, in parts, of the rows that were
+    normed (the norm's weight has to be in ``a`` already).  ``sumsq_out`` [M, ceil(N / 16)] with ``add``: the kernel
+    also leaves the sums of squares of the rows of the updated ``out``, 16 columns a part; ``copy_out`` [M, N] bfloat16
+    with ``add``: the updated ``out`` once more, every column multiplied by its ``copy_scale`` (bfloat16 [N], the weight
+    of the norm that reads ``out`` next; None: as it is) and rounded: what ``row_scale`` of the next product takes.
     """
     scale_sumsq, scale_eps = row_scale if row_scale is not None else (None, 0.0)
-    _gpu("gemm_skinny", a, w, out, sumsq_out, copy_out, scale_sumsq)
+    _gpu("gemm_skinny", a, w, out, sumsq_out, copy_out, scale_sumsq, copy_scale)
     _need(gemm_skinny_ok(a, w), "gemm_skinny: needs bfloat16 operands with at most 64 rows, K a multiple of 8, "
           "contiguous 16-byte aligned rows")
     m, k = a.shape
@@ -232,6 +233,9 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool =
         _need(add and copy_out.dtype == torch.bfloat16 and tuple(copy_out.shape) == (m, n) and copy_out.stride(1) == 1,
               f"gemm_skinny: copy_out must be bfloat16 [{m}, {n}] and comes with add")
     ldcopy = 0 if copy_out is None else (copy_out.stride(0) if m > 1 else n)
+    _need(copy_scale is None or (copy_out is not None and copy_scale.dtype == torch.bfloat16 and copy_scale.numel() == n
+                                 and copy_scale.is_contiguous()),
+          f"gemm_skinny: copy_scale must hold {n} bfloat16 values and comes with copy_out")
     scale_parts = 0
     if scale_sumsq is not None:
         _need(scale_sumsq.dtype == torch.float32 and scale_sumsq.dim() == 2 and scale_sumsq.shape[0] >= m
@@ -241,7 +245,7 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool =
     call("pulse_gemm_skinny_fused", _ptr(a), _i64(ldx), _ptr(w), _i64(w.stride(0) if n > 1 else k), _ptr(out),
          _i64(out.stride(0) if m > 1 else cols), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(1 if swiglu else 0),
          _i32(tune), _ptr(scale_sumsq), _i32(scale_parts), _f32(scale_eps), _ptr(sumsq_out), _ptr(copy_out),
-         _i64(ldcopy), _stream(), label=f"N={n} K={k}")
+         _i64(ldcopy), _ptr(copy_scale), _stream(), label=f"N={n} K={k}")
 
 
 MID_MAX_ROWS = 192

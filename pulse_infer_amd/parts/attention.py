@@ -90,11 +90,8 @@ class PagedAttention(Part):
     accepts_lazy_input = True   # the first product may take rows that are not normalised yet and scale its result
     records_cleanly = True      # positions, tables and work lists are read on the device
 
-    def fold_input_weight(self, scale: torch.Tensor) -> bool:
-        """Column factors of the input (the weight of the norm before) go into the q, k and v weights."""
-        return self.qkv.fold_input_weight(scale)
-
-    def forward(self, x, ctx: StepContext, cache: PagedCacheView, residual: Optional[torch.Tensor] = None):
+    def forward(self, x, ctx: StepContext, cache: PagedCacheView, residual: Optional[torch.Tensor] = None,
+                next_scale: Optional[torch.Tensor] = None):
         tokens = x.shape[0]
         ws = ctx.workspace
         write = cache.writable
@@ -119,7 +116,7 @@ class PagedAttention(Part):
             self.attend(qkv, attn, ctx, cache, table)
         out = ws.buffer("attention.proj", tokens, self.hidden, self.act_dtype)
         if residual is not None:
-            return self.o.add_into(attn, residual, out, ws)
+            return self.o.add_into(attn, residual, out, ws, next_scale)
         return self.o.forward(attn, out)
 
     def uses_matrix_cores(self, q: torch.Tensor, cache: PagedCacheView) -> bool:

@@ -176,20 +176,23 @@ class StepContext:
 @dataclass
 class RowStats:
     """What a part that added into the residual itself knows about the new rows: their sums of squares, in parts
-    (``sumsq`` [rows, parts] float32), and the rows themselves once more, rounded to the activations' type
-    (``rounded`` [rows, H]).  A norm that only divides a row by a figure of its own can then be left to its consumer."""
+    (``sumsq`` [rows, parts] float32), and the rows themselves once more, every column multiplied by ``scaled_by``
+    (the weight of the norm that was expected to read them next; None: as they are) and rounded to the activations'
+    type (``rounded`` [rows, H]).  What is left of that norm, a division of each row, can then move behind its
+    consumer's first product."""
 
     sumsq: torch.Tensor
     rounded: Optional[torch.Tensor] = None
+    scaled_by: Optional[torch.Tensor] = None
 
 
 @dataclass
 class LazyNorm:
-    """A normalised input that has not been computed: the rows of ``x`` (the residual ``h``, rounded) each divided by
-    sqrt(mean of its squares + eps), the mean taken from the sums of squares in ``sumsq`` [rows, parts].  A consumer
-    whose first product is linear (``accepts_lazy_input``) multiplies the rows of that product's result instead, which
-    is the same and costs nothing.  The norm has no weight of its own then: the consumer's first product holds it
-    (``fold_input_weight``).  ``materialize`` computes the input the ordinary way."""
+    """A normalised input that has not been computed: the rows of ``x`` (the residual ``h`` times the norm's weight,
+    rounded) each still to be divided by sqrt(mean of the squares of its row of ``h`` + eps), the mean taken from the
+    sums of squares in ``sumsq`` [rows, parts].  A consumer whose first product is linear (``accepts_lazy_input``)
+    multiplies the rows of that product's result instead, which is the same and costs nothing.  ``materialize``
+    computes the input the ordinary way."""
 
     x: torch.Tensor
     sumsq: torch.Tensor
@@ -216,6 +219,8 @@ class ResidualStream:
         self.h = h
         self.pending: Optional[torch.Tensor] = None
         self.stats: Optional[RowStats] = None
+        self.after_block: Any = None   # the norm that reads the residual first once the block in hand is through
+                                       # (set by whoever runs the blocks; None: unknown, or no norm)
 
     def pending_for(self, norm: Any) -> Optional[torch.Tensor]:
         """The update not yet added, in a form ``norm`` takes: an update in parts ([parts, T, H] float32, the shares of

@@ -44,13 +44,6 @@ class PreNormBlock(Part):
         self.ffn = FEED_FORWARDS.get(layer.ffn.kind)(layer.ffn.params,
                                                      joined(layer.prefix, layer.ffn.params.get("prefix", "")), build)
         self.act_dtype = build.act_dtype
-        # A norm that scales columns and a part whose first product is linear: the product's weight takes the norm's
-        # over (W diag(w)), and what is left of the norm, a division of each row, can move behind that product.
-        for norm, part in ((self.mixer_norm, self.mixer), (self.ffn_norm, self.ffn)):
-            if hasattr(norm, "foldable_weight") and hasattr(part, "fold_input_weight"):
-                weight = norm.foldable_weight()
-                if weight is not None and part.fold_input_weight(weight):
-                    norm.weight_folded()
 
     def cache_spec(self) -> Optional[Any]:
         return self.mixer.cache_spec()
@@ -69,15 +62,24 @@ class PreNormBlock(Part):
         x = ctx.workspace.buffer("block.normed", ctx.num_tokens, stream.h.shape[1], self.act_dtype)
         return stream.normed(norm, x)
 
+    def entry_norm(self) -> Any:
+        """The norm that reads the residual first in this block."""
+        return self.mixer_norm
+
+    @staticmethod
+    def _scale_of(norm: Any) -> Any:
+        return norm.column_scale() if norm is not None and hasattr(norm, "column_scale") else None
+
     def forward(self, stream: ResidualStream, ctx: StepContext, cache: Any) -> None:
         x = self._input(stream, self.mixer_norm, self.mixer, ctx)
-        # a part that says so may add its result into the residual itself and return None (or the new rows' statistics)
+        # a part that says so may add its result into the residual itself and return None (or the new rows' statistics,
+        # for which it is told the column factors of the norm that reads the residual next)
         if getattr(self.mixer, "accepts_residual", False):
-            stream.push(self.mixer.forward(x, ctx, cache, residual=stream.h))
+            stream.push(self.mixer.forward(x, ctx, cache, residual=stream.h, next_scale=self._scale_of(self.ffn_norm)))
         else:
             stream.push(self.mixer.forward(x, ctx, cache))
         x = self._input(stream, self.ffn_norm, self.ffn, ctx)
         if getattr(self.ffn, "accepts_residual", False):
-            stream.push(self.ffn.forward(x, ctx, residual=stream.h))
+            stream.push(self.ffn.forward(x, ctx, residual=stream.h, next_scale=self._scale_of(stream.after_block)))
         else:
             stream.push(self.ffn.forward(x, ctx))

@@ -33,22 +33,6 @@ class Linear:
         self.mode = mode
         self.library = mode == "bfloat16" and weight.dtype == torch.bfloat16
 
-    def fold_input_weight(self, scale: torch.Tensor) -> bool:
-        """W <- W diag(scale), rounded once: a factor of every input column (the weight of the norm before) becomes
-        part of this product.  Only bfloat16 products of a width for which the product exists that scales its rows
-        (``takes_lazy``) do that: the folded weight is rounded once more than the weight and the normalised input
-        each are, which is paid for only where it saves the norm's kernel.  False otherwise."""
-        if (not self.library or scale.numel() != self.in_features
-                or not kernels.gemm_skinny_fusable(1, self.out_features, self.in_features)):
-            return False
-        folded = torch.empty_like(self.weight)
-        factor = scale.to(torch.float32).view(1, -1)
-        step = max(1, (1 << 26) // self.in_features)   # a quarter of a gigabyte of float32 at a time
-        for r0 in range(0, self.out_features, step):
-            folded[r0:r0 + step] = (self.weight[r0:r0 + step].to(torch.float32) * factor).to(self.weight.dtype)
-        self.weight = folded
-        return True
-
     def takes_lazy(self, x: LazyNorm, rows: Optional[int] = None) -> bool:
         """Whether the product can take rows that have not been normalised yet and scale its result instead."""
         n = self.out_features if rows is None else rows
@@ -104,10 +88,11 @@ class Linear:
         return out
 
     def add_into(self, x: torch.Tensor, residual: torch.Tensor, scratch: torch.Tensor,
-                 workspace: Optional[Workspace] = None):
+                 workspace: Optional[Workspace] = None, next_scale: Optional[torch.Tensor] = None):
         """residual += x W^T, in one of five ways.  Few rows: the kernel adds into the residual itself and None is
         returned, or, given a workspace and a shape the fused kernel takes, the ``RowStats`` of the updated rows (their
-        sums of squares and a rounded copy, with which the next product can do without a norm kernel before it).  17 to
+        sums of squares and a rounded copy, multiplied column by column by ``next_scale``, the weight of the norm that
+        reads the residual next: with these the next product can do without a norm kernel before it).  17 to
         192 rows, given a workspace: the product's inner dimension is shared out over workgroups and the shares' float32
         results [parts, rows, out] are returned as the update, which the next norm adds up in order; more rows of a
         product with a wide inner dimension and a narrow output: the same through the library's batched product.
@@ -142,8 +127,11 @@ class Linear:
                                         torch.float32)
                 rounded = workspace.buffer(f"linear.rounded.{self.out_features}", x.shape[0], self.out_features,
                                            torch.bfloat16)
-                kernels.gemm_skinny(x, self.weight, residual, add=True, sumsq_out=sums, copy_out=rounded)
-                return RowStats(sums, rounded)
+                scaled = next_scale is not None and next_scale.dtype == torch.bfloat16 \
+                    and next_scale.numel() == self.out_features and next_scale.is_contiguous()
+                kernels.gemm_skinny(x, self.weight, residual, add=True, sumsq_out=sums, copy_out=rounded,
+                                    copy_scale=next_scale if scaled else None)
+                return RowStats(sums, rounded, next_scale if scaled else None)
             kernels.gemm_skinny(x, self.weight, residual, add=True)
             return None
         return self.forward(x, scratch)

@@ -53,11 +53,8 @@ class GatedMLP(Part):
     accepts_lazy_input = True   # the first product may take rows that are not normalised yet and scale its result
     records_cleanly = True
 
-    def fold_input_weight(self, scale: torch.Tensor) -> bool:
-        """Column factors of the input (the weight of the norm before) go into the gate+up weight."""
-        return self.gate_up.fold_input_weight(scale)
-
-    def forward(self, x, ctx: StepContext, residual: Optional[torch.Tensor] = None):
+    def forward(self, x, ctx: StepContext, residual: Optional[torch.Tensor] = None,
+                next_scale: Optional[torch.Tensor] = None):
         tokens = x.shape[0]
         ws = ctx.workspace
         z = ws.buffer("mlp.act", tokens, self.inter, self.act_dtype)
@@ -76,5 +73,5 @@ class GatedMLP(Part):
             kernels.swiglu(gu, z, slab=self.slab)
         out = ws.buffer("mlp.out", tokens, self.hidden, self.act_dtype)
         if residual is not None:
-            return self.down.add_into(z, residual, out, ws)
+            return self.down.add_into(z, residual, out, ws, next_scale)
         return self.down.forward(z, out)

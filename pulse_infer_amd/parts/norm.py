@@ -21,7 +21,6 @@ class RMSNorm(Part):
         self.size = int(params["size"])
         self.eps = float(params["eps"])
         self.weight = build.loader.get(f"{prefix}.weight")
-        self.folded = False   # True: the weight has gone into the consumer's first product, this norm only divides
 
     records_cleanly = True
     takes_parts = True   # delta may be [parts, T, H] float32: the kernel adds the parts in order
@@ -32,18 +31,14 @@ class RMSNorm(Part):
         kernels.add_rmsnorm(h, delta, self.weight, self.eps, out, rows=rows)
         return out
 
-    def foldable_weight(self) -> Optional[torch.Tensor]:
-        """The factor of every column, for a consumer that can multiply it into its first product's weight."""
-        return None if self.folded else self.weight
-
-    def weight_folded(self) -> None:
-        """The consumer has taken the weight over: from now on this norm is x / sqrt(mean(x^2) + eps) alone."""
-        self.weight = torch.ones_like(self.weight)
-        self.folded = True
+    def column_scale(self) -> Optional[torch.Tensor]:
+        """The factor of every column: whoever writes the rows that this norm reads next may multiply it in as it
+        writes a rounded copy of them (``RowStats``), and leave the rest of the norm to the consumer."""
+        return self.weight
 
     def lazy(self, h: torch.Tensor, stats: RowStats) -> Optional[LazyNorm]:
-        """This norm as an input that its consumer computes: possible once the weight is the consumer's, since
-        dividing a row by a number commutes with a linear product."""
-        if not self.folded or stats.rounded is None:
+        """This norm as an input that its consumer finishes: the rows already carry this norm's weight, and dividing
+        a row by a number commutes with a linear product."""
+        if stats.rounded is None or stats.scaled_by is not self.weight:
             return None
         return LazyNorm(stats.rounded, stats.sumsq, self.eps, h, self)

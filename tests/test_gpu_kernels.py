@@ -853,6 +853,12 @@ def test_gemm_skinny_rounded_copy_and_rows_scaled_behind_the_product(k, m, n, kk
     assert torch.equal(h, plain)
     assert torch.equal(rounded[:m], h.to(torch.bfloat16))
     assert bool(torch.isnan(rounded[m]).all())        # nothing beyond the rows
+    # with column factors (the weight of the norm that reads h next): multiplied in before the one rounding
+    cs, _ = as_stored(1 + 0.5 * rnd(kk, seed=94), torch.bfloat16)
+    again, weighted = h.clone(), torch.empty(m, kk, dtype=torch.bfloat16, device=DEV)
+    k.gemm_skinny(a, wo, again, add=True, copy_out=weighted, copy_scale=cs)
+    assert torch.equal(weighted, (again * cs.float()).to(torch.bfloat16))
+    again = None
     want_sums = (h.cpu().to(F64) ** 2).view(m, kk // 16, 16).sum(-1)
     assert torch.allclose(sums.cpu().to(F64), want_sums, rtol=1e-5, atol=1e-6)      # 16 columns a part
     # the mean comes from the float32 rows, the product from their rounded copy

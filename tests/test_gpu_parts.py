@@ -114,57 +114,62 @@ def test_feed_forward_part(gpu, mode):
         FEED_FORWARDS.get("gated_mlp")({"hidden_size": hidden, "intermediate_size": inter, "activation": "relu"}, "m", build)
 
 
-@pytest.mark.parametrize("mode", ["float32", "bfloat16"])
 @pytest.mark.parametrize("rows", [1, 7, 16, 20])
-def test_a_norm_hands_its_weight_to_the_product_behind_it(gpu, mode, rows):
-    """The protocol that takes the norm kernels out of a decoding step, on a feed-forward with a width the fused
-    product takes: the feed-forward folds the norm's weight into its first product (bfloat16 only), the norm then
-    only divides, and given the rows' sums of squares and their rounded copy (what the product before leaves) the
-    feed-forward takes rows that were never normalised.  The norm's weights are far from 1 and differ by column,
-    so that a weight applied twice, not at all or to the wrong operand shows."""
+def test_a_norm_is_finished_behind_the_product_that_consumes_it(gpu, rows):
+    """The protocol that takes the norm kernels out of a decoding step, on real parts of a width the fused products
+    take: the product that adds into the residual is told the weight of the norm that reads the residual next and
+    leaves, beside the new rows, their sums of squares and a rounded copy with that weight multiplied in; the norm
+    recognises its weight in them and hands the feed-forward rows that are only divided by their root mean square
+    behind its first product.  The norm's weights are far from 1 and differ by column, so that a weight applied twice,
+    not at all or to the wrong operand shows."""
     from pulse_infer_amd.ops import kernels
-    from pulse_infer_amd.parts.base import FEED_FORWARDS, NORMS, ResidualStream, RowStats
-    hidden, inter, eps = 1024, 96, 1e-5
+    from pulse_infer_amd.parts.base import FEED_FORWARDS, NORMS, LazyNorm, ResidualStream, RowStats
+    from pulse_infer_amd.parts.linear import Linear
+    hidden, inter, inner, eps, mode = 1024, 96, 2048, 1e-5, "bfloat16"
     nw = (torch.linspace(0.25, 4.0, hidden) * torch.tensor([1.0, -1.0]).repeat(hidden // 2)).to(torch.bfloat16)
     ws = {"m.gate_proj.weight": rnd(inter, hidden, seed=3, scale=hidden ** -0.5),
           "m.up_proj.weight": rnd(inter, hidden, seed=4, scale=hidden ** -0.5),
-          "m.down_proj.weight": rnd(hidden, inter, seed=5, scale=inter ** -0.5), "n.weight": nw}
+          "m.down_proj.weight": rnd(hidden, inter, seed=5, scale=inter ** -0.5), "n.weight": nw, "other.weight": nw.clone()}
     build = build_ctx(ws, mode)
     mlp = FEED_FORWARDS.get("gated_mlp")({"hidden_size": hidden, "intermediate_size": inter, "activation": "silu"}, "m", build)
     norm = NORMS.get("rmsnorm")({"size": hidden, "eps": eps}, "n", build)
-    took = mlp.fold_input_weight(norm.foldable_weight())
-    assert took == (mode == "bfloat16")
-    # a width for which no product scales its rows keeps the norm's weight in the norm: folding rounds once more
-    # and would buy nothing there
-    narrow = {"m.gate_proj.weight": rnd(96, 72, seed=3), "m.up_proj.weight": rnd(96, 72, seed=4),
-              "m.down_proj.weight": rnd(72, 96, seed=5)}
-    small = FEED_FORWARDS.get("gated_mlp")({"hidden_size": 72, "intermediate_size": 96, "activation": "silu"}, "m",
-                                           build_ctx(narrow, mode))
-    assert not small.fold_input_weight(torch.ones(72, dtype=torch.bfloat16, device=DEV))
-    if took:
-        norm.weight_folded()
-        assert norm.foldable_weight() is None              # it can be given away once
+    other = NORMS.get("rmsnorm")({"size": hidden, "eps": eps}, "other", build)
+    # the product before: h += a o^T, told who reads h next
+    o = Linear(rnd(hidden, inner, seed=7, scale=inner ** -0.5).to(DEV), mode)
+    a = rnd(rows, inner, seed=8).to(DEV)
     h = (torch.randn(rows, hidden, generator=torch.Generator().manual_seed(6)) * 3).to(DEV)
+    before = h.clone()
+    scratch = torch.empty(rows, hidden, dtype=torch.bfloat16, device=DEV)
+    left = o.add_into(a, h, scratch, build.workspace, next_scale=norm.column_scale())
+    ctx = step_ctx(build, list(range(rows)), [0] * rows, [[0]])
+    if rows > kernels.SKINNY_FAST_ROWS:
+        assert not isinstance(left, RowStats)          # more rows: an update in parts, which the norm's kernel adds up
+        return
+    assert isinstance(left, RowStats) and left.scaled_by is norm.weight
+    assert torch.allclose(h.double(), before.double() + a.double() @ o.weight.double().T, atol=1e-3, rtol=1e-4)
+    assert torch.equal(left.rounded, (h * nw.to(DEV).float()).to(torch.bfloat16))       # the weight is in, rounded once
+    want_sums = (h.double() ** 2).view(rows, hidden // 16, 16).sum(-1)
+    assert torch.allclose(left.sumsq.double(), want_sums, rtol=1e-5, atol=1e-6)
     want = P.gated_mlp(P.rms_norm(h.cpu().to(F64), nw.to(F64), eps),
                        *(ws[f"m.{n}_proj.weight"].to(F64) for n in ("gate", "up", "down")))
-    ctx = step_ctx(build, list(range(rows)), [0] * rows, [[0]])
-    # 1. through the norm's own kernel (what prompt portions do): the weight is applied exactly once either way
-    x = torch.empty(rows, hidden, dtype=build.act_dtype, device=DEV)
-    norm.apply(h, None, x)
-    out = mlp.forward(x, ctx)
     scale = float(want.abs().max())
-    assert float((out.cpu().to(F64) - want).abs().max()) <= (3e-5 if mode == "float32" else 3e-2) * scale
-    # 2. as a decoding step does it: the rows as the product before left them, normalised behind the first product
     stream = ResidualStream(h)
-    sums = (h.double() ** 2).view(rows, hidden // 16, 16).sum(-1).float().contiguous()
-    stream.push(RowStats(sums, h.to(torch.bfloat16)))
+    stream.push(left)
+    assert stream.lazy(other) is None                  # a norm with another weight does not take them for its own
     lazy = stream.lazy(norm)
-    if mode == "float32" or rows > kernels.SKINNY_FAST_ROWS:
-        assert lazy is None or not mlp.gate_up.takes_lazy(lazy)     # the norm's kernel it is
-        return
-    assert lazy is not None and mlp.gate_up.takes_lazy(lazy)
+    assert isinstance(lazy, LazyNorm) and mlp.gate_up.takes_lazy(lazy)
     out = mlp.forward(lazy, ctx)
     assert float((out.cpu().to(F64) - want).abs().max()) <= 3e-2 * scale
+    # the ordinary way gives the same within rounding
+    x = torch.empty(rows, hidden, dtype=build.act_dtype, device=DEV)
+    norm.apply(h, None, x)
+    plain_way = mlp.forward(x, ctx)
+    assert float((out.float() - plain_way.float()).abs().max()) <= 2e-2 * scale
+    # rows left as they are (nobody said who reads next) are nobody's
+    left = o.add_into(a, h, scratch, build.workspace)
+    assert isinstance(left, RowStats) and left.scaled_by is None
+    stream.push(left)
+    assert stream.lazy(norm) is None
 
 
 @pytest.mark.parametrize("mode", ["float32", "bfloat16"])
