@@ -373,15 +373,28 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
         float mass = 0.f;
         sweep(row, threadIdx.x, vocab, SAMPLE_THREADS, [&](int, float x) { mass += weight_of(x); });
         const float want = p * block_sum_f(mass, sf);
+        // The largest threshold whose kept mass still reaches `want`, four bits of it a pass over the row: the masses
+        // above the fifteen candidates of a digit are summed side by side (each in the order in which a pass for it
+        // alone would sum it, so the choice is that of a search bit by bit, in an eighth of the passes).
         uint32_t thr = 0u;
-        for (int bit = 31; bit >= 0; --bit) {
-            const uint32_t cand = thr | (1u << bit);
-            const uint32_t lim = cand > keep ? cand : keep;
-            float part_mass = 0.f;
+        for (int shift = 28; shift >= 0; shift -= 4) {
+            float above[15];
+#pragma unroll
+            for (int j = 0; j < 15; ++j) above[j] = 0.f;
             sweep(row, threadIdx.x, vocab, SAMPLE_THREADS, [&](int, float x) {
-                if (x != -INFINITY && order_key(x) >= lim) part_mass += expf((x - best) * inv_t);
+                if (x == -INFINITY) return;
+                const uint32_t key = order_key(x);
+                if (key < keep || key < (thr | (1u << shift))) return;
+                const float w = expf((x - best) * inv_t);
+#pragma unroll
+                for (int j = 0; j < 15; ++j)
+                    if (key >= (thr | (static_cast<uint32_t>(j + 1) << shift))) above[j] += w;
             });
-            if (block_sum_f(part_mass, sf) >= want) thr = cand;
+            uint32_t digit = 0u;
+#pragma unroll
+            for (int j = 0; j < 15; ++j)
+                if (block_sum_f(above[j], sf) >= want) digit = static_cast<uint32_t>(j + 1);
+            thr |= digit << shift;
         }
         if (thr > keep) keep = thr;
     }
