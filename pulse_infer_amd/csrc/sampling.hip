@@ -493,6 +493,166 @@ __global__ __launch_bounds__(PULSE_WAVE) void argmax_merge_kernel(const float* _
     if (threadIdx.x == 0) out[r] = best_i == 0x7fffffff ? -1 : best_i;
 }
 
+// ---- rows without top-k and top-p, in chunks -------------------------------------------------------------------
+// A workgroup a row reads its row at the rate of one compute unit.  Without top-k and top-p nothing has to be
+// known about the row as a whole but its maximum and its mass, so the row is cut into chunks of SIMPLE_CHUNK logits
+// with a workgroup each: the chunk's maximum (with its lowest index); then, the row's maximum known, the chunk's
+// mass; then one wavefront a row finds the chunk in which u * mass falls (chunk masses summed in chunk order) and
+// walks that chunk alone.  The steps and their meaning are those of sample_kernel; sums are taken in another order.
+constexpr int SIMPLE_CHUNK = 2048;
+constexpr int SIMPLE_THREADS = 256;
+
+__device__ __forceinline__ RowView simple_row(const float* logits, int r, int64_t row_stride, int vocab,
+                                              const float* penalty, const int* seen_row, const uint32_t* seen_masks,
+                                              const uint32_t* banned, int mask_words) {
+    RowView row;
+    row.logits = logits + r * row_stride;
+    row.vocab = vocab;
+    row.banned = banned;
+    row.penalty = penalty ? penalty[r] : 0.f;
+    row.seen = (seen_masks && seen_row && seen_row[r] >= 0 && row.penalty > 0.f)
+                   ? seen_masks + static_cast<int64_t>(seen_row[r]) * mask_words : nullptr;
+    return row;
+}
+
+__global__ __launch_bounds__(SIMPLE_THREADS) void simple_max_kernel(
+    const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ penalty,
+    const int* __restrict__ seen_row, const uint32_t* __restrict__ seen_masks, const uint32_t* __restrict__ banned,
+    int mask_words, float* __restrict__ part_max, int* __restrict__ part_idx) {
+    __shared__ float sv[SIMPLE_THREADS / PULSE_WAVE];
+    __shared__ int si[SIMPLE_THREADS / PULSE_WAVE];
+    const int r = blockIdx.y, chunk = blockIdx.x, chunks = gridDim.x;
+    const RowView row = simple_row(logits, r, row_stride, vocab, penalty, seen_row, seen_masks, banned, mask_words);
+    const int begin = chunk * SIMPLE_CHUNK, end = min(vocab, begin + SIMPLE_CHUNK);
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    sweep(row, begin + static_cast<int>(threadIdx.x), end, SIMPLE_THREADS, [&](int i, float x) {
+        if (x > best) { best = x; best_i = i; }   // a thread's indices rise: the first of equals stays
+    });
+    const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off, PULSE_WAVE);
+        const int oi = __shfl_xor(best_i, off, PULSE_WAVE);
+        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    if (lane == 0) { sv[wave] = best; si[wave] = best_i; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < SIMPLE_THREADS / PULSE_WAVE; ++w)
+            if (sv[w] > best || (sv[w] == best && si[w] < best_i)) { best = sv[w]; best_i = si[w]; }
+        part_max[r * chunks + chunk] = best;
+        part_idx[r * chunks + chunk] = best_i;
+    }
+}
+
+// The row's maximum from the chunks' (every lane gets it).
+__device__ __forceinline__ float simple_row_max(const float* part_max, int chunks) {
+    float best = -INFINITY;
+    for (int c = threadIdx.x % PULSE_WAVE; c < chunks; c += PULSE_WAVE) best = fmaxf(best, part_max[c]);
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) best = fmaxf(best, __shfl_xor(best, off, PULSE_WAVE));
+    return best;
+}
+
+__global__ __launch_bounds__(SIMPLE_THREADS) void simple_mass_kernel(
+    const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ temperature,
+    const float* __restrict__ penalty, const int* __restrict__ seen_row, const uint32_t* __restrict__ seen_masks,
+    const uint32_t* __restrict__ banned, int mask_words, const float* __restrict__ part_max,
+    float* __restrict__ part_mass) {
+    __shared__ float sf[SIMPLE_THREADS / PULSE_WAVE];
+    const int r = blockIdx.y, chunk = blockIdx.x, chunks = gridDim.x;
+    const float temp = temperature ? temperature[r] : 0.f;
+    if (!(temp > 0.f)) return;   // the largest logit wins: no mass is asked for
+    const float best = simple_row_max(part_max + r * chunks, chunks);
+    if (best == -INFINITY) return;
+    const float inv_t = 1.0f / temp;
+    const RowView row = simple_row(logits, r, row_stride, vocab, penalty, seen_row, seen_masks, banned, mask_words);
+    const int begin = chunk * SIMPLE_CHUNK, end = min(vocab, begin + SIMPLE_CHUNK);
+    float mass = 0.f;
+    sweep(row, begin + static_cast<int>(threadIdx.x), end, SIMPLE_THREADS, [&](int, float x) {
+        if (x != -INFINITY) mass += expf((x - best) * inv_t);
+    });
+    const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) mass += __shfl_xor(mass, off, PULSE_WAVE);
+    if (lane == 0) sf[wave] = mass;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float total = 0.f;
+        for (int w = 0; w < SIMPLE_THREADS / PULSE_WAVE; ++w) total += sf[w];
+        part_mass[r * chunks + chunk] = total;
+    }
+}
+
+__global__ __launch_bounds__(PULSE_WAVE) void simple_pick_kernel(
+    const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ temperature,
+    const float* __restrict__ uniform, const float* __restrict__ penalty, const int* __restrict__ seen_row,
+    const uint32_t* __restrict__ seen_masks, const uint32_t* __restrict__ banned, int mask_words,
+    const float* __restrict__ part_max, const int* __restrict__ part_idx, const float* __restrict__ part_mass,
+    int chunks, int* __restrict__ out) {
+    const int r = blockIdx.x, lane = threadIdx.x;
+    part_max += r * chunks;
+    part_idx += r * chunks;
+    part_mass += r * chunks;
+    // the largest logit, the lowest index among equals
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int c = lane; c < chunks; c += PULSE_WAVE) {
+        const float v = part_max[c];
+        const int i = part_idx[c];
+        if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+    }
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off, PULSE_WAVE);
+        const int oi = __shfl_xor(best_i, off, PULSE_WAVE);
+        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    if (best_i == 0x7fffffff) {   // everything banned or NaN
+        if (lane == 0) out[r] = -1;
+        return;
+    }
+    const float temp = temperature ? temperature[r] : 0.f;
+    if (!(temp > 0.f)) {
+        if (lane == 0) out[r] = best_i;
+        return;
+    }
+    // the chunk in which the draw falls: chunk masses in chunk order, as a walk over them
+    int last_chunk;
+    float total = 0.f;
+    for (int c = lane; c < chunks; c += PULSE_WAVE) total += part_mass[c];
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) total += __shfl_xor(total, off, PULSE_WAVE);
+    const float target = uniform[r] * total;
+    // running sum over the chunks before the one that is hit, in chunk order (one lane's work: a few dozen additions)
+    float run = 0.f;
+    int who = -1;
+    last_chunk = -1;
+    for (int c = 0; c < chunks; ++c) {
+        const float m = part_mass[c];
+        if (m > 0.f) {
+            last_chunk = c;
+            if (target < run + m) { who = c; break; }
+        }
+        run += m;
+    }
+    float rest = target - run;
+    if (who < 0) {  // rounding left the target beyond the last chunk with mass: its last kept entry
+        who = last_chunk;
+        rest = INFINITY;
+    }
+    const float inv_t = 1.0f / temp;
+    const RowView row = simple_row(logits, r, row_stride, vocab, penalty, seen_row, seen_masks, banned, mask_words);
+    const int begin = who * SIMPLE_CHUNK, end = min(vocab, begin + SIMPLE_CHUNK);
+    int last;
+    const int e = wave_walk(begin, end, rest, [&](int i) {
+        const float x = row.at(i);
+        return x != -INFINITY ? expf((x - best) * inv_t) : 0.f;
+    }, last);
+    if (lane == 0) out[r] = e >= 0 ? e : (last >= 0 ? last : best_i);
+}
+
 }  // namespace
 
 // out[r] = index of the largest logit of row r, the lowest index among equals, -1 if none is a number.
@@ -580,6 +740,38 @@ extern "C" int pulse_sample(const float* logits, int rows, int vocab, int64_t ro
     hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, row_stride,
                        temperature, top_k, top_p, uniform, penalty, seen_row, seen_masks, banned, mask_words, out);
     PULSE_LAUNCH_CHECK("sample");
+    return 0;
+}
+
+// The same for rows none of which asks for top-k or top-p (greedy rows and rows that sample from the whole
+// vocabulary at their temperature), in chunks of the vocabulary with a workgroup each.  part_max, part_idx and
+// part_mass: scratch of rows * pulse_sample_simple_chunks(vocab) entries each.
+extern "C" int pulse_sample_simple_chunks(int vocab) { return (vocab + SIMPLE_CHUNK - 1) / SIMPLE_CHUNK; }
+
+extern "C" int pulse_sample_simple(const float* logits, int rows, int vocab, int64_t row_stride, const float* temperature,
+                                   const float* uniform, const float* penalty, const int* seen_row,
+                                   const uint32_t* seen_masks, const uint32_t* banned, int mask_words, float* part_max,
+                                   int* part_idx, float* part_mass, int* out, hipStream_t stream) {
+    PULSE_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "sample_simple: bad sizes rows=%d V=%d", rows, vocab);
+    PULSE_REQUIRE(rows < 65536, "sample_simple: at most 65535 rows");
+    PULSE_REQUIRE(logits && out && part_max && part_idx && part_mass, "sample_simple: null pointer");
+    PULSE_REQUIRE(!temperature || uniform, "sample_simple: temperature sampling needs uniform numbers");
+    PULSE_REQUIRE((!seen_masks && !banned) || mask_words * 32 >= vocab, "sample_simple: masks cover %d tokens, "
+                  "vocabulary has %d", mask_words * 32, vocab);
+    if (rows == 0) return 0;
+    const int chunks = pulse_sample_simple_chunks(vocab);
+    hipLaunchKernelGGL(simple_max_kernel, dim3(chunks, rows), dim3(SIMPLE_THREADS), 0, stream, logits, vocab, row_stride,
+                       penalty, seen_row, seen_masks, banned, mask_words, part_max, part_idx);
+    PULSE_LAUNCH_CHECK("sample_simple (maxima)");
+    if (temperature) {
+        hipLaunchKernelGGL(simple_mass_kernel, dim3(chunks, rows), dim3(SIMPLE_THREADS), 0, stream, logits, vocab,
+                           row_stride, temperature, penalty, seen_row, seen_masks, banned, mask_words, part_max, part_mass);
+        PULSE_LAUNCH_CHECK("sample_simple (masses)");
+    }
+    hipLaunchKernelGGL(simple_pick_kernel, dim3(rows), dim3(PULSE_WAVE), 0, stream, logits, vocab, row_stride, temperature,
+                       uniform, penalty, seen_row, seen_masks, banned, mask_words, part_max, part_idx, part_mass, chunks,
+                       out);
+    PULSE_LAUNCH_CHECK("sample_simple (pick)");
     return 0;
 }
 

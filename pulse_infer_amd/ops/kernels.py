@@ -385,6 +385,48 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.
          _ptr(banned), _i32(words), _ptr(out), _stream())
 
 
+SAMPLE_SIMPLE_CHUNK = 2048   # as SIMPLE_CHUNK of sampling.hip
+
+
+def sample_simple_chunks(vocab: int) -> int:
+    """Chunks of the vocabulary that ``sample_simple`` cuts a row into (its scratch holds rows * chunks entries)."""
+    return (vocab + SAMPLE_SIMPLE_CHUNK - 1) // SAMPLE_SIMPLE_CHUNK
+
+
+def sample_simple(logits: torch.Tensor, out: torch.Tensor, part_max: torch.Tensor, part_idx: torch.Tensor,
+                  part_mass: torch.Tensor, temperature: Optional[torch.Tensor] = None,
+                  uniform: Optional[torch.Tensor] = None, penalty: Optional[torch.Tensor] = None,
+                  seen_row: Optional[torch.Tensor] = None, seen_masks: Optional[torch.Tensor] = None,
+                  banned: Optional[torch.Tensor] = None) -> None:
+    """``sample`` for rows none of which asks for top-k or top-p: the largest logit where the temperature is absent
+    or <= 0, else a draw from the whole vocabulary at the row's temperature; in chunks of the vocabulary with a
+    workgroup each instead of a workgroup a row."""
+    _gpu("sample_simple", logits, out, part_max, part_idx, part_mass, temperature, uniform, penalty, seen_row, seen_masks,
+         banned)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1,
+          "sample_simple: logits must be float32 [R, V]")
+    rows, vocab = logits.shape
+    _int_vec("sample_simple: out", out, rows)
+    for name, t, dt in (("temperature", temperature, torch.float32), ("uniform", uniform, torch.float32),
+                        ("penalty", penalty, torch.float32), ("seen_row", seen_row, torch.int32)):
+        if t is not None:
+            _need(t.dtype == dt and t.is_contiguous() and t.numel() >= rows, f"sample_simple: {name} must be {dt}[{rows}]")
+    need = rows * sample_simple_chunks(vocab)
+    for name, t, dt in (("part_max", part_max, torch.float32), ("part_idx", part_idx, torch.int32),
+                        ("part_mass", part_mass, torch.float32)):
+        _need(t.dtype == dt and t.is_contiguous() and t.numel() >= need, f"sample_simple: {name} must hold {need} {dt}")
+    words = 0
+    for name, t in (("seen_masks", seen_masks), ("banned", banned)):
+        if t is not None:
+            _need(t.dtype == torch.int32 and t.is_contiguous(), f"sample_simple: {name} must be contiguous int32 words")
+            w = t.shape[-1]
+            _need(words in (0, w), "sample_simple: masks differ in width")
+            words = w
+    call("pulse_sample_simple", _ptr(logits), _i32(rows), _i32(vocab), _i64(logits.stride(0) if rows > 1 else vocab),
+         _ptr(temperature), _ptr(uniform), _ptr(penalty), _ptr(seen_row), _ptr(seen_masks), _ptr(banned), _i32(words),
+         _ptr(part_max), _ptr(part_idx), _ptr(part_mass), _ptr(out), _stream())
+
+
 def argmax(logits: torch.Tensor, out: torch.Tensor, part_val: torch.Tensor, part_idx: torch.Tensor) -> None:
     """out[r] = index of the largest logit of row r, lowest index among equals (two-stage, for few rows of a wide vocabulary)."""
     _gpu("argmax", logits, out, part_val, part_idx)

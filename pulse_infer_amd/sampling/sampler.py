@@ -27,6 +27,9 @@ class Sampler:
         self.banned: Optional[torch.Tensor] = None
         self._part_val: Optional[torch.Tensor] = None
         self._part_idx: Optional[torch.Tensor] = None
+        self._part_mass: Optional[torch.Tensor] = None   # scratch of the sampling in chunks (with _part_max, _part_at)
+        self._part_max: Optional[torch.Tensor] = None
+        self._part_at: Optional[torch.Tensor] = None
         if banned_tokens:
             host = torch.zeros(self.words, dtype=torch.int64)
             for tok in banned_tokens:
@@ -82,7 +85,18 @@ class Sampler:
         top_k = dev[1]
         penalty = dev[4].view(torch.float32) if use_penalty else None
         seen_row = dev[5] if use_penalty else None
+        seen = self.seen if penalty is not None else None
+        if all(p.top_k == 0 and not 0.0 < p.top_p < 1.0 for p in params):
+            # nothing but temperatures: the rows go through the kernels that cut a row into chunks
+            need = rows * kernels.sample_simple_chunks(logits.shape[1])
+            if self._part_mass is None or self._part_mass.numel() < need:
+                self._part_mass = torch.empty(need, dtype=torch.float32, device=self.device)
+                self._part_max = torch.empty(need, dtype=torch.float32, device=self.device)
+                self._part_at = torch.empty(need, dtype=torch.int32, device=self.device)
+            kernels.sample_simple(logits, out, self._part_max, self._part_at, self._part_mass, temperature=temperature,
+                                  uniform=uniform, penalty=penalty, seen_row=seen_row, seen_masks=seen,
+                                  banned=self.banned)
+            return out.tolist()
         kernels.sample(logits, out, temperature=temperature, top_k=top_k, top_p=top_p, uniform=uniform,
-                       penalty=penalty, seen_row=seen_row, seen_masks=self.seen if penalty is not None else None,
-                       banned=self.banned)
+                       penalty=penalty, seen_row=seen_row, seen_masks=seen, banned=self.banned)
         return out.tolist()

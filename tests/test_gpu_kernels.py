@@ -401,6 +401,91 @@ def test_sampling_at_a_real_vocabulary(k, mode):
     assert again.item() == got[5]
 
 
+def _simple_scratch(k, rows, vocab):
+    n = rows * k.sample_simple_chunks(vocab)
+    return (torch.full((n,), float("nan"), device=DEV), torch.full((n,), -7, dtype=torch.int32, device=DEV),
+            torch.full((n,), float("nan"), device=DEV))
+
+
+@pytest.mark.parametrize("vocab", [151936, 2048, 2049, 700])
+def test_sampling_in_chunks(k, vocab):
+    """Rows without top-k and top-p through the kernels that cut a row into chunks (a workgroup a chunk): greedy rows
+    (ties, NaN, all banned) beside rows at a temperature, a presence penalty and banned ids; every draw against the
+    same steps in float64, as for the kernel that takes a workgroup a row, and the same draw whatever else is batched."""
+    rows = 40
+    gen = torch.Generator().manual_seed(21)
+    logits = torch.randn(rows, vocab, generator=gen) * 2.5
+    logits[0, 17] = logits[0, vocab - 3] = 50.0            # greedy: the lowest index among equals
+    logits[1, vocab - 1] = 60.0
+    logits[2, 5] = float("nan")
+    temp = torch.full((rows,), 0.7)
+    temp[:4] = 0.0                                          # rows 0 to 3 are greedy
+    temp[4] = 5.0                                           # a flat row
+    uniform = torch.rand(rows, generator=gen)
+    uniform[5] = 0.0
+    uniform[6] = 0.99999994                                 # the last kept token, not beyond it
+    words = (vocab + 31) // 32
+    banned = torch.zeros(words, dtype=torch.int64)
+    for tok in (3, 40, vocab - 1):
+        banned[tok >> 5] |= 1 << (tok & 31)
+    banned = torch.where(banned >= 2 ** 31, banned - 2 ** 32, banned).to(torch.int32)
+    seen = torch.zeros(rows, words, dtype=torch.int32, device=DEV)
+    best = torch.argmax(torch.nan_to_num(logits, nan=-1e30), dim=1).to(torch.int32)
+    k.mark_seen(seen, torch.arange(rows, dtype=torch.int32, device=DEV), best.to(DEV), vocab)
+    penalty = torch.zeros(rows)
+    penalty[10:20] = 1.5
+    ref = torch.nan_to_num(logits.to(F64), nan=float("-inf")).clone()
+    ref[torch.arange(10, 20), best[10:20].long()] -= 1.5
+    ref[:, [3, 40, vocab - 1]] = float("-inf")
+    dev = lambda t: t.to(DEV)
+    kw = dict(temperature=dev(temp), uniform=dev(uniform), penalty=dev(penalty),
+              seen_row=torch.arange(rows, dtype=torch.int32, device=DEV), seen_masks=seen, banned=dev(banned))
+    out = torch.full((rows,), -5, dtype=torch.int32, device=DEV)
+    k.sample_simple(dev(logits), out, *_simple_scratch(k, rows, vocab), **kw)
+    got = out.cpu().tolist()
+    for r in range(rows):
+        x = ref[r]
+        if float(temp[r]) <= 0:
+            assert got[r] == int(torch.argmax(x)), r       # torch.argmax: the first of equals
+            continue
+        w = torch.exp((x - x.max()) / float(temp[r]))
+        cum = torch.cumsum(w, 0)
+        target = float(uniform[r]) * float(cum[-1])
+        t = got[r]
+        slack = 2e-5 * float(cum[-1])
+        assert float(w[t]) > 0 and t not in (3, 40, vocab - 1), (r, t)
+        assert float(cum[t]) - float(w[t]) - slack <= target <= float(cum[t]) + slack, (r, t)
+    # the kernel with a workgroup a row agrees (its sums run in another order: draws at an interval's edge may differ)
+    other = torch.empty(rows, dtype=torch.int32, device=DEV)
+    k.sample(dev(logits), other, **kw)
+    assert sum(a != b for a, b in zip(got, other.cpu().tolist())) <= 1
+    # a row's draw does not depend on the other rows
+    again = torch.empty(1, dtype=torch.int32, device=DEV)
+    one = {n: v[12:13] for n, v in kw.items() if n not in ("seen_masks", "banned")}
+    one["seen_row"] = torch.tensor([12], dtype=torch.int32, device=DEV)
+    k.sample_simple(dev(logits[12:13]), again, *_simple_scratch(k, 1, vocab), seen_masks=seen, banned=dev(banned), **one)
+    assert again.item() == got[12]
+    # nothing left of a row: -1
+    everything = torch.full((words,), -1, dtype=torch.int32, device=DEV)
+    k.sample_simple(dev(logits[:2]), out[:2], *_simple_scratch(k, 2, vocab), temperature=dev(temp[4:6]),
+                    uniform=dev(uniform[:2]), banned=everything)
+    assert out[:2].tolist() == [-1, -1]
+
+
+def test_temperature_sampling_in_chunks_follows_the_softmax(k):
+    vocab, rows = 5000, 4000
+    base = torch.full((vocab,), -30.0)
+    base[[5, 2047, 2048, 4999]] = torch.tensor([1.0, 2.0, 0.5, 1.5])     # on both sides of a chunk's edge
+    logits = base.repeat(rows, 1).to(DEV)
+    temperature = torch.full((rows,), 0.8, device=DEV)
+    uniform = torch.rand(rows, generator=torch.Generator().manual_seed(1)).to(DEV)
+    out = torch.empty(rows, dtype=torch.int32, device=DEV)
+    k.sample_simple(logits, out, *_simple_scratch(k, rows, vocab), temperature=temperature, uniform=uniform)
+    counts = torch.bincount(out.cpu().long(), minlength=vocab).double() / rows
+    want = torch.softmax(base.double() / 0.8, dim=0)
+    assert torch.allclose(counts, want, atol=0.03)
+
+
 def test_kernels_refuse_what_they_cannot_do(k):
     from pulse_infer_amd.ops import KernelError
     with pytest.raises(KernelError, match="GPU"):
