@@ -146,14 +146,87 @@ constexpr int WAVE_CAP = 128;                           // candidates a wavefron
 constexpr int LIST_CAP = SAMPLE_WAVES * WAVE_CAP;       // candidates of a row
 constexpr int LIST_PER_LANE = LIST_CAP / PULSE_WAVE;
 
+// The end of the choice on a short list in LDS, by one wavefront: `n` candidates in vocabulary order (`list_i`, their
+// values `list_x`, which are overwritten), among them every token that top-k keeps.  The k-th largest value by a
+// search bit by bit, then top-p on what that kept (relative to its mass; without top-k relative to `whole`, the mass
+// of the whole row, and only if the list holds that much: else false and nothing is chosen), then the walk along the
+// cumulative sum.  Every lane returns the same.  PER: entries a lane takes (n <= PER * 64).
+template <int PER>
+__device__ bool finish_on_list(const int* list_i, float* list_x, int n, bool by_k, int k, bool use_p, float p, float whole,
+                               float best, float inv_t, float u, int best_i, int& token) {
+    const int lane = threadIdx.x % PULSE_WAVE;
+    auto lane_sum_i = [&](int v) {
+#pragma unroll
+        for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, PULSE_WAVE);
+        return v;
+    };
+    auto lane_sum_f = [&](float v) {
+#pragma unroll
+        for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, PULSE_WAVE);
+        return v;
+    };
+    uint32_t keys[PER];
+    float wts[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int e = lane + j * PULSE_WAVE;
+        keys[j] = e < n ? order_key(list_x[e]) : 0u;
+        wts[j] = e < n ? expf((list_x[e] - best) * inv_t) : 0.f;
+    }
+    // the k-th largest key, bit by bit
+    uint32_t keep = 0u;
+    if (by_k) {
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = keep | (1u << bit);
+            int c = 0;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) c += (lane + j * PULSE_WAVE < n && keys[j] >= cand) ? 1 : 0;
+            if (lane_sum_i(c) >= k) keep = cand;
+        }
+    }
+    if (use_p) {
+        float mass = 0.f;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) mass += keys[j] >= keep ? wts[j] : 0.f;
+        mass = lane_sum_f(mass);
+        const float want = p * (by_k ? mass : whole);
+        if (!by_k && !(mass >= want)) return false;   // without top-k the list must hold all of the top_p set
+        uint32_t thr = 0u;
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = thr | (1u << bit);
+            const uint32_t lim = cand > keep ? cand : keep;
+            float part_mass = 0.f;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) part_mass += keys[j] >= lim ? wts[j] : 0.f;
+            if (lane_sum_f(part_mass) >= want) thr = cand;
+        }
+        if (thr > keep) keep = thr;
+    }
+    // what is kept, as weights in the list's place of x, then the walk
+    float kept = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int e = lane + j * PULSE_WAVE;
+        const float w = (e < n && keys[j] >= keep) ? wts[j] : 0.f;
+        if (e < n) list_x[e] = w;
+        kept += w;
+    }
+    kept = lane_sum_f(kept);
+    int last;
+    const int e = wave_walk(0, n, u * kept, [&](int q) { return list_x[q]; }, last);
+    token = e >= 0 ? list_i[e] : (last >= 0 ? list_i[last] : best_i);
+    return true;
+}
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
     const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ uniform,
     const float* __restrict__ penalty, const int* __restrict__ seen_row, const uint32_t* __restrict__ seen_masks,
-    const uint32_t* __restrict__ banned, int mask_words, int* __restrict__ out) {
+    const uint32_t* __restrict__ banned, int mask_words, int* __restrict__ out, const int* __restrict__ done) {
     __shared__ float sf[SAMPLE_WAVES];
     __shared__ int si[SAMPLE_WAVES];
     __shared__ int hist[HIST_BINS];
+    if (done && done[blockIdx.x]) return;   // the kernels that work in chunks have chosen this row's token already
     __shared__ int wave_bins[SAMPLE_WAVES];
     __shared__ int region_i[SAMPLE_WAVES][WAVE_CAP];
     __shared__ float region_x[SAMPLE_WAVES][WAVE_CAP];
@@ -281,74 +354,13 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(
                 __syncthreads();
                 // the first wavefront finishes alone (lane l holds entries l, l + 64, ..); the others wait for its word
                 if (wave == 0) {
-                auto lane_sum_i = [&](int v) {
-#pragma unroll
-                    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, PULSE_WAVE);
-                    return v;
-                };
-                auto lane_sum_f = [&](float v) {
-#pragma unroll
-                    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, PULSE_WAVE);
-                    return v;
-                };
-                uint32_t keys[LIST_PER_LANE];
-                float wts[LIST_PER_LANE];
-#pragma unroll
-                for (int j = 0; j < LIST_PER_LANE; ++j) {
-                    const int e = lane + j * PULSE_WAVE;
-                    keys[j] = e < n ? order_key(list_x[e]) : 0u;
-                    wts[j] = e < n ? expf((list_x[e] - best) * inv_t) : 0.f;
-                }
-                // the k-th largest key, bit by bit
-                uint32_t keep = 0u;
-                if (by_k) {
-                    for (int bit = 31; bit >= 0; --bit) {
-                        const uint32_t cand = keep | (1u << bit);
-                        int c = 0;
-#pragma unroll
-                        for (int j = 0; j < LIST_PER_LANE; ++j) c += (lane + j * PULSE_WAVE < n && keys[j] >= cand) ? 1 : 0;
-                        if (lane_sum_i(c) >= k) keep = cand;
+                    int token;
+                    const bool enough = finish_on_list<LIST_PER_LANE>(list_i, list_x, n, by_k, k, use_p, p, whole, best, inv_t, uniform[r],
+                                                       best_i, token);
+                    if (lane == 0) {
+                        if (enough) out[r] = token;   // else (only without top-k) the list is too short: the passes
+                        list_done = enough ? 1 : 0;   // over the whole vocabulary
                     }
-                }
-                bool enough = true;
-                if (use_p) {
-                    float mass = 0.f;
-#pragma unroll
-                    for (int j = 0; j < LIST_PER_LANE; ++j) mass += keys[j] >= keep ? wts[j] : 0.f;
-                    mass = lane_sum_f(mass);
-                    const float want = p * (by_k ? mass : whole);
-                    enough = by_k || mass >= want;   // without top-k the list must hold all of the top_p set
-                    uint32_t thr = 0u;
-                    for (int bit = 31; bit >= 0; --bit) {
-                        const uint32_t cand = thr | (1u << bit);
-                        const uint32_t lim = cand > keep ? cand : keep;
-                        float part_mass = 0.f;
-#pragma unroll
-                        for (int j = 0; j < LIST_PER_LANE; ++j) part_mass += keys[j] >= lim ? wts[j] : 0.f;
-                        if (lane_sum_f(part_mass) >= want) thr = cand;
-                    }
-                    if (thr > keep) keep = thr;
-                }
-                if (!enough) {   // (only without top-k) the list is too short: the passes over the whole vocabulary
-                    if (lane == 0) list_done = 0;
-                } else {
-                // what is kept, as weights in the list's place of x, then the walk
-                float kept = 0.f;
-#pragma unroll
-                for (int j = 0; j < LIST_PER_LANE; ++j) {
-                    const int e = lane + j * PULSE_WAVE;
-                    const float w = (e < n && keys[j] >= keep) ? wts[j] : 0.f;
-                    if (e < n) list_x[e] = w;
-                    kept += w;
-                }
-                kept = lane_sum_f(kept);
-                int last;
-                const int e = wave_walk(0, n, uniform[r] * kept, [&](int q) { return list_x[q]; }, last);
-                if (lane == 0) {
-                    out[r] = e >= 0 ? list_i[e] : (last >= 0 ? list_i[last] : best_i);
-                    list_done = 1;
-                }
-                }
                 }
                 __syncthreads();
                 if (list_done) return;
@@ -653,6 +665,159 @@ __global__ __launch_bounds__(PULSE_WAVE) void simple_pick_kernel(
     if (lane == 0) out[r] = e >= 0 ? e : (last >= 0 ? last : best_i);
 }
 
+// ---- rows with top-k, in chunks -------------------------------------------------------------------------------
+// With a small k the candidates can be found chunk by chunk as well.  The k-th largest of the chunks' maxima is a
+// lower bound of the k-th largest logit (that many logits, the maxima themselves, reach it), so everything that
+// top-k keeps lies at or above it, and little else: a workgroup a chunk collects what it has there, in vocabulary
+// order, into its own short segment; a wavefront a row strings the segments together in LDS and finishes on that list
+// as sample_kernel does on its own (finish_on_list).  A row that does not fit (k above the number of chunks, a chunk
+// with more candidates than its segment holds: many equal values) is left to sample_kernel, which runs behind and
+// skips the rows that are done.
+constexpr int TOPK_SEGMENT = 32;   // candidates a chunk may leave
+
+__global__ __launch_bounds__(SIMPLE_THREADS) void topk_collect_kernel(
+    const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ penalty, const int* __restrict__ seen_row,
+    const uint32_t* __restrict__ seen_masks, const uint32_t* __restrict__ banned, int mask_words,
+    const float* __restrict__ part_max, int* __restrict__ seg_i, float* __restrict__ seg_x, int* __restrict__ seg_n) {
+    constexpr int WAVES = SIMPLE_THREADS / PULSE_WAVE;
+    constexpr int PER = SIMPLE_CHUNK / SIMPLE_THREADS;   // consecutive logits a thread takes
+    __shared__ float s_bound;
+    __shared__ int s_count[WAVES];
+    const int r = blockIdx.y, chunk = blockIdx.x, chunks = gridDim.x;
+    const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
+    const int k = top_k[r];
+    const float temp = temperature ? temperature[r] : 0.f;
+    int* my_n = seg_n + r * chunks + chunk;
+    if (!(temp > 0.f) || k <= 0 || k > chunks || chunks > 2 * PULSE_WAVE) {   // greedy rows need no candidates; the others are not for these kernels
+        if (threadIdx.x == 0) *my_n = 0;
+        return;
+    }
+    // the k-th largest of the chunks' maxima, bit by bit (chunks <= 2 * 64: two a lane)
+    if (wave == 0) {
+        uint32_t keys[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int c = lane + j * PULSE_WAVE;
+            keys[j] = c < chunks ? order_key(part_max[r * chunks + c]) : 0u;
+        }
+        uint32_t bound = 0u;
+        for (int bit = 31; bit >= 0; --bit) {
+            const uint32_t cand = bound | (1u << bit);
+            int c = (keys[0] >= cand ? 1 : 0) + (keys[1] >= cand ? 1 : 0);
+#pragma unroll
+            for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) c += __shfl_xor(c, off, PULSE_WAVE);
+            if (c >= k) bound = cand;
+        }
+        // back to the value whose key it is (a maximum of -inf, a chunk with nothing left, has the key of -inf)
+        float value = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int c = lane + j * PULSE_WAVE;
+            if (c < chunks && keys[j] == bound) value = part_max[r * chunks + c];
+        }
+#pragma unroll
+        for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) value = fmaxf(value, __shfl_xor(value, off, PULSE_WAVE));
+        if (lane == 0) s_bound = value;
+    }
+    __syncthreads();
+    const float bound = s_bound;
+    const RowView row = simple_row(logits, r, row_stride, vocab, penalty, seen_row, seen_masks, banned, mask_words);
+    const int begin = chunk * SIMPLE_CHUNK + static_cast<int>(threadIdx.x) * PER;
+    float xs[PER];
+    int mine = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = begin + j;
+        xs[j] = i < vocab ? row.at(i) : -INFINITY;
+        mine += (xs[j] != -INFINITY && xs[j] >= bound) ? 1 : 0;
+    }
+    // where this thread's candidates go: an exclusive sum over the threads, in thread order (vocabulary order)
+    int pre = mine;
+#pragma unroll
+    for (int off = 1; off < PULSE_WAVE; off <<= 1) {
+        const int up = __shfl_up(pre, off, PULSE_WAVE);
+        if (lane >= off) pre += up;
+    }
+    if (lane == PULSE_WAVE - 1) s_count[wave] = pre;
+    __syncthreads();
+    int at = pre - mine, total = 0;
+    for (int w = 0; w < WAVES; ++w) {
+        if (w < wave) at += s_count[w];
+        total += s_count[w];
+    }
+    int* out_i = seg_i + (static_cast<int64_t>(r) * chunks + chunk) * TOPK_SEGMENT;
+    float* out_x = seg_x + (static_cast<int64_t>(r) * chunks + chunk) * TOPK_SEGMENT;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        if (xs[j] != -INFINITY && xs[j] >= bound) {
+            if (at < TOPK_SEGMENT) { out_i[at] = begin + j; out_x[at] = xs[j]; }
+            ++at;
+        }
+    }
+    if (threadIdx.x == 0) *my_n = total;   // more than TOPK_SEGMENT: the row does not fit
+}
+
+__global__ __launch_bounds__(PULSE_WAVE) void topk_finish_kernel(
+    const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
+    const float* __restrict__ uniform, const float* __restrict__ part_max, const int* __restrict__ part_idx,
+    const int* __restrict__ seg_i, const float* __restrict__ seg_x, const int* __restrict__ seg_n, int chunks,
+    int* __restrict__ out, int* __restrict__ done) {
+    __shared__ int list_i[LIST_CAP];
+    __shared__ float list_x[LIST_CAP];
+    const int r = blockIdx.x, lane = threadIdx.x;
+    part_max += r * chunks;
+    part_idx += r * chunks;
+    seg_n += r * chunks;
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int c = lane; c < chunks; c += PULSE_WAVE) {
+        const float v = part_max[c];
+        const int i = part_idx[c];
+        if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+    }
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(best, off, PULSE_WAVE);
+        const int oi = __shfl_xor(best_i, off, PULSE_WAVE);
+        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    const float temp = temperature ? temperature[r] : 0.f;
+    if (best_i == 0x7fffffff || !(temp > 0.f)) {   // everything banned or NaN, or the largest logit wins
+        if (lane == 0) { out[r] = best_i == 0x7fffffff ? -1 : best_i; done[r] = 1; }
+        return;
+    }
+    const int k = top_k[r];
+    // the segments' places in the list: an exclusive sum over the chunks, in chunk order (two chunks a lane)
+    int n0 = lane < chunks ? seg_n[lane] : 0, n1 = lane + PULSE_WAVE < chunks ? seg_n[lane + PULSE_WAVE] : 0;
+    const bool over = n0 > TOPK_SEGMENT || n1 > TOPK_SEGMENT;
+    int pre0 = n0, pre1 = n1;
+#pragma unroll
+    for (int off = 1; off < PULSE_WAVE; off <<= 1) {
+        const int u0 = __shfl_up(pre0, off, PULSE_WAVE), u1 = __shfl_up(pre1, off, PULSE_WAVE);
+        if (lane >= off) { pre0 += u0; pre1 += u1; }
+    }
+    const int first = __shfl(pre0, PULSE_WAVE - 1, PULSE_WAVE);      // candidates of chunks 0 .. 63
+    const int n = first + __shfl(pre1, PULSE_WAVE - 1, PULSE_WAVE);
+    if (k <= 0 || k > chunks || chunks > 2 * PULSE_WAVE || __ballot(over) != 0ull || n > LIST_CAP || n < k) {
+        if (lane == 0) done[r] = 0;   // not a row for these kernels: sample_kernel takes it
+        return;
+    }
+    const int64_t seg0 = (static_cast<int64_t>(r) * chunks + lane) * TOPK_SEGMENT;
+    for (int e = 0; e < n0; ++e) { list_i[pre0 - n0 + e] = seg_i[seg0 + e]; list_x[pre0 - n0 + e] = seg_x[seg0 + e]; }
+    const int64_t seg1 = seg0 + static_cast<int64_t>(PULSE_WAVE) * TOPK_SEGMENT;
+    for (int e = 0; e < n1; ++e) { list_i[first + pre1 - n1 + e] = seg_i[seg1 + e]; list_x[first + pre1 - n1 + e] = seg_x[seg1 + e]; }
+    __syncthreads();
+    const float p = top_p ? top_p[r] : 0.f;
+    int token;
+    const bool use_p = p > 0.f && p < 1.f;
+    if (n <= 4 * PULSE_WAVE)   // the usual case: a few dozen candidates, a few a lane
+        finish_on_list<4>(list_i, list_x, n, true, k, use_p, p, 0.f, best, 1.0f / temp, uniform[r], best_i, token);
+    else
+        finish_on_list<LIST_PER_LANE>(list_i, list_x, n, true, k, use_p, p, 0.f, best, 1.0f / temp, uniform[r], best_i, token);
+    if (lane == 0) { out[r] = token; done[r] = 1; }
+}
+
 }  // namespace
 
 // out[r] = index of the largest logit of row r, the lowest index among equals, -1 if none is a number.
@@ -738,7 +903,8 @@ extern "C" int pulse_sample(const float* logits, int rows, int vocab, int64_t ro
                   mask_words * 32, vocab);
     if (rows == 0) return 0;
     hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, row_stride,
-                       temperature, top_k, top_p, uniform, penalty, seen_row, seen_masks, banned, mask_words, out);
+                       temperature, top_k, top_p, uniform, penalty, seen_row, seen_masks, banned, mask_words, out,
+                       static_cast<const int*>(nullptr));
     PULSE_LAUNCH_CHECK("sample");
     return 0;
 }
@@ -772,6 +938,41 @@ extern "C" int pulse_sample_simple(const float* logits, int rows, int vocab, int
                        uniform, penalty, seen_row, seen_masks, banned, mask_words, part_max, part_idx, part_mass, chunks,
                        out);
     PULSE_LAUNCH_CHECK("sample_simple (pick)");
+    return 0;
+}
+
+// The same for steps with top-k (every row of which is tried in chunks first: see topk_collect_kernel; rows without
+// top-k, with a k above the number of chunks or with too many equal values go through the kernel of pulse_sample
+// afterwards).  part_max, part_idx, seg_n: rows * chunks entries; seg_i, seg_x: rows * chunks *
+// pulse_sample_topk_segment() entries; done: rows entries (chunks = pulse_sample_simple_chunks(vocab)).
+extern "C" int pulse_sample_topk_segment() { return TOPK_SEGMENT; }
+
+extern "C" int pulse_sample_topk(const float* logits, int rows, int vocab, int64_t row_stride, const float* temperature,
+                                 const int* top_k, const float* top_p, const float* uniform, const float* penalty,
+                                 const int* seen_row, const uint32_t* seen_masks, const uint32_t* banned, int mask_words,
+                                 float* part_max, int* part_idx, int* seg_i, float* seg_x, int* seg_n, int* done, int* out,
+                                 hipStream_t stream) {
+    PULSE_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "sample_topk: bad sizes rows=%d V=%d", rows, vocab);
+    PULSE_REQUIRE(rows < 65536, "sample_topk: at most 65535 rows");
+    PULSE_REQUIRE(logits && out && top_k && temperature && uniform && part_max && part_idx && seg_i && seg_x && seg_n && done,
+                  "sample_topk: null pointer");
+    PULSE_REQUIRE((!seen_masks && !banned) || mask_words * 32 >= vocab, "sample_topk: masks cover %d tokens, "
+                  "vocabulary has %d", mask_words * 32, vocab);
+    if (rows == 0) return 0;
+    const int chunks = pulse_sample_simple_chunks(vocab);
+    hipLaunchKernelGGL(simple_max_kernel, dim3(chunks, rows), dim3(SIMPLE_THREADS), 0, stream, logits, vocab, row_stride,
+                       penalty, seen_row, seen_masks, banned, mask_words, part_max, part_idx);
+    PULSE_LAUNCH_CHECK("sample_topk (maxima)");
+    hipLaunchKernelGGL(topk_collect_kernel, dim3(chunks, rows), dim3(SIMPLE_THREADS), 0, stream, logits, vocab, row_stride,
+                       temperature, top_k, penalty, seen_row, seen_masks, banned, mask_words, part_max, seg_i, seg_x, seg_n);
+    PULSE_LAUNCH_CHECK("sample_topk (candidates)");
+    hipLaunchKernelGGL(topk_finish_kernel, dim3(rows), dim3(PULSE_WAVE), 0, stream, temperature, top_k, top_p, uniform,
+                       part_max, part_idx, seg_i, seg_x, seg_n, chunks, out, done);
+    PULSE_LAUNCH_CHECK("sample_topk (choice)");
+    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, row_stride,
+                       temperature, top_k, top_p, uniform, penalty, seen_row, seen_masks, banned, mask_words, out,
+                       static_cast<const int*>(done));
+    PULSE_LAUNCH_CHECK("sample_topk (the rest)");
     return 0;
 }
 

@@ -30,6 +30,7 @@ class Sampler:
         self._part_mass: Optional[torch.Tensor] = None   # scratch of the sampling in chunks (with _part_max, _part_at)
         self._part_max: Optional[torch.Tensor] = None
         self._part_at: Optional[torch.Tensor] = None
+        self._topk: Optional[dict] = None                # scratch of the top-k sampling in chunks
         if banned_tokens:
             host = torch.zeros(self.words, dtype=torch.int64)
             for tok in banned_tokens:
@@ -96,6 +97,13 @@ class Sampler:
             kernels.sample_simple(logits, out, self._part_max, self._part_at, self._part_mass, temperature=temperature,
                                   uniform=uniform, penalty=penalty, seen_row=seen_row, seen_masks=seen,
                                   banned=self.banned)
+            return out.tolist()
+        if any(p.top_k > 0 for p in params):
+            # top-k somewhere: candidates are found in chunks of the vocabulary first
+            if self._topk is None or self._topk["done"].numel() < rows:
+                self._topk = kernels.sample_topk_scratch(rows, logits.shape[1], self.device)
+            kernels.sample_topk(logits, out, self._topk, temperature=temperature, top_k=top_k, uniform=uniform,
+                                top_p=top_p, penalty=penalty, seen_row=seen_row, seen_masks=seen, banned=self.banned)
             return out.tolist()
         kernels.sample(logits, out, temperature=temperature, top_k=top_k, top_p=top_p, uniform=uniform,
                        penalty=penalty, seen_row=seen_row, seen_masks=seen, banned=self.banned)

@@ -341,20 +341,27 @@ def test_top_k_top_p_penalty_and_banned(k):
     assert greedy[0].item() == second
 
 
-@pytest.mark.parametrize("mode", ["temperature", "top_k", "top_k_top_p", "top_p", "top_p_peaked", "ties", "penalty"])
-def test_sampling_at_a_real_vocabulary(k, mode):
+@pytest.mark.parametrize("mode,vocab,chunked", [
+    ("temperature", 151936, False), ("top_k", 151936, False), ("top_k_top_p", 151936, False), ("top_p", 151936, False),
+    ("top_p_peaked", 151936, False), ("ties", 151936, False), ("many_ties", 151936, False), ("penalty", 151936, False),
+    # candidates found in chunks of the vocabulary: rows that fit, rows with too many equal values (left to the kernel
+    # with a workgroup a row), a vocabulary of fewer chunks than k (the same), one of barely more
+    ("top_k", 151936, True), ("top_k_top_p", 151936, True), ("ties", 151936, True), ("many_ties", 151936, True),
+    ("penalty", 151936, True),
+    ("top_k", 5000, True), ("top_k_top_p", 43000, True), ("top_k", 2048 * 20, True)])
+def test_sampling_at_a_real_vocabulary(k, mode, vocab, chunked):
     """The draw of every row against the same steps in float64: kept set by thresholds (top-k, then top-p on what
     top-k kept), cumulative walk in vocabulary order.  The chosen token must be kept and the draw must fall into its
     interval of the cumulative sum (up to float32 rounding of the sums)."""
-    vocab, rows = 151936, 48
+    rows = 48
     gen = torch.Generator().manual_seed(11)
     # flat enough that top-p alone needs thousands of tokens (the passes over the whole vocabulary), or peaked so that
     # a thousand hold its mass (the short list)
     logits = torch.randn(rows, vocab, generator=gen) * (8.0 if mode == "top_p_peaked" else 2.5)
-    if mode == "ties":                       # the k-th largest value many times: all of its copies are kept
-        logits[:, ::97] = 6.0
+    if mode in ("ties", "many_ties"):        # the k-th largest value many times: all of its copies are kept
+        logits[:, ::(97 if mode == "ties" else 40)] = 20.0
     temp = 0.7
-    top_k = {"top_k": 20, "top_k_top_p": 50, "ties": 40, "penalty": 20}.get(mode, 0)
+    top_k = {"top_k": 20, "top_k_top_p": 50, "ties": 40, "many_ties": 40, "penalty": 20}.get(mode, 0)
     top_p = {"top_k_top_p": 0.9, "top_p": 0.8, "top_p_peaked": 0.9, "penalty": 0.95}.get(mode, 0.0)
     uniform = torch.rand(rows, generator=gen)
     dev = lambda t: t.to(DEV)
@@ -372,8 +379,21 @@ def test_sampling_at_a_real_vocabulary(k, mode):
         kw.update(penalty=dev(torch.full((rows,), 1.5)), seen_row=torch.arange(rows, dtype=torch.int32, device=DEV),
                   seen_masks=seen)
         ref[torch.arange(rows), best.long()] -= 1.5
-    out = torch.empty(rows, dtype=torch.int32, device=DEV)
-    k.sample(dev(logits), out, **kw)
+    out = torch.full((rows,), -9, dtype=torch.int32, device=DEV)
+
+    def draw(logits_dev, out_dev, **args):
+        if not chunked:
+            return k.sample(logits_dev, out_dev, **args)
+        scratch = k.sample_topk_scratch(out_dev.numel(), vocab, DEV)
+        for t in scratch.values():
+            t.fill_(-3)                                               # nothing that was not written is used
+        k.sample_topk(logits_dev, out_dev, scratch, **args)
+        if mode in ("top_k", "top_k_top_p", "penalty", "ties") and vocab >= 2048 * 50:
+            assert bool((scratch["done"][: out_dev.numel()] == 1).all())     # these rows fit: no row was left over
+        if mode == "many_ties" or vocab == 5000:
+            assert bool((scratch["done"][: out_dev.numel()] == 0).all())     # and these did not
+
+    draw(dev(logits), out, **kw)
     got = out.cpu().tolist()
     for r in range(rows):
         x = ref[r]
@@ -397,7 +417,7 @@ def test_sampling_at_a_real_vocabulary(k, mode):
     one = {n: v[5:6] for n, v in kw.items() if n not in ("seen_masks",)}
     if "seen_masks" in kw:
         one["seen_masks"] = kw["seen_masks"]
-    k.sample(dev(logits[5:6]), again, **one)
+    draw(dev(logits[5:6]), again, **one)
     assert again.item() == got[5]
 
 
