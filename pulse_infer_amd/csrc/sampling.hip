@@ -505,12 +505,13 @@ __global__ __launch_bounds__(PULSE_WAVE) void argmax_merge_kernel(const float* _
     if (threadIdx.x == 0) out[r] = best_i == 0x7fffffff ? -1 : best_i;
 }
 
-// ---- rows without top-k and top-p, in chunks -------------------------------------------------------------------
+// ---- rows in chunks ----------------------------------------------------------------------------------------------
 // A workgroup a row reads its row at the rate of one compute unit.  Without top-k and top-p nothing has to be
 // known about the row as a whole but its maximum and its mass, so the row is cut into chunks of SIMPLE_CHUNK logits
 // with a workgroup each: the chunk's maximum (with its lowest index); then, the row's maximum known, the chunk's
 // mass; then one wavefront a row finds the chunk in which u * mass falls (chunk masses summed in chunk order) and
-// walks that chunk alone.  The steps and their meaning are those of sample_kernel; sums are taken in another order.
+// walks that chunk alone (chunked_choose_kernel).  The steps and their meaning are those of sample_kernel; sums are
+// taken in another order.
 constexpr int SIMPLE_CHUNK = 2048;
 constexpr int SIMPLE_THREADS = 256;
 
@@ -569,6 +570,7 @@ __device__ __forceinline__ float simple_row_max(const float* part_max, int chunk
 
 __global__ __launch_bounds__(SIMPLE_THREADS) void simple_mass_kernel(
     const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ top_p,
     const float* __restrict__ penalty, const int* __restrict__ seen_row, const uint32_t* __restrict__ seen_masks,
     const uint32_t* __restrict__ banned, int mask_words, const float* __restrict__ part_max,
     float* __restrict__ part_mass) {
@@ -576,6 +578,8 @@ __global__ __launch_bounds__(SIMPLE_THREADS) void simple_mass_kernel(
     const int r = blockIdx.y, chunk = blockIdx.x, chunks = gridDim.x;
     const float temp = temperature ? temperature[r] : 0.f;
     if (!(temp > 0.f)) return;   // the largest logit wins: no mass is asked for
+    const float p = top_p ? top_p[r] : 0.f;
+    if ((top_k && top_k[r] > 0) || (p > 0.f && p < 1.f)) return;   // not a row that draws from the whole vocabulary
     const float best = simple_row_max(part_max + r * chunks, chunks);
     if (best == -INFINITY) return;
     const float inv_t = 1.0f / temp;
@@ -595,74 +599,6 @@ __global__ __launch_bounds__(SIMPLE_THREADS) void simple_mass_kernel(
         for (int w = 0; w < SIMPLE_THREADS / PULSE_WAVE; ++w) total += sf[w];
         part_mass[r * chunks + chunk] = total;
     }
-}
-
-__global__ __launch_bounds__(PULSE_WAVE) void simple_pick_kernel(
-    const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ temperature,
-    const float* __restrict__ uniform, const float* __restrict__ penalty, const int* __restrict__ seen_row,
-    const uint32_t* __restrict__ seen_masks, const uint32_t* __restrict__ banned, int mask_words,
-    const float* __restrict__ part_max, const int* __restrict__ part_idx, const float* __restrict__ part_mass,
-    int chunks, int* __restrict__ out) {
-    const int r = blockIdx.x, lane = threadIdx.x;
-    part_max += r * chunks;
-    part_idx += r * chunks;
-    part_mass += r * chunks;
-    // the largest logit, the lowest index among equals
-    float best = -INFINITY;
-    int best_i = 0x7fffffff;
-    for (int c = lane; c < chunks; c += PULSE_WAVE) {
-        const float v = part_max[c];
-        const int i = part_idx[c];
-        if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
-    }
-#pragma unroll
-    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(best, off, PULSE_WAVE);
-        const int oi = __shfl_xor(best_i, off, PULSE_WAVE);
-        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
-    }
-    if (best_i == 0x7fffffff) {   // everything banned or NaN
-        if (lane == 0) out[r] = -1;
-        return;
-    }
-    const float temp = temperature ? temperature[r] : 0.f;
-    if (!(temp > 0.f)) {
-        if (lane == 0) out[r] = best_i;
-        return;
-    }
-    // the chunk in which the draw falls: chunk masses in chunk order, as a walk over them
-    int last_chunk;
-    float total = 0.f;
-    for (int c = lane; c < chunks; c += PULSE_WAVE) total += part_mass[c];
-#pragma unroll
-    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) total += __shfl_xor(total, off, PULSE_WAVE);
-    const float target = uniform[r] * total;
-    // running sum over the chunks before the one that is hit, in chunk order (one lane's work: a few dozen additions)
-    float run = 0.f;
-    int who = -1;
-    last_chunk = -1;
-    for (int c = 0; c < chunks; ++c) {
-        const float m = part_mass[c];
-        if (m > 0.f) {
-            last_chunk = c;
-            if (target < run + m) { who = c; break; }
-        }
-        run += m;
-    }
-    float rest = target - run;
-    if (who < 0) {  // rounding left the target beyond the last chunk with mass: its last kept entry
-        who = last_chunk;
-        rest = INFINITY;
-    }
-    const float inv_t = 1.0f / temp;
-    const RowView row = simple_row(logits, r, row_stride, vocab, penalty, seen_row, seen_masks, banned, mask_words);
-    const int begin = who * SIMPLE_CHUNK, end = min(vocab, begin + SIMPLE_CHUNK);
-    int last;
-    const int e = wave_walk(begin, end, rest, [&](int i) {
-        const float x = row.at(i);
-        return x != -INFINITY ? expf((x - best) * inv_t) : 0.f;
-    }, last);
-    if (lane == 0) out[r] = e >= 0 ? e : (last >= 0 ? last : best_i);
 }
 
 // ---- rows with top-k, in chunks -------------------------------------------------------------------------------
@@ -686,7 +622,7 @@ __global__ __launch_bounds__(SIMPLE_THREADS) void topk_collect_kernel(
     __shared__ int s_count[WAVES];
     const int r = blockIdx.y, chunk = blockIdx.x, chunks = gridDim.x;
     const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
-    const int k = top_k[r];
+    const int k = top_k ? top_k[r] : 0;
     const float temp = temperature ? temperature[r] : 0.f;
     int* my_n = seg_n + r * chunks + chunk;
     if (!(temp > 0.f) || k <= 0 || k > chunks || chunks > 2 * PULSE_WAVE) {   // greedy rows need no candidates; the others are not for these kernels
@@ -758,17 +694,26 @@ __global__ __launch_bounds__(SIMPLE_THREADS) void topk_collect_kernel(
     if (threadIdx.x == 0) *my_n = total;   // more than TOPK_SEGMENT: the row does not fit
 }
 
-__global__ __launch_bounds__(PULSE_WAVE) void topk_finish_kernel(
-    const float* __restrict__ temperature, const int* __restrict__ top_k, const float* __restrict__ top_p,
-    const float* __restrict__ uniform, const float* __restrict__ part_max, const int* __restrict__ part_idx,
-    const int* __restrict__ seg_i, const float* __restrict__ seg_x, const int* __restrict__ seg_n, int chunks,
-    int* __restrict__ out, int* __restrict__ done) {
+// The choice of every row from what the kernels before left, a wavefront a row: the largest logit for greedy rows;
+// for rows with top-k the candidates' segments strung together in LDS and finished there; for rows that draw from the
+// whole vocabulary the chunk in which u * mass falls (chunk masses in chunk order), walked alone.  done[r] says
+// whether the row's token is chosen; the others (top-p alone, or a row that did not fit) are sample_kernel's.
+__global__ __launch_bounds__(PULSE_WAVE) void chunked_choose_kernel(
+    const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ uniform,
+    const float* __restrict__ penalty, const int* __restrict__ seen_row, const uint32_t* __restrict__ seen_masks,
+    const uint32_t* __restrict__ banned, int mask_words, const float* __restrict__ part_max,
+    const int* __restrict__ part_idx, const float* __restrict__ part_mass, const int* __restrict__ seg_i,
+    const float* __restrict__ seg_x, const int* __restrict__ seg_n, int chunks, int* __restrict__ out,
+    int* __restrict__ done) {
     __shared__ int list_i[LIST_CAP];
     __shared__ float list_x[LIST_CAP];
     const int r = blockIdx.x, lane = threadIdx.x;
     part_max += r * chunks;
     part_idx += r * chunks;
+    part_mass += r * chunks;
     seg_n += r * chunks;
+    // the largest logit, the lowest index among equals
     float best = -INFINITY;
     int best_i = 0x7fffffff;
     for (int c = lane; c < chunks; c += PULSE_WAVE) {
@@ -787,35 +732,72 @@ __global__ __launch_bounds__(PULSE_WAVE) void topk_finish_kernel(
         if (lane == 0) { out[r] = best_i == 0x7fffffff ? -1 : best_i; done[r] = 1; }
         return;
     }
-    const int k = top_k[r];
-    // the segments' places in the list: an exclusive sum over the chunks, in chunk order (two chunks a lane)
-    int n0 = lane < chunks ? seg_n[lane] : 0, n1 = lane + PULSE_WAVE < chunks ? seg_n[lane + PULSE_WAVE] : 0;
-    const bool over = n0 > TOPK_SEGMENT || n1 > TOPK_SEGMENT;
-    int pre0 = n0, pre1 = n1;
+    const int k = top_k ? top_k[r] : 0;
+    const float p = top_p ? top_p[r] : 0.f;
+    const bool use_p = p > 0.f && p < 1.f;
+    const float inv_t = 1.0f / temp;
+    if (k > 0) {
+        // the segments' places in the list: an exclusive sum over the chunks, in chunk order (two chunks a lane)
+        const int n0 = lane < chunks ? seg_n[lane] : 0, n1 = lane + PULSE_WAVE < chunks ? seg_n[lane + PULSE_WAVE] : 0;
+        const bool over = n0 > TOPK_SEGMENT || n1 > TOPK_SEGMENT;
+        int pre0 = n0, pre1 = n1;
 #pragma unroll
-    for (int off = 1; off < PULSE_WAVE; off <<= 1) {
-        const int u0 = __shfl_up(pre0, off, PULSE_WAVE), u1 = __shfl_up(pre1, off, PULSE_WAVE);
-        if (lane >= off) { pre0 += u0; pre1 += u1; }
-    }
-    const int first = __shfl(pre0, PULSE_WAVE - 1, PULSE_WAVE);      // candidates of chunks 0 .. 63
-    const int n = first + __shfl(pre1, PULSE_WAVE - 1, PULSE_WAVE);
-    if (k <= 0 || k > chunks || chunks > 2 * PULSE_WAVE || __ballot(over) != 0ull || n > LIST_CAP || n < k) {
-        if (lane == 0) done[r] = 0;   // not a row for these kernels: sample_kernel takes it
+        for (int off = 1; off < PULSE_WAVE; off <<= 1) {
+            const int u0 = __shfl_up(pre0, off, PULSE_WAVE), u1 = __shfl_up(pre1, off, PULSE_WAVE);
+            if (lane >= off) { pre0 += u0; pre1 += u1; }
+        }
+        const int first = __shfl(pre0, PULSE_WAVE - 1, PULSE_WAVE);      // candidates of chunks 0 .. 63
+        const int n = first + __shfl(pre1, PULSE_WAVE - 1, PULSE_WAVE);
+        if (k > chunks || chunks > 2 * PULSE_WAVE || __ballot(over) != 0ull || n > LIST_CAP || n < k) {
+            if (lane == 0) done[r] = 0;   // not a row for these kernels: sample_kernel takes it
+            return;
+        }
+        const int64_t seg0 = (static_cast<int64_t>(r) * chunks + lane) * TOPK_SEGMENT;
+        for (int e = 0; e < n0; ++e) { list_i[pre0 - n0 + e] = seg_i[seg0 + e]; list_x[pre0 - n0 + e] = seg_x[seg0 + e]; }
+        const int64_t seg1 = seg0 + static_cast<int64_t>(PULSE_WAVE) * TOPK_SEGMENT;
+        for (int e = 0; e < n1; ++e) { list_i[first + pre1 - n1 + e] = seg_i[seg1 + e]; list_x[first + pre1 - n1 + e] = seg_x[seg1 + e]; }
+        __syncthreads();
+        int token;
+        if (n <= 4 * PULSE_WAVE)   // the usual case: a few dozen candidates, a few a lane
+            finish_on_list<4>(list_i, list_x, n, true, k, use_p, p, 0.f, best, inv_t, uniform[r], best_i, token);
+        else
+            finish_on_list<LIST_PER_LANE>(list_i, list_x, n, true, k, use_p, p, 0.f, best, inv_t, uniform[r], best_i, token);
+        if (lane == 0) { out[r] = token; done[r] = 1; }
         return;
     }
-    const int64_t seg0 = (static_cast<int64_t>(r) * chunks + lane) * TOPK_SEGMENT;
-    for (int e = 0; e < n0; ++e) { list_i[pre0 - n0 + e] = seg_i[seg0 + e]; list_x[pre0 - n0 + e] = seg_x[seg0 + e]; }
-    const int64_t seg1 = seg0 + static_cast<int64_t>(PULSE_WAVE) * TOPK_SEGMENT;
-    for (int e = 0; e < n1; ++e) { list_i[first + pre1 - n1 + e] = seg_i[seg1 + e]; list_x[first + pre1 - n1 + e] = seg_x[seg1 + e]; }
-    __syncthreads();
-    const float p = top_p ? top_p[r] : 0.f;
-    int token;
-    const bool use_p = p > 0.f && p < 1.f;
-    if (n <= 4 * PULSE_WAVE)   // the usual case: a few dozen candidates, a few a lane
-        finish_on_list<4>(list_i, list_x, n, true, k, use_p, p, 0.f, best, 1.0f / temp, uniform[r], best_i, token);
-    else
-        finish_on_list<LIST_PER_LANE>(list_i, list_x, n, true, k, use_p, p, 0.f, best, 1.0f / temp, uniform[r], best_i, token);
-    if (lane == 0) { out[r] = token; done[r] = 1; }
+    if (use_p) {   // top-p alone: the set it keeps has no bound that these kernels could use
+        if (lane == 0) done[r] = 0;
+        return;
+    }
+    // a draw from the whole vocabulary: the chunk in which it falls, chunk masses in chunk order
+    float total = 0.f;
+    for (int c = lane; c < chunks; c += PULSE_WAVE) total += part_mass[c];
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) total += __shfl_xor(total, off, PULSE_WAVE);
+    const float target = uniform[r] * total;
+    float run = 0.f;
+    int who = -1, last_chunk = -1;
+    for (int c = 0; c < chunks; ++c) {   // (every lane the same few dozen additions)
+        const float m = part_mass[c];
+        if (m > 0.f) {
+            last_chunk = c;
+            if (target < run + m) { who = c; break; }
+        }
+        run += m;
+    }
+    float rest = target - run;
+    if (who < 0) {  // rounding left the target beyond the last chunk with mass: its last kept entry
+        who = last_chunk;
+        rest = INFINITY;
+    }
+    const RowView row = simple_row(logits, r, row_stride, vocab, penalty, seen_row, seen_masks, banned, mask_words);
+    const int begin = who * SIMPLE_CHUNK, end = min(vocab, begin + SIMPLE_CHUNK);
+    int last;
+    const int e = wave_walk(begin, end, rest, [&](int i) {
+        const float x = row.at(i);
+        return x != -INFINITY ? expf((x - best) * inv_t) : 0.f;
+    }, last);
+    if (lane == 0) { out[r] = e >= 0 ? e : (last >= 0 ? last : best_i); done[r] = 1; }
 }
 
 }  // namespace
@@ -909,70 +891,56 @@ extern "C" int pulse_sample(const float* logits, int rows, int vocab, int64_t ro
     return 0;
 }
 
-// The same for rows none of which asks for top-k or top-p (greedy rows and rows that sample from the whole
-// vocabulary at their temperature), in chunks of the vocabulary with a workgroup each.  part_max, part_idx and
-// part_mass: scratch of rows * pulse_sample_simple_chunks(vocab) entries each.
-extern "C" int pulse_sample_simple_chunks(int vocab) { return (vocab + SIMPLE_CHUNK - 1) / SIMPLE_CHUNK; }
+// The same in chunks of the vocabulary with a workgroup each, which reads a row many times faster than the
+// workgroup a row of pulse_sample does.  Greedy rows, rows that draw from the whole vocabulary at their temperature
+// and rows with top-k (and top-p on what it keeps) whose k is at most the number of chunks are chosen by these
+// kernels; rows with top-p alone, and rows that do not fit (many equal values around the k-th largest), by the kernel
+// of pulse_sample behind them, which skips the rows that are done.  What a row's choice is does not depend on the
+// other rows.  Scratch, with chunks = pulse_sample_chunks(vocab): part_max, part_mass (float32), part_idx, seg_n
+// (int32) of rows * chunks entries; seg_i (int32), seg_x (float32) of rows * chunks * pulse_sample_segment()
+// entries; done (int32) of rows entries.
+extern "C" int pulse_sample_chunks(int vocab) { return (vocab + SIMPLE_CHUNK - 1) / SIMPLE_CHUNK; }
+extern "C" int pulse_sample_segment() { return TOPK_SEGMENT; }
 
-extern "C" int pulse_sample_simple(const float* logits, int rows, int vocab, int64_t row_stride, const float* temperature,
-                                   const float* uniform, const float* penalty, const int* seen_row,
-                                   const uint32_t* seen_masks, const uint32_t* banned, int mask_words, float* part_max,
-                                   int* part_idx, float* part_mass, int* out, hipStream_t stream) {
-    PULSE_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "sample_simple: bad sizes rows=%d V=%d", rows, vocab);
-    PULSE_REQUIRE(rows < 65536, "sample_simple: at most 65535 rows");
-    PULSE_REQUIRE(logits && out && part_max && part_idx && part_mass, "sample_simple: null pointer");
-    PULSE_REQUIRE(!temperature || uniform, "sample_simple: temperature sampling needs uniform numbers");
-    PULSE_REQUIRE((!seen_masks && !banned) || mask_words * 32 >= vocab, "sample_simple: masks cover %d tokens, "
+extern "C" int pulse_sample_chunked(const float* logits, int rows, int vocab, int64_t row_stride, const float* temperature,
+                                    const int* top_k, const float* top_p, const float* uniform, const float* penalty,
+                                    const int* seen_row, const uint32_t* seen_masks, const uint32_t* banned,
+                                    int mask_words, float* part_max, int* part_idx, float* part_mass, int* seg_i,
+                                    float* seg_x, int* seg_n, int* done, int* out, hipStream_t stream) {
+    PULSE_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "sample_chunked: bad sizes rows=%d V=%d", rows, vocab);
+    PULSE_REQUIRE(rows < 65536, "sample_chunked: at most 65535 rows");
+    PULSE_REQUIRE(logits && out && part_max && part_idx && part_mass && seg_i && seg_x && seg_n && done,
+                  "sample_chunked: null pointer");
+    PULSE_REQUIRE(!temperature || uniform, "sample_chunked: temperature sampling needs uniform numbers");
+    PULSE_REQUIRE((!seen_masks && !banned) || mask_words * 32 >= vocab, "sample_chunked: masks cover %d tokens, "
                   "vocabulary has %d", mask_words * 32, vocab);
     if (rows == 0) return 0;
-    const int chunks = pulse_sample_simple_chunks(vocab);
+    const int chunks = pulse_sample_chunks(vocab);
     hipLaunchKernelGGL(simple_max_kernel, dim3(chunks, rows), dim3(SIMPLE_THREADS), 0, stream, logits, vocab, row_stride,
                        penalty, seen_row, seen_masks, banned, mask_words, part_max, part_idx);
-    PULSE_LAUNCH_CHECK("sample_simple (maxima)");
+    PULSE_LAUNCH_CHECK("sample_chunked (maxima)");
     if (temperature) {
         hipLaunchKernelGGL(simple_mass_kernel, dim3(chunks, rows), dim3(SIMPLE_THREADS), 0, stream, logits, vocab,
-                           row_stride, temperature, penalty, seen_row, seen_masks, banned, mask_words, part_max, part_mass);
-        PULSE_LAUNCH_CHECK("sample_simple (masses)");
+                           row_stride, temperature, top_k, top_p, penalty, seen_row, seen_masks, banned, mask_words,
+                           part_max, part_mass);
+        PULSE_LAUNCH_CHECK("sample_chunked (masses)");
+        if (top_k) {
+            hipLaunchKernelGGL(topk_collect_kernel, dim3(chunks, rows), dim3(SIMPLE_THREADS), 0, stream, logits, vocab,
+                               row_stride, temperature, top_k, penalty, seen_row, seen_masks, banned, mask_words, part_max,
+                               seg_i, seg_x, seg_n);
+            PULSE_LAUNCH_CHECK("sample_chunked (candidates)");
+        }
     }
-    hipLaunchKernelGGL(simple_pick_kernel, dim3(rows), dim3(PULSE_WAVE), 0, stream, logits, vocab, row_stride, temperature,
-                       uniform, penalty, seen_row, seen_masks, banned, mask_words, part_max, part_idx, part_mass, chunks,
-                       out);
-    PULSE_LAUNCH_CHECK("sample_simple (pick)");
-    return 0;
-}
-
-// The same for steps with top-k (every row of which is tried in chunks first: see topk_collect_kernel; rows without
-// top-k, with a k above the number of chunks or with too many equal values go through the kernel of pulse_sample
-// afterwards).  part_max, part_idx, seg_n: rows * chunks entries; seg_i, seg_x: rows * chunks *
-// pulse_sample_topk_segment() entries; done: rows entries (chunks = pulse_sample_simple_chunks(vocab)).
-extern "C" int pulse_sample_topk_segment() { return TOPK_SEGMENT; }
-
-extern "C" int pulse_sample_topk(const float* logits, int rows, int vocab, int64_t row_stride, const float* temperature,
-                                 const int* top_k, const float* top_p, const float* uniform, const float* penalty,
-                                 const int* seen_row, const uint32_t* seen_masks, const uint32_t* banned, int mask_words,
-                                 float* part_max, int* part_idx, int* seg_i, float* seg_x, int* seg_n, int* done, int* out,
-                                 hipStream_t stream) {
-    PULSE_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "sample_topk: bad sizes rows=%d V=%d", rows, vocab);
-    PULSE_REQUIRE(rows < 65536, "sample_topk: at most 65535 rows");
-    PULSE_REQUIRE(logits && out && top_k && temperature && uniform && part_max && part_idx && seg_i && seg_x && seg_n && done,
-                  "sample_topk: null pointer");
-    PULSE_REQUIRE((!seen_masks && !banned) || mask_words * 32 >= vocab, "sample_topk: masks cover %d tokens, "
-                  "vocabulary has %d", mask_words * 32, vocab);
-    if (rows == 0) return 0;
-    const int chunks = pulse_sample_simple_chunks(vocab);
-    hipLaunchKernelGGL(simple_max_kernel, dim3(chunks, rows), dim3(SIMPLE_THREADS), 0, stream, logits, vocab, row_stride,
-                       penalty, seen_row, seen_masks, banned, mask_words, part_max, part_idx);
-    PULSE_LAUNCH_CHECK("sample_topk (maxima)");
-    hipLaunchKernelGGL(topk_collect_kernel, dim3(chunks, rows), dim3(SIMPLE_THREADS), 0, stream, logits, vocab, row_stride,
-                       temperature, top_k, penalty, seen_row, seen_masks, banned, mask_words, part_max, seg_i, seg_x, seg_n);
-    PULSE_LAUNCH_CHECK("sample_topk (candidates)");
-    hipLaunchKernelGGL(topk_finish_kernel, dim3(rows), dim3(PULSE_WAVE), 0, stream, temperature, top_k, top_p, uniform,
-                       part_max, part_idx, seg_i, seg_x, seg_n, chunks, out, done);
-    PULSE_LAUNCH_CHECK("sample_topk (choice)");
-    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, row_stride,
-                       temperature, top_k, top_p, uniform, penalty, seen_row, seen_masks, banned, mask_words, out,
-                       static_cast<const int*>(done));
-    PULSE_LAUNCH_CHECK("sample_topk (the rest)");
+    hipLaunchKernelGGL(chunked_choose_kernel, dim3(rows), dim3(PULSE_WAVE), 0, stream, logits, vocab, row_stride,
+                       temperature, top_k, top_p, uniform, penalty, seen_row, seen_masks, banned, mask_words, part_max,
+                       part_idx, part_mass, seg_i, seg_x, seg_n, chunks, out, done);
+    PULSE_LAUNCH_CHECK("sample_chunked (choice)");
+    if (temperature && (top_k || top_p)) {   // (without them every row is done)
+        hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, vocab, row_stride,
+                           temperature, top_k, top_p, uniform, penalty, seen_row, seen_masks, banned, mask_words, out,
+                           static_cast<const int*>(done));
+        PULSE_LAUNCH_CHECK("sample_chunked (the rest)");
+    }
     return 0;
 }
 

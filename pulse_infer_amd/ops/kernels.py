@@ -385,98 +385,65 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.
          _ptr(banned), _i32(words), _ptr(out), _stream())
 
 
-SAMPLE_SIMPLE_CHUNK = 2048   # as SIMPLE_CHUNK of sampling.hip
+SAMPLE_CHUNK = 2048      # as SIMPLE_CHUNK of sampling.hip
+SAMPLE_SEGMENT = 32      # as TOPK_SEGMENT of sampling.hip
 
 
-def sample_simple_chunks(vocab: int) -> int:
-    """Chunks of the vocabulary that ``sample_simple`` cuts a row into (its scratch holds rows * chunks entries)."""
-    return (vocab + SAMPLE_SIMPLE_CHUNK - 1) // SAMPLE_SIMPLE_CHUNK
+def sample_chunks(vocab: int) -> int:
+    """Chunks of the vocabulary that ``sample_chunked`` cuts a row into."""
+    return (vocab + SAMPLE_CHUNK - 1) // SAMPLE_CHUNK
 
 
-def sample_simple(logits: torch.Tensor, out: torch.Tensor, part_max: torch.Tensor, part_idx: torch.Tensor,
-                  part_mass: torch.Tensor, temperature: Optional[torch.Tensor] = None,
-                  uniform: Optional[torch.Tensor] = None, penalty: Optional[torch.Tensor] = None,
-                  seen_row: Optional[torch.Tensor] = None, seen_masks: Optional[torch.Tensor] = None,
-                  banned: Optional[torch.Tensor] = None) -> None:
-    """``sample`` for rows none of which asks for top-k or top-p: the largest logit where the temperature is absent
-    or <= 0, else a draw from the whole vocabulary at the row's temperature; in chunks of the vocabulary with a
-    workgroup each instead of a workgroup a row."""
-    _gpu("sample_simple", logits, out, part_max, part_idx, part_mass, temperature, uniform, penalty, seen_row, seen_masks,
-         banned)
+def sample_chunked_scratch(rows: int, vocab: int, device) -> dict:
+    """Scratch tensors of the sizes ``sample_chunked`` asks for."""
+    per_row = sample_chunks(vocab)
+    f32 = lambda n: torch.empty(n, dtype=torch.float32, device=device)
+    i32 = lambda n: torch.empty(n, dtype=torch.int32, device=device)
+    return {"part_max": f32(rows * per_row), "part_idx": i32(rows * per_row), "part_mass": f32(rows * per_row),
+            "seg_n": i32(rows * per_row), "done": i32(rows), "seg_i": i32(rows * per_row * SAMPLE_SEGMENT),
+            "seg_x": f32(rows * per_row * SAMPLE_SEGMENT)}
+
+
+def sample_chunked(logits: torch.Tensor, out: torch.Tensor, scratch: dict, temperature: Optional[torch.Tensor] = None,
+                   top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
+                   uniform: Optional[torch.Tensor] = None, penalty: Optional[torch.Tensor] = None,
+                   seen_row: Optional[torch.Tensor] = None, seen_masks: Optional[torch.Tensor] = None,
+                   banned: Optional[torch.Tensor] = None) -> None:
+    """``sample`` in chunks of the vocabulary with a workgroup each instead of a workgroup a row: greedy rows, rows
+    that draw from the whole vocabulary and rows with top-k (k at most the number of chunks) are chosen from what the
+    chunks leave; rows with top-p alone, and what does not fit, go through the kernel of ``sample`` behind them.
+    Which way a row goes depends on the row alone.  ``scratch`` as ``sample_chunked_scratch`` makes it."""
+    names = ("part_max", "part_idx", "part_mass", "seg_i", "seg_x", "seg_n", "done")
+    _gpu("sample_chunked", logits, out, temperature, top_k, top_p, uniform, penalty, seen_row, seen_masks, banned,
+         *(scratch[n] for n in names))
     _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1,
-          "sample_simple: logits must be float32 [R, V]")
+          "sample_chunked: logits must be float32 [R, V]")
     rows, vocab = logits.shape
-    _int_vec("sample_simple: out", out, rows)
-    for name, t, dt in (("temperature", temperature, torch.float32), ("uniform", uniform, torch.float32),
-                        ("penalty", penalty, torch.float32), ("seen_row", seen_row, torch.int32)):
-        if t is not None:
-            _need(t.dtype == dt and t.is_contiguous() and t.numel() >= rows, f"sample_simple: {name} must be {dt}[{rows}]")
-    need = rows * sample_simple_chunks(vocab)
-    for name, t, dt in (("part_max", part_max, torch.float32), ("part_idx", part_idx, torch.int32),
-                        ("part_mass", part_mass, torch.float32)):
-        _need(t.dtype == dt and t.is_contiguous() and t.numel() >= need, f"sample_simple: {name} must hold {need} {dt}")
-    words = 0
-    for name, t in (("seen_masks", seen_masks), ("banned", banned)):
-        if t is not None:
-            _need(t.dtype == torch.int32 and t.is_contiguous(), f"sample_simple: {name} must be contiguous int32 words")
-            w = t.shape[-1]
-            _need(words in (0, w), "sample_simple: masks differ in width")
-            words = w
-    call("pulse_sample_simple", _ptr(logits), _i32(rows), _i32(vocab), _i64(logits.stride(0) if rows > 1 else vocab),
-         _ptr(temperature), _ptr(uniform), _ptr(penalty), _ptr(seen_row), _ptr(seen_masks), _ptr(banned), _i32(words),
-         _ptr(part_max), _ptr(part_idx), _ptr(part_mass), _ptr(out), _stream())
-
-
-SAMPLE_TOPK_SEGMENT = 32     # as TOPK_SEGMENT of sampling.hip
-
-
-def sample_topk(logits: torch.Tensor, out: torch.Tensor, scratch: dict, temperature: torch.Tensor, top_k: torch.Tensor,
-                uniform: torch.Tensor, top_p: Optional[torch.Tensor] = None, penalty: Optional[torch.Tensor] = None,
-                seen_row: Optional[torch.Tensor] = None, seen_masks: Optional[torch.Tensor] = None,
-                banned: Optional[torch.Tensor] = None) -> None:
-    """``sample`` for steps with top-k: the rows' candidates are found in chunks of the vocabulary, a workgroup each
-    (for rows whose k is at most the number of chunks); what does not fit goes through the kernel of ``sample`` behind
-    them.  ``scratch`` holds part_max (float32), part_idx, seg_n (int32) of rows * chunks entries, seg_i (int32) and
-    seg_x (float32) of rows * chunks * SAMPLE_TOPK_SEGMENT entries and done (int32) of rows entries."""
-    parts = [scratch[n] for n in ("part_max", "part_idx", "seg_i", "seg_x", "seg_n", "done")]
-    _gpu("sample_topk", logits, out, temperature, top_k, top_p, uniform, penalty, seen_row, seen_masks, banned, *parts)
-    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1,
-          "sample_topk: logits must be float32 [R, V]")
-    rows, vocab = logits.shape
-    _int_vec("sample_topk: out", out, rows)
+    _int_vec("sample_chunked: out", out, rows)
     for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
                         ("top_p", top_p, torch.float32), ("uniform", uniform, torch.float32),
                         ("penalty", penalty, torch.float32), ("seen_row", seen_row, torch.int32)):
         if t is not None:
-            _need(t.dtype == dt and t.is_contiguous() and t.numel() >= rows, f"sample_topk: {name} must be {dt}[{rows}]")
-    per_row = sample_simple_chunks(vocab)
+            _need(t.dtype == dt and t.is_contiguous() and t.numel() >= rows, f"sample_chunked: {name} must be {dt}[{rows}]")
+    per_row = sample_chunks(vocab)
     for name, dt, need in (("part_max", torch.float32, rows * per_row), ("part_idx", torch.int32, rows * per_row),
-                           ("seg_n", torch.int32, rows * per_row), ("done", torch.int32, rows),
-                           ("seg_i", torch.int32, rows * per_row * SAMPLE_TOPK_SEGMENT),
-                           ("seg_x", torch.float32, rows * per_row * SAMPLE_TOPK_SEGMENT)):
+                           ("part_mass", torch.float32, rows * per_row), ("seg_n", torch.int32, rows * per_row),
+                           ("done", torch.int32, rows), ("seg_i", torch.int32, rows * per_row * SAMPLE_SEGMENT),
+                           ("seg_x", torch.float32, rows * per_row * SAMPLE_SEGMENT)):
         t = scratch[name]
-        _need(t.dtype == dt and t.is_contiguous() and t.numel() >= need, f"sample_topk: {name} must hold {need} {dt}")
+        _need(t.dtype == dt and t.is_contiguous() and t.numel() >= need, f"sample_chunked: {name} must hold {need} {dt}")
     words = 0
     for name, t in (("seen_masks", seen_masks), ("banned", banned)):
         if t is not None:
-            _need(t.dtype == torch.int32 and t.is_contiguous(), f"sample_topk: {name} must be contiguous int32 words")
+            _need(t.dtype == torch.int32 and t.is_contiguous(), f"sample_chunked: {name} must be contiguous int32 words")
             w = t.shape[-1]
-            _need(words in (0, w), "sample_topk: masks differ in width")
+            _need(words in (0, w), "sample_chunked: masks differ in width")
             words = w
-    call("pulse_sample_topk", _ptr(logits), _i32(rows), _i32(vocab), _i64(logits.stride(0) if rows > 1 else vocab),
+    call("pulse_sample_chunked", _ptr(logits), _i32(rows), _i32(vocab), _i64(logits.stride(0) if rows > 1 else vocab),
          _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(uniform), _ptr(penalty), _ptr(seen_row), _ptr(seen_masks),
-         _ptr(banned), _i32(words), _ptr(scratch["part_max"]), _ptr(scratch["part_idx"]), _ptr(scratch["seg_i"]),
-         _ptr(scratch["seg_x"]), _ptr(scratch["seg_n"]), _ptr(scratch["done"]), _ptr(out), _stream())
-
-
-def sample_topk_scratch(rows: int, vocab: int, device) -> dict:
-    """Scratch tensors of the sizes ``sample_topk`` asks for."""
-    per_row = sample_simple_chunks(vocab)
-    f32 = lambda n: torch.empty(n, dtype=torch.float32, device=device)
-    i32 = lambda n: torch.empty(n, dtype=torch.int32, device=device)
-    return {"part_max": f32(rows * per_row), "part_idx": i32(rows * per_row), "seg_n": i32(rows * per_row),
-            "done": i32(rows), "seg_i": i32(rows * per_row * SAMPLE_TOPK_SEGMENT),
-            "seg_x": f32(rows * per_row * SAMPLE_TOPK_SEGMENT)}
+         _ptr(banned), _i32(words), _ptr(scratch["part_max"]), _ptr(scratch["part_idx"]), _ptr(scratch["part_mass"]),
+         _ptr(scratch["seg_i"]), _ptr(scratch["seg_x"]), _ptr(scratch["seg_n"]), _ptr(scratch["done"]), _ptr(out),
+         _stream())
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor, part_val: torch.Tensor, part_idx: torch.Tensor) -> None:

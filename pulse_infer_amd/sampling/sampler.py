@@ -27,10 +27,7 @@ class Sampler:
         self.banned: Optional[torch.Tensor] = None
         self._part_val: Optional[torch.Tensor] = None
         self._part_idx: Optional[torch.Tensor] = None
-        self._part_mass: Optional[torch.Tensor] = None   # scratch of the sampling in chunks (with _part_max, _part_at)
-        self._part_max: Optional[torch.Tensor] = None
-        self._part_at: Optional[torch.Tensor] = None
-        self._topk: Optional[dict] = None                # scratch of the top-k sampling in chunks
+        self._chunked: Optional[dict] = None             # scratch of the sampling in chunks
         if banned_tokens:
             host = torch.zeros(self.words, dtype=torch.int64)
             for tok in banned_tokens:
@@ -87,24 +84,14 @@ class Sampler:
         penalty = dev[4].view(torch.float32) if use_penalty else None
         seen_row = dev[5] if use_penalty else None
         seen = self.seen if penalty is not None else None
-        if all(p.top_k == 0 and not 0.0 < p.top_p < 1.0 for p in params):
-            # nothing but temperatures: the rows go through the kernels that cut a row into chunks
-            need = rows * kernels.sample_simple_chunks(logits.shape[1])
-            if self._part_mass is None or self._part_mass.numel() < need:
-                self._part_mass = torch.empty(need, dtype=torch.float32, device=self.device)
-                self._part_max = torch.empty(need, dtype=torch.float32, device=self.device)
-                self._part_at = torch.empty(need, dtype=torch.int32, device=self.device)
-            kernels.sample_simple(logits, out, self._part_max, self._part_at, self._part_mass, temperature=temperature,
-                                  uniform=uniform, penalty=penalty, seen_row=seen_row, seen_masks=seen,
-                                  banned=self.banned)
-            return out.tolist()
-        if any(p.top_k > 0 for p in params):
-            # top-k somewhere: candidates are found in chunks of the vocabulary first
-            if self._topk is None or self._topk["done"].numel() < rows:
-                self._topk = kernels.sample_topk_scratch(rows, logits.shape[1], self.device)
-            kernels.sample_topk(logits, out, self._topk, temperature=temperature, top_k=top_k, uniform=uniform,
-                                top_p=top_p, penalty=penalty, seen_row=seen_row, seen_masks=seen, banned=self.banned)
-            return out.tolist()
-        kernels.sample(logits, out, temperature=temperature, top_k=top_k, top_p=top_p, uniform=uniform,
-                       penalty=penalty, seen_row=seen_row, seen_masks=seen, banned=self.banned)
+        # in chunks of the vocabulary; which way a row goes there depends on its own options alone, so a seeded
+        # request draws the same tokens whatever else is in the batch.  An option that no row uses is left out
+        # (a kernel less), which changes no row's choice.
+        if self._chunked is None or self._chunked["done"].numel() < rows:
+            self._chunked = kernels.sample_chunked_scratch(rows, logits.shape[1], self.device)
+        kernels.sample_chunked(logits, out, self._chunked, temperature=temperature,
+                               top_k=top_k if any(p.top_k > 0 for p in params) else None,
+                               top_p=top_p if any(0.0 < p.top_p < 1.0 for p in params) else None,
+                               uniform=uniform, penalty=penalty, seen_row=seen_row, seen_masks=seen,
+                               banned=self.banned)
         return out.tolist()

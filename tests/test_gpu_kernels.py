@@ -347,7 +347,7 @@ def test_top_k_top_p_penalty_and_banned(k):
     # candidates found in chunks of the vocabulary: rows that fit, rows with too many equal values (left to the kernel
     # with a workgroup a row), a vocabulary of fewer chunks than k (the same), one of barely more
     ("top_k", 151936, True), ("top_k_top_p", 151936, True), ("ties", 151936, True), ("many_ties", 151936, True),
-    ("penalty", 151936, True),
+    ("penalty", 151936, True), ("temperature", 151936, True), ("top_p", 151936, True),
     ("top_k", 5000, True), ("top_k_top_p", 43000, True), ("top_k", 2048 * 20, True)])
 def test_sampling_at_a_real_vocabulary(k, mode, vocab, chunked):
     """The draw of every row against the same steps in float64: kept set by thresholds (top-k, then top-p on what
@@ -384,13 +384,11 @@ def test_sampling_at_a_real_vocabulary(k, mode, vocab, chunked):
     def draw(logits_dev, out_dev, **args):
         if not chunked:
             return k.sample(logits_dev, out_dev, **args)
-        scratch = k.sample_topk_scratch(out_dev.numel(), vocab, DEV)
-        for t in scratch.values():
-            t.fill_(-3)                                               # nothing that was not written is used
-        k.sample_topk(logits_dev, out_dev, scratch, **args)
-        if mode in ("top_k", "top_k_top_p", "penalty", "ties") and vocab >= 2048 * 50:
+        scratch = _chunked_scratch(k, out_dev.numel(), vocab)
+        k.sample_chunked(logits_dev, out_dev, scratch, **args)
+        if mode in ("top_k", "top_k_top_p", "penalty", "ties", "temperature") and vocab >= 2048 * 50:
             assert bool((scratch["done"][: out_dev.numel()] == 1).all())     # these rows fit: no row was left over
-        if mode == "many_ties" or vocab == 5000:
+        if mode in ("many_ties", "top_p") or vocab == 5000:
             assert bool((scratch["done"][: out_dev.numel()] == 0).all())     # and these did not
 
     draw(dev(logits), out, **kw)
@@ -421,10 +419,11 @@ def test_sampling_at_a_real_vocabulary(k, mode, vocab, chunked):
     assert again.item() == got[5]
 
 
-def _simple_scratch(k, rows, vocab):
-    n = rows * k.sample_simple_chunks(vocab)
-    return (torch.full((n,), float("nan"), device=DEV), torch.full((n,), -7, dtype=torch.int32, device=DEV),
-            torch.full((n,), float("nan"), device=DEV))
+def _chunked_scratch(k, rows, vocab):
+    scratch = k.sample_chunked_scratch(rows, vocab, DEV)
+    for t in scratch.values():                             # nothing that was not written is used
+        t.fill_(float("nan") if t.dtype == torch.float32 else -3)
+    return scratch
 
 
 @pytest.mark.parametrize("vocab", [151936, 2048, 2049, 700])
@@ -461,7 +460,7 @@ def test_sampling_in_chunks(k, vocab):
     kw = dict(temperature=dev(temp), uniform=dev(uniform), penalty=dev(penalty),
               seen_row=torch.arange(rows, dtype=torch.int32, device=DEV), seen_masks=seen, banned=dev(banned))
     out = torch.full((rows,), -5, dtype=torch.int32, device=DEV)
-    k.sample_simple(dev(logits), out, *_simple_scratch(k, rows, vocab), **kw)
+    k.sample_chunked(dev(logits), out, _chunked_scratch(k, rows, vocab), **kw)
     got = out.cpu().tolist()
     for r in range(rows):
         x = ref[r]
@@ -483,13 +482,50 @@ def test_sampling_in_chunks(k, vocab):
     again = torch.empty(1, dtype=torch.int32, device=DEV)
     one = {n: v[12:13] for n, v in kw.items() if n not in ("seen_masks", "banned")}
     one["seen_row"] = torch.tensor([12], dtype=torch.int32, device=DEV)
-    k.sample_simple(dev(logits[12:13]), again, *_simple_scratch(k, 1, vocab), seen_masks=seen, banned=dev(banned), **one)
+    k.sample_chunked(dev(logits[12:13]), again, _chunked_scratch(k, 1, vocab), seen_masks=seen, banned=dev(banned), **one)
     assert again.item() == got[12]
     # nothing left of a row: -1
     everything = torch.full((words,), -1, dtype=torch.int32, device=DEV)
-    k.sample_simple(dev(logits[:2]), out[:2], *_simple_scratch(k, 2, vocab), temperature=dev(temp[4:6]),
-                    uniform=dev(uniform[:2]), banned=everything)
+    k.sample_chunked(dev(logits[:2]), out[:2], _chunked_scratch(k, 2, vocab), temperature=dev(temp[4:6]),
+                     uniform=dev(uniform[:2]), banned=everything)
     assert out[:2].tolist() == [-1, -1]
+
+
+@pytest.mark.parametrize("vocab", [151936, 43000])
+def test_rows_of_every_kind_in_one_step_draw_what_they_draw_alone(k, vocab):
+    """Greedy rows, rows at a temperature, with top-k, with top-k and top-p, with top-p alone and rows whose
+    candidates do not fit, in one call: every row draws the token that it draws in a call of its own, with and
+    without the options that it does not use (a seeded request does not depend on what it is batched with)."""
+    rows = 24
+    gen = torch.Generator().manual_seed(5)
+    logits = torch.randn(rows, vocab, generator=gen) * 2.5
+    logits[20:, ::40] = 20.0                                # rows 20 to 23: too many equal values for a segment
+    temp = torch.full((rows,), 0.8)
+    temp[0:4] = 0.0
+    top_k = torch.zeros(rows, dtype=torch.int32)
+    top_k[8:16] = 20
+    top_k[20:] = 40
+    top_p = torch.zeros(rows)
+    top_p[12:20] = 0.9
+    uniform = torch.rand(rows, generator=gen)
+    dev = lambda t: t.to(DEV)
+    out = torch.full((rows,), -5, dtype=torch.int32, device=DEV)
+    scratch = _chunked_scratch(k, rows, vocab)
+    k.sample_chunked(dev(logits), out, scratch, temperature=dev(temp), top_k=dev(top_k), top_p=dev(top_p),
+                     uniform=dev(uniform))
+    got = out.cpu().tolist()
+    assert scratch["done"].cpu().tolist() == [1] * 16 + [0] * 8
+    for r in range(rows):
+        alone = torch.empty(1, dtype=torch.int32, device=DEV)
+        kw = dict(temperature=dev(temp[r:r + 1]), uniform=dev(uniform[r:r + 1]))
+        if int(top_k[r]):
+            kw["top_k"] = dev(top_k[r:r + 1])
+        if float(top_p[r]):
+            kw["top_p"] = dev(top_p[r:r + 1])
+        k.sample_chunked(dev(logits[r:r + 1]), alone, _chunked_scratch(k, 1, vocab), **kw)
+        assert alone.item() == got[r], r
+        if float(temp[r]) <= 0:
+            assert got[r] == int(torch.argmax(logits[r]))
 
 
 def test_temperature_sampling_in_chunks_follows_the_softmax(k):
@@ -500,7 +536,7 @@ def test_temperature_sampling_in_chunks_follows_the_softmax(k):
     temperature = torch.full((rows,), 0.8, device=DEV)
     uniform = torch.rand(rows, generator=torch.Generator().manual_seed(1)).to(DEV)
     out = torch.empty(rows, dtype=torch.int32, device=DEV)
-    k.sample_simple(logits, out, *_simple_scratch(k, rows, vocab), temperature=temperature, uniform=uniform)
+    k.sample_chunked(logits, out, _chunked_scratch(k, rows, vocab), temperature=temperature, uniform=uniform)
     counts = torch.bincount(out.cpu().long(), minlength=vocab).double() / rows
     want = torch.softmax(base.double() / 0.8, dim=0)
     assert torch.allclose(counts, want, atol=0.03)
