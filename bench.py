@@ -158,7 +158,8 @@ def serving(args, cfg, model, full_layers: int) -> int:
                    "output_tokens": args.output_tokens, "chunk": args.chunk, "token_budget": engine.scheduler.max_num_batched_tokens,
                    "temperature": args.temperature,
                    "prompt_tokens": sum(lengths), "preemptions": stats.num_preemptions},
-        "seconds": round(seconds, 3), "tokens_computed": stats.tokens_computed}))
+        "seconds": round(seconds, 3), "tokens_computed": stats.tokens_computed,
+        "steps_recorded": engine.runner.graph_records, "steps_replayed": engine.runner.graph_replays}))
     return 0
 
 

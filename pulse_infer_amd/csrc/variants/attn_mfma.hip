@@ -73,6 +73,7 @@ struct MfmaArgs {
     const int* block_table;
     const int* items;  // [n_items, 4]: first token row, number of tokens, row of the block table, 0
     int bt_width;
+    int n_items;
     int nq, nkv, group;
     int gp;           // columns per token: the group size rounded up to a power of two, at most 16
     int head_chunks;  // ceil(group / 16)
@@ -86,6 +87,12 @@ struct MfmaArgs {
     // up to n_splits * split_size; with this the kernel of decoded tokens cuts the keys that are there into n_splits
     // even splits instead (see live_split_size), so that no split stands empty while another walks its full length.
     const int* live_context;
+    // Or null: the step's plan (made by attn_plan_kernel from the contexts as they are now), which takes the place
+    // of the even cut above.  plan[0] (item, split) pairs in the order the workgroups take them, pair k as
+    // plan[1 + k] = item * n_splits + split (workgroups beyond the count leave at once); behind the n_items *
+    // n_splits places for pairs, every item's own split size: its keys are cut into as many splits as its length
+    // asks for, an item of one split is finished by its workgroup, and no workgroup stands empty.
+    const int* plan;
     // Only for the kernel that prepares q and the step's own key itself (decoded tokens): then q points at the raw
     // projection output [T, (nq + 2 nkv) D] (q heads, k heads, v heads), as the kernel of qk_rope_kv.hip takes it.
     const bf16_t* q_w;     // per-head RMSNorm weights [D], or null for no norm
@@ -226,8 +233,15 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     // as many compute units as it has workgroups.
     const int heads = a.nkv * a.head_chunks;
     const int hy = blockIdx.x % heads;
-    const int split = (blockIdx.x / heads) % a.n_splits;
-    const int item = blockIdx.x / heads / a.n_splits;
+    int split = (blockIdx.x / heads) % a.n_splits;
+    int item = blockIdx.x / heads / a.n_splits;
+    if (a.plan) {
+        const int k = blockIdx.x / heads;
+        if (k >= a.plan[0]) return;
+        const int s = a.plan[1 + k];
+        item = s / a.n_splits;
+        split = s % a.n_splits;
+    }
     const int g = hy / a.head_chunks;       // kv head
     const int chunk = hy % a.head_chunks;   // which 16 heads of the group
     const int tid = threadIdx.x;
@@ -243,7 +257,8 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     const int ntok = a.items[4 * item + 1];
     const int* bt = a.block_table + static_cast<int64_t>(a.items[4 * item + 2]) * a.bt_width;
     const int hi = a.positions[row0 + ntok - 1];    // last key any column of the item may see
-    const int split_size = (a.live_context && a.n_splits > 1)
+    const int split_size = a.plan ? a.plan[1 + a.n_items * a.n_splits + item]
+                           : (a.live_context && a.n_splits > 1)
                                ? live_split_size(uniform(*a.live_context), a.n_splits, a.split_size) : a.split_size;
     const int split_begin = split * split_size;
     int split_end = 0;                              // set once hi has arrived
@@ -573,7 +588,7 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     }
     const int64_t row = row0 + tc2;
     const int head = g * a.group + hc2;
-    if (a.n_splits == 1) {
+    if (a.n_splits == 1 || (a.plan && hi < split_size)) {   // the only split of its item: nothing to merge
         const float inv = ll > 0.f ? 1.0f / ll : 0.f;
         bf16_t* dst = a.out + row * a.o_stride + static_cast<int64_t>(head) * D;
         for (int ch = dd; ch < D; ch += 16) {
@@ -1294,16 +1309,19 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
                                                                          const int* __restrict__ items, int per,
                                                                          bf16_t* __restrict__ out, int64_t o_stride, int nq,
                                                                          int n_splits, int static_split_size, int hpw_log2,
-                                                                         const int* __restrict__ live_context) {
-    const int split_size = live_context ? live_split_size(*live_context, n_splits, static_split_size) : static_split_size;
+                                                                         const int* __restrict__ live_context,
+                                                                         const int* __restrict__ plan, int n_items) {
+    const int item = blockIdx.x / per;
+    const int split_size = plan ? plan[1 + n_items * n_splits + item]
+                           : live_context ? live_split_size(*live_context, n_splits, static_split_size) : static_split_size;
     __shared__ float s_w[MAX_SPLITS];      // hpw * n_splits <= MAX_SPLITS (hpw > 1 only with few splits)
     __shared__ float s_l[MAX_SPLITS];
     __shared__ f32x4 s_acc[REDUCE_GROUPS][REDUCE_QUADS];
     // only the rows of this launch's items have partial results
-    const int item = blockIdx.x / per;
     const int tok = blockIdx.x % per;
     if (tok >= items[4 * item + 1]) return;
     const int64_t row = items[4 * item] + tok;
+    if (plan && positions[items[4 * item] + items[4 * item + 1] - 1] < split_size) return;   // finished by its only split
     const int hpw = 1 << hpw_log2;            // heads of this workgroup
     const int head0 = blockIdx.y * hpw;
     const int valid = min(n_splits, positions[row] / split_size + 1);
@@ -1368,6 +1386,119 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
     }
 }
 
+// The plan of a step of decoded tokens and short portions whose contexts differ much: how many splits every item's
+// keys are cut into, and in which order the workgroups take the (item, split) pairs.  The smallest split length T
+// (whole 32-key blocks, at least min_keys) with sum_i min(n_splits, ceil(context_i / T)) <= slots is found; item i
+// is cut evenly into that many splits; the pairs are ordered by their lengths, longest first, the second
+// `first_wave` of them the other way round: consecutive workgroups go to different compute units until every unit
+// has one, so the longest walks start first, each on a unit of its own, and the unit that got the longest gets the
+// shortest of the second round.  One workgroup; n_items * n_splits <= PLAN_MAX_PAIRS.
+constexpr int PLAN_THREADS = 256;
+constexpr int PLAN_MAX_PAIRS = 1024;
+
+__global__ __launch_bounds__(PLAN_THREADS) void attn_plan_kernel(const int* __restrict__ items,
+                                                                  const int* __restrict__ positions, int n_items,
+                                                                  int n_splits, int slots, int first_wave, int min_keys,
+                                                                  int* __restrict__ plan) {
+    __shared__ int s_ctx[PLAN_MAX_PAIRS];
+    __shared__ int s_size[PLAN_MAX_PAIRS];
+    __shared__ int s_len[PLAN_MAX_PAIRS];
+    __shared__ int s_pair[PLAN_MAX_PAIRS];
+    __shared__ int s_red[PLAN_THREADS / PULSE_WAVE];
+    const int tid = threadIdx.x, lane = tid % PULSE_WAVE, wave = tid / PULSE_WAVE;
+    constexpr int WV = PLAN_THREADS / PULSE_WAVE;
+    // a sum or a maximum over the workgroup, the same in every thread
+    auto all_sum = [&](int v) {
+#pragma unroll
+        for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, PULSE_WAVE);
+        __syncthreads();   // (the last round's reads of s_red are over)
+        if (lane == 0) s_red[wave] = v;
+        __syncthreads();
+        int t = 0;
+#pragma unroll
+        for (int w = 0; w < WV; ++w) t += s_red[w];
+        return t;
+    };
+    int longest = 1;
+    for (int i = tid; i < n_items; i += PLAN_THREADS) {
+        const int c = positions[items[4 * i] + items[4 * i + 1] - 1] + 1;
+        s_ctx[i] = c;
+        longest = max(longest, c);
+    }
+#pragma unroll
+    for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) longest = max(longest, __shfl_xor(longest, off, PULSE_WAVE));
+    if (lane == 0) s_red[wave] = longest;
+    __syncthreads();
+    longest = 0;
+#pragma unroll
+    for (int w = 0; w < WV; ++w) longest = max(longest, s_red[w]);
+    // T in blocks of 32 keys: the smallest in [lo, hi] whose pairs fit the slots (hi: every item whole)
+    int lo = max(1, (min_keys + 31) / 32), hi = (longest + 31) / 32;
+    lo = min(lo, hi);
+    while (lo < hi) {
+        const int mid = (lo + hi) / 2, t = mid * 32;
+        int mine = 0;
+        for (int i = tid; i < n_items; i += PLAN_THREADS) mine += min(n_splits, (s_ctx[i] + t - 1) / t);
+        if (all_sum(mine) <= slots) hi = mid; else lo = mid + 1;
+    }
+    const int T = lo * 32;
+    // every item's split size and number of pairs; the pairs' places by a running sum over the items
+    constexpr int PER = PLAN_MAX_PAIRS / PLAN_THREADS;   // consecutive items a thread
+    int counts[PER], run = 0;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+        const int i = tid * PER + e;
+        counts[e] = 0;
+        if (i < n_items) {
+            const int c = s_ctx[i];
+            const int n = min(n_splits, (c + T - 1) / T);
+            const int size = ((c + n - 1) / n + 31) / 32 * 32;
+            s_size[i] = size;
+            plan[1 + n_items * n_splits + i] = size;
+            counts[e] = (c + size - 1) / size;
+        }
+        run += counts[e];
+    }
+    int incl = run;   // inclusive sum over the threads before: within the wavefront, then over the wavefronts
+#pragma unroll
+    for (int off = 1; off < PULSE_WAVE; off <<= 1) {
+        const int up = __shfl_up(incl, off, PULSE_WAVE);
+        if (lane >= off) incl += up;
+    }
+    __syncthreads();
+    if (lane == PULSE_WAVE - 1) s_red[wave] = incl;
+    __syncthreads();
+    int before = incl - run, total = 0;
+#pragma unroll
+    for (int w = 0; w < WV; ++w) {
+        if (w < wave) before += s_red[w];
+        total += s_red[w];
+    }
+#pragma unroll
+    for (int e = 0; e < PER; ++e) {
+        const int i = tid * PER + e;
+        if (i < n_items) {
+            const int c = s_ctx[i], size = s_size[i];
+            for (int z = 0; z < counts[e]; ++z) {
+                s_len[before + z] = min(size, c - z * size);
+                s_pair[before + z] = i * n_splits + z;
+            }
+            before += counts[e];
+        }
+    }
+    __syncthreads();
+    // a pair's place: how many are longer (or as long and earlier); the second round turned round
+    const int second_end = min(2 * first_wave, total);
+    for (int j = tid; j < total; j += PLAN_THREADS) {
+        const int mine = s_len[j];
+        int rank = 0;
+        for (int k = 0; k < total; ++k) rank += (s_len[k] > mine || (s_len[k] == mine && k < j)) ? 1 : 0;
+        const int place = (rank >= first_wave && rank < second_end) ? first_wave + (second_end - 1 - rank) : rank;
+        plan[1 + place] = s_pair[j];
+    }
+    if (tid == 0) plan[0] = total;
+}
+
 }  // namespace
 
 extern "C" int pulse_attn_mfma_head_dim() { return D; }
@@ -1387,7 +1518,7 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
                      const void* vcache, const int* positions, const int* block_table, int bt_width, const int* items,
                      int n_items, int tokens, int nq, int nkv, int page_size, int num_pages, float scale, int window,
                      int split_size, int n_splits, int max_context, float* part_o, float* part_ml,
-                     const Preparation* prep, const int* live_context, hipStream_t stream) {
+                     const Preparation* prep, const int* live_context, const int* plan, hipStream_t stream) {
     PULSE_REQUIRE(tokens >= 0 && n_items >= 0 && nq > 0 && nkv > 0, "attn_mfma: bad sizes");
     PULSE_REQUIRE(nq % nkv == 0, "attn_mfma: %d query heads are not a multiple of %d kv heads", nq, nkv);
     PULSE_REQUIRE(page_size > 0 && page_size % 16 == 0, "attn_mfma: page size %d must be a multiple of 16", page_size);
@@ -1421,6 +1552,8 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
     a.scale_log2e = scale * 1.4426950408889634f;
     a.window = window; a.split_size = split_size; a.n_splits = n_splits;
     a.live_context = n_splits > 1 ? live_context : nullptr;
+    a.plan = n_splits > 1 ? plan : nullptr;
+    a.n_items = n_items;
     a.q_w = a.k_w = nullptr; a.cos_t = a.sin_t = nullptr; a.eps = 0.f; a.rotary_dim = 0; a.pairing = 0; a.new_key = 0;
     if (prep) {
         a.q_w = static_cast<const bf16_t*>(prep->q_w); a.k_w = static_cast<const bf16_t*>(prep->k_w);
@@ -1439,7 +1572,7 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
         while (hpw * 2 * n_splits <= REDUCE_GROUPS && hpw * 2 <= nq) { hpw *= 2; ++hpw_log2; }
         hipLaunchKernelGGL(attn_mfma_reduce_kernel, dim3(n_items * per, (nq + hpw - 1) / hpw), dim3(REDUCE_THREADS), 0, stream,
                            part_o, part_ml, positions, items, per, a.out, o_stride, nq, n_splits, split_size, hpw_log2,
-                           a.live_context);
+                           a.live_context, a.plan, n_items);
         PULSE_LAUNCH_CHECK("attn_mfma_reduce");
     }
     return 0;
@@ -1451,15 +1584,34 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
 // live_context (device, or null): the longest context (last position + 1) among ALL items of this call as the step
 // has it; split_size and n_splits say what the launch is made for (max_context), and with live_context the kernel cuts
 // the keys that are there evenly into the same number of splits.  A value below an item's context loses keys.
+// plan (device, or null): what pulse_attn_plan made of these items and positions for this n_splits; it takes the
+// place of that even cut (every item then has a split size of its own and the workgroups an order).
 extern "C" int pulse_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_stride, const void* kcache,
                                const void* vcache, const int* positions, const int* block_table, int bt_width,
                                const int* items, int n_items, int tokens, int nq,
                                int nkv, int page_size, int num_pages, float scale, int window, int split_size,
                                int n_splits, int max_context, float* part_o, float* part_ml, const int* live_context,
-                               hipStream_t stream) {
+                               const int* plan, hipStream_t stream) {
     return launch_attn_mfma(q, q_stride, out, o_stride, kcache, vcache, positions, block_table, bt_width, items, n_items,
                             tokens, nq, nkv, page_size, num_pages, scale, window, split_size, n_splits, max_context,
-                            part_o, part_ml, nullptr, live_context, stream);
+                            part_o, part_ml, nullptr, live_context, plan, stream);
+}
+
+// The plan of a step (see attn_plan_kernel) for pulse_attn_mfma / pulse_attn_decode with the same items and n_splits:
+// plan holds 1 + n_items * n_splits + n_items ints.  slots: how many workgroups a kv head's walks should be cut into
+// at most (what the compute units hold at a time); first_wave: how many of them land on units of their own.
+extern "C" int pulse_attn_plan_max_pairs() { return PLAN_MAX_PAIRS; }
+
+extern "C" int pulse_attn_plan(const int* items, const int* positions, int n_items, int n_splits, int slots,
+                               int first_wave, int min_keys, int* plan, hipStream_t stream) {
+    PULSE_REQUIRE(items && positions && plan, "attn_plan: null pointer");
+    PULSE_REQUIRE(n_items >= 1 && n_splits >= 1 && static_cast<int64_t>(n_items) * n_splits <= PLAN_MAX_PAIRS,
+                  "attn_plan: %d items in up to %d splits are more than %d pairs", n_items, n_splits, PLAN_MAX_PAIRS);
+    PULSE_REQUIRE(slots >= 1 && first_wave >= 1 && min_keys >= 1, "attn_plan: slots, first_wave and min_keys must be positive");
+    hipLaunchKernelGGL(attn_plan_kernel, dim3(1), dim3(PLAN_THREADS), 0, stream, items, positions, n_items, n_splits,
+                       slots, first_wave, min_keys, plan);
+    PULSE_LAUNCH_CHECK("attn_plan");
+    return 0;
 }
 
 // Whether pulse_attn_decode takes a rotation: whole 8-element slices, and for pairs (i, i + rotary_dim / 2) a
@@ -1482,7 +1634,7 @@ extern "C" int pulse_attn_decode(const void* qkv, int64_t qkv_stride, void* out,
                                  int num_pages, float scale, int window, int split_size, int n_splits, int max_context,
                                  float* part_o, float* part_ml, const void* q_w, const void* k_w, float eps,
                                  const float* cos_t, const float* sin_t, int rotary_dim, int pairing, int new_key,
-                                 const int* live_context, hipStream_t stream) {
+                                 const int* live_context, const int* plan, hipStream_t stream) {
     PULSE_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attn_decode: cos and sin come together");
     if (!cos_t) rotary_dim = 0;
     PULSE_REQUIRE(pulse_attn_decode_takes(rotary_dim, pairing), "attn_decode: rotation of %d channels with pairing %d is not "
@@ -1496,7 +1648,7 @@ extern "C" int pulse_attn_decode(const void* qkv, int64_t qkv_stride, void* out,
     Preparation prep{q_w, k_w, cos_t, sin_t, eps, rotary_dim, pairing, new_key ? 1 : 0};
     return launch_attn_mfma(qkv, qkv_stride, out, o_stride, kcache, vcache, positions, block_table, bt_width, items,
                             n_items, tokens, nq, nkv, page_size, num_pages, scale, window, split_size, n_splits,
-                            max_context, part_o, part_ml, &prep, live_context, stream);
+                            max_context, part_o, part_ml, &prep, live_context, plan, stream);
 }
 
 // Keys a split of the prompt-portion kernel must be a multiple of; 0 when this head size's kernel has no splits.
@@ -1546,6 +1698,7 @@ extern "C" int pulse_attn_prefill(const void* q, int64_t q_stride, void* out, in
     a.scale_log2e = scale * 1.4426950408889634f;
     a.window = window; a.split_size = n_splits > 1 ? split_size : 0; a.n_splits = n_splits;
     a.live_context = nullptr;
+    a.plan = nullptr;
     a.part_o = n_splits > 1 ? part_o : nullptr; a.part_ml = n_splits > 1 ? part_ml : nullptr;
 #if PULSE_WIDE
     hipLaunchKernelGGL((attn_prefill_wide_kernel<WIDE_CT, 4, WIDE_NW>), dim3(n_items, nkv * a.head_chunks, n_splits),

@@ -22,7 +22,7 @@ import torch
 
 from ..cache.manager import CacheManager, PagedKVSpec, StateSpec
 from ..models.causal_lm import CausalLM
-from ..parts.base import EntryMeta, PagedCacheView, StateView, StepContext
+from ..parts.base import EntryMeta, PagedCacheView, StateView, StepContext, contexts_uneven
 
 
 class StepError(ValueError):
@@ -195,7 +195,7 @@ class ModelRunner:
         flat[offsets[8 + len(widths)]] = max(m.start + m.count for m in metas)
 
     def _context(self, dev: torch.Tensor, offsets: np.ndarray, metas: List[EntryMeta], wanted: int,
-                 widths: Sequence[int], workspace, max_context: int) -> StepContext:
+                 widths: Sequence[int], workspace, max_context: int, uneven: bool) -> StepContext:
         total, batch = metas[-1].first_row + metas[-1].count, len(metas)
         part = [dev[offsets[i]:offsets[i + 1]] for i in range(len(offsets) - 1)]
         return StepContext(
@@ -204,6 +204,7 @@ class ModelRunner:
             block_tables={gi: part[8 + gi].view(batch, w) for gi, w in enumerate(widths)},
             want_rows=part[7], num_wanted=wanted, workspace=workspace,
             max_count=max(m.count for m in metas), max_context=max_context, live_context=part[8 + len(widths)],
+            uneven=uneven,
             upload=self._staging.upload_values)   # (the staging's method, not a closure over the step function: a
                                                    # recording keeps its context, and would keep the step function
                                                    # that holds it alive in a circle that only the collector ends)
@@ -219,15 +220,16 @@ class ModelRunner:
         total = row
         want_rows = [m.first_row + int(w) for e, m in zip(entries, metas) for w in e.want]
         max_context = max(m.start + m.count for m in metas)
-        if self._graph_ok(entries, metas) and self._graph_ready(len(metas), max_context):
-            logits = self._step_captured(entries, metas, want_rows, max_context)
+        uneven = contexts_uneven(metas)
+        if self._graph_ok(entries, metas) and self._graph_ready(len(metas), max_context, uneven):
+            logits = self._step_captured(entries, metas, want_rows, max_context, uneven)
         else:
             widths = [max(1, max(g.pages_for(m.start + m.count) for m in metas)) for g in cache.groups]
             offsets = self._layout(total, len(metas), len(want_rows), widths)
             flat = np.zeros(int(offsets[-1]), dtype=np.int32)
             self._fill(flat, offsets, entries, metas, want_rows, widths)
             dev = self._staging.upload(flat)
-            ctx = self._context(dev, offsets, metas, len(want_rows), widths, self.model.workspace, max_context)
+            ctx = self._context(dev, offsets, metas, len(want_rows), widths, self.model.workspace, max_context, uneven)
             logits = self.model.forward(ctx, self.views)
         for m in metas:
             cache.advance(m.request, m.start + m.count)
@@ -237,8 +239,9 @@ class ModelRunner:
 
     # ------------------------------------------------------- captured decoding
     # A step of single tokens (one per request, each wanting its logits) has the same launches every time,
-    # so it is recorded once per (batch, context bucket) as a HIP graph over buffers of its own and replayed:
-    # the host then only copies the step's integers and starts the graph.
+    # so it is recorded once per (batch, context bucket, whether the contexts differ much: parts may share their work
+    # out differently then) as a HIP graph over buffers of its own and replayed: the host then only copies the
+    # step's integers and starts the graph.
     GRAPH_MAX_BATCH = 64        # up to here every product can be this package's own kernel; a shape whose step does
                                 # call the vendor library (seen when it is first run for recording) stays eager
     GRAPH_CONTEXT_BUCKET = 1024
@@ -250,14 +253,14 @@ class ModelRunner:
             return False
         return all(m.count == 1 for m in metas) and all(list(e.want) == [0] for e in entries)
 
-    def _graph_key(self, batch: int, max_context: int):
+    def _graph_key(self, batch: int, max_context: int, uneven: bool):
         bucket = (max_context + self.GRAPH_CONTEXT_BUCKET - 1) // self.GRAPH_CONTEXT_BUCKET * self.GRAPH_CONTEXT_BUCKET
-        return batch, min(bucket, max(self.max_positions, max_context))
+        return batch, min(bucket, max(self.max_positions, max_context)), uneven
 
-    def _graph_ready(self, batch: int, max_context: int) -> bool:
+    def _graph_ready(self, batch: int, max_context: int, uneven: bool) -> bool:
         """A shape is recorded when it comes for the GRAPH_AFTER_STEPS-th time: recording costs about as much as a
         dozen steps, which a shape that a draining batch passes through once or twice never pays back."""
-        key = self._graph_key(batch, max_context)
+        key = self._graph_key(batch, max_context, uneven)
         if key in self._graphs:
             return True
         if key in self._graph_refused:
@@ -267,8 +270,8 @@ class ModelRunner:
         return seen >= self.GRAPH_AFTER_STEPS
 
     def _step_captured(self, entries: Sequence[StepEntry], metas: List[EntryMeta], want_rows: List[int],
-                       max_context: int) -> torch.Tensor:
-        key = self._graph_key(len(metas), max_context)
+                       max_context: int, uneven: bool) -> torch.Tensor:
+        key = self._graph_key(len(metas), max_context, uneven)
         rec = self._graphs.get(key)
         if rec is None:
             # The step that meets a new shape runs eagerly (over the recording's own buffers, which sizes them) and is
@@ -293,7 +296,7 @@ class ModelRunner:
     def _capture(self, key, entries, metas, want_rows):
         from ..parts.base import Workspace
 
-        batch, bucket = key
+        batch, bucket, uneven = key
         widths = [max(1, g.pages_for(bucket)) for g in self.cache.groups]
         offsets = self._layout(batch, batch, batch, widths)
         n = int(offsets[-1])
@@ -301,7 +304,7 @@ class ModelRunner:
         dev = torch.zeros(n, dtype=torch.int32, device=self.device)
         rec = _Captured(host=host, host_np=host.numpy(), dev=dev, offsets=offsets, widths=widths)
         workspace = Workspace(self.device)
-        ctx = self._context(dev, offsets, metas, batch, widths, workspace, bucket)
+        ctx = self._context(dev, offsets, metas, batch, widths, workspace, bucket, uneven)
         self._fill(rec.host_np, offsets, entries, metas, want_rows, widths)
         dev.copy_(host, non_blocking=True)
         # the step itself, eagerly: it sizes the workspace and lets parts build what depends only on the step's shape

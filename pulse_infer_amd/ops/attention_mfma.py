@@ -109,12 +109,14 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
               vcache: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
               items: torch.Tensor, scale: float, window: int, split_size: int, n_splits: int, max_context: int,
               part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor],
-              live_context: Optional[torch.Tensor] = None) -> None:
+              live_context: Optional[torch.Tensor] = None, plan: Optional[torch.Tensor] = None) -> None:
     """Attention of decoded tokens and short portions.  ``split_size`` x ``n_splits`` is what the launch is made for
     (contexts up to ``max_context``); ``live_context`` (one int32 on the device: the longest context among the step's
-    entries as it is now) lets the kernel cut the keys that are there evenly into the same number of splits."""
-    _gpu("attn_mfma", q, out, kcache, vcache, positions, block_table, items, part_o, part_ml, live_context)
+    entries as it is now) lets the kernel cut the keys that are there evenly into the same number of splits;
+    ``plan`` (what ``attn_plan`` made of these items for this ``n_splits``) takes the place of that even cut."""
+    _gpu("attn_mfma", q, out, kcache, vcache, positions, block_table, items, part_o, part_ml, live_context, plan)
     _live(live_context)
+    _planned(plan, items.numel() // ITEM_INTS, n_splits)
     tokens = q.shape[0]
     _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and q.stride(1) == 1 and out.stride(1) == 1,
           "attn_mfma: q and out must be bfloat16 matrices with contiguous rows")
@@ -138,7 +140,53 @@ def attn_mfma(q: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kca
             _ptr(vcache), _ptr(positions), _ptr(block_table), _i32(block_table.shape[1]),
             _ptr(items), _i32(n_items), _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages), _f32(scale),
             _i32(window), _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml),
-            _ptr(live_context), _stream())
+            _ptr(live_context), _ptr(plan), _stream())
+
+
+PLAN_MIN_KEYS = 256      # no split of a plan is shorter (what a workgroup costs beside its walk, in keys walked)
+PLAN_SPLITS = 8          # most splits of an item in a planned step
+
+
+def plan_ints(n_items: int, n_splits: int) -> int:
+    """int32 values of a plan for ``n_items`` items in up to ``n_splits`` splits."""
+    return 1 + n_items * n_splits + n_items
+
+
+def plan_slots(nkv: int, group: int) -> Tuple[int, int]:
+    """(slots, first_wave) for ``attn_plan``: the workgroups of one kv head (and chunk of 16 heads) that the compute
+    units hold at a time, two a unit, and how many of them land on a unit of their own."""
+    heads = nkv * ((group + 15) // 16)
+    first = max(1, compute_units() // heads)
+    return 2 * first, first
+
+
+def plan_fits(n_items: int, n_splits: int) -> bool:
+    return 1 <= n_items and n_items * n_splits <= 1024     # PLAN_MAX_PAIRS of attn_mfma.hip
+
+
+def attn_plan(items: torch.Tensor, positions: torch.Tensor, n_splits: int, slots: int, first_wave: int,
+              plan: torch.Tensor, d: int, min_keys: int = PLAN_MIN_KEYS) -> None:
+    """The plan of a step whose contexts differ much (on the device, from ``positions`` as they are now): every
+    item's keys are cut into min(n_splits, ceil(context / T)) even splits, T the smallest length with at most
+    ``slots`` (item, split) pairs in all, and the pairs are put in the order the workgroups take them, longest first.
+    ``plan``: int32 [plan_ints(items, n_splits)], to be passed to ``attn_mfma`` / ``attn_decode`` with the same items,
+    positions and n_splits."""
+    _gpu("attn_plan", items, positions, plan)
+    n_items = items.numel() // ITEM_INTS
+    _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() % ITEM_INTS == 0,
+          "attn_plan: items must be int32 quadruples")
+    _need(positions.dtype == torch.int32 and positions.is_contiguous(), "attn_plan: positions must be contiguous int32")
+    _need(plan_fits(n_items, n_splits), f"attn_plan: {n_items} items in up to {n_splits} splits do not fit a plan")
+    _planned(plan, n_items, n_splits)
+    lib = load_variant("attn_mfma", {"PULSE_HEAD_DIM": d})
+    call_in(lib, "pulse_attn_plan", _ptr(items), _ptr(positions), _i32(n_items), _i32(n_splits), _i32(slots),
+            _i32(first_wave), _i32(min_keys), _ptr(plan), _stream())
+
+
+def _planned(plan: Optional[torch.Tensor], n_items: int, n_splits: int) -> None:
+    _need(plan is None or (plan.dtype == torch.int32 and plan.is_contiguous()
+                           and plan.numel() >= plan_ints(n_items, n_splits)),
+          f"attention: a plan must hold {plan_ints(n_items, n_splits)} contiguous int32 values")
 
 
 def _live(live_context: Optional[torch.Tensor]) -> None:
@@ -251,13 +299,15 @@ def attn_decode(qkv: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int,
                 scale: float, window: int, split_size: int, n_splits: int, max_context: int,
                 part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor], q_w: Optional[torch.Tensor],
                 k_w: Optional[torch.Tensor], eps: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
-                rotary_dim: int, pairing: int, new_key: bool, live_context: Optional[torch.Tensor] = None) -> None:
+                rotary_dim: int, pairing: int, new_key: bool, live_context: Optional[torch.Tensor] = None,
+                plan: Optional[torch.Tensor] = None) -> None:
     """Attention for decoded tokens from the raw projection output ``qkv`` [tokens, (nq + 2 nkv) d]: per-head norm
     and rotation of q and of the token's own key happen inside the kernel; with ``new_key`` key and value are also
-    written to the token's page.  Every item must hold one token.  ``live_context``: as for ``attn_mfma``."""
+    written to the token's page.  Every item must hold one token.  ``live_context``, ``plan``: as for ``attn_mfma``."""
     _gpu("attn_decode", qkv, out, kcache, vcache, positions, block_table, items, part_o, part_ml, q_w, k_w, cos, sin,
-         live_context)
+         live_context, plan)
     _live(live_context)
+    _planned(plan, items.numel() // ITEM_INTS, n_splits)
     tokens = qkv.shape[0]
     _need(qkv.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and qkv.stride(1) == 1 and out.stride(1) == 1,
           "attn_decode: qkv and out must be bfloat16 matrices with contiguous rows")
@@ -291,4 +341,4 @@ def attn_decode(qkv: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int,
             _i32(tokens), _i32(nq), _i32(nkv), _i32(page_size), _i32(pages), _f32(scale), _i32(window),
             _i32(split_size), _i32(n_splits), _i32(max_context), _ptr(part_o), _ptr(part_ml), _ptr(q_w), _ptr(k_w),
             _f32(eps), _ptr(cos), _ptr(sin), _i32(rotary_dim if cos is not None else 0), _i32(pairing),
-            _i32(1 if new_key else 0), _ptr(live_context), _stream())
+            _i32(1 if new_key else 0), _ptr(live_context), _ptr(plan), _stream())

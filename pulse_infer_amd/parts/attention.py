@@ -176,8 +176,24 @@ class PagedAttention(Part):
         if short_items is not None:
             # a recorded step passes its context bucket as max_context: its splits must cover that
             max_context = ctx.max_context if long_items is None else short_context
-            split_size, n_splits = attention_mfma.choose_splits(short_items.numel() // attention_mfma.ITEM_INTS, self.nkv, group,
-                                                                      max_context)
+            n_items = short_items.numel() // attention_mfma.ITEM_INTS
+            split_size, n_splits = attention_mfma.choose_splits(n_items, self.nkv, group, max_context)
+            plan = None
+            if ctx.uneven and long_items is None and not window:
+                # contexts that differ much: every request's keys cut by its own length, the workgroups in an order
+                # that starts the longest walks first (the plan is made on the device, once a step for all layers)
+                planned = min(attention_mfma.PLAN_SPLITS, 1024 // n_items)
+                if planned > 1 and attention_mfma.plan_fits(n_items, planned):
+                    n_splits = planned
+                    split_size = max(32, ((max_context + n_splits - 1) // n_splits + 31) // 32 * 32)
+                    slots, first = attention_mfma.plan_slots(self.nkv, group)
+                    pkey = f"attention.plan:{per}:{n_splits}:{slots}:{first}"
+                    if pkey not in ctx.extras:
+                        made = ctx.workspace.buffer(f"attention.plan:{n_splits}:{slots}:{first}",
+                                                    attention_mfma.plan_ints(n_items, n_splits), 1, torch.int32)
+                        attention_mfma.attn_plan(short_items, ctx.positions, n_splits, slots, first, made, self.d)
+                        ctx.extras[pkey] = made
+                    plan = ctx.extras[pkey]
             part_o = part_ml = None
             if n_splits > 1:
                 rows = ctx.num_tokens * self.nq * n_splits
@@ -190,8 +206,9 @@ class PagedAttention(Part):
                     self.scale, window, split_size, n_splits, max_context, part_o, part_ml, self.q_w, self.k_w,
                     self.eps, tables.cos if tables is not None else None, tables.sin if tables is not None else None,
                     tables.rotary_dim if tables is not None else 0, tables.pairing if tables is not None else 0,
-                    new_key=write, live_context=ctx.live_context)
+                    new_key=write, live_context=ctx.live_context if plan is None else None, plan=plan)
                 return
             attention_mfma.attn_mfma(q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions,
                                      table, short_items, self.scale, window, split_size, n_splits,
-                                     max_context, part_o, part_ml, live_context=ctx.live_context)
+                                     max_context, part_o, part_ml,
+                                     live_context=ctx.live_context if plan is None else None, plan=plan)

@@ -133,6 +133,23 @@ class StateView:
     state: torch.Tensor    # [slots, *shape]
 
 
+UNEVEN_CONTEXTS = 1.5     # longest context / mean context from which a step counts as uneven
+UNEVEN_MIN_ENTRIES = 3
+
+
+def contexts_uneven(entries: List[EntryMeta]) -> bool:
+    """Whether a step's requests hold contexts that differ much (``StepContext.uneven``)."""
+    if len(entries) < UNEVEN_MIN_ENTRIES:
+        return False
+    longest = total = 0
+    for e in entries:
+        c = e.start + e.count
+        total += c
+        if c > longest:
+            longest = c
+    return longest * len(entries) >= UNEVEN_CONTEXTS * total
+
+
 @dataclass
 class StepContext:
     """Everything a part may need to know about the step being run."""
@@ -155,6 +172,9 @@ class StepContext:
                                  # (of a recorded step: the most its replays may bring)
     live_context: Optional[torch.Tensor] = None   # int32 [1] on the device: the longest context as it is in this
                                                   # step (at most max_context), for kernels that shape their work by it
+    uneven: bool = False         # the requests' contexts differ much (the longest at least UNEVEN_CONTEXTS times
+                                 # their mean): a part may share its work out differently then; a recorded step is
+                                 # recorded for one case or the other
     extras: Dict[str, Any] = field(default_factory=dict)  # per-step products of position encodings etc.
     upload: Optional[Callable[[List[int]], torch.Tensor]] = None   # integers of a part's own to the device, through the
                                                                    # step function's pinned staging (no synchronous copy)

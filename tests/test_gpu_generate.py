@@ -201,6 +201,62 @@ def test_captured_decode_steps_replay_like_eager_ones(gpu, model_folders, plain_
             close(row_g[None], row_e[None], "bfloat16", f"captured against eager {k}@{pos_g}", SPLIT_TOL)
 
 
+def test_steps_of_uneven_contexts_are_recorded_apart(gpu, model_folders, plain_logits):
+    """When the longest context of a decoding step is well above the mean, attention shares its work out by a plan
+    made on the device (every request cut by its own length, the longest walks first), and such a step has a recording
+    of its own.  A batch that goes from uneven to even and back, with another request in between: three recordings,
+    every replay against the eager step and the plain implementation."""
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from test_gpu_model import SPLIT_TOL, close
+
+    cfg, page = TINY["B"]
+    _, model = load_model(model_folders["B"], mode="bfloat16")
+    lens = {"a": 200, "b": 20, "c": 24, "d": 18, "e": 150, "f": 25}
+    ids = {k: token_ids(cfg["vocab_size"], n + 30, seed=70 + n) for k, n in lens.items()}
+    got = []
+    for graphs in (True, False):
+        runner = ModelRunner(model, page_size=16, num_pages=40, max_requests=4, use_graphs=graphs)
+        runner.GRAPH_AFTER_STEPS = 1
+        fed, rows = {}, []
+
+        def start(k):
+            runner.add_request(k)
+            runner.reserve(k, lens[k] + 30)
+            runner.step([StepEntry(k, ids[k][:lens[k]], [])])
+            fed[k] = lens[k]
+
+        def decode(names, steps):
+            for _ in range(steps):
+                logits = runner.step([StepEntry(k, ids[k][fed[k]:fed[k] + 1], [0]) for k in names])
+                for row, k in enumerate(names):
+                    rows.append((k, fed[k], logits[row]))
+                    fed[k] += 1
+
+        for k in "abcd":
+            start(k)
+        decode("abcd", 5)            # uneven: one of 200 among three of 20
+        runner.free_request("a")
+        decode("bcd", 5)             # even
+        start("e")
+        decode("ebcd", 5)            # uneven again, another request in another place: the first recording
+        runner.free_request("e")
+        start("f")
+        decode("bcdf", 5)            # four even ones
+        assert runner.graph_records == (3 if graphs else 0)
+        assert runner.graph_replays == (20 - 3 if graphs else 0)
+        for k in "bcdf":
+            runner.free_request(k)
+        runner.cache.check()
+        got.append(rows)
+    assert any(name.startswith("attention.plan") for name, _ in model.workspace._flat)   # the eager steps planned too
+    for (k, pos, recorded), (k2, pos2, eager) in zip(*got):
+        assert (k, pos) == (k2, pos2)
+        want = plain_logits("B", ids[k])                 # (causal: the logits at pos do not see what follows)
+        close(recorded[None], want[pos][None], "bfloat16", f"uneven {k}@{pos}")
+        close(recorded[None], eager[None], "bfloat16", f"uneven against eager {k}@{pos}", SPLIT_TOL)
+
+
 def test_the_collector_rests_while_a_step_is_recorded(gpu, model_folders):
     """No graph may be destroyed while a stream records, and Python's collector, which may find dropped recordings (of
     a step function that is no longer used, of the caller), runs whenever it likes: the step function lets it run

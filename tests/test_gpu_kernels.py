@@ -558,11 +558,12 @@ def test_kernels_refuse_what_they_cannot_do(k):
 
 
 # ------------------------------------------------------- matrix-core attention
-def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0, portion_split=0, made_for=None):
+def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0, portion_split=0, made_for=None, planned=None):
     """Requests with contexts `lens`; request 0 brings its last `portion` tokens, the others one token each.
     ``portion_split``: request 0's portion goes through the prompt-portion kernel with its keys in splits of that size.
     ``made_for = (context, splits)``: the launch is made for contexts up to that (as a recorded step's is for its
-    bucket) and is told the longest context there is through ``live_context``."""
+    bucket) and is told the longest context there is through ``live_context``.  ``planned = (slots, first_wave,
+    min_keys)``: such a launch with a plan made on the device instead."""
     from pulse_infer_amd.ops import attention_mfma as M
     dtype = torch.bfloat16
     pages_per = [(n + bs - 1) // bs for n in lens]
@@ -599,7 +600,7 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0, portion_
     if made_for is not None:
         max_ctx, n = made_for
         split = ((max_ctx + n - 1) // n + 31) // 32 * 32
-        live = torch.tensor([max(lens)], dtype=torch.int32, device=DEV)
+        live = torch.tensor([max(lens)], dtype=torch.int32, device=DEV) if planned is None else None
     if split is None or split == "portion" or portion_split:
         split_size, n_splits = M.choose_splits(items.numel() // M.ITEM_INTS, nkv, group, max_ctx)
     else:
@@ -625,8 +626,13 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0, portion_
             M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), small, scale, window, split_size,
                         n_splits, max_ctx, part_o, part_ml)
     else:
+        plan = None
+        if planned is not None:
+            n_items = items.numel() // M.ITEM_INTS
+            plan = torch.full((M.plan_ints(n_items, n_splits),), -77, dtype=torch.int32, device=DEV)
+            M.attn_plan(items, pos_t, n_splits, planned[0], planned[1], plan, d, min_keys=planned[2])
         M.attn_mfma(q, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), items, scale, window, split_size,
-                    n_splits, max_ctx, part_o, part_ml, live_context=live)
+                    n_splits, max_ctx, part_o, part_ml, live_context=live, plan=plan)
     got = out.cpu().to(F64).reshape(-1, nq, d)
     for t, (p, e) in enumerate(zip(positions, entry)):
         kref, vref = refs[e]
@@ -662,6 +668,57 @@ def test_attn_mfma_made_for_longer_contexts_than_the_step_has(k, case, made_for)
     """A launch shaped for a context bucket (its number of splits, its scratch) that is told the longest context of the
     step: the kernel and the merge cut the keys that are there into even splits, and both must agree on where."""
     _mfma_case(k, split=None, made_for=made_for, **case)
+
+
+@pytest.mark.parametrize("case", [
+    dict(nq=32, nkv=8, d=128, bs=16, window=0, lens=[300, 513, 512, 31], portion=3),
+    dict(nq=6, nkv=3, d=48, bs=32, window=24, lens=[170, 90, 24, 25], portion=1),     # splits that lie below the window
+    dict(nq=8, nkv=2, d=64, bs=16, window=0, lens=[5, 1, 2], portion=1),
+    dict(nq=4, nkv=2, d=32, bs=16, window=0, lens=[1500, 40, 33, 900, 64, 65, 7], portion=1),
+])
+@pytest.mark.parametrize("planned", [(4, 2, 32), (9, 3, 64), (64, 32, 256), (1000, 1, 32)])
+def test_attn_mfma_with_a_plan_of_the_step(k, case, planned):
+    """The kernel for decoded tokens and short portions with a plan made on the device from the step's positions:
+    every item cut into as many splits as its length asks for, the (item, split) pairs in the plan's order; items of
+    one split are finished by their workgroup, the others by the merge (the scratch starts as NaN)."""
+    _mfma_case(k, split=None, made_for=(2048, 6), planned=planned, **case)
+
+
+def test_attn_plan_cuts_and_orders(k):
+    """The plan itself against the rule it follows: the smallest split length T (whole blocks of 32, at least
+    min_keys) with at most `slots` pairs in all, items cut evenly into min(n_splits, ceil(context / T)) splits, pairs
+    by length, longest first (ties: the earlier pair), the second `first_wave` turned round."""
+    from pulse_infer_amd.ops import attention_mfma as M
+    gen = torch.Generator().manual_seed(3)
+    for n_items, n_splits, slots, first, min_keys, hi in ((32, 8, 64, 32, 256, 2304), (5, 4, 7, 2, 32, 700), (48, 8, 64, 32, 256, 4096),
+                                                         (128, 8, 64, 32, 256, 3000), (3, 6, 64, 32, 256, 90), (20, 8, 64, 32, 256, 8000),
+                                                         (64, 16, 100, 8, 128, 50000)):
+        ctx = torch.randint(1, hi + 1, (n_items,), generator=gen).tolist()
+        rows = torch.randperm(n_items, generator=gen).tolist()            # items in another order than their rows
+        positions = torch.zeros(n_items, dtype=torch.int32)
+        items = []
+        for i, r in enumerate(rows):
+            positions[r] = ctx[i] - 1
+            items.extend((r, 1, i, 0))
+        items = torch.tensor(items, dtype=torch.int32, device=DEV)
+        plan = torch.full((M.plan_ints(n_items, n_splits),), -77, dtype=torch.int32, device=DEV)
+        M.attn_plan(items, positions.to(DEV), n_splits, slots, first, plan, 128, min_keys=min_keys)
+        got = plan.cpu().tolist()
+        count = lambda t: sum(min(n_splits, -(-c // t)) for c in ctx)
+        top = (max(ctx) + 31) // 32 * 32
+        T = next(t for t in range(min((min_keys + 31) // 32 * 32, top), top + 1, 32) if count(t) <= slots or t == top)
+        sizes, pairs = [], []
+        for i, c in enumerate(ctx):
+            n = min(n_splits, -(-c // T))
+            size = (-(-c // n) + 31) // 32 * 32
+            sizes.append(size)
+            pairs.extend((min(size, c - z * size), i * n_splits + z) for z in range(-(-c // size)))
+        order = sorted(range(len(pairs)), key=lambda j: (-pairs[j][0], j))
+        end = min(2 * first, len(order))
+        order = order[:first] + order[first:end][::-1] + order[end:]
+        assert got[0] == len(pairs)
+        assert got[1:1 + len(pairs)] == [pairs[j][1] for j in order]
+        assert got[1 + n_items * n_splits:] == sizes
 
 
 @pytest.mark.parametrize("case", [
@@ -808,14 +865,17 @@ def test_attn_mfma_refuses_other_sizes(k):
     dict(nq=16, nkv=1, d=224, rot=224, pairing="interleaved", norm=True, bs=16, window=100, lens=[260, 130]),
     dict(nq=40, nkv=2, d=64, rot=32, pairing="interleaved", norm=True, bs=64, window=0, lens=[200, 77, 64]),  # 20 heads a kv head: two chunks
 ])
-@pytest.mark.parametrize("split", [None, 32, 128, "bucket"])
+@pytest.mark.parametrize("split", [None, 32, 128, "bucket", "planned", "planned_short"])
 @pytest.mark.parametrize("new_key", [True, False])
 def test_attn_decode_from_raw(k, case, split, new_key):
     """Decoded tokens straight from the raw projection output: per-head norm, rotation, the token's own key and
     value (used from registers, written to the page) inside the attention kernel, against the plain formulas and
     against what the separate preparation kernel writes.  With new_key False the pages already hold the token.
     "bucket": the launch is made for contexts of up to 2,048 in five splits, as a recorded step's is, and told the
-    longest context there is: the split that holds a token's position, whose workgroup writes its key, moves with it."""
+    longest context there is: the split that holds a token's position, whose workgroup writes its key, moves with it.
+    "planned": the same launch with a plan made on the device from the positions (every item its own split size, the
+    workgroups in the plan's order, items of one split finished without the merge); "planned_short": splits down to a
+    block of keys, so that every item is cut as far as the launch allows."""
     from pulse_infer_amd.ops import attention_mfma as M
     nq, nkv, d, rot, bs, window, lens = (case[x] for x in ("nq", "nkv", "d", "rot", "bs", "window", "lens"))
     pairing = 0 if case["pairing"] == "interleaved" else 1
@@ -873,15 +933,27 @@ def test_attn_decode_from_raw(k, case, split, new_key):
         live = torch.tensor([max_ctx], dtype=torch.int32, device=DEV)
         max_ctx, n_splits = 2048, 5
         split_size = 416
+    elif split in ("planned", "planned_short"):
+        max_ctx, n_splits = 2048, 5
+        split_size = 416
     else:
         split_size, n_splits = split, (max_ctx + split - 1) // split
     part_o = torch.full((n * nq * n_splits, d), float("nan"), device=DEV)
     part_ml = torch.full((n * nq * n_splits, 2), float("nan"), device=DEV)
     out = torch.zeros(n, nq * d, dtype=dtype, device=DEV)
     pos_t = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    plan = None
+    if split in ("planned", "planned_short"):
+        plan = torch.full((M.plan_ints(n, n_splits),), -77, dtype=torch.int32, device=DEV)
+        slots = 2 * n if split == "planned" else 1000
+        M.attn_plan(items, pos_t, n_splits, slots, 2, plan, d, min_keys=64 if split == "planned" else 32)
+        sizes = plan[1 + n * n_splits:].tolist()
+        assert all(sz % 32 == 0 and sz * n_splits >= c for sz, c in zip(sizes, lens))
+        if split == "planned_short":
+            assert sizes == [max(32, ((c + n_splits - 1) // n_splits + 31) // 32 * 32) for c in lens]
     raw = qkv.clone()
     M.attn_decode(qkv, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), items, scale, window, split_size, n_splits,
-                  max_ctx, part_o, part_ml, qw, kw, eps, cos, sin, rot, pairing, new_key, live_context=live)
+                  max_ctx, part_o, part_ml, qw, kw, eps, cos, sin, rot, pairing, new_key, live_context=live, plan=plan)
     assert torch.equal(qkv, raw)                   # the projection output stays raw
     got = out.cpu().to(F64).reshape(n, nq, d)
     for t, p in enumerate(positions):
