@@ -570,7 +570,7 @@ __device__ __forceinline__ float simple_row_max(const float* part_max, int chunk
 
 __global__ __launch_bounds__(SIMPLE_THREADS) void simple_mass_kernel(
     const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ temperature,
-    const int* __restrict__ top_k, const float* __restrict__ top_p,
+    const int* __restrict__ top_k,
     const float* __restrict__ penalty, const int* __restrict__ seen_row, const uint32_t* __restrict__ seen_masks,
     const uint32_t* __restrict__ banned, int mask_words, const float* __restrict__ part_max,
     float* __restrict__ part_mass) {
@@ -578,8 +578,7 @@ __global__ __launch_bounds__(SIMPLE_THREADS) void simple_mass_kernel(
     const int r = blockIdx.y, chunk = blockIdx.x, chunks = gridDim.x;
     const float temp = temperature ? temperature[r] : 0.f;
     if (!(temp > 0.f)) return;   // the largest logit wins: no mass is asked for
-    const float p = top_p ? top_p[r] : 0.f;
-    if ((top_k && top_k[r] > 0) || (p > 0.f && p < 1.f)) return;   // not a row that draws from the whole vocabulary
+    if (top_k && top_k[r] > 0) return;   // what top-k keeps is weighed on the short list
     const float best = simple_row_max(part_max + r * chunks, chunks);
     if (best == -INFINITY) return;
     const float inv_t = 1.0f / temp;
@@ -611,18 +610,28 @@ __global__ __launch_bounds__(SIMPLE_THREADS) void simple_mass_kernel(
 // skips the rows that are done.
 constexpr int TOPK_SEGMENT = 32;   // candidates a chunk may leave
 
+// A row with top-p alone takes the same way with what lies at or above one of the lower chunk maxima (seven eighths
+// of the chunks have a larger one): some hundreds of the largest logits of a vocabulary of 150,000, which hold the
+// top_p share of a distribution as peaked as a language model's; if they do not (or a chunk has more than its segment
+// holds), the row is left to sample_kernel too.  The mass of the whole row, which top_p refers to, comes from
+// simple_mass_kernel.
+__device__ __forceinline__ int top_p_bound_rank(int chunks) { return max(1, chunks - chunks / 8); }
+
 __global__ __launch_bounds__(SIMPLE_THREADS) void topk_collect_kernel(
     const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ temperature,
-    const int* __restrict__ top_k, const float* __restrict__ penalty, const int* __restrict__ seen_row,
-    const uint32_t* __restrict__ seen_masks, const uint32_t* __restrict__ banned, int mask_words,
-    const float* __restrict__ part_max, int* __restrict__ seg_i, float* __restrict__ seg_x, int* __restrict__ seg_n) {
+    const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ penalty,
+    const int* __restrict__ seen_row, const uint32_t* __restrict__ seen_masks, const uint32_t* __restrict__ banned,
+    int mask_words, const float* __restrict__ part_max, int* __restrict__ seg_i, float* __restrict__ seg_x,
+    int* __restrict__ seg_n) {
     constexpr int WAVES = SIMPLE_THREADS / PULSE_WAVE;
     constexpr int PER = SIMPLE_CHUNK / SIMPLE_THREADS;   // consecutive logits a thread takes
     __shared__ float s_bound;
     __shared__ int s_count[WAVES];
     const int r = blockIdx.y, chunk = blockIdx.x, chunks = gridDim.x;
     const int lane = threadIdx.x % PULSE_WAVE, wave = threadIdx.x / PULSE_WAVE;
-    const int k = top_k ? top_k[r] : 0;
+    int k = top_k ? top_k[r] : 0;
+    const float p = top_p ? top_p[r] : 0.f;
+    if (k <= 0 && p > 0.f && p < 1.f) k = top_p_bound_rank(chunks);   // top-p alone: see top_p_bound_rank
     const float temp = temperature ? temperature[r] : 0.f;
     int* my_n = seg_n + r * chunks + chunk;
     if (!(temp > 0.f) || k <= 0 || k > chunks || chunks > 2 * PULSE_WAVE) {   // greedy rows need no candidates; the others are not for these kernels
@@ -697,7 +706,7 @@ __global__ __launch_bounds__(SIMPLE_THREADS) void topk_collect_kernel(
 // The choice of every row from what the kernels before left, a wavefront a row: the largest logit for greedy rows;
 // for rows with top-k the candidates' segments strung together in LDS and finished there; for rows that draw from the
 // whole vocabulary the chunk in which u * mass falls (chunk masses in chunk order), walked alone.  done[r] says
-// whether the row's token is chosen; the others (top-p alone, or a row that did not fit) are sample_kernel's.
+// whether the row's token is chosen; the others (rows that did not fit) are sample_kernel's.
 __global__ __launch_bounds__(PULSE_WAVE) void chunked_choose_kernel(
     const float* __restrict__ logits, int vocab, int64_t row_stride, const float* __restrict__ temperature,
     const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ uniform,
@@ -736,7 +745,8 @@ __global__ __launch_bounds__(PULSE_WAVE) void chunked_choose_kernel(
     const float p = top_p ? top_p[r] : 0.f;
     const bool use_p = p > 0.f && p < 1.f;
     const float inv_t = 1.0f / temp;
-    if (k > 0) {
+    if (k > 0 || use_p) {
+        const bool by_k = k > 0;
         // the segments' places in the list: an exclusive sum over the chunks, in chunk order (two chunks a lane)
         const int n0 = lane < chunks ? seg_n[lane] : 0, n1 = lane + PULSE_WAVE < chunks ? seg_n[lane + PULSE_WAVE] : 0;
         const bool over = n0 > TOPK_SEGMENT || n1 > TOPK_SEGMENT;
@@ -748,9 +758,15 @@ __global__ __launch_bounds__(PULSE_WAVE) void chunked_choose_kernel(
         }
         const int first = __shfl(pre0, PULSE_WAVE - 1, PULSE_WAVE);      // candidates of chunks 0 .. 63
         const int n = first + __shfl(pre1, PULSE_WAVE - 1, PULSE_WAVE);
-        if (k > chunks || chunks > 2 * PULSE_WAVE || __ballot(over) != 0ull || n > LIST_CAP || n < k) {
+        if (k > chunks || chunks > 2 * PULSE_WAVE || __ballot(over) != 0ull || n > LIST_CAP || n < k || n == 0) {
             if (lane == 0) done[r] = 0;   // not a row for these kernels: sample_kernel takes it
             return;
+        }
+        float whole = 0.f;   // without top-k: the mass of the whole row, chunk masses in chunk order
+        if (!by_k) {
+            for (int c = lane; c < chunks; c += PULSE_WAVE) whole += part_mass[c];
+#pragma unroll
+            for (int off = PULSE_WAVE / 2; off > 0; off >>= 1) whole += __shfl_xor(whole, off, PULSE_WAVE);
         }
         const int64_t seg0 = (static_cast<int64_t>(r) * chunks + lane) * TOPK_SEGMENT;
         for (int e = 0; e < n0; ++e) { list_i[pre0 - n0 + e] = seg_i[seg0 + e]; list_x[pre0 - n0 + e] = seg_x[seg0 + e]; }
@@ -758,15 +774,14 @@ __global__ __launch_bounds__(PULSE_WAVE) void chunked_choose_kernel(
         for (int e = 0; e < n1; ++e) { list_i[first + pre1 - n1 + e] = seg_i[seg1 + e]; list_x[first + pre1 - n1 + e] = seg_x[seg1 + e]; }
         __syncthreads();
         int token;
-        if (n <= 4 * PULSE_WAVE)   // the usual case: a few dozen candidates, a few a lane
-            finish_on_list<4>(list_i, list_x, n, true, k, use_p, p, 0.f, best, inv_t, uniform[r], best_i, token);
-        else
-            finish_on_list<LIST_PER_LANE>(list_i, list_x, n, true, k, use_p, p, 0.f, best, inv_t, uniform[r], best_i, token);
-        if (lane == 0) { out[r] = token; done[r] = 1; }
-        return;
-    }
-    if (use_p) {   // top-p alone: the set it keeps has no bound that these kernels could use
-        if (lane == 0) done[r] = 0;
+        const bool enough =   // (false only without top-k: the list does not hold top_p of the row)
+            n <= 4 * PULSE_WAVE   // the usual case with top-k: a few dozen candidates, a few a lane
+                ? finish_on_list<4>(list_i, list_x, n, by_k, k, use_p, p, whole, best, inv_t, uniform[r], best_i, token)
+                : finish_on_list<LIST_PER_LANE>(list_i, list_x, n, by_k, k, use_p, p, whole, best, inv_t, uniform[r], best_i, token);
+        if (lane == 0) {
+            if (enough) out[r] = token;
+            done[r] = enough ? 1 : 0;
+        }
         return;
     }
     // a draw from the whole vocabulary: the chunk in which it falls, chunk masses in chunk order
@@ -893,9 +908,10 @@ extern "C" int pulse_sample(const float* logits, int rows, int vocab, int64_t ro
 
 // The same in chunks of the vocabulary with a workgroup each, which reads a row many times faster than the
 // workgroup a row of pulse_sample does.  Greedy rows, rows that draw from the whole vocabulary at their temperature
-// and rows with top-k (and top-p on what it keeps) whose k is at most the number of chunks are chosen by these
-// kernels; rows with top-p alone, and rows that do not fit (many equal values around the k-th largest), by the kernel
-// of pulse_sample behind them, which skips the rows that are done.  What a row's choice is does not depend on the
+// rows with top-k (and top-p on what it keeps) whose k is at most the number of chunks and rows with top-p alone whose
+// top_p share lies in some hundreds of the largest logits are chosen by these kernels; rows that do not fit (many
+// equal values around the k-th largest, a distribution too flat for top-p alone) by the kernel of pulse_sample behind
+// them, which skips the rows that are done.  What a row's choice is does not depend on the
 // other rows.  Scratch, with chunks = pulse_sample_chunks(vocab): part_max, part_mass (float32), part_idx, seg_n
 // (int32) of rows * chunks entries; seg_i (int32), seg_x (float32) of rows * chunks * pulse_sample_segment()
 // entries; done (int32) of rows entries.
@@ -921,13 +937,13 @@ extern "C" int pulse_sample_chunked(const float* logits, int rows, int vocab, in
     PULSE_LAUNCH_CHECK("sample_chunked (maxima)");
     if (temperature) {
         hipLaunchKernelGGL(simple_mass_kernel, dim3(chunks, rows), dim3(SIMPLE_THREADS), 0, stream, logits, vocab,
-                           row_stride, temperature, top_k, top_p, penalty, seen_row, seen_masks, banned, mask_words,
+                           row_stride, temperature, top_k, penalty, seen_row, seen_masks, banned, mask_words,
                            part_max, part_mass);
         PULSE_LAUNCH_CHECK("sample_chunked (masses)");
-        if (top_k) {
+        if (top_k || top_p) {
             hipLaunchKernelGGL(topk_collect_kernel, dim3(chunks, rows), dim3(SIMPLE_THREADS), 0, stream, logits, vocab,
-                               row_stride, temperature, top_k, penalty, seen_row, seen_masks, banned, mask_words, part_max,
-                               seg_i, seg_x, seg_n);
+                               row_stride, temperature, top_k, top_p, penalty, seen_row, seen_masks, banned, mask_words,
+                               part_max, seg_i, seg_x, seg_n);
             PULSE_LAUNCH_CHECK("sample_chunked (candidates)");
         }
     }

@@ -345,9 +345,11 @@ def test_top_k_top_p_penalty_and_banned(k):
     ("temperature", 151936, False), ("top_k", 151936, False), ("top_k_top_p", 151936, False), ("top_p", 151936, False),
     ("top_p_peaked", 151936, False), ("ties", 151936, False), ("many_ties", 151936, False), ("penalty", 151936, False),
     # candidates found in chunks of the vocabulary: rows that fit, rows with too many equal values (left to the kernel
-    # with a workgroup a row), a vocabulary of fewer chunks than k (the same), one of barely more
+    # with a workgroup a row), a vocabulary of fewer chunks than k (the same), one of barely more; top-p alone on
+    # peaked rows (the short list holds its share) and on flat ones (it does not)
     ("top_k", 151936, True), ("top_k_top_p", 151936, True), ("ties", 151936, True), ("many_ties", 151936, True),
-    ("penalty", 151936, True), ("temperature", 151936, True), ("top_p", 151936, True),
+    ("penalty", 151936, True), ("temperature", 151936, True), ("top_p", 151936, True), ("top_p_peaked", 151936, True),
+    ("top_p_flat", 151936, True), ("top_p_peaked", 43000, True),
     ("top_k", 5000, True), ("top_k_top_p", 43000, True), ("top_k", 2048 * 20, True)])
 def test_sampling_at_a_real_vocabulary(k, mode, vocab, chunked):
     """The draw of every row against the same steps in float64: kept set by thresholds (top-k, then top-p on what
@@ -357,12 +359,12 @@ def test_sampling_at_a_real_vocabulary(k, mode, vocab, chunked):
     gen = torch.Generator().manual_seed(11)
     # flat enough that top-p alone needs thousands of tokens (the passes over the whole vocabulary), or peaked so that
     # a thousand hold its mass (the short list)
-    logits = torch.randn(rows, vocab, generator=gen) * (8.0 if mode == "top_p_peaked" else 2.5)
+    logits = torch.randn(rows, vocab, generator=gen) * {"top_p_peaked": 8.0, "top_p_flat": 0.5}.get(mode, 2.5)
     if mode in ("ties", "many_ties"):        # the k-th largest value many times: all of its copies are kept
         logits[:, ::(97 if mode == "ties" else 40)] = 20.0
     temp = 0.7
     top_k = {"top_k": 20, "top_k_top_p": 50, "ties": 40, "many_ties": 40, "penalty": 20}.get(mode, 0)
-    top_p = {"top_k_top_p": 0.9, "top_p": 0.8, "top_p_peaked": 0.9, "penalty": 0.95}.get(mode, 0.0)
+    top_p = {"top_k_top_p": 0.9, "top_p": 0.8, "top_p_peaked": 0.9, "top_p_flat": 0.9, "penalty": 0.95}.get(mode, 0.0)
     uniform = torch.rand(rows, generator=gen)
     dev = lambda t: t.to(DEV)
     kw = dict(temperature=dev(torch.full((rows,), temp)), uniform=dev(uniform))
@@ -386,10 +388,11 @@ def test_sampling_at_a_real_vocabulary(k, mode, vocab, chunked):
             return k.sample(logits_dev, out_dev, **args)
         scratch = _chunked_scratch(k, out_dev.numel(), vocab)
         k.sample_chunked(logits_dev, out_dev, scratch, **args)
-        if mode in ("top_k", "top_k_top_p", "penalty", "ties", "temperature") and vocab >= 2048 * 50:
+        if mode in ("top_k", "top_k_top_p", "penalty", "ties", "temperature", "top_p_peaked") and vocab >= 2048 * 50:
             assert bool((scratch["done"][: out_dev.numel()] == 1).all())     # these rows fit: no row was left over
-        if mode in ("many_ties", "top_p") or vocab == 5000:
-            assert bool((scratch["done"][: out_dev.numel()] == 0).all())     # and these did not
+        if mode in ("many_ties", "top_p_flat") or vocab == 5000:
+            assert bool((scratch["done"][: out_dev.numel()] == 0).all())     # and these did not (top-p alone on a flat
+                                                                             # row: thousands of tokens hold its share)
 
     draw(dev(logits), out, **kw)
     got = out.cpu().tolist()
@@ -514,7 +517,8 @@ def test_rows_of_every_kind_in_one_step_draw_what_they_draw_alone(k, vocab):
     k.sample_chunked(dev(logits), out, scratch, temperature=dev(temp), top_k=dev(top_k), top_p=dev(top_p),
                      uniform=dev(uniform))
     got = out.cpu().tolist()
-    assert scratch["done"].cpu().tolist() == [1] * 16 + [0] * 8
+    done = scratch["done"].cpu().tolist()
+    assert done[:16] == [1] * 16 and done[20:] == [0] * 4       # (top-p alone, rows 16 to 19: as the row's shape has it)
     for r in range(rows):
         alone = torch.empty(1, dtype=torch.int32, device=DEV)
         kw = dict(temperature=dev(temp[r:r + 1]), uniform=dev(uniform[r:r + 1]))
