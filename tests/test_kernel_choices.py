@@ -35,6 +35,35 @@ def test_decode_splits_cover_the_context_in_whole_blocks(units):
     assert n == 1
 
 
+def test_a_plan_for_uneven_contexts_has_room_for_every_pair(units):
+    from pulse_infer_amd.ops import attention_mfma as M
+
+    for nkv, group in ((8, 4), (1, 6), (2, 20), (16, 1)):
+        slots, first = M.plan_slots(nkv, group)
+        heads = nkv * ((group + 15) // 16)
+        assert first >= 1 and slots == 2 * first and first * heads <= max(units, heads)   # one round fills the units once
+    for items, splits in ((1, 8), (64, 8), (128, 8), (200, 5), (1024, 1)):
+        assert M.plan_fits(items, splits)
+        assert M.plan_ints(items, splits) == 1 + items * splits + items                    # count, pairs, split sizes
+    assert not M.plan_fits(129, 8) and not M.plan_fits(0, 8)
+
+
+def test_a_step_counts_as_uneven_by_its_longest_context_over_the_mean():
+    from pulse_infer_amd.parts.base import UNEVEN_CONTEXTS, EntryMeta, contexts_uneven
+
+    def metas(contexts):
+        return [EntryMeta(i, i, c - 1, 1, i) for i, c in enumerate(contexts)]
+
+    assert not contexts_uneven(metas([4096] * 8))
+    assert not contexts_uneven(metas([9000, 10]))                     # two requests: nothing to order
+    assert contexts_uneven(metas([4096, 200, 200, 200]))
+    assert contexts_uneven(metas([1500, 1000, 500]))                  # exactly 1.5 times the mean
+    assert not contexts_uneven(metas([1499, 1000, 500]))
+    assert UNEVEN_CONTEXTS == 1.5
+    # portions count with what they bring: a context is start + count
+    assert contexts_uneven([EntryMeta(0, 0, 0, 900, 0), EntryMeta(1, 1, 99, 1, 900), EntryMeta(2, 2, 49, 1, 901)])
+
+
 def test_prefill_splits_are_chosen_for_long_walks(units):
     from pulse_infer_amd.ops import attention_mfma as M
 
