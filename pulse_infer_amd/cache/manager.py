@@ -105,6 +105,8 @@ class _Request:
     slot: int
     computed: int = 0   # tokens whose keys are in the cache
     reserved: int = 0   # tokens that pages are reserved for
+    capacity: int = 0   # tokens that the pages it has can hold (the fewest over the groups)
+    stamp: int = 0      # changes whenever one of its block tables does (never the same for two requests)
 
 
 class CacheManager:
@@ -140,6 +142,11 @@ class CacheManager:
         self.requests: Dict[Hashable, _Request] = {}
         self.state: Dict[int, object] = {}  # run -> [slots, *shape] array
         self.max_requests = int(max_requests)
+        self._clock = 0     # source of the requests' stamps
+
+    def _tick(self) -> int:
+        self._clock += 1
+        return self._clock
 
     # ------------------------------------------------------------------ storage
     def allocate_storage(self, device, dtype) -> None:
@@ -163,7 +170,7 @@ class CacheManager:
         if request in self.requests:
             raise CacheError(f"request {request!r} is already live")
         slot = self.slots.take(request)
-        self.requests[request] = _Request(slot)
+        self.requests[request] = _Request(slot, stamp=self._tick())
         for g in self.groups:
             g.tables[request] = []
         return slot
@@ -179,6 +186,12 @@ class CacheManager:
 
     def reserved(self, request: Hashable) -> int:
         return self._req(request).reserved
+
+    def tables_stamp(self, request: Hashable) -> int:
+        """A number that changes whenever a block table of the request changes (a page more, pages given back below
+        a window) and that no other request, before or after, has had: who copies the tables elsewhere can tell by
+        it whether the copy still holds."""
+        return self._req(request).stamp
 
     def _req(self, request: Hashable) -> _Request:
         try:
@@ -196,6 +209,9 @@ class CacheManager:
         return [g.pages_for(length) for g in self.groups]
 
     def can_reserve(self, request: Optional[Hashable], length: int, spare: Optional[List[int]] = None) -> bool:
+        live = self.requests.get(request) if request is not None else None
+        if live is not None and length <= live.capacity:
+            return True      # the pages it has hold that many tokens
         need = self.pages_needed(request, length) if request in self.requests else self.pages_needed_new(length)
         free = spare if spare is not None else [g.pool.num_free for g in self.groups]
         return all(n <= f for n, f in zip(need, free))
@@ -206,6 +222,9 @@ class CacheManager:
     def reserve(self, request: Hashable, length: int) -> None:
         """Make sure pages exist for tokens [0, length) in every group; all or nothing."""
         req = self._req(request)
+        if length <= req.capacity:   # the pages it has hold that many tokens
+            req.reserved = max(req.reserved, length)
+            return
         need = self.pages_needed(request, length)
         for g, n in zip(self.groups, need):
             if n > g.pool.num_free:
@@ -214,6 +233,8 @@ class CacheManager:
         for g, n in zip(self.groups, need):
             g.tables[request].extend(g.pool.allocate(n))
         req.reserved = max(req.reserved, length)
+        req.capacity = min((len(g.tables[request]) * g.page_size for g in self.groups), default=1 << 62)
+        req.stamp = self._tick()
 
     def advance(self, request: Hashable, computed: int) -> None:
         """Tokens [0, computed) are now in the cache; give back pages that a window has passed."""
@@ -233,6 +254,7 @@ class CacheManager:
                 g.pool.release(gone)
                 for i in range(dead):
                     table[i] = -1
+                req.stamp = self._tick()
 
     def free_request(self, request: Hashable) -> None:
         """Give back everything the request holds (finish or preemption)."""

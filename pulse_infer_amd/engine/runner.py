@@ -80,6 +80,7 @@ class _Captured:
     workspace: Any = None
     context: Any = None   # kept alive: the graph reads tensors that the context's parts created (work lists, tables)
     event: Any = None
+    row_stamps: Any = None   # per row of the block tables: the stamp of the request's tables when the row was written
 
     def wait(self) -> None:
         if self.event is not None:
@@ -194,6 +195,29 @@ class ModelRunner:
             flat[offsets[8 + gi]:offsets[9 + gi]] = table.reshape(-1)
         flat[offsets[8 + len(widths)]] = max(m.start + m.count for m in metas)
 
+    def _refill(self, rec: "_Captured", entries: Sequence[StepEntry], metas: List[EntryMeta]) -> None:
+        """The integers of a step of single tokens in a recording's buffer: only what changes from one such step to
+        the next (ids, positions, slots, the longest context) and the block-table rows of requests whose tables have
+        changed since the row was written (a request gets a page every ``page_size`` steps).  Token-to-entry map,
+        counts, first rows and wanted rows are the same for every step of the recording's batch size."""
+        flat, o, cache = rec.host_np, rec.offsets, self.cache
+        starts = [m.start for m in metas]
+        flat[o[0]:o[1]] = [e.tokens[0] for e in entries]
+        flat[o[1]:o[2]] = starts
+        flat[o[3]:o[4]] = starts
+        flat[o[6]:o[7]] = [m.slot for m in metas]
+        stamps = rec.row_stamps
+        for i, m in enumerate(metas):
+            stamp = cache.tables_stamp(m.request)
+            if stamps[i] != stamp:
+                stamps[i] = stamp
+                for gi, w in enumerate(rec.widths):
+                    pages = cache.table(gi, m.request)[:w]
+                    at = int(o[8 + gi]) + i * w
+                    flat[at:at + len(pages)] = pages
+                    flat[at + len(pages):at + w] = -1
+        flat[o[8 + len(rec.widths)]] = max(starts) + 1
+
     def _context(self, dev: torch.Tensor, offsets: np.ndarray, metas: List[EntryMeta], wanted: int,
                  widths: Sequence[int], workspace, max_context: int, uneven: bool) -> StepContext:
         total, batch = metas[-1].first_row + metas[-1].count, len(metas)
@@ -286,7 +310,7 @@ class ModelRunner:
                 self._graphs.pop(next(iter(self._graphs)))
             return logits
         rec.wait()
-        self._fill(rec.host_np, rec.offsets, entries, metas, want_rows, rec.widths)
+        self._refill(rec, entries, metas)
         rec.dev.copy_(rec.host, non_blocking=True)
         rec.graph.replay()
         rec.mark()
@@ -306,6 +330,7 @@ class ModelRunner:
         workspace = Workspace(self.device)
         ctx = self._context(dev, offsets, metas, batch, widths, workspace, bucket, uneven)
         self._fill(rec.host_np, offsets, entries, metas, want_rows, widths)
+        rec.row_stamps = [self.cache.tables_stamp(m.request) for m in metas]
         dev.copy_(host, non_blocking=True)
         # the step itself, eagerly: it sizes the workspace and lets parts build what depends only on the step's shape
         from ..parts import linear

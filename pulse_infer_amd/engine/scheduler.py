@@ -172,12 +172,19 @@ class ContinuousBatchScheduler:
     def _fill(self, batch: ScheduledBatch) -> None:
         """One pass of the three phases, adding to ``batch``."""
         budget = self.max_num_batched_tokens
+        # who decodes and who is in a prompt (or is being recomputed), looked at once: in order of admission
+        decoding: List[InferenceRequest] = []
+        prompting: List[InferenceRequest] = []
+        for request in self.running:
+            pending = request.num_pending_tokens
+            if pending == 1 and not request.is_prefill:
+                decoding.append(request)
+            elif pending >= 1:
+                prompting.append(request)
 
         # 1. running requests that decode: one token each, preempting the newest when pages run out
-        for request in list(self.running):
-            if request not in self.running:  # preempted a moment ago
-                continue
-            if request.num_pending_tokens != 1 or request.is_prefill:
+        for request in decoding:
+            if request.state is not RequestState.RUNNING:  # preempted a moment ago
                 continue
             if budget <= 0 or batch.batch_size() >= self.max_batch_size:
                 break
@@ -201,13 +208,11 @@ class ContinuousBatchScheduler:
             budget -= 1
 
         # 2. running requests with more than one pending token (prefill, or recomputation after preemption)
-        for request in list(self.running):
-            if request.num_pending_tokens < 1 or (request.num_pending_tokens == 1 and not request.is_prefill):
+        for request in prompting:
+            if request.state is not RequestState.RUNNING:
                 continue
             if budget <= 0 or batch.batch_size() >= self.max_batch_size:
                 break
-            if any(p.request is request for p in batch.portions):
-                continue
             want = min(self.chunk_size, request.num_pending_tokens, budget)
             count = self._largest_fitting(request, want)
             if count <= 0:
@@ -247,6 +252,8 @@ class ContinuousBatchScheduler:
         for i, portion in enumerate(batch.portions):
             if budget <= 0:
                 break
+            if portion.samples:   # it brings all that its request has pending
+                continue
             request, have = portion.request, len(portion.tokens)
             more = min(request.num_pending_tokens - have, budget)
             if more <= 0:
