@@ -97,6 +97,43 @@ def test_window_pages_are_given_back_as_the_window_passes():
     assert m.groups[0].pool.num_free == 6
 
 
+def test_a_stamp_tells_when_a_requests_tables_have_changed():
+    """Who keeps a copy of a request's block tables (a recorded step's buffer) compares stamps: the stamp moves with
+    every page taken and every page given back below a window, stays while a reservation fits the pages that are
+    there, and is never that of another request, not even of a later one with the same name."""
+    m = CacheManager([FULL, WIN], page_size=4, num_pages=12, max_requests=2)
+    m.add_request("a")
+    m.add_request("b")
+    seen = {m.tables_stamp("a"), m.tables_stamp("b")}
+    assert len(seen) == 2
+    m.reserve("a", 3)
+    first = m.tables_stamp("a")
+    assert first not in seen and m.table(0, "a") != []
+    seen.add(first)
+    free = m.free_pages()
+    for length in (4, 2, 4):                      # inside the page it has: nothing is taken, nothing changes
+        assert m.can_reserve("a", length)
+        m.reserve("a", length)
+        assert m.tables_stamp("a") == first and m.free_pages() == free
+    assert m.reserved("a") == 4
+    m.reserve("a", 5)                             # a second page in both groups
+    second = m.tables_stamp("a")
+    assert second not in seen and m.free_pages() == [f - 1 for f in free]
+    seen.add(second)
+    m.reserve("a", 16)
+    seen.add(m.tables_stamp("a"))
+    m.advance("a", 8)                             # the window (10 keys) still reaches the first page
+    before = m.tables_stamp("a")
+    m.advance("a", 14)                            # now it does not: the window group's first page goes back
+    assert m.table(1, "a")[0] == -1 and m.tables_stamp("a") != before and m.tables_stamp("a") not in seen
+    seen.add(m.tables_stamp("a"))
+    assert m.tables_stamp("b") in seen            # b was never touched
+    m.free_request("a")
+    m.add_request("a")
+    assert m.tables_stamp("a") not in seen and not m.can_reserve("a", 4 * 12 + 1) and m.can_reserve("a", 4)
+    m.check()
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_random_orders_keep_every_page_accounted_for(seed):
     rng = random.Random(seed)
