@@ -138,26 +138,31 @@ class ModelRunner:
         self.cache.reserve(request, length)
 
     # --------------------------------------------------------------------- step
-    def _check(self, entries: Sequence[StepEntry]) -> None:
+    def _check(self, entries: Sequence[StepEntry]) -> List[EntryMeta]:
+        """Refuses what a step cannot run; returns every entry's share of the step."""
         if not entries:
             raise StepError("a step needs at least one entry")
         seen = set()
         vocab = self.model.vocab_size
+        live = self.cache.requests
+        metas: List[EntryMeta] = []
+        row = 0
         for e in entries:
             if e.request in seen:
                 raise StepError(f"request {e.request!r} appears twice in one step")
             seen.add(e.request)
-            if not self.cache.has_request(e.request):
+            held = live.get(e.request)
+            if held is None:
                 raise StepError(f"request {e.request!r} is not live (add_request first)")
             n = len(e.tokens)
             if n == 0:
                 raise StepError(f"request {e.request!r} brings no tokens")
-            start = self.cache.computed(e.request)
+            start = held.computed
             if start + n > self.max_positions:
                 raise StepError(f"request {e.request!r} would reach position {start + n - 1}, the model allows "
                                 f"{self.max_positions} positions")
-            if self.cache.reserved(e.request) < start + n:
-                raise StepError(f"request {e.request!r}: pages are reserved for {self.cache.reserved(e.request)} "
+            if held.reserved < start + n:
+                raise StepError(f"request {e.request!r}: pages are reserved for {held.reserved} "
                                 f"tokens, the step needs {start + n}")
             if min(e.tokens) < 0 or max(e.tokens) >= vocab:
                 bad = next(tok for tok in e.tokens if not 0 <= int(tok) < vocab)
@@ -165,6 +170,9 @@ class ModelRunner:
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise StepError(f"request {e.request!r}: wanted place {w} is outside its {n} tokens")
+            metas.append(EntryMeta(e.request, held.slot, start, n, row))
+            row += n
+        return metas
 
     def _layout(self, total: int, batch: int, wanted: int, widths: Sequence[int]) -> np.ndarray:
         """Offsets of the step's integer arrays in one flat buffer:
@@ -234,14 +242,9 @@ class ModelRunner:
                                                    # that holds it alive in a circle that only the collector ends)
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        self._check(entries)
+        metas = self._check(entries)
         cache = self.cache
-        metas: List[EntryMeta] = []
-        row = 0
-        for e in entries:
-            metas.append(EntryMeta(e.request, cache.slot_of(e.request), cache.computed(e.request), len(e.tokens), row))
-            row += len(e.tokens)
-        total = row
+        total = metas[-1].first_row + metas[-1].count
         want_rows = [m.first_row + int(w) for e, m in zip(entries, metas) for w in e.want]
         max_context = max(m.start + m.count for m in metas)
         uneven = contexts_uneven(metas)
