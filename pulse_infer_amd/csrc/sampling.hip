@@ -119,24 +119,35 @@ __device__ void block_argmax(float& v, int& idx, float* sv, int* si) {
 template <typename Weight>
 __device__ int wave_walk(int begin, int end, float rest, Weight weight, int& last) {
     const int lane = threadIdx.x % PULSE_WAVE;
+    constexpr int AHEAD = 8;   // steps of 64 entries whose weights are asked for together (a step's trip to memory
+                               // would otherwise be waited for before the next one starts)
     float run = 0.f;
     last = -1;
-    for (int base = begin; base < end; base += PULSE_WAVE) {
-        const int i = base + lane;
-        const float w = i < end ? weight(i) : 0.f;
-        const unsigned long long has = __ballot(w > 0.f);
-        if (has == 0ull) continue;
-        last = base + (63 - __builtin_clzll(has));
-        // inclusive prefix over the lanes, in lane order
-        float pre = w;
+    for (int first = begin; first < end; first += AHEAD * PULSE_WAVE) {
+        float ws[AHEAD];
 #pragma unroll
-        for (int off = 1; off < PULSE_WAVE; off <<= 1) {
-            const float up = __shfl_up(pre, off, PULSE_WAVE);
-            if (lane >= off) pre += up;
+        for (int u = 0; u < AHEAD; ++u) {
+            const int i = first + u * PULSE_WAVE + lane;
+            ws[u] = i < end ? weight(i) : 0.f;
         }
-        const unsigned long long hit = __ballot(w > 0.f && rest < run + pre);
-        if (hit != 0ull) return base + __builtin_ctzll(hit);
-        run += __shfl(pre, PULSE_WAVE - 1, PULSE_WAVE);
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) {
+            const int base = first + u * PULSE_WAVE;
+            const float w = ws[u];
+            const unsigned long long has = __ballot(w > 0.f);
+            if (has == 0ull) continue;
+            last = base + (63 - __builtin_clzll(has));
+            // inclusive prefix over the lanes, in lane order
+            float pre = w;
+#pragma unroll
+            for (int off = 1; off < PULSE_WAVE; off <<= 1) {
+                const float up = __shfl_up(pre, off, PULSE_WAVE);
+                if (lane >= off) pre += up;
+            }
+            const unsigned long long hit = __ballot(w > 0.f && rest < run + pre);
+            if (hit != 0ull) return base + __builtin_ctzll(hit);
+            run += __shfl(pre, PULSE_WAVE - 1, PULSE_WAVE);
+        }
     }
     return -1;
 }
@@ -638,6 +649,15 @@ __global__ __launch_bounds__(SIMPLE_THREADS) void topk_collect_kernel(
         if (threadIdx.x == 0) *my_n = 0;
         return;
     }
+    // the chunk's logits are asked for first: they travel while the bound is searched
+    const RowView row = simple_row(logits, r, row_stride, vocab, penalty, seen_row, seen_masks, banned, mask_words);
+    const int begin = chunk * SIMPLE_CHUNK + static_cast<int>(threadIdx.x) * PER;
+    float xs[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = begin + j;
+        xs[j] = i < vocab ? row.at(i) : -INFINITY;
+    }
     // the k-th largest of the chunks' maxima, bit by bit (chunks <= 2 * 64: two a lane)
     if (wave == 0) {
         uint32_t keys[2];
@@ -667,16 +687,9 @@ __global__ __launch_bounds__(SIMPLE_THREADS) void topk_collect_kernel(
     }
     __syncthreads();
     const float bound = s_bound;
-    const RowView row = simple_row(logits, r, row_stride, vocab, penalty, seen_row, seen_masks, banned, mask_words);
-    const int begin = chunk * SIMPLE_CHUNK + static_cast<int>(threadIdx.x) * PER;
-    float xs[PER];
     int mine = 0;
 #pragma unroll
-    for (int j = 0; j < PER; ++j) {
-        const int i = begin + j;
-        xs[j] = i < vocab ? row.at(i) : -INFINITY;
-        mine += (xs[j] != -INFINITY && xs[j] >= bound) ? 1 : 0;
-    }
+    for (int j = 0; j < PER; ++j) mine += (xs[j] != -INFINITY && xs[j] >= bound) ? 1 : 0;
     // where this thread's candidates go: an exclusive sum over the threads, in thread order (vocabulary order)
     int pre = mine;
 #pragma unroll
@@ -792,13 +805,19 @@ __global__ __launch_bounds__(PULSE_WAVE) void chunked_choose_kernel(
     const float target = uniform[r] * total;
     float run = 0.f;
     int who = -1, last_chunk = -1;
-    for (int c = 0; c < chunks; ++c) {   // (every lane the same few dozen additions)
-        const float m = part_mass[c];
-        if (m > 0.f) {
-            last_chunk = c;
-            if (target < run + m) { who = c; break; }
+    // (every lane the same few dozen additions; the masses come 64 at a time, one a lane, so that the additions do
+    // not each wait for a trip to memory)
+    for (int base = 0; base < chunks && who < 0; base += PULSE_WAVE) {
+        const float mine = base + lane < chunks ? part_mass[base + lane] : 0.f;
+        const int n = min(PULSE_WAVE, chunks - base);
+        for (int j = 0; j < n; ++j) {
+            const float m = __shfl(mine, j, PULSE_WAVE);
+            if (m > 0.f) {
+                last_chunk = base + j;
+                if (target < run + m) { who = base + j; break; }
+            }
+            run += m;
         }
-        run += m;
     }
     float rest = target - run;
     if (who < 0) {  // rounding left the target beyond the last chunk with mass: its last kept entry
