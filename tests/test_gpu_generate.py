@@ -128,6 +128,21 @@ def test_seeded_sampling_does_not_depend_on_the_batch(gpu, model_folders):
     other = make_llm(model_folders["B"], max_batch_size=3, chunk_size=16, page_size=page, num_pages=32).generate(
         prompts, max_new_tokens=12, sampling=[SamplingParams(temperature=0.8, seed=900 + i, ignore_eos=True) for i in range(3)])
     assert other != together                                          # another seed, another path
+    # requests with options of different kinds in one batch: each draws what it draws alone (which kernels choose a
+    # row's token depends on the row's own options)
+    kinds = [SamplingParams(temperature=0.9, seed=31, ignore_eos=True),
+             SamplingParams(temperature=0.9, top_k=7, seed=32, ignore_eos=True),
+             SamplingParams(temperature=1.1, top_k=20, top_p=0.9, seed=33, ignore_eos=True),
+             SamplingParams(temperature=1.0, top_p=0.8, seed=34, ignore_eos=True),
+             SamplingParams(ignore_eos=True),
+             SamplingParams(temperature=0.7, presence_penalty=1.5, seed=36, ignore_eos=True)]
+    many = [token_ids(cfg["vocab_size"], n, seed=40 + n) for n in (6, 13, 3, 18, 8, 11)]
+    mixed = make_llm(model_folders["B"], max_batch_size=6, chunk_size=16, page_size=page, num_pages=48).generate(
+        many, max_new_tokens=10, sampling=kinds)
+    for i in range(6):
+        alone = make_llm(model_folders["B"], max_batch_size=1, chunk_size=16, page_size=page, num_pages=32).generate(
+            [many[i]], max_new_tokens=10, sampling=[kinds[i]])[0]
+        assert alone == mixed[i], i
     # temperature near zero is greedy; top_k = 1 is greedy whatever the temperature
     greedy = make_llm(model_folders["B"], page_size=page, num_pages=32).generate(prompts, max_new_tokens=6, ignore_eos=True)
     topk1 = make_llm(model_folders["B"], page_size=page, num_pages=32).generate(
