@@ -28,6 +28,8 @@ class Sampler:
         self._part_val: Optional[torch.Tensor] = None
         self._part_idx: Optional[torch.Tensor] = None
         self._chunked: Optional[dict] = None             # scratch of the sampling in chunks
+        self._options_host: Optional[torch.Tensor] = None  # pinned [6, rows] int32 and its device twin: a step's
+        self._options_dev: Optional[torch.Tensor] = None   # per-row options go up without the host waiting
         if banned_tokens:
             host = torch.zeros(self.words, dtype=torch.int64)
             for tok in banned_tokens:
@@ -69,7 +71,11 @@ class Sampler:
             return out.tolist()
         # every per-row option in one upload: rows of a [6, R] int32 array, the float ones as their bit patterns
         use_penalty = self.seen is not None and any(p.presence_penalty > 0.0 for p in params)
-        host = np.empty((6, rows), dtype=np.int32)
+        if self._options_host is None or self._options_host.shape[1] < rows:
+            self._options_host = torch.empty((6, max(rows, 64)), dtype=torch.int32, pin_memory=True)
+            self._options_dev = torch.empty((6, max(rows, 64)), dtype=torch.int32, device=self.device)
+        # (the last call's copy out of the pinned rows has finished: that call waited for its tokens)
+        host = self._options_host.numpy()[:, :rows]
         as_float = host.view(np.float32)
         as_float[0] = [p.temperature for p in params]
         host[1] = [p.top_k for p in params]
@@ -78,11 +84,12 @@ class Sampler:
                        for p, c, d in zip(params, counters, default_seeds)]
         as_float[4] = [p.presence_penalty for p in params]
         host[5] = [s if p.presence_penalty > 0.0 else -1 for p, s in zip(params, slots)]
-        dev = torch.from_numpy(host).to(self.device)
-        temperature, top_p, uniform = (dev[i].view(torch.float32) for i in (0, 2, 3))
-        top_k = dev[1]
-        penalty = dev[4].view(torch.float32) if use_penalty else None
-        seen_row = dev[5] if use_penalty else None
+        self._options_dev.copy_(self._options_host, non_blocking=True)
+        dev = self._options_dev
+        temperature, top_p, uniform = (dev[i, :rows].view(torch.float32) for i in (0, 2, 3))
+        top_k = dev[1, :rows]
+        penalty = dev[4, :rows].view(torch.float32) if use_penalty else None
+        seen_row = dev[5, :rows] if use_penalty else None
         seen = self.seen if penalty is not None else None
         # in chunks of the vocabulary; which way a row goes there depends on its own options alone, so a seeded
         # request draws the same tokens whatever else is in the batch.  An option that no row uses is left out
