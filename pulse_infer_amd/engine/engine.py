@@ -24,6 +24,18 @@ from .scheduler import ContinuousBatchScheduler, ScheduledBatch, Stats
 DEFAULT_MAX_SEQUENCES = 32  # reference: src/scheduler/continuous_batch_engine.cpp:73
 
 
+class _InFlight:
+    """A step that has been queued: who draws a token in it, where the tokens will be, and where they belong."""
+
+    def __init__(self, batch: ScheduledBatch, sampled: list, live: list):
+        self.batch, self.sampled, self.live = batch, sampled, live
+        self.tokens: Optional[torch.Tensor] = None    # int32 on the device, one a drawing request
+        self.rows: Dict[int, int] = {}                # request id -> its row of ``tokens``
+        self.landing: Optional[torch.Tensor] = None   # pinned host memory the tokens are copied to
+        self.landed: Optional[torch.cuda.Event] = None
+        self.places: list = []                        # (request, index in its generated tokens, row)
+
+
 class ContinuousBatchEngine:
     def __init__(self, model: Any, max_batch_size: int, chunk_size: int, *, page_size: int = 16,
                  num_pages: int = 1024, max_sequences: int = DEFAULT_MAX_SEQUENCES,
@@ -39,6 +51,8 @@ class ContinuousBatchEngine:
         self.eos_token_ids = list(eos_token_ids)
         self.seed = int(seed)
         self.last_batch: Optional[ScheduledBatch] = None
+        self._landing: List[Optional[torch.Tensor]] = [None, None]   # pinned buffers for a step's tokens, in turn
+        self._turn = 0
 
     # ------------------------------------------------------------------ intake
     def add_request(self, prompt_tokens: Sequence[int], max_new_tokens: int,
@@ -92,15 +106,130 @@ class ContinuousBatchEngine:
         self.scheduler.update_after_step(finished)
         return batch
 
-    def run_until_complete(self, print_progress: bool = False) -> None:
+    # ------------------------------------------------------- the loop, one step ahead
+    # ``step`` leaves the GPU idle while the host takes a step's tokens, decides the next step and fills its arrays.
+    # ``run_until_complete`` therefore runs one step ahead: step k is decided and queued while step k - 1 is still
+    # computed, with the tokens of step k - 1 fed to it on the device, and only then are those tokens waited for.
+    # What a step's tokens can change in the step after it is little: a request that drew an end-of-sequence id
+    # (or had no token left to draw) has one token too many computed, which is dropped; that it ends by its length
+    # is known without the token.  Every request draws what it draws with ``step``.
+    def _launch(self, batch: ScheduledBatch, before: Optional["_InFlight"]) -> "_InFlight":
+        """Queue a step and its sampling; nothing is waited for."""
+        cache = self.runner.cache
+        fed = before.rows if before is not None else {}
+        for request in batch.admitted:
+            slot = cache.slot_of(request.request_id)
+            tokens = request.prompt_tokens + request.generated_tokens
+            if request.request_id in fed:   # (preempted and admitted again at once: its last token is on the device)
+                self.sampler.start_request(slot, request.sampling, tokens[:-1])
+                if request.sampling.presence_penalty > 0.0:
+                    row = fed[request.request_id]
+                    self.sampler.note_on_device(self._ints([slot]), before.tokens[row:row + 1])
+            else:
+                self.sampler.start_request(slot, request.sampling, tokens)
+        entries, places, rows, at = [], [], [], 0
+        for p in batch.portions:
+            entries.append(StepEntry(p.request.request_id, p.tokens, [len(p.tokens) - 1] if p.samples else []))
+            at += len(p.tokens)
+            if p.request.request_id in fed and p.start + len(p.tokens) == p.request.total_input_tokens:
+                places.append(at - 1)       # the portion ends with the token that the step before drew
+                rows.append(fed[p.request.request_id])
+        logits = self.runner.step(entries, feed=(before.tokens, places, rows) if places else None)
+        self.scheduler.tokens_computed += batch.num_tokens()
+        sampled = [p for p in batch.portions if p.samples]
+        live = [(row, p.request) for row, p in enumerate(sampled) if p.request.can_generate_more]
+        flight = _InFlight(batch, sampled, live)
+        if live:
+            picked = logits if len(live) == logits.shape[0] else logits[[r for r, _ in live]]
+            requests = [q for _, q in live]
+            slots = [cache.slot_of(q.request_id) for q in requests]
+            flight.tokens = self.sampler.launch(
+                picked, [q.sampling for q in requests], slots, [q.num_generated for q in requests],
+                [self.seed + q.request_id for q in requests])
+            if any(q.sampling.presence_penalty > 0.0 for q in requests):
+                self.sampler.note_on_device(
+                    self._ints([s if q.sampling.presence_penalty > 0.0 else -1 for s, q in zip(slots, requests)]),
+                    flight.tokens)
+            flight.rows = {q.request_id: i for i, q in enumerate(requests)}
+            turn = self._turn = 1 - self._turn
+            if self._landing[turn] is None or self._landing[turn].numel() < len(live):
+                self._landing[turn] = torch.empty(max(64, len(live)), dtype=torch.int32, pin_memory=True)
+            flight.landing = self._landing[turn][:len(live)]
+            flight.landing.copy_(flight.tokens, non_blocking=True)
+            flight.landed = torch.cuda.Event()
+            flight.landed.record()
+        return flight
+
+    def _ints(self, values: List[int]) -> torch.Tensor:
+        return self.runner._staging.upload_values(values)
+
+    def _assume(self, flight: "_InFlight") -> None:
+        """What a queued step does to its requests as far as it is known without its tokens: the cursors move,
+        every drawing request has one token more (its value follows), and who reaches its length ends."""
+        finished: List[int] = []
+        for p in flight.batch.portions:
+            if not p.request.is_finished:      # (ended meanwhile by the token it drew in the step before)
+                p.request.add_computed_tokens(len(p.tokens))
+        drawing = {id(q) for _, q in flight.live}
+        for p in flight.sampled:
+            if id(p.request) not in drawing and not p.request.is_finished:   # nothing more to generate
+                p.request.finish("length")
+                finished.append(p.request.request_id)
+        for row, (_, q) in enumerate(flight.live):
+            if q.is_finished:
+                continue
+            if not q.add_sampled_token(0, ()):      # (any valid id holds the place)
+                finished.append(q.request_id)
+            flight.places.append((q, len(q.generated_tokens) - 1, row))
+        self.scheduler.update_after_step(finished)
+
+    def _settle(self, flight: "_InFlight") -> None:
+        """The tokens of a step have arrived: they take their places, and who drew an end ends."""
+        if flight.landed is None:
+            return
+        flight.landed.synchronize()
+        tokens = flight.landing.tolist()
+        finished: List[int] = []
+        for q, index, row in flight.places:
+            tok = tokens[row]
+            q.generated_tokens[index] = tok
+            reason = None
+            if tok == -1:
+                reason = "no_token"
+            elif tok in self.eos_token_ids and not q.sampling.ignore_eos:
+                reason = "eos"
+            if reason is None:
+                continue
+            if q.is_finished:
+                q.finish_reason = reason     # it reached its length with this token; the token's reason comes first
+            else:
+                q.finish(reason)
+                finished.append(q.request_id)
+        if finished:
+            self.scheduler.update_after_step(finished, count_step=False)
+
+    def run_until_complete(self, print_progress: bool = False, one_step_ahead: bool = True) -> None:
         step = 0
-        while self.scheduler.has_work():
-            if print_progress and step % 10 == 0:
+        flight: Optional[_InFlight] = None
+        while True:
+            if print_progress and step % 10 == 0 and self.scheduler.has_work():
                 s = self.scheduler.get_stats()
                 print(f"[pulse_infer_amd] step {step}: {s.num_running} requests running, {s.num_waiting} waiting, "
                       f"{s.num_finished} finished", file=sys.stderr, flush=True)
-            if self.step().empty():
+            if not one_step_ahead:
+                if not self.scheduler.has_work() or self.step().empty():
+                    break
+                step += 1
+                continue
+            batch = self.scheduler.schedule_next_batch() if self.scheduler.has_work() else None
+            self.last_batch = batch if batch is not None else self.last_batch
+            queued = self._launch(batch, flight) if batch is not None and not batch.empty() else None
+            if flight is not None:
+                self._settle(flight)
+            if queued is None:     # nothing left, or nothing that can be scheduled (as ``step`` returning an empty batch)
                 break
+            self._assume(queued)
+            flight = queued
             step += 1
         if print_progress:
             s = self.scheduler.get_stats()

@@ -241,7 +241,25 @@ class ModelRunner:
                                                    # recording keeps its context, and would keep the step function
                                                    # that holds it alive in a circle that only the collector ends)
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def _feed(self, ids: torch.Tensor, feed) -> None:
+        """Token ids that are still on the device (the tokens the step before sampled, which the host has not seen
+        yet) go into the step's ids there: ``feed = (source, places, rows)`` puts ``source[rows[i]]`` at
+        ``ids[places[i]]``.  The entries hold any valid id at those places."""
+        if feed is None:
+            return
+        source, places, rows = feed
+        n = len(places)
+        if n == 0:
+            return
+        if n == ids.numel() == source.numel() and places == rows == list(range(n)):
+            ids.copy_(source)      # the same requests in the same order: the usual decoding step
+            return
+        both = self._staging.upload_values(list(places) + list(rows)).long()
+        ids.index_copy_(0, both[:n], source.index_select(0, both[n:]))
+
+    def step(self, entries: Sequence[StepEntry], feed=None) -> torch.Tensor:
+        """One step of the model over the entries' tokens, from the cache; the logits at the wanted places.
+        ``feed``: see ``_feed``."""
         metas = self._check(entries)
         cache = self.cache
         total = metas[-1].first_row + metas[-1].count
@@ -249,13 +267,14 @@ class ModelRunner:
         max_context = max(m.start + m.count for m in metas)
         uneven = contexts_uneven(metas)
         if self._graph_ok(entries, metas) and self._graph_ready(len(metas), max_context, uneven):
-            logits = self._step_captured(entries, metas, want_rows, max_context, uneven)
+            logits = self._step_captured(entries, metas, want_rows, max_context, uneven, feed)
         else:
             widths = [max(1, max(g.pages_for(m.start + m.count) for m in metas)) for g in cache.groups]
             offsets = self._layout(total, len(metas), len(want_rows), widths)
             flat = np.zeros(int(offsets[-1]), dtype=np.int32)
             self._fill(flat, offsets, entries, metas, want_rows, widths)
             dev = self._staging.upload(flat)
+            self._feed(dev[offsets[0]:offsets[1]], feed)
             ctx = self._context(dev, offsets, metas, len(want_rows), widths, self.model.workspace, max_context, uneven)
             logits = self.model.forward(ctx, self.views)
         for m in metas:
@@ -297,13 +316,13 @@ class ModelRunner:
         return seen >= self.GRAPH_AFTER_STEPS
 
     def _step_captured(self, entries: Sequence[StepEntry], metas: List[EntryMeta], want_rows: List[int],
-                       max_context: int, uneven: bool) -> torch.Tensor:
+                       max_context: int, uneven: bool, feed=None) -> torch.Tensor:
         key = self._graph_key(len(metas), max_context, uneven)
         rec = self._graphs.get(key)
         if rec is None:
             # The step that meets a new shape runs eagerly (over the recording's own buffers, which sizes them) and is
             # recorded afterwards without being run again: a part with state of its own must see every step once.
-            rec, logits = self._capture(key, entries, metas, want_rows)
+            rec, logits = self._capture(key, entries, metas, want_rows, feed)
             if rec is None:
                 self._graph_refused.add(key)
                 return logits
@@ -315,12 +334,13 @@ class ModelRunner:
         rec.wait()
         self._refill(rec, entries, metas)
         rec.dev.copy_(rec.host, non_blocking=True)
+        rec.mark()      # (the pinned buffer is free again once this copy has run, whatever the graph still does)
+        self._feed(rec.dev[rec.offsets[0]:rec.offsets[1]], feed)
         rec.graph.replay()
-        rec.mark()
         self.graph_replays += 1
         return rec.logits.clone()
 
-    def _capture(self, key, entries, metas, want_rows):
+    def _capture(self, key, entries, metas, want_rows, feed=None):
         from ..parts.base import Workspace
 
         batch, bucket, uneven = key
@@ -335,6 +355,7 @@ class ModelRunner:
         self._fill(rec.host_np, offsets, entries, metas, want_rows, widths)
         rec.row_stamps = [self.cache.tables_stamp(m.request) for m in metas]
         dev.copy_(host, non_blocking=True)
+        self._feed(dev[offsets[0]:offsets[1]], feed)
         # the step itself, eagerly: it sizes the workspace and lets parts build what depends only on the step's shape
         from ..parts import linear
 

@@ -266,17 +266,25 @@ class ContinuousBatchScheduler:
                                                  request.num_computed_tokens, count == request.num_pending_tokens)
             budget -= count - have
 
-    def update_after_step(self, finished_ids: Sequence[int]) -> None:
+    def update_after_step(self, finished_ids: Sequence[int], count_step: bool = True) -> None:
         """Take finished requests out of the running list and give their cache back
-        (reference: continuous_batch_scheduler.hpp:75-89)."""
-        self.num_steps += 1
+        (reference: continuous_batch_scheduler.hpp:75-89).  ``count_step`` False: requests whose end became known
+        after the step had been counted (a loop that learns a step's tokens while the next step runs); such a
+        request may have been preempted meanwhile and wait in the queue, from which it is taken too."""
+        if count_step:
+            self.num_steps += 1
         for request_id in finished_ids:
             request = self.request_map.get(request_id)
-            if request is None or request not in self.running:
+            if request is None:
+                continue
+            if request in self.running:
+                self.running.remove(request)
+            elif request in self.waiting:
+                self.waiting.remove(request)
+            else:
                 continue
             if not request.is_finished:
                 request.finish()
-            self.running.remove(request)
             if self.cache is not None and self.cache.has_request(request_id):
                 self.cache.free_request(request_id)
 

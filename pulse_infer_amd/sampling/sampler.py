@@ -28,8 +28,12 @@ class Sampler:
         self._part_val: Optional[torch.Tensor] = None
         self._part_idx: Optional[torch.Tensor] = None
         self._chunked: Optional[dict] = None             # scratch of the sampling in chunks
-        self._options_host: Optional[torch.Tensor] = None  # pinned [6, rows] int32 and its device twin: a step's
-        self._options_dev: Optional[torch.Tensor] = None   # per-row options go up without the host waiting
+        # pinned [6, rows] int32 and device twins, two of each used in turn: a step's per-row options go up without
+        # the host waiting, and a caller may queue a step's sampling while it still waits for the tokens of the step
+        # before (not for older ones: a pair is used again two calls later)
+        self._options_host: List[Optional[torch.Tensor]] = [None, None]
+        self._options_dev: List[Optional[torch.Tensor]] = [None, None]
+        self._turn = 0
         if banned_tokens:
             host = torch.zeros(self.words, dtype=torch.int64)
             for tok in banned_tokens:
@@ -54,28 +58,43 @@ class Sampler:
         both = torch.tensor([list(slots), list(tokens)], dtype=torch.int32).to(self.device)   # one upload
         kernels.mark_seen(self.seen, both[0], both[1], self.vocab)
 
+    def note_on_device(self, slots: torch.Tensor, tokens: torch.Tensor) -> None:
+        """``note_tokens`` for tokens that are still on the device (``launch``'s result): ``slots`` int32 on the
+        device, -1 where a row's request keeps no seen set; rows without a token (-1) mark nothing."""
+        if self.seen is not None and slots.numel():
+            kernels.mark_seen(self.seen, slots, tokens, self.vocab)
+
     # ---------------------------------------------------------------- sampling
     def sample(self, logits: torch.Tensor, params: Sequence[SamplingParams], slots: Sequence[int],
                counters: Sequence[int], default_seeds: Sequence[int]) -> List[int]:
         """One token per row.  ``counters[r]`` is how many tokens row r's request has drawn before."""
-        rows = logits.shape[0]
-        if rows == 0:
+        if logits.shape[0] == 0:
             return []
+        return self.launch(logits, params, slots, counters, default_seeds).tolist()
+
+    def launch(self, logits: torch.Tensor, params: Sequence[SamplingParams], slots: Sequence[int],
+               counters: Sequence[int], default_seeds: Sequence[int]) -> torch.Tensor:
+        """``sample`` without waiting: the tokens as an int32 vector on the device, the kernels only queued."""
+        rows = logits.shape[0]
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        if rows == 0:
+            return out
         if all(p.greedy and p.presence_penalty == 0.0 for p in params) and self.banned is None:
             need = rows * kernels.argmax_chunks(logits.shape[1])
             if self._part_val is None or self._part_val.numel() < need:
                 self._part_val = torch.empty(need, dtype=torch.float32, device=self.device)
                 self._part_idx = torch.empty(need, dtype=torch.int32, device=self.device)
             kernels.argmax(logits, out, self._part_val, self._part_idx)
-            return out.tolist()
+            return out
         # every per-row option in one upload: rows of a [6, R] int32 array, the float ones as their bit patterns
         use_penalty = self.seen is not None and any(p.presence_penalty > 0.0 for p in params)
-        if self._options_host is None or self._options_host.shape[1] < rows:
-            self._options_host = torch.empty((6, max(rows, 64)), dtype=torch.int32, pin_memory=True)
-            self._options_dev = torch.empty((6, max(rows, 64)), dtype=torch.int32, device=self.device)
-        # (the last call's copy out of the pinned rows has finished: that call waited for its tokens)
-        host = self._options_host.numpy()[:, :rows]
+        turn = self._turn
+        self._turn = 1 - turn
+        if self._options_host[turn] is None or self._options_host[turn].shape[1] < rows:
+            self._options_host[turn] = torch.empty((6, max(rows, 64)), dtype=torch.int32, pin_memory=True)
+            self._options_dev[turn] = torch.empty((6, max(rows, 64)), dtype=torch.int32, device=self.device)
+        # (the copy out of these pinned rows two calls ago has run: its tokens have been waited for)
+        host = self._options_host[turn].numpy()[:, :rows]
         as_float = host.view(np.float32)
         as_float[0] = [p.temperature for p in params]
         host[1] = [p.top_k for p in params]
@@ -84,8 +103,8 @@ class Sampler:
                        for p, c, d in zip(params, counters, default_seeds)]
         as_float[4] = [p.presence_penalty for p in params]
         host[5] = [s if p.presence_penalty > 0.0 else -1 for p, s in zip(params, slots)]
-        self._options_dev.copy_(self._options_host, non_blocking=True)
-        dev = self._options_dev
+        self._options_dev[turn].copy_(self._options_host[turn], non_blocking=True)
+        dev = self._options_dev[turn]
         temperature, top_p, uniform = (dev[i, :rows].view(torch.float32) for i in (0, 2, 3))
         top_k = dev[1, :rows]
         penalty = dev[4, :rows].view(torch.float32) if use_penalty else None
@@ -101,4 +120,4 @@ class Sampler:
                                top_p=top_p if any(0.0 < p.top_p < 1.0 for p in params) else None,
                                uniform=uniform, penalty=penalty, seen_row=seen_row, seen_masks=seen,
                                banned=self.banned)
-        return out.tolist()
+        return out

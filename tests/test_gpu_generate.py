@@ -154,6 +154,53 @@ def test_seeded_sampling_does_not_depend_on_the_batch(gpu, model_folders):
     assert len(set(fresh)) == 30 and not set(fresh) & set(prompts[1])
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_loop_one_step_ahead_gives_what_the_loop_step_by_step_gives(gpu, model_folders, dtype):
+    """``run_until_complete`` queues a step before it has seen the tokens of the step before (they are fed to it on
+    the device).  Requests of every kind: ended by an end-of-sequence id that is drawn often, by their length, by
+    both at once, with a presence penalty, greedy and seeded, in a pool so small that requests are preempted and
+    computed again: every request's tokens, reasons and results are those of the loop that waits for every step.
+    In 32-bit, where a draw does not depend on what else a step holds; in bfloat16 (recorded steps, whose ids are fed
+    on the device) no request ends early and the pool is large, so that both loops run the same steps."""
+    from pulse_infer_amd import SamplingParams
+    from pulse_infer_amd.engine.engine import ContinuousBatchEngine
+    from pulse_infer_amd.models.factory import load_model
+
+    cfg, page = TINY["B"]
+    _, model = load_model(model_folders["B"], mode=dtype)
+    vocab = cfg["vocab_size"]
+    exact = dtype == "float32"
+    eos = list(range(0, vocab, 9)) if exact else []   # one id in nine ends a request: many end early, at any step
+    prompts = [token_ids(vocab, n, seed=200 + n) for n in (5, 33, 17, 2, 40, 11, 26, 8, 19, 3)]
+    kinds = [SamplingParams(temperature=0.9, seed=11), SamplingParams(), SamplingParams(temperature=1.2, top_k=12, seed=12),
+             SamplingParams(temperature=0.8, presence_penalty=2.0, seed=13), SamplingParams(temperature=1.0, top_p=0.9, seed=14),
+             SamplingParams(temperature=0.9, seed=15, ignore_eos=True), SamplingParams(presence_penalty=50.0),
+             SamplingParams(temperature=1.5, top_k=30, top_p=0.8, seed=16), SamplingParams(temperature=0.7, seed=17),
+             SamplingParams(temperature=1.1, seed=18, ignore_eos=True)]
+    lengths = [30, 12, 25, 40, 9, 16, 33, 1, 22, 14]
+    results = []
+    for ahead in (True, False):
+        engine = ContinuousBatchEngine(model, max_batch_size=6, chunk_size=8, page_size=page, num_pages=5 if exact else 64,
+                                       max_sequences=6, eos_token_ids=eos, seed=3)
+        engine.runner.GRAPH_AFTER_STEPS = 1
+        ids = [engine.add_request(p, n, k) for p, n, k in zip(prompts, lengths, kinds)]
+        engine.run_until_complete(one_step_ahead=ahead)
+        stats = engine.get_stats()
+        assert stats.num_finished == len(ids) and stats.num_running == 0 and stats.num_waiting == 0
+        engine.runner.cache.check()
+        assert all(g.pool.num_held == 0 for g in engine.runner.cache.groups)
+        results.append([(engine.get_request(i).generated_tokens, engine.get_request(i).finish_reason,
+                         engine.get_result(i)) for i in ids])
+        if ahead and exact:
+            assert stats.num_preemptions > 0                       # the pool of 5 pages made requests give way
+        if not exact:
+            assert engine.runner.graph_replays > 20
+    for i, (a, b) in enumerate(zip(*results)):
+        assert a == b, i
+    reasons = {reason for _, reason, _ in results[0]}
+    assert ({"eos", "length"} if exact else {"length"}) <= reasons
+
+
 def test_command_line(gpu, model_folders, plain_models, capsys):
     from pulse_infer_amd import cli
     cfg, page = TINY["A"]
