@@ -101,20 +101,21 @@ def trajectory(args, cfg, model, batch: int, prompt_tokens: int, new_tokens: int
                            SamplingParams(ignore_eos=True))
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    t_decode, decode_steps = None, 0
-    while engine.scheduler.has_work():
-        if t_decode is None and not any(r.is_prefill for r in engine.scheduler.running + list(engine.scheduler.waiting)):
-            torch.cuda.synchronize()
-            t_decode = time.perf_counter()
+    # the prompts step by step (so that the moment the last one is through can be told), then the engine's own loop
+    while engine.scheduler.has_work() and any(r.is_prefill for r in engine.scheduler.running + list(engine.scheduler.waiting)):
         if engine.step().empty():
             break
-        decode_steps += t_decode is not None
+    torch.cuda.synchronize()
+    t_decode = time.perf_counter()
+    steps_before = engine.get_stats().num_steps
+    engine.run_until_complete()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     stats = engine.get_stats()
     total = stats.tokens_generated
     assert total == batch * new_tokens, (total, batch, new_tokens)
-    decode_s = t1 - (t_decode if t_decode is not None else t0)
+    decode_s = t1 - t_decode
+    decode_steps = stats.num_steps - steps_before
     del engine
     torch.cuda.empty_cache()
     return {"value": round(total / (t1 - t0), 2), "decode_value": round(batch * decode_steps / decode_s, 2),
@@ -289,18 +290,37 @@ def main() -> int:
             tokens = torch.randint(0, cfg.vocab_size, (batch,), generator=gen).tolist()
             slots = [runner.cache.slot_of(n) for n in names]
 
-            def one_step(toks):
-                logits = runner.step([StepEntry(n, [t], [0]) for n, t in zip(names, toks)])
-                return sampler.sample(logits, greedy, slots, [0] * batch, [0] * batch)
+            # As the engine's loop does, a step is queued while the step before it is computed: that step's tokens go
+            # into the new step's ids on the device, and come back to the host (every step's do) while it runs.
+            same = list(range(batch))
+            landing = [torch.empty(batch, dtype=torch.int32, pin_memory=True) for _ in range(2)]
 
-            for _ in range(warmup):
-                tokens = one_step(tokens)
+            def queue(toks, before, turn):
+                feed = (before[0], same, same) if before is not None else None
+                logits = runner.step([StepEntry(n, [t], [0]) for n, t in zip(names, toks)], feed=feed)
+                out = sampler.launch(logits, greedy, slots, [0] * batch, [0] * batch)
+                landing[turn].copy_(out, non_blocking=True)
+                landed = torch.cuda.Event()
+                landed.record()
+                return out, landing[turn], landed
+
+            def run_steps(count, toks):
+                flight = queue(toks, None, 0)
+                for i in range(1, count):
+                    ahead = queue([0] * batch, flight, i % 2)
+                    flight[2].synchronize()
+                    toks = flight[1].tolist()           # the tokens of the step before, on the host
+                    flight = ahead
+                flight[2].synchronize()
+                return flight[1].tolist()
+
+            if warmup:
+                tokens = run_steps(warmup, tokens)
             first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             first.record()
-            for _ in range(steps):
-                tokens = one_step(tokens)
+            tokens = run_steps(steps, tokens)
             last.record()
             torch.cuda.synchronize()
             host.append((time.perf_counter() - t0) / steps)
