@@ -321,8 +321,8 @@ def test_steps_of_uneven_contexts_are_recorded_apart(gpu, model_folders, plain_l
 
 def test_the_collector_rests_while_a_step_is_recorded(gpu, model_folders):
     """No graph may be destroyed while a stream records, and Python's collector, which may find dropped recordings (of
-    a step function that is no longer used, of the caller), runs whenever it likes: the step function lets it run
-    before it records and keeps it off meanwhile.  A dropped step function itself goes at once: nothing points back at it
+    a step function that is no longer used, of the caller), runs whenever it likes: the step function keeps it off
+    while it records.  A dropped step function itself goes at once: nothing points back at it
     in a circle."""
     import gc
     import weakref
