@@ -154,20 +154,21 @@ def test_seeded_sampling_does_not_depend_on_the_batch(gpu, model_folders):
     assert len(set(fresh)) == 30 and not set(fresh) & set(prompts[1])
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_the_loop_one_step_ahead_gives_what_the_loop_step_by_step_gives(gpu, model_folders, dtype):
+@pytest.mark.parametrize("name,dtype", [("B", "float32"), ("B", "bfloat16"), ("W", "float32")])
+def test_the_loop_one_step_ahead_gives_what_the_loop_step_by_step_gives(gpu, model_folders, name, dtype):
     """``run_until_complete`` queues a step before it has seen the tokens of the step before (they are fed to it on
     the device).  Requests of every kind: ended by an end-of-sequence id that is drawn often, by their length, by
     both at once, with a presence penalty, greedy and seeded, in a pool so small that requests are preempted and
     computed again: every request's tokens, reasons and results are those of the loop that waits for every step.
     In 32-bit, where a draw does not depend on what else a step holds; in bfloat16 (recorded steps, whose ids are fed
-    on the device) no request ends early and the pool is large, so that both loops run the same steps."""
+    on the device) no request ends early and the pool is large, so that both loops run the same steps.  "W": layers
+    with a window, whose pages go back to the pool while requests run."""
     from pulse_infer_amd import SamplingParams
     from pulse_infer_amd.engine.engine import ContinuousBatchEngine
     from pulse_infer_amd.models.factory import load_model
 
-    cfg, page = TINY["B"]
-    _, model = load_model(model_folders["B"], mode=dtype)
+    cfg, page = TINY[name]
+    _, model = load_model(model_folders[name], mode=dtype, config_overrides=OVERRIDES.get(name))
     vocab = cfg["vocab_size"]
     exact = dtype == "float32"
     eos = list(range(0, vocab, 9)) if exact else []   # one id in nine ends a request: many end early, at any step
@@ -180,7 +181,8 @@ def test_the_loop_one_step_ahead_gives_what_the_loop_step_by_step_gives(gpu, mod
     lengths = [30, 12, 25, 40, 9, 16, 33, 1, 22, 14]
     results = []
     for ahead in (True, False):
-        engine = ContinuousBatchEngine(model, max_batch_size=6, chunk_size=8, page_size=page, num_pages=5 if exact else 64,
+        engine = ContinuousBatchEngine(model, max_batch_size=6, chunk_size=8, page_size=page,
+                                       num_pages=(80 // page if exact else 64),
                                        max_sequences=6, eos_token_ids=eos, seed=3)
         engine.runner.GRAPH_AFTER_STEPS = 1
         ids = [engine.add_request(p, n, k) for p, n, k in zip(prompts, lengths, kinds)]
