@@ -51,6 +51,7 @@ constexpr int PREFILL_TILES = PULSE_WIDE ? WIDE_CT : 1;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
@@ -1311,27 +1312,32 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
                                                                          int n_splits, int static_split_size, int hpw_log2,
                                                                          const int* __restrict__ live_context,
                                                                          const int* __restrict__ plan, int n_items) {
-    const int item = blockIdx.x / per;
-    const int split_size = plan ? plan[1 + n_items * n_splits + item]
-                           : live_context ? live_split_size(*live_context, n_splits, static_split_size) : static_split_size;
     __shared__ float s_w[MAX_SPLITS];      // hpw * n_splits <= MAX_SPLITS (hpw > 1 only with few splits)
     __shared__ float s_l[MAX_SPLITS];
     __shared__ f32x4 s_acc[REDUCE_GROUPS][REDUCE_QUADS];
-    // only the rows of this launch's items have partial results
+    // The kernel is a chain of trips to memory and little else, so it is kept to two: the item (and what says how its
+    // keys were cut), then everything that needs only the row: its position, the item's last position, the (m, l)
+    // pairs of every split and the first partial outputs.  What of that a row does not use is read and dropped.
+    const int item = blockIdx.x / per;
     const int tok = blockIdx.x % per;
-    if (tok >= items[4 * item + 1]) return;
-    const int64_t row = items[4 * item] + tok;
-    if (plan && positions[items[4 * item] + items[4 * item + 1] - 1] < split_size) return;   // finished by its only split
+    const int row0 = items[4 * item], ntok = items[4 * item + 1];
+    const int split_size = plan ? plan[1 + n_items * n_splits + item]
+                           : live_context ? live_split_size(*live_context, n_splits, static_split_size) : static_split_size;
+    if (tok >= ntok) return;   // only the rows of this launch's items have partial results
+    const int64_t row = row0 + tok;
     const int hpw = 1 << hpw_log2;            // heads of this workgroup
     const int head0 = blockIdx.y * hpw;
-    const int valid = min(n_splits, positions[row] / split_size + 1);
-    for (int i = threadIdx.x; i < hpw * valid; i += REDUCE_THREADS) {
+    const int pos_row = positions[row];
+    const int pos_last = positions[row0 + ntok - 1];
+    constexpr int ML_PER = MAX_SPLITS / REDUCE_THREADS;
+    f32x2 ml[ML_PER];
+#pragma unroll
+    for (int j = 0; j < ML_PER; ++j) {
+        const int i = threadIdx.x + j * REDUCE_THREADS;
         const int hs = i & (hpw - 1), z = i >> hpw_log2;
-        if (head0 + hs < nq) {
-            const int64_t at = (row * nq + head0 + hs) * n_splits + z;
-            s_w[hs * n_splits + z] = part_ml[2 * at];
-            s_l[hs * n_splits + z] = part_ml[2 * at + 1];
-        }
+        ml[j] = f32x2{0.f, 0.f};
+        if (i < hpw * n_splits && head0 + hs < nq)
+            ml[j] = *reinterpret_cast<const f32x2*>(part_ml + 2 * ((row * nq + head0 + hs) * n_splits + z));
     }
     // group `grp` of threads takes head grp % hpw and of its splits sg = grp / hpw, sg + gph, ..; a thread four
     // channels of them.
@@ -1354,6 +1360,17 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
         // a split without keys of the row left nothing behind: what is read there is not used (z < valid below)
         first[i] = (works && z < n_splits) ? *reinterpret_cast<const f32x4*>(part_o + (base + z) * D + 4 * quad)
                                            : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (plan && pos_last < split_size) return;   // the item was finished by its only split
+    const int valid = min(n_splits, pos_row / split_size + 1);
+#pragma unroll
+    for (int j = 0; j < ML_PER; ++j) {
+        const int i = threadIdx.x + j * REDUCE_THREADS;
+        const int hs2 = i & (hpw - 1), z = i >> hpw_log2;
+        if (i < hpw * valid && head0 + hs2 < nq) {
+            s_w[hs2 * n_splits + z] = ml[j][0];
+            s_l[hs2 * n_splits + z] = ml[j][1];
+        }
     }
     __syncthreads();
     float inv = 0.f;
