@@ -62,7 +62,8 @@ def split_entries(entries: Sequence):
 
 
 SPLIT_OVERHEAD_KEYS = 256      # what a workgroup costs beside its walk (start-up, merge inside it), in keys walked
-MERGE_OVERHEAD_KEYS = 700      # what splitting at all costs (partial results through memory, the second kernel)
+MERGE_OVERHEAD_KEYS = 350      # what splitting at all costs (partial results through memory, the second kernel)
+MIN_SPLIT_KEYS = 64            # no split is shorter
 MAX_CHOSEN_SPLITS = 64
 
 
@@ -77,7 +78,9 @@ def choose_splits(num_items: int, nkv: int, group: int, max_context: int) -> Tup
     one (160 to 256 workgroups; two splits are 10 to 25% slower), 40 in 4 and 48 in 2 (a multiple of the units
     again), 64 in one.  Walks of 4,096 keys and more stream better with two workgroups a unit (16 requests at 8,192:
     4 splits 95.9 us, 2 splits 97.6; at 4,096, walks of 2,048 keys, 2 splits 51.9 us and 4 splits 53.8), so a choice
-    that gives every unit one such walk is cut in two once more."""
+    that gives every unit one such walk is cut in two once more.  Short contexts (the merge's cost as it was measured
+    there, 5 to 6 us, about 350 keys' worth of a walk): 8 requests of 512 keys 15.0 us whole and 13.1 in four splits,
+    16 of 1,024 25.0 whole and 21.8 in two, one of 1,024 11.6 in 8 splits and 10.3 in 16."""
     units = compute_units()        # the split kernel's workgroups are counted against them
     groups = num_items * nkv * ((group + 15) // 16)
     whole = (max_context + BLOCK_KEYS - 1) // BLOCK_KEYS * BLOCK_KEYS
@@ -90,10 +93,13 @@ def choose_splits(num_items: int, nkv: int, group: int, max_context: int) -> Tup
     best = None
     for n in range(1, MAX_CHOSEN_SPLITS + 1):
         size = split_size(n)
-        if n > 1 and (size < 128 or (n - 1) * size >= max_context):
+        if n > 1 and (size < MIN_SPLIT_KEYS or (n - 1) * size >= max_context):
             continue
         on_a_unit = (groups * n + units - 1) // units
-        cost = on_a_unit * (size + SPLIT_OVERHEAD_KEYS) + (MERGE_OVERHEAD_KEYS if n > 1 else 0)
+        # (more workgroups than the units hold at a time, two each, wait for one another: 24 requests of 4,096 keys
+        # take 79 us whole and 85 in four splits, which this rule's sums alone would prefer)
+        merge = 0 if n == 1 else MERGE_OVERHEAD_KEYS * (2 if groups * n > 2 * units else 1)
+        cost = on_a_unit * (size + SPLIT_OVERHEAD_KEYS) + merge
         if best is None or cost < best[0]:
             best = (cost, n)
     n = best[1]

@@ -29,7 +29,7 @@ def test_decode_splits_cover_the_context_in_whole_blocks(units):
         assert size * n >= context and size * (n - 1) < max(context, 1)          # every key once, no empty last split
         assert n <= 2 * M.MAX_CHOSEN_SPLITS
         if n > 1:
-            assert size >= 128                                                   # a split is worth its workgroup
+            assert size >= M.MIN_SPLIT_KEYS                                      # a split is worth its workgroup
     # more work than the chip has units is never cut finer than one split a unit would need
     size, n = M.choose_splits(4 * units, 8, 4, 2048)
     assert n == 1
