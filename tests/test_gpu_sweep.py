@@ -108,6 +108,63 @@ def test_random_configurations_continuous_batching_and_preemption(tmp_path, seed
 
 
 @pytest.mark.parametrize("seed", range(6))
+def test_random_workloads_through_the_loop_one_step_ahead_and_step_by_step(tmp_path, seed):
+    """Random requests (sampling options of every kind, seeded; lengths from none to thirty; end-of-sequence ids that
+    are drawn often; banned ids; a pool that holds little more than the longest request, so requests are preempted,
+    some of them while their last token is still on the device) through the serving loop that queues a step ahead
+    and through the loop that waits for every step, in 32-bit: the same tokens, finish reasons and results."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from pulse_infer_amd import SamplingParams
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.engine.engine import ContinuousBatchEngine
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.weights import write_model_folder
+
+    rng = random.Random(5000 + seed)
+    cfg, options = random_config(rng, [64, 128], max_positions=512)
+    vocab = cfg["vocab_size"]
+    folder = write_model_folder(Qwen3Config.from_dict(cfg), str(tmp_path / "m"), seed=80 + seed)
+    _, model = load_model(folder, mode="float32", config_overrides=options)
+    page = rng.choice([8, 16])
+    count = rng.randint(4, 12)
+    prompts = [token_ids(vocab, rng.randint(1, 60), seed=seed * 100 + i) for i in range(count)]
+    lengths = [rng.randint(0, 30) for _ in range(count)]
+    eos = rng.sample(range(vocab), k=rng.choice([0, vocab // 12, vocab // 5]))
+    banned = rng.sample(range(vocab), k=rng.choice([0, 3]))
+
+    def options_of(i):
+        r = random.Random(seed * 1000 + i)
+        kind = r.choice(["greedy", "temperature", "top_k", "top_p", "both", "penalty"])
+        common = dict(seed=r.randint(0, 10 ** 6), ignore_eos=r.random() < 0.2)
+        if kind == "greedy":
+            return SamplingParams(ignore_eos=common["ignore_eos"], presence_penalty=r.choice([0.0, 3.0]))
+        t = r.uniform(0.5, 1.5)
+        return {"temperature": SamplingParams(temperature=t, **common),
+                "top_k": SamplingParams(temperature=t, top_k=r.choice([1, 5, 40]), **common),
+                "top_p": SamplingParams(temperature=t, top_p=r.uniform(0.3, 0.95), **common),
+                "both": SamplingParams(temperature=t, top_k=r.choice([3, 20]), top_p=r.uniform(0.5, 0.95), **common),
+                "penalty": SamplingParams(temperature=t, presence_penalty=r.uniform(0.5, 4.0), **common)}[kind]
+
+    longest = max(len(p) + n for p, n in zip(prompts, lengths))
+    pages = max((longest + page - 1) // page + 1, rng.choice([4, 6, 8]))
+    batch, chunk = rng.choice([2, 4, 8]), rng.choice([4, 16, 64])
+    results = []
+    for ahead in (True, False):
+        engine = ContinuousBatchEngine(model, max_batch_size=batch, chunk_size=chunk, page_size=page, num_pages=pages,
+                                       max_sequences=8, eos_token_ids=eos, banned_tokens=banned or None, seed=5)
+        ids = [engine.add_request(p, n, options_of(i)) for i, (p, n) in enumerate(zip(prompts, lengths))]
+        engine.run_until_complete(one_step_ahead=ahead)
+        stats = engine.get_stats()
+        assert stats.num_finished == count and stats.num_running == 0 and stats.num_waiting == 0
+        engine.runner.cache.check()
+        assert all(g.pool.num_held == 0 for g in engine.runner.cache.groups)
+        results.append([(engine.get_request(i).generated_tokens, engine.get_request(i).finish_reason,
+                         engine.get_result(i)) for i in ids])
+    assert results[0] == results[1]
+
+
+@pytest.mark.parametrize("seed", range(6))
 def test_random_configurations_mixed_batches_with_page_reuse(tmp_path, seed):
     """Up to four live requests, portions of some beside single tokens of others, in a pool of 256 tokens whose
     pages are used again, for random configurations in both storage types."""
