@@ -1023,7 +1023,14 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
         asm volatile("s_load_dword %0, %1, 0x0" : "=s"(page) : "s"(entry) : "memory");
         return page;
     };
+    // The register a load was asked into holds nothing until the wait: between the two it must not be copied, which
+    // the compiler, to whom the load's result looks ready at once, is free to do wherever values meet (the head of a
+    // loop, the end of a branch).  So a load and its wait stand in the same straight piece of code, with nothing but
+    // the wait touching the variable in between, and only landed values are carried round the loop.
     auto page_landed = [&](int& page) { asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(page) : : "memory"); };
+    auto pages_landed = [&](int& one, int& two) {
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(one), "+s"(two) : : "memory");
+    };
     const int64_t page_elems = static_cast<int64_t>(a.nkv) * a.page_size * D;  // of K and of V alike
     const int head_elems = g * a.page_size * D;
     auto fetch = [&](int b, int page_read, int stage) {
@@ -1192,12 +1199,13 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
     const int first_block = max(lo_item, split_begin) / BK;
     const int last_block = split_last / BK;
     // (a split that lies below the item's window has no block to walk: nothing is fetched, its columns stay empty)
-    int page_next = 0;
+    int page_next = 0;   // the page of block b + 1, landed
     if (first_block <= last_block) {
         int page_first = page_ahead(first_block);
-        page_landed(page_first);
+        int page_second = page_ahead(first_block + 1);
+        pages_landed(page_first, page_second);
         fetch(first_block, page_first, 0);
-        page_next = page_ahead(first_block + 1);
+        page_next = page_second;
     }
     for (int b = first_block; b <= last_block; ++b) {
         const int stage = (b - first_block) & 1;
@@ -1205,17 +1213,18 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) PULSE_WIDE_WAVES_PER_EU void attn_p
         // count of loads.
         asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
         __syncthreads();  // every wavefront's part of this block has landed
-        if (b < last_block) {
-            page_landed(page_next);
+        if (b < last_block)
             fetch(b + 1, page_next, stage ^ 1);  // that stage was read a block ago; the barrier that ended that block released it
-            page_next = page_ahead(b + 2);       // used an iteration later
-        }
+        int page_after = page_ahead(b + 2);      // asked for now (past the walk's end it reads an entry nobody uses),
+                                                 // waited for at the end of this block, used in the next
         // a wavefront skips blocks that none of its columns sees (above its diagonal, below its window)
         if (b * BK + BK - 1 > hi || b * BK < lo_item) {   // the same for the whole workgroup
             clear_stale(b, stage);
             __syncthreads();
         }
         if (w_hi >= 0 && b * BK <= w_hi && b * BK + BK - 1 >= w_lo) compute(b, stage);
+        page_landed(page_after);
+        page_next = page_after;
         __syncthreads();  // everybody has read this block
     }
 

@@ -33,14 +33,17 @@ def test_greedy_generation_matches_the_plain_implementation(gpu, model_folders, 
     assert not llm.engine.runner.cache.requests                       # everything was given back
     # bfloat16: the same tokens wherever the plain top-two margin is clear of bfloat16's error
     llm16 = make_llm(model_folders[name], "bfloat16", name, max_batch_size=3, chunk_size=8, page_size=page, num_pages=64)
+    clear = 0
     for prompt, out in zip(prompts, llm16.generate(prompts, max_new_tokens=8, ignore_eos=True)):
-        ids = list(prompt)
-        for tok in out:
-            row = plain_models[name].logits(ids)[-1]
+        assert len(out) == 8
+        rows = plain_models[name].logits(list(prompt) + out)[len(prompt) - 1:-1]   # along the engine's own path
+        for tok, row in zip(out, rows):
             top = torch.topk(row, 2)
             if float(top.values[0] - top.values[1]) > 0.25:
                 assert tok == int(top.indices[0])
-            ids.append(tok)                                           # follow the engine's own path
+                clear += 1
+            assert float(row[tok]) >= float(row.max()) - 3e-2 * float(row.abs().max())   # never far from the best
+    assert clear >= 5, f"only {clear} of 24 tokens had a margin that bfloat16 cannot blur: the check says too little"
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -201,6 +204,134 @@ def test_the_loop_one_step_ahead_gives_what_the_loop_step_by_step_gives(gpu, mod
         assert a == b, i
     reasons = {reason for _, reason, _ in results[0]}
     assert ({"eos", "length"} if exact else {"length"}) <= reasons
+
+
+def _sweep_model(tmp_path, seed):
+    """A seeded random configuration of the architecture (as the sweep's), its folder and its plain twin."""
+    import random
+    from plain.qwen3_plain import PlainQwen3
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.weights import write_model_folder
+    from test_gpu_sweep import random_config
+
+    rng = random.Random(seed)
+    cfg, options = random_config(rng, [128, 256], max_positions=512)
+    folder = write_model_folder(Qwen3Config.from_dict(cfg), str(tmp_path / "m"), seed=seed)
+    plain = PlainQwen3.from_folder(folder, windows=(options or {}).get("layer_windows"))
+    return cfg, options, folder, plain, rng.choice([16, 32])
+
+
+@pytest.mark.parametrize("which", ["B", "sweep"])
+def test_the_loop_one_step_ahead_in_bfloat16_with_recorded_steps_early_ends_and_preemption(
+        gpu, model_folders, plain_models, tmp_path, which):
+    """The serving loop as it serves (reference loop: src/scheduler/continuous_batch_engine.cpp:186-252): bfloat16,
+    every step of single tokens recorded at once and replayed with its ids fed on the device, end-of-sequence ids that
+    are drawn often (a request ends while the step that already holds its next token is queued) and a pool so tight
+    that requests are preempted and computed again (some with their last token still on the device).  In bfloat16 the
+    tokens need not be those of the loop that waits for every step, so what must hold is asserted instead: every
+    request finishes, everything is given back, an end-of-sequence id is only ever a request's last token, and every
+    greedy token, along the engine's own path, is the plain implementation's best or within bfloat16's error of it."""
+    from pulse_infer_amd import SamplingParams
+    from pulse_infer_amd.engine.engine import ContinuousBatchEngine
+    from pulse_infer_amd.models.factory import load_model
+
+    if which == "B":
+        (cfg, page), options, folder, plain = TINY["B"], None, model_folders["B"], plain_models["B"]
+    else:
+        cfg, options, folder, plain, page = _sweep_model(tmp_path, 7003)
+    vocab = cfg["vocab_size"]
+    _, model = load_model(folder, mode="bfloat16", config_overrides=options)
+    eos = list(range(0, vocab, 9))
+    sizes = (5, 33, 17, 2, 40, 11, 26, 8, 19, 3, 30, 14)
+    prompts = [token_ids(vocab, n, seed=600 + n) for n in sizes]
+    lengths = [30, 12, 25, 40, 9, 16, 33, 1, 22, 14, 35, 28]
+    kinds = [SamplingParams() for _ in sizes]
+    kinds[3] = SamplingParams(ignore_eos=True)
+    kinds[6] = SamplingParams(ignore_eos=True)
+    kinds[2] = SamplingParams(temperature=0.9, top_k=12, seed=21)              # three that draw: their tokens are
+    kinds[5] = SamplingParams(temperature=0.8, presence_penalty=2.0, seed=22)  # checked for form only
+    kinds[9] = SamplingParams(temperature=1.1, top_p=0.9, seed=23)
+    longest = max(len(p) + n for p, n in zip(prompts, lengths))
+    pages = (longest + page - 1) // page + 1
+    engine = ContinuousBatchEngine(model, max_batch_size=6, chunk_size=8, page_size=page, num_pages=pages,
+                                   max_sequences=6, eos_token_ids=eos, seed=3)
+    engine.runner.GRAPH_AFTER_STEPS = 1
+    ids = [engine.add_request(p, n, k) for p, n, k in zip(prompts, lengths, kinds)]
+    engine.run_until_complete(one_step_ahead=True)
+    stats = engine.get_stats()
+    assert stats.num_finished == len(ids) and stats.num_running == 0 and stats.num_waiting == 0
+    engine.runner.cache.check()
+    assert all(g.pool.num_held == 0 for g in engine.runner.cache.groups) and not engine.runner.cache.requests
+    assert engine.runner.graph_records > 0 and engine.runner.graph_replays > 0
+    assert stats.num_preemptions > 0, "the pool was meant to run out"
+    reasons, checked = set(), 0
+    for rid, prompt, most, kind in zip(ids, prompts, lengths, kinds):
+        request = engine.get_request(rid)
+        out = request.generated_tokens
+        reasons.add(request.finish_reason)
+        assert 1 <= len(out) <= most and all(0 <= t < vocab for t in out)
+        if kind.ignore_eos:
+            assert len(out) == most and request.finish_reason == "length"
+        else:
+            assert not any(t in eos for t in out[:-1])                   # an end-of-sequence id ends its request
+            assert (out[-1] in eos) == (request.finish_reason == "eos")
+            assert len(out) == most or request.finish_reason == "eos"
+            assert engine.get_result(rid) == (out[:-1] if out[-1] in eos else out)
+        if kind.greedy and kind.presence_penalty == 0.0:
+            rows = plain.logits(list(prompt) + out)[len(prompt) - 1:-1]
+            for t, (tok, row) in enumerate(zip(out, rows)):
+                slack = 3e-2 * float(row.abs().max())
+                assert float(row[tok]) >= float(row.max()) - slack, (
+                    f"request {rid}, token {t}: logit {float(row[tok]):.4f} against the best {float(row.max()):.4f}")
+                checked += 1
+    assert {"eos", "length"} <= reasons and checked > 60
+
+
+def test_a_fed_token_that_is_no_token_spoils_only_its_own_request(gpu, model_folders, plain_logits):
+    """A request for which no token is allowed draws -1, and the loop one step ahead has by then queued a step that is
+    fed that -1 on the device: its embedding row is NaN and so are the key and value that the step writes into the
+    request's page.  The request ends there; nothing of it may reach another request, neither the one beside it in
+    the step nor the one that gets its pages next (whose slots beyond its own context still hold the NaN).  Eager and
+    recorded steps, against the plain implementation."""
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+    from test_gpu_model import close
+
+    cfg, page = TINY["B"]
+    vocab = cfg["vocab_size"]
+    ids = {k: token_ids(vocab, n, seed=800 + n) for k, n in (("good", 60), ("bad", 41), ("next", 47))}
+    want = {k: plain_logits("B", v) for k, v in ids.items() if k != "bad"}
+    for dtype, graphs in (("float32", False), ("bfloat16", False), ("bfloat16", True)):
+        _, model = load_model(model_folders["B"], mode=dtype)
+        runner = ModelRunner(model, page_size=page, num_pages=8, max_requests=3, use_graphs=graphs)
+        runner.GRAPH_AFTER_STEPS = 1
+        for k, n in (("good", 30), ("bad", 37)):
+            runner.add_request(k)
+            runner.reserve(k, 60 if k == "good" else n + 4)
+            runner.step([StepEntry(k, ids[k][:n], [])])
+        none = torch.tensor([7, -1], dtype=torch.int32, device=model.device)    # what the step before "drew"
+        got = []
+        for s in range(4):         # "bad" is fed -1 from the device in every one of them; the host holds a valid id
+            feed = (none, [1], [1])
+            logits = runner.step([StepEntry("good", [ids["good"][30 + s]], [0]), StepEntry("bad", [0], [0])], feed=feed)
+            got.append(logits[0])
+            assert bool(torch.isnan(logits[1]).all())            # no token can be chosen from this row
+        assert model.embedding.saw_bad_id()
+        bad_pages = set(runner.cache.table(0, "bad"))
+        runner.free_request("bad")
+        runner.add_request("next")
+        runner.reserve("next", 47)
+        assert bad_pages & set(runner.cache.table(0, "next"))    # the pages with NaN in them are used again
+        first = runner.step([StepEntry("next", ids["next"][:21], list(range(21)))])
+        rest = [runner.step([StepEntry("good", [ids["good"][34 + s]], [0]),
+                             StepEntry("next", [ids["next"][21 + s]], [0])]) for s in range(26)]
+        if graphs:
+            assert runner.graph_replays >= 20
+        close(torch.stack(got + [r[0] for r in rest]), want["good"][30:60], dtype, f"beside the spoiled request ({dtype})")
+        close(torch.cat([first, torch.stack([r[1] for r in rest])]), want["next"], dtype,
+              f"in the spoiled request's pages ({dtype})")
+        runner.cache.reset()
+        runner.cache.check()
 
 
 def test_command_line(gpu, model_folders, plain_models, capsys):

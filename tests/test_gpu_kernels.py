@@ -135,6 +135,26 @@ def _cache(pages, nkv, bs, d, dtype):
             torch.zeros(pages, nkv, d, bs, dtype=dtype, device=DEV))
 
 
+def _stale(kc, vc, seed=0):
+    """What pages hold that have been used before, and worse: every page, its slots beyond a request's context
+    included, is filled with ordinary values, with NaN, with +Inf or with -Inf before the requests' keys and values
+    go in (a request that was fed an id outside the table leaves NaN behind).  Nothing of it may reach an output: a
+    stale value times a weight of zero is not zero."""
+    kinds = torch.randint(0, 4, (kc.shape[0],), generator=torch.Generator().manual_seed(1000 + seed)).tolist()
+    kc.normal_()
+    vc.normal_()
+    for page, kind in enumerate(kinds):
+        if kind:
+            value = (float("nan"), float("inf"), float("-inf"))[kind - 1]
+            kc[page].fill_(value)
+            vc[page].fill_(value)
+
+
+def _bits(t):
+    """The tensor's bit patterns, so that NaN compares equal to itself."""
+    return t.cpu().contiguous().view(torch.int16 if t.element_size() == 2 else torch.int32)
+
+
 def _tables(k, positions, theta, rot):
     inv = torch.pow(torch.tensor(theta, dtype=F64), -torch.arange(rot // 2, dtype=F64) * 2 / rot).to(DEV)
     cos = torch.empty(len(positions), rot // 2, device=DEV)
@@ -218,6 +238,7 @@ def test_attn_generic(k, dtype, case):
              [2 * i + 1 for i in range((lens[1] + bs - 1) // bs)]]         # ascending odd pages
     width = max(len(p) for p in pages)
     kc, vc = _cache(128, nkv, bs, d, dtype)
+    _stale(kc, vc)
     refs = []
     for r, n in enumerate(lens):
         ks, kref = as_stored(rnd(n, nkv, d, seed=20 + r), dtype)
@@ -574,8 +595,7 @@ def _mfma_case(k, nq, nkv, d, bs, window, lens, portion, split, seed=0, portion_
     total = sum(pages_per) + 3
     perm = torch.randperm(total, generator=torch.Generator().manual_seed(seed)).tolist()
     kc, vc = _cache(total, nkv, bs, d, dtype)
-    kc.normal_()                      # stale data everywhere, as in pages that are used again
-    vc.normal_()
+    _stale(kc, vc, seed)              # stale data everywhere, as in pages that are used again
     width = max(pages_per)
     table = torch.full((len(lens), width), -1, dtype=torch.int32)
     refs, start = [], 0
@@ -751,8 +771,7 @@ def test_attn_prefill_at_the_benchmark_shape(k, n):
     pages = n // bs
     perm = torch.randperm(pages + 3, generator=torch.Generator().manual_seed(9)).tolist()[:pages]
     kc, vc = _cache(pages + 3, nkv, bs, d, dtype)
-    kc.normal_()
-    vc.normal_()
+    _stale(kc, vc)
     ks, kref = as_stored(rnd(n, nkv, d, seed=501), dtype)
     vs, vref = as_stored(rnd(n, nkv, d, seed=502), dtype)
     _fill_cache(kc, vc, ks, vs, perm, bs)
@@ -890,8 +909,7 @@ def test_attn_decode_from_raw(k, case, split, new_key):
     total = sum(pages_per) + 2
     perm = torch.randperm(total, generator=torch.Generator().manual_seed(5)).tolist()
     kc, vc = _cache(total, nkv, bs, d, dtype)
-    kc.normal_()                                   # stale data, also in the slot the new key goes to
-    vc.normal_()
+    _stale(kc, vc)                                 # stale data, also in the slot the new key goes to
     table = torch.full((n, max(pages_per)), -1, dtype=torch.int32)
     positions = [c - 1 for c in lens]
     qkv, ref = as_stored(rnd(n, (nq + 2 * nkv) * d + 8, seed=41), dtype)
@@ -973,13 +991,14 @@ def test_attn_decode_from_raw(k, case, split, new_key):
         assert torch.allclose(kcpu[page, :, slot, :], knew[t], atol=2e-2, rtol=2e-2)
         assert torch.equal(vcpu[page, :, :, slot], vnew[t])
     same = ~touched.unsqueeze(1).expand(-1, nkv, -1)
-    assert torch.equal(kc.cpu()[same], before_k.cpu()[same])
-    assert torch.equal(vc.cpu().transpose(2, 3)[same], before_v.cpu().transpose(2, 3)[same])
+    assert torch.equal(_bits(kc)[same], _bits(before_k)[same])
+    assert torch.equal(_bits(vc).transpose(2, 3)[same], _bits(before_v).transpose(2, 3)[same])
     if new_key:
         # the separate preparation kernel writes the same pages (up to the last bit of a sum in another order)
         k.qk_rope_kv(raw, nq, nkv, d, qw, kw, eps, cos, sin, rot, pairing, before_k, before_v, pos_t,
                      torch.arange(n, dtype=torch.int32, device=DEV), table.to(DEV))
-        assert torch.allclose(kc.float(), before_k.float(), atol=0, rtol=2 ** -7) and torch.equal(vc, before_v)
+        assert torch.allclose(kc.float(), before_k.float(), atol=0, rtol=2 ** -7, equal_nan=True)
+        assert torch.equal(_bits(vc), _bits(before_v))
 
 
 def test_attn_decode_refuses_rotations_it_cannot_prepare(k):

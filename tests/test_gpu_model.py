@@ -295,6 +295,112 @@ def test_benchmark_layer_sizes_recorded_decode_steps(layer_shape, batch):
     torch.cuda.empty_cache()
 
 
+# One layer of the benchmark's sizes under the benchmark's vocabulary: the head's products at the size they are timed
+# at (151,936 rows of 4,096), and contexts up to the model's 4,096 positions.
+HEAD_SHAPE = dict(LAYER_SHAPE, num_hidden_layers=1, vocab_size=151936)
+
+
+@pytest.fixture(scope="module")
+def head_shape(tmp_path_factory):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU visible")
+    from plain.qwen3_plain import PlainQwen3
+    from pulse_infer_amd.config import Qwen3Config
+    from pulse_infer_amd.weights import write_model_folder
+
+    folder = str(tmp_path_factory.mktemp("head_shape"))
+    write_model_folder(Qwen3Config.from_dict(HEAD_SHAPE), folder, seed=43)
+    return folder, PlainQwen3.from_folder(folder)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_head_at_the_benchmark_vocabulary(head_shape, dtype):
+    """The logits of the last row of a whole prompt, of a step of 8 decoded tokens and of a step of 24 (in bfloat16
+    three products: the streaming one for few rows, the same at 8 rows, the one for 17 to 64 rows with a float32
+    result), at a vocabulary of 151,936, against the plain implementation."""
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+
+    folder, plain = head_shape
+    vocab = HEAD_SHAPE["vocab_size"]
+    _, model = load_model(folder, mode=dtype)
+    runner = ModelRunner(model, page_size=16, num_pages=80, max_requests=24)
+    prompt = token_ids(vocab, 70, seed=44)
+    runner.add_request("p")
+    runner.reserve("p", 70)
+    got = runner.step([StepEntry("p", prompt, [69])])
+    runner.free_request("p")
+    assert got.shape == (1, vocab)
+    close(got, plain.logits(prompt, rows=[69]), dtype, "head, last row of a prompt")
+    for batch in (8, 24):
+        lengths = [3 + (11 * i) % 29 for i in range(batch)]
+        ids = [token_ids(vocab, n + 1, seed=500 + 10 * batch + i) for i, n in enumerate(lengths)]
+        for r, n in enumerate(lengths):
+            runner.add_request(r)
+            runner.reserve(r, n + 1)
+        runner.step([StepEntry(r, ids[r][:n], []) for r, n in enumerate(lengths)])
+        got = runner.step([StepEntry(r, [ids[r][n]], [0]) for r, n in enumerate(lengths)])
+        assert got.shape == (batch, vocab)
+        want = torch.cat([plain.logits(ids[r], rows=[n]) for r, n in enumerate(lengths)])
+        close(got, want, dtype, f"head, {batch} decoded rows")
+        assert torch.equal(got.argmax(dim=1).cpu(), want.argmax(dim=1)) or dtype == "bfloat16"
+        for r in range(batch):
+            runner.free_request(r)
+    runner.cache.check()
+    del runner, model
+    torch.cuda.empty_cache()
+
+
+def test_recorded_decode_steps_at_the_benchmark_contexts(head_shape):
+    """Three requests decode from 3,065 to 3,085 keys and, after a prompt portion each, from 4,075 to 4,090: into and
+    inside the context bucket of 4,096 keys, the model's last positions, whose recording cuts every request's keys into
+    the splits chosen for 4,096.  Every replay against the eager step and the plain implementation."""
+    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.models.factory import load_model
+
+    folder, plain = head_shape
+    vocab = HEAD_SHAPE["vocab_size"]
+    legs = ((3065, 20), (4075, 15))
+    shift = (0, 1, 40)                           # the requests' contexts differ a little
+    ids = [token_ids(vocab, 4090 - s, seed=700 + r) for r, s in enumerate(shift)]
+    _, model = load_model(folder, mode="bfloat16")
+    results, rows_of = [], {r: [] for r in range(3)}
+    for graphs in (True, False):
+        runner = ModelRunner(model, page_size=16, num_pages=3 * 256 + 2, max_requests=3, use_graphs=graphs)
+        runner.GRAPH_AFTER_STEPS = 1
+        fed, got = [0, 0, 0], {r: [] for r in range(3)}
+        for r in range(3):
+            runner.add_request(r)
+            runner.reserve(r, len(ids[r]))
+        for start, steps in legs:
+            for r, s in enumerate(shift):
+                runner.step([StepEntry(r, ids[r][fed[r]:start - s], [])])
+                fed[r] = start - s
+            for _ in range(steps):
+                logits = runner.step([StepEntry(r, [ids[r][fed[r]]], [0]) for r in range(3)])
+                for r in range(3):
+                    got[r].append(logits[r])
+                    if graphs:
+                        rows_of[r].append(fed[r])
+                    fed[r] += 1
+        assert fed == [len(x) for x in ids]
+        # (the first leg walks from the bucket of 3,072 keys into that of 4,096: two recordings)
+        assert runner.graph_records == (2 if graphs else 0) and runner.graph_replays == (33 if graphs else 0)
+        results.append({r: torch.stack(v) for r, v in got.items()})
+        runner.cache.reset()
+        runner.cache.check()
+        del runner
+    recorded, eager = results
+    for r in range(3):
+        want = plain.logits(ids[r], rows=rows_of[r])
+        close(recorded[r], want, "bfloat16", f"recorded at the benchmark's contexts, request {r}")
+        close(eager[r], want, "bfloat16", f"eager at the benchmark's contexts, request {r}")
+        close(recorded[r], eager[r], "bfloat16", f"recorded against eager at the benchmark's contexts, request {r}",
+              SPLIT_TOL)
+    del model
+    torch.cuda.empty_cache()
+
+
 FAR_PAGES = dict(
     architectures=["Qwen3ForCausalLM"], model_type="qwen3", vocab_size=300, hidden_size=512, intermediate_size=768,
     num_hidden_layers=1, num_attention_heads=16, num_key_value_heads=8, head_dim=128, max_position_embeddings=512,
