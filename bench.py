@@ -267,8 +267,8 @@ def main() -> int:
                + [(n + page - 1) // page + 1 for n in [args.prefill_tokens] + list(prefill_points.values())])
     runner = ModelRunner(model, page_size=page, num_pages=pool, max_requests=max_batch + 1)
     for g in runner.cache.groups:  # a cache that looks computed: random keys and values
-        g.keys.normal_(0.0, 1.0)
-        g.values.normal_(0.0, 1.0)
+        for t in g.spec.tensors(g.storage):
+            t.normal_(0.0, 1.0)
     sampler = Sampler(cfg.vocab_size, max_batch + 1, device)
     gen = torch.Generator().manual_seed(args.seed)
 

@@ -3,15 +3,13 @@ one pool per group of runs with the same needs, and slots of fixed size for
 per-request state.
 
 What a run (an entry of the model's execution order) needs is said by its
-mixer as a spec:
+mixer as a cache spec (``cache/specs.py``): something for every token, in pages
+(with a window, pages wholly below it are given back while the request still
+runs), or one array of fixed shape per request, or ``None`` (nothing, or the
+run reads another run's cache).  The manager asks a spec what it stores, how
+much, and what view a run gets; it holds no knowledge of keys and values.
 
-* ``PagedKVSpec`` — keys and values of every token, in pages.  ``window`` set:
-  only the last ``window`` keys are ever read, so pages wholly below the
-  window are given back while the request is still running.
-* ``StateSpec`` — one array of fixed shape per request.
-* ``None`` — nothing (or the run reads another run's cache).
-
-Runs with an equal ``PagedKVSpec`` form a group: one page pool and one block
+Runs with equal per-token specs form a group: one page pool and one block
 table per request serve all of them, and page ``p`` means slice ``p`` of every
 run of the group (reference: src/runtime/kv_cache_manager.cpp:56-76, one group
 of all layers; growth and release there: :83-173, :175-204).  Groups with
@@ -24,25 +22,10 @@ never allocates.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Any, Dict, Hashable, List, Optional, Sequence, Tuple
 
 from .page_pool import OutOfPages, PageError, PagePool
-
-
-@dataclass(frozen=True)
-class PagedKVSpec:
-    num_kv_heads: int
-    head_dim: int
-    window: Optional[int] = None  # None: all keys
-
-    def bytes_per_token(self, element_size: int) -> int:
-        return 2 * self.num_kv_heads * self.head_dim * element_size
-
-
-@dataclass(frozen=True)
-class StateSpec:
-    shape: Tuple[int, ...]
-    dtype: str = "float32"
+from .specs import PagedKVSpec, StateSpec, check_spec  # noqa: F401  (the two specs are part of this module's names)
 
 
 class CacheError(RuntimeError):
@@ -82,22 +65,25 @@ class CacheGroup:
     """Runs that share a page pool and block tables."""
 
     index: int
-    spec: PagedKVSpec
+    spec: Any              # the per-token cache spec that all its runs share
     page_size: int
     runs: List[int]
     pool: PagePool
     tables: Dict[Hashable, List[int]] = field(default_factory=dict)  # -1: page given back (below the window)
-    keys: object = None    # [runs, pages, kv_heads, page_size, head_dim]
-    values: object = None  # [runs, pages, kv_heads, head_dim, page_size]
+    storage: Any = None    # what the spec allocated for all runs of the group
+
+    @property
+    def window(self) -> Optional[int]:
+        return getattr(self.spec, "window", None)
 
     def pages_for(self, length: int) -> int:
         return (length + self.page_size - 1) // self.page_size
 
     def first_needed_token(self, computed: int) -> int:
         """The lowest key position that a token at position >= computed can still read."""
-        if self.spec.window is None:
+        if self.window is None:
             return 0
-        return max(0, computed - self.spec.window + 1)
+        return max(0, computed - self.window + 1)
 
 
 @dataclass
@@ -111,8 +97,8 @@ class _Request:
 
 class CacheManager:
     def __init__(self, run_specs: Sequence[object], page_size: int, num_pages: int, max_requests: int,
-                 group_pages: Optional[Dict[PagedKVSpec, int]] = None):
-        """``run_specs[r]`` is the spec of run ``r`` (PagedKVSpec, StateSpec or None).
+                 group_pages: Optional[Dict[Any, int]] = None):
+        """``run_specs[r]`` is the cache spec of run ``r``, or None.
 
         ``num_pages`` is the pool size of every paged group unless ``group_pages`` names one for a spec.
         """
@@ -122,10 +108,13 @@ class CacheManager:
         self.run_specs = list(run_specs)
         self.groups: List[CacheGroup] = []
         self.run_group: Dict[int, Tuple[int, int]] = {}   # run -> (group, index within group)
-        self.state_runs: Dict[int, StateSpec] = {}
-        by_spec: Dict[PagedKVSpec, CacheGroup] = {}
+        self.state_runs: Dict[int, Any] = {}
+        by_spec: Dict[Any, CacheGroup] = {}
         for run, spec in enumerate(self.run_specs):
-            if isinstance(spec, PagedKVSpec):
+            if spec is None:
+                continue
+            check_spec(spec, run)
+            if spec.per_token:
                 group = by_spec.get(spec)
                 if group is None:
                     pages = (group_pages or {}).get(spec, num_pages)
@@ -134,10 +123,8 @@ class CacheManager:
                     self.groups.append(group)
                 self.run_group[run] = (group.index, len(group.runs))
                 group.runs.append(run)
-            elif isinstance(spec, StateSpec):
+            else:
                 self.state_runs[run] = spec
-            elif spec is not None:
-                raise TypeError(f"run {run}: unknown cache spec {spec!r}")
         self.slots = StateSlots(max_requests)
         self.requests: Dict[Hashable, _Request] = {}
         self.state: Dict[int, object] = {}  # run -> [slots, *shape] array
@@ -150,16 +137,22 @@ class CacheManager:
 
     # ------------------------------------------------------------------ storage
     def allocate_storage(self, device, dtype) -> None:
-        """Create the page and state arrays (torch tensors) on ``device``."""
-        import torch
-
+        """Create the page and state arrays on ``device``: every spec allocates its own."""
         for g in self.groups:
-            n, p, s = len(g.runs), g.pool.num_pages, g.spec
-            g.keys = torch.zeros((n, p, s.num_kv_heads, g.page_size, s.head_dim), dtype=dtype, device=device)
-            g.values = torch.zeros((n, p, s.num_kv_heads, s.head_dim, g.page_size), dtype=dtype, device=device)
+            g.storage = g.spec.allocate(len(g.runs), g.pool.num_pages, g.page_size, device, dtype)
         for run, spec in self.state_runs.items():
-            self.state[run] = torch.zeros((self.slots.num_slots, *spec.shape), dtype=getattr(torch, spec.dtype),
-                                          device=device)
+            self.state[run] = spec.allocate(1, self.slots.num_slots, self.page_size, device, dtype)
+
+    def view(self, run: int, writable: bool = True) -> Any:
+        """What run ``run`` is handed as its cache in a step (None for a run that keeps nothing)."""
+        spec = self.run_specs[run]
+        if spec is None:
+            return None
+        if spec.per_token:
+            g, i = self.run_group[run]
+            group = self.groups[g]
+            return spec.view(group.storage, i, g, group.page_size, writable)
+        return spec.view(self.state[run], 0, -1, self.page_size, writable)
 
     def storage_bytes(self, element_size: int) -> int:
         return sum(len(g.runs) * g.pool.num_pages * g.page_size * g.spec.bytes_per_token(element_size)
@@ -245,7 +238,7 @@ class CacheManager:
             raise CacheError(f"request {request!r} computed {computed} tokens but pages are reserved for {req.reserved}")
         req.computed = computed
         for g in self.groups:
-            if g.spec.window is None:
+            if g.window is None:
                 continue
             table = g.tables[request]
             dead = min(g.first_needed_token(computed) // g.page_size, len(table))

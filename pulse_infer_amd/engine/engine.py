@@ -211,26 +211,37 @@ class ContinuousBatchEngine:
     def run_until_complete(self, print_progress: bool = False, one_step_ahead: bool = True) -> None:
         step = 0
         flight: Optional[_InFlight] = None
-        while True:
-            if print_progress and step % 10 == 0 and self.scheduler.has_work():
-                s = self.scheduler.get_stats()
-                print(f"[pulse_infer_amd] step {step}: {s.num_running} requests running, {s.num_waiting} waiting, "
-                      f"{s.num_finished} finished", file=sys.stderr, flush=True)
-            if not one_step_ahead:
-                if not self.scheduler.has_work() or self.step().empty():
+        try:
+            while True:
+                if print_progress and step % 10 == 0 and self.scheduler.has_work():
+                    s = self.scheduler.get_stats()
+                    print(f"[pulse_infer_amd] step {step}: {s.num_running} requests running, {s.num_waiting} waiting, "
+                          f"{s.num_finished} finished", file=sys.stderr, flush=True)
+                if not one_step_ahead:
+                    if not self.scheduler.has_work() or self.step().empty():
+                        break
+                    step += 1
+                    continue
+                batch = self.scheduler.schedule_next_batch() if self.scheduler.has_work() else None
+                self.last_batch = batch if batch is not None else self.last_batch
+                queued = self._launch(batch, flight) if batch is not None and not batch.empty() else None
+                if flight is not None:
+                    settling, flight = flight, None
+                    self._settle(settling)
+                if queued is None:     # nothing left, or nothing that can be scheduled (as ``step`` returning an empty batch)
                     break
+                self._assume(queued)
+                flight = queued
                 step += 1
-                continue
-            batch = self.scheduler.schedule_next_batch() if self.scheduler.has_work() else None
-            self.last_batch = batch if batch is not None else self.last_batch
-            queued = self._launch(batch, flight) if batch is not None and not batch.empty() else None
+        finally:
+            # Only an error leaves a step in flight here (the scheduler's, a kernel's, an interrupt, between the step's
+            # launch and the arrival of its tokens): the tokens are still taken, so that no request keeps a
+            # place-holder for a token, or a finish reason that only the place-holder gave it.
             if flight is not None:
-                self._settle(flight)
-            if queued is None:     # nothing left, or nothing that can be scheduled (as ``step`` returning an empty batch)
-                break
-            self._assume(queued)
-            flight = queued
-            step += 1
+                try:
+                    self._settle(flight)
+                except Exception:      # (the device may be what failed; the error under way says more than this one)
+                    pass
         if print_progress:
             s = self.scheduler.get_stats()
             print(f"[pulse_infer_amd] all {s.total_requests} requests finished after {step} steps", file=sys.stderr,

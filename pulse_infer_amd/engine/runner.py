@@ -20,9 +20,9 @@ from typing import Any, Hashable, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..cache.manager import CacheManager, PagedKVSpec, StateSpec
+from ..cache.manager import CacheManager
 from ..models.causal_lm import CausalLM
-from ..parts.base import EntryMeta, PagedCacheView, StateView, StepContext, contexts_uneven
+from ..parts.base import EntryMeta, StepContext, contexts_uneven
 
 
 class StepError(ValueError):
@@ -99,25 +99,12 @@ class ModelRunner:
         self.device = model.device
         self.cache = CacheManager(model.run_cache_specs(), page_size, num_pages, max_requests)
         self.cache.allocate_storage(self.device, model.act_dtype)
-        self.views: List[Any] = []
-        order = model.spec.order
-        for index, run in enumerate(order):
-            source = run.cache_of if run.cache_of is not None else index
-            spec = self.cache.run_specs[source]
-            if isinstance(spec, PagedKVSpec):
-                g, i = self.cache.run_group[source]
-                group = self.cache.groups[g]
-                self.views.append(PagedCacheView(group=g, keys=group.keys[i], values=group.values[i],
-                                                 page_size=group.page_size, writable=run.cache_of is None))
-            elif isinstance(spec, StateSpec):
-                self.views.append(StateView(self.cache.state[source]))
-            else:
-                self.views.append(None)
+        # what every run of the order is handed as its cache: a view of its own storage, or of the run's it reads
+        self.views: List[Any] = [
+            self.cache.view(run.cache_of if run.cache_of is not None else index, writable=run.cache_of is None)
+            for index, run in enumerate(model.spec.order)]
         self._staging = _Staging(self.device)
-        # a step is recorded only if every part it runs says that it records cleanly (Part.records_cleanly)
-        clean = all(getattr(model.blocks[run.layer], "records_cleanly", lambda: False)() for run in order) and all(
-            getattr(p, "records_cleanly", False) for p in getattr(model, "positions", {}).values())
-        self.use_graphs = bool(use_graphs) and model.options.get("decode_graph", True) and clean
+        self.use_graphs = bool(use_graphs) and model.options.get("decode_graph", True)
         self._graphs: dict = {}
         self._graph_seen: dict = {}
         self._graph_refused: set = set()   # shapes whose step holds a library call: no library call is ever recorded
@@ -288,16 +275,19 @@ class ModelRunner:
     # so it is recorded once per (batch, context bucket, whether the contexts differ much: parts may share their work
     # out differently then) as a HIP graph over buffers of its own and replayed: the host then only copies the
     # step's integers and starts the graph.
-    GRAPH_MAX_BATCH = 64        # up to here every product can be this package's own kernel; a shape whose step does
-                                # call the vendor library (seen when it is first run for recording) stays eager
     GRAPH_CONTEXT_BUCKET = 1024
     GRAPH_LIMIT = 64            # recordings kept
     GRAPH_AFTER_STEPS = 4       # a (batch, context bucket) is recorded when it comes for this many-th time
 
     def _graph_ok(self, entries: Sequence[StepEntry], metas: List[EntryMeta]) -> bool:
-        if not self.use_graphs or self.model.mode != "bfloat16" or len(metas) > self.GRAPH_MAX_BATCH:
+        """A step can be replayed if it has the form whose integers ``_refill`` rewrites (a token a request, every one
+        wanting its logits) and the model says that such a step records (``recordable``: its parts issue the same
+        launches whatever the step's values are, in this run mode, at this many rows)."""
+        if not self.use_graphs:
             return False
-        return all(m.count == 1 for m in metas) and all(list(e.want) == [0] for e in entries)
+        if not (all(m.count == 1 for m in metas) and all(list(e.want) == [0] for e in entries)):
+            return False
+        return self.model.recordable(metas)
 
     def _graph_key(self, batch: int, max_context: int, uneven: bool):
         bucket = (max_context + self.GRAPH_CONTEXT_BUCKET - 1) // self.GRAPH_CONTEXT_BUCKET * self.GRAPH_CONTEXT_BUCKET

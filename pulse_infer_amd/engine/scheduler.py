@@ -114,7 +114,7 @@ class ContinuousBatchScheduler:
             raise SchedulerError(f"request needs {longest} positions, the model allows {self.max_positions}")
         if self.cache is not None:
             for g, need in zip(self.cache.groups, self.cache.pages_needed_new(longest)):
-                if g.spec.window is None and need > g.pool.num_pages:
+                if g.window is None and need > g.pool.num_pages:
                     raise SchedulerError(f"request needs {need} cache pages of {g.page_size} tokens, "
                                          f"the pool has {g.pool.num_pages}")
         self.next_request_id += 1

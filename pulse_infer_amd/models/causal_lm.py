@@ -13,8 +13,8 @@ from typing import Any, Dict, List, Optional
 
 import torch
 
-from ..parts.base import BLOCKS, NORMS, POSITIONS, BuildContext, ResidualStream, StepContext, Workspace, joined
-from ..parts.embedding import OutputHead, TokenEmbedding
+from ..parts.base import (BLOCKS, EMBEDDINGS, HEADS, NORMS, POSITIONS, BuildContext, EntryMeta, ResidualStream,
+                          StepContext, Workspace, joined, says)
 from ..weights.store import TensorSpec, WeightLoader
 from .spec import ModelSpec
 
@@ -24,12 +24,12 @@ ACT_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 def expected_tensors(spec: ModelSpec) -> Dict[str, TensorSpec]:
     """Every tensor the model loads, by checkpoint name."""
     out: Dict[str, TensorSpec] = {}
-    out.update(TokenEmbedding.weight_specs(spec.embedding.params))
+    out.update(EMBEDDINGS.get(spec.embedding.kind).weight_specs(spec.embedding.params))
     for layer in spec.layers:
         out.update(BLOCKS.get(layer.block.kind).layer_weight_specs(layer))
     for name, ts in NORMS.get(spec.final_norm.kind).weight_specs(spec.final_norm.params).items():
         out[joined(spec.final_norm_prefix, name)] = ts
-    for name, ts in OutputHead.weight_specs(spec.head.params).items():
+    for name, ts in HEADS.get(spec.head.kind).weight_specs(spec.head.params).items():
         out.setdefault(name, ts)
     return out
 
@@ -54,12 +54,13 @@ class CausalLM:
             params.setdefault("name", name)
             build.positions[name] = POSITIONS.get(part.kind)(params, build)
         self.positions = build.positions
-        self.embedding = TokenEmbedding(spec.embedding.params, build)
+        self.embedding = EMBEDDINGS.get(spec.embedding.kind)(spec.embedding.params, build)
         self.blocks = [BLOCKS.get(layer.block.kind)(layer, build) for layer in spec.layers]
         self.final_norm = NORMS.get(spec.final_norm.kind)(spec.final_norm.params, spec.final_norm_prefix, build)
-        self.head = OutputHead(spec.head.params, build, self.embedding)
+        self.head = HEADS.get(spec.head.kind)(spec.head.params, build, self.embedding)
         self.vocab_size = spec.vocab_size
         self.hidden_size = spec.hidden_size
+        self._clean: Optional[bool] = None
 
     # ------------------------------------------------------------------- caches
     def run_cache_specs(self) -> List[Any]:
@@ -68,6 +69,26 @@ class CausalLM:
         for run in self.spec.order:
             out.append(None if run.cache_of is not None else self.blocks[run.layer].cache_spec())
         return out
+
+    # ---------------------------------------------------------------- recording
+    MAX_RECORDED_ROWS = 64      # up to here every product of a step of single tokens can be this package's own kernel;
+                                # a shape whose step does call the vendor library (seen when it is first run for
+                                # recording) stays eager
+
+    def records_cleanly(self) -> bool:
+        """Whether every part of the model says that its launches do not depend on a step's values
+        (``Part.records_cleanly``, an attribute or a method)."""
+        if self._clean is None:
+            parts: List[Any] = [self.embedding, self.final_norm, self.head]
+            parts += [self.blocks[run.layer] for run in self.spec.order]
+            parts += list(self.positions.values())
+            self._clean = all(says(part, "records_cleanly") for part in parts)
+        return self._clean
+
+    def recordable(self, entries: List[EntryMeta]) -> bool:
+        """Whether a step of these entries (one token each, every one wanting its logits: the form the step function
+        can replay) may be recorded as a graph and replayed with other values."""
+        return self.mode == "bfloat16" and len(entries) <= self.MAX_RECORDED_ROWS and self.records_cleanly()
 
     # --------------------------------------------------------------------- step
     def forward(self, ctx: StepContext, cache_views: List[Any]) -> torch.Tensor:

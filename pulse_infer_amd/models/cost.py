@@ -6,7 +6,7 @@ from __future__ import annotations
 
 from typing import List, Tuple
 
-from ..parts.base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, StepCost
+from ..parts.base import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, StepCost
 from .spec import ModelSpec
 
 
@@ -17,10 +17,7 @@ def step_cost(spec: ModelSpec, entries: List[Tuple[int, int]], wanted: int, weig
 
     Weights count once a step (every run of the order that names a layer again reads them again); the embedding
     table counts its gathered rows only; the head counts its whole matrix and the arithmetic of the wanted rows."""
-    rows = sum(count for _, count in entries)
-    cost = StepCost()
-    hidden, vocab = spec.hidden_size, spec.vocab_size
-    cost.weight_bytes += rows * hidden * weight_bytes                      # embedding rows
+    cost = EMBEDDINGS.get(spec.embedding.kind).step_cost(spec.embedding.params, entries, weight_bytes, cache_bytes)
     for run in spec.order:
         layer = spec.layers[run.layer]
         block = BLOCKS.get(layer.block.kind)
@@ -32,6 +29,4 @@ def step_cost(spec: ModelSpec, entries: List[Tuple[int, int]], wanted: int, weig
             cost = cost + NORMS.get(norm.kind).step_cost(norm.params, entries, weight_bytes, cache_bytes)
     cost = cost + NORMS.get(spec.final_norm.kind).step_cost(spec.final_norm.params, [(0, wanted)], weight_bytes,
                                                              cache_bytes)
-    cost.weight_bytes += float(vocab) * hidden * weight_bytes              # the head's matrix (tied or its own)
-    cost.flops += 2.0 * wanted * vocab * hidden
-    return cost
+    return cost + HEADS.get(spec.head.kind).step_cost(spec.head.params, [(0, wanted)], weight_bytes, cache_bytes)

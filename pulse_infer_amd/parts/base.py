@@ -13,6 +13,11 @@ and built from a ``PartSpec`` (its kind and its parameters):
   mixers consume (rotation tables here).
 * **block** — the arrangement of the above around the residual stream.
 
+Two more kinds stand at the model's ends: the **embedding**
+(``forward(ids, out)`` fills the float32 residual) and the **output head**
+(``forward(x, out)`` gives float32 logits for the normed rows it is handed; it
+is built with the embedding at hand, for weights the two share).
+
 Every part states the tensors it loads with ``weight_specs(params)`` (names
 relative to its prefix), so the loader can check a checkpoint, and the random
 initialiser can create one, before anything is built.  No part knows which
@@ -25,6 +30,7 @@ from typing import Any, Callable, Dict, List, Optional, Tuple
 
 import torch
 
+from ..cache.specs import PagedCacheView, StateView  # noqa: F401  (what a mixer is handed as its cache)
 from ..weights.store import TensorSpec, WeightLoader
 
 
@@ -62,6 +68,8 @@ FEED_FORWARDS = Registry("feed-forward")
 NORMS = Registry("norm")
 POSITIONS = Registry("position encoding")
 BLOCKS = Registry("block")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("output head")
 
 
 class Workspace:
@@ -113,24 +121,6 @@ class EntryMeta:
     start: int      # position of its first token in this step = tokens already in the cache
     count: int      # tokens in this step
     first_row: int  # where they start among the step's tokens
-
-
-@dataclass
-class PagedCacheView:
-    """The pages of one run of a paged group."""
-
-    group: int
-    keys: torch.Tensor     # [pages, kv_heads, page_size, head_dim]
-    values: torch.Tensor   # [pages, kv_heads, head_dim, page_size]
-    page_size: int
-    writable: bool = True  # False: the run reads a cache that another run writes
-
-
-@dataclass
-class StateView:
-    """The per-request state of one run: row ``slot`` belongs to the request in that slot."""
-
-    state: torch.Tensor    # [slots, *shape]
 
 
 UNEVEN_CONTEXTS = 1.5     # longest context / mean context from which a step counts as uneven
@@ -323,6 +313,13 @@ class Part:
             if len(spec.shape) == 2 and spec.kind == "linear":
                 cost.flops += 2.0 * rows * n
         return cost
+
+
+def says(part: Any, name: str) -> bool:
+    """A part's yes or no to ``name``, whether it gives it as an attribute or as a method; a part that does not say
+    is a no."""
+    value = getattr(part, name, False)
+    return bool(value() if callable(value) else value)
 
 
 def joined(prefix: str, name: str) -> str:

@@ -10,7 +10,7 @@ from typing import Any, Dict, Optional
 
 from ..models.spec import LayerSpec
 from ..weights.store import TensorSpec
-from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BuildContext, Part, ResidualStream, StepContext, joined
+from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, BuildContext, Part, ResidualStream, StepContext, joined, says
 
 
 @BLOCKS.register("prenorm")
@@ -50,7 +50,7 @@ class PreNormBlock(Part):
 
     def records_cleanly(self) -> bool:
         """Whether a step of this block may be recorded as a graph and replayed: every part of it says so."""
-        return all(getattr(part, "records_cleanly", False)
+        return all(says(part, "records_cleanly")
                    for part in (self.mixer, self.ffn, self.mixer_norm, self.ffn_norm))
 
     def _input(self, stream: ResidualStream, norm: Any, part: Any, ctx: StepContext) -> Any:

@@ -7,21 +7,31 @@ checkpoint holds it, else the embedding table when the configuration ties them
 """
 from __future__ import annotations
 
-from typing import Any, Dict
+from typing import Any, Dict, List, Tuple
 
 import torch
 
 from ..ops import kernels
 from ..weights.store import TensorSpec
-from .base import BuildContext, Part
+from .base import EMBEDDINGS, HEADS, BuildContext, Part, StepCost
 from .linear import Linear
 
 
+@EMBEDDINGS.register("embedding")
 class TokenEmbedding(Part):
+    records_cleanly = True
+
     @classmethod
     def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
         return {params["name"]: TensorSpec((params["vocab_size"], params["hidden_size"]), kind="embedding",
                                            fan_in=params["hidden_size"])}
+
+    @classmethod
+    def step_cost(cls, params: Dict[str, Any], entries: List[Tuple[int, int]], weight_bytes: int,
+                  cache_bytes: int) -> StepCost:
+        """Only the gathered rows of the table are read."""
+        rows = sum(count for _, count in entries)
+        return StepCost(weight_bytes=float(rows) * params["hidden_size"] * weight_bytes)
 
     def __init__(self, params: Dict[str, Any], build: BuildContext):
         self.vocab = int(params["vocab_size"])
@@ -43,7 +53,18 @@ class TokenEmbedding(Part):
         return seen
 
 
+@HEADS.register("lm_head")
 class OutputHead(Part):
+    records_cleanly = True
+
+    @classmethod
+    def step_cost(cls, params: Dict[str, Any], entries: List[Tuple[int, int]], weight_bytes: int,
+                  cache_bytes: int) -> StepCost:
+        """The whole matrix (tied or its own) is read once; ``entries`` holds the wanted rows as one entry."""
+        rows = sum(count for _, count in entries)
+        size = float(params["vocab_size"]) * params["hidden_size"]
+        return StepCost(flops=2.0 * rows * size, weight_bytes=size * weight_bytes)
+
     @classmethod
     def weight_specs(cls, params: Dict[str, Any]) -> Dict[str, TensorSpec]:
         # with tied embeddings the head's own tensor may be absent; if present it is used
