@@ -3,18 +3,21 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-A "step" is one decode step of the whole batch: the step function on one token
-per request, the argmax kernel, and the tokens' way back to the host and into
-the next step.  Weights are random (made on the GPU), token ids are seeded
-synthetic ids, and for the fixed-context points the cache of the context before
-the timed steps is filled with random keys and values instead of being computed
-(its content does not change the work of a decode step).  Every point is timed
-three times and the median is reported; ``value`` is the batch over the median
-step time of ``--steps`` steps at contexts ending at ``--context``.  ``trajectory``
-is the workload as stated, end to end: every request a prompt of ``--prefill-tokens``
-tokens and as many greedy tokens, through the scheduler, the step function and
-the sampler.  Bytes and arithmetic of the rooflines come from the model's own
-description (``models/cost.py``), not from formulas of one architecture.
+A "step" is one decode step of the whole batch, as the engine's own serving loop
+runs it (``ContinuousBatchEngine.run_until_complete``): the scheduler's decision,
+the step function on one token per request, the argmax kernel, and the tokens'
+way back to the host and into the next step, which is queued while this one is
+computed.  Weights are random (made on the GPU), token ids are seeded synthetic
+ids, and for the fixed-context points the requests are admitted with the context
+before the timed steps counting as computed, over a cache filled with random
+keys and values (its content does not change the work of a decode step).  Every
+point is timed three times and the median is reported; ``value`` is the batch
+over the median step time of ``--steps`` steps at contexts ending at
+``--context``.  ``trajectory`` is the workload as stated, end to end: every
+request a prompt of ``--prefill-tokens`` tokens and as many greedy tokens;
+``serving`` is continuous batching of 32 requests with seeded prompt lengths.
+Bytes and arithmetic of the rooflines come from the model's own description
+(``models/cost.py``), not from formulas of one architecture.
 ``--kernels`` prints where one decode step's time goes, entry point by entry
 point.  Prints one JSON line.
 """
@@ -67,10 +70,12 @@ def parse_args() -> argparse.Namespace:
     p.add_argument("--prefill-tokens", type=int, default=2048)
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--dtype", choices=["bfloat16", "float32"], default="bfloat16")
-    p.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
+    p.add_argument("--no-points", action="store_true",
+                   help="skip the further points (batch 1 / 16 / 32 / 64, batch 8 at a context of 16,384, prompts of "
+                        "512 and 8,192 tokens)")
     p.add_argument("--more-points", action="store_true",
-                   help="further points: batch 8 at contexts of 1,024 / 16,384 / 40,000, batch 16 / 32 / 128 at the "
-                        "context, prompts of 512 and 8,192 tokens")
+                   help="points that need a larger cache pool: batch 8 at contexts of 1,024 and 40,000, batch 128")
+    p.add_argument("--no-serving", action="store_true", help="skip the serving workload at the end of the default run")
     p.add_argument("--no-prefill", action="store_true")
     p.add_argument("--no-trajectory", action="store_true",
                    help="skip the end-to-end run (prompt + as many greedy tokens per request through the scheduler)")
@@ -123,8 +128,9 @@ def trajectory(args, cfg, model, batch: int, prompt_tokens: int, new_tokens: int
             "decode_ms_per_step": round(decode_s * 1e3 / max(1, decode_steps), 4), "steps": stats.num_steps}
 
 
-def serving(args, cfg, model, full_layers: int) -> int:
-    """Continuous batching end to end: every request through the scheduler, the step function and the sampler."""
+def serving(args, cfg, model, full_layers: int) -> dict:
+    """Continuous batching end to end: every request through the scheduler, the step function and the sampler.
+    Returns the record of the run (the whole JSON line of ``--workload serving``)."""
     import torch
 
     from pulse_infer_amd.engine.engine import ContinuousBatchEngine
@@ -157,7 +163,7 @@ def serving(args, cfg, model, full_layers: int) -> int:
     stats.num_steps -= before.num_steps
     stats.tokens_computed -= before.tokens_computed
     total = stats.tokens_generated - before.tokens_generated
-    print(json.dumps({
+    record = {
         "metric": f"qwen3_{args.model}_serving_output_tokens_per_s", "value": round(total / seconds, 2), "unit": "tokens/s",
         "n_gpus": 1, "steps": stats.num_steps, "warmup": before.num_steps, "ms_per_step": round(seconds * 1e3 / max(1, stats.num_steps), 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
@@ -168,8 +174,10 @@ def serving(args, cfg, model, full_layers: int) -> int:
                    "temperature": args.temperature,
                    "prompt_tokens": sum(lengths), "preemptions": stats.num_preemptions},
         "seconds": round(seconds, 3), "tokens_computed": stats.tokens_computed,
-        "steps_recorded": engine.runner.graph_records, "steps_replayed": engine.runner.graph_replays}))
-    return 0
+        "steps_recorded": engine.runner.graph_records, "steps_replayed": engine.runner.graph_replays}
+    del engine
+    torch.cuda.empty_cache()
+    return record
 
 
 def long_prompt(args, cfg, model, full_layers: int) -> int:
@@ -223,10 +231,9 @@ def main() -> int:
 
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     from pulse_infer_amd.config import Qwen3Config
-    from pulse_infer_amd.engine.runner import ModelRunner, StepEntry
+    from pulse_infer_amd.engine.engine import ContinuousBatchEngine
     from pulse_infer_amd.models.causal_lm import expected_tensors
     from pulse_infer_amd.models.factory import build_model
-    from pulse_infer_amd.sampling.sampler import Sampler
     from pulse_infer_amd.sampling.params import SamplingParams
     from pulse_infer_amd.weights.random_init import RandomSource
 
@@ -243,7 +250,8 @@ def main() -> int:
     model = build_model(cfg, source, mode=args.dtype, device=device)
 
     if args.workload == "serving":
-        return serving(args, cfg, model, full_layers)
+        print(json.dumps(serving(args, cfg, model, full_layers)))
+        return 0
     if args.workload == "long-prompt":
         return long_prompt(args, cfg, model, full_layers)
 
@@ -252,81 +260,56 @@ def main() -> int:
     spec = cfg.model_spec()
     peak_flops = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
     # (batch, context) of every decode point, prompt lengths of every prefill point
-    decode_points = {} if args.no_points else {"decode_b1": (1, args.context), "decode_b64": (64, args.context)}
-    prefill_points = {}
-    if args.more_points:
-        for ctx in (1024, 16384, 40000):
-            decode_points[f"decode_b8_ctx{ctx}"] = (8, ctx)
-        for b in (16, 32, 128):
-            decode_points[f"decode_b{b}"] = (b, args.context)
+    decode_points, prefill_points = {}, {}
+    if not args.no_points:
+        decode_points = {"decode_b1": (1, args.context), "decode_b64": (64, args.context),
+                         "decode_b16": (16, args.context), "decode_b32": (32, args.context),
+                         "decode_b8_ctx16384": (8, 16384)}
         prefill_points = {"prefill_512": 512, "prefill_8192": 8192}
+    if args.more_points:
+        for ctx in (1024, 40000):
+            decode_points[f"decode_b8_ctx{ctx}"] = (8, ctx)
+        decode_points["decode_b128"] = (128, args.context)
     shapes = [(args.batch, args.context)] + list(decode_points.values())
     max_batch = max(b for b, _ in shapes)
     page = args.page_size
-    pool = max([b * ((c + page - 1) // page + 1) for b, c in shapes]
-               + [(n + page - 1) // page + 1 for n in [args.prefill_tokens] + list(prefill_points.values())])
-    runner = ModelRunner(model, page_size=page, num_pages=pool, max_requests=max_batch + 1)
+    prompts = [args.prefill_tokens] + list(prefill_points.values())
+    pool = max([b * ((c + page - 1) // page + 1) for b, c in shapes] + [(n + page - 1) // page + 1 for n in prompts])
+    # every point runs through the engine's own serving loop; a prompt that has a step to itself runs in one portion
+    engine = ContinuousBatchEngine(model, max_batch_size=max_batch, chunk_size=512, page_size=page, num_pages=pool,
+                                   max_sequences=max_batch, max_num_batched_tokens=max(prompts), seed=args.seed)
+    runner = engine.runner
     for g in runner.cache.groups:  # a cache that looks computed: random keys and values
         for t in g.spec.tensors(g.storage):
             t.normal_(0.0, 1.0)
-    sampler = Sampler(cfg.vocab_size, max_batch + 1, device)
     gen = torch.Generator().manual_seed(args.seed)
+    greedy = SamplingParams(ignore_eos=True)
 
     def decode_run(batch: int, context: int, steps: int, warmup: int, runs: int):
         """``runs`` timings of ``steps`` decode steps of ``batch`` requests whose contexts end at ``context`` (every run
-        walks the same contexts).  Returns (median seconds a step by the host's clock between two synchronisations,
-        the same by GPU events, every run's host figure)."""
+        walks the same contexts), through ``run_until_complete``.  Returns (median seconds a step by the host's clock
+        between two synchronisations, the same by GPU events, every run's host figure)."""
         start = context - (steps + warmup)
         if start < 1:
             raise SystemExit(f"a context of {context} is too short for {steps} + {warmup} steps")
-        names = [f"d{batch}_{i}" for i in range(batch)]
-        greedy = [SamplingParams()] * batch
         host, events = [], []
         for _ in range(runs):
-            for n in names:
-                runner.add_request(n)
-                runner.reserve(n, context)
-                runner.cache.advance(n, start)          # the context so far counts as computed
-            tokens = torch.randint(0, cfg.vocab_size, (batch,), generator=gen).tolist()
-            slots = [runner.cache.slot_of(n) for n in names]
-
-            # As the engine's loop does, a step is queued while the step before it is computed: that step's tokens go
-            # into the new step's ids on the device, and come back to the host (every step's do) while it runs.
-            same = list(range(batch))
-            landing = [torch.empty(batch, dtype=torch.int32, pin_memory=True) for _ in range(2)]
-
-            def queue(toks, before, turn):
-                feed = (before[0], same, same) if before is not None else None
-                logits = runner.step([StepEntry(n, [t], [0]) for n, t in zip(names, toks)], feed=feed)
-                out = sampler.launch(logits, greedy, slots, [0] * batch, [0] * batch)
-                landing[turn].copy_(out, non_blocking=True)
-                landed = torch.cuda.Event()
-                landed.record()
-                return out, landing[turn], landed
-
-            def run_steps(count, toks):
-                flight = queue(toks, None, 0)
-                for i in range(1, count):
-                    ahead = queue([0] * batch, flight, i % 2)
-                    flight[2].synchronize()
-                    toks = flight[1].tolist()           # the tokens of the step before, on the host
-                    flight = ahead
-                flight[2].synchronize()
-                return flight[1].tolist()
-
+            for _ in range(batch):
+                rid = engine.add_request(torch.randint(0, cfg.vocab_size, (start + 1,), generator=gen).tolist(),
+                                         steps + warmup, greedy)
+                engine.admit_as_computed(rid, start)        # the context so far counts as computed
             if warmup:
-                tokens = run_steps(warmup, tokens)
+                assert engine.run_until_complete(max_steps=warmup) == warmup
             first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             first.record()
-            tokens = run_steps(steps, tokens)
+            ran = engine.run_until_complete()
             last.record()
             torch.cuda.synchronize()
+            assert ran == steps and not engine.scheduler.has_work(), (ran, steps)
             host.append((time.perf_counter() - t0) / steps)
             events.append(first.elapsed_time(last) * 1e-3 / steps)
-            for n in names:
-                runner.free_request(n)
         return statistics.median(host), statistics.median(events), host
 
     def decode_bytes(batch: int, context: int, steps: int) -> float:
@@ -339,21 +322,19 @@ def main() -> int:
         ids = torch.randint(0, cfg.vocab_size, (tokens,), generator=gen).tolist()
         times = []
         for r in range(runs + 1):  # the first run warms up
-            runner.add_request("p")
-            runner.reserve("p", tokens)
+            engine.add_request(ids, 1, greedy)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            logits = runner.step([StepEntry("p", ids, [tokens - 1])])
-            sampler.sample(logits, [SamplingParams()], [0], [0], [0])
+            ran = engine.run_until_complete()    # one step of the whole prompt, its last row's token back on the host
             torch.cuda.synchronize()
             seconds = time.perf_counter() - t0
-            runner.free_request("p")
+            assert ran == 1, ran
             if r > 0:
                 times.append(seconds)
         return statistics.median(times)
 
     if args.kernels:
-        return kernel_table(args, cfg, runner, sampler, gen)
+        return kernel_table(args, cfg, runner, engine.sampler, gen)
 
     step_s, step_gpu_s, all_runs = decode_run(args.batch, args.context, args.steps, args.warmup, args.runs)
     value = args.batch / step_s
@@ -395,11 +376,19 @@ def main() -> int:
             fracs[name] = round(step_cost(spec, [(0, n)], 1, element, element).flops / t / peak_flops, 4)
         result["points"] = points
         result["points_frac"] = fracs     # of 8 TB/s for decoding, of the dense matrix-core peak for prompts
+    del runner, engine
+    torch.cuda.empty_cache()
     if not args.no_trajectory:
-        del runner, sampler
-        torch.cuda.empty_cache()
         new_tokens = args.trajectory_tokens or args.prefill_tokens
         result["trajectory"] = trajectory(args, cfg, model, args.batch, args.prefill_tokens, new_tokens)
+    if not args.no_serving:
+        record = serving(args, cfg, model, full_layers)
+        result["serving"] = {"value": record["value"], "unit": "output tokens/s", "requests": args.requests,
+                             "prompt_min": args.prompt_range[0], "prompt_max": args.prompt_range[1],
+                             "output_tokens": args.output_tokens, "chunk": args.chunk,
+                             "token_budget": record["config"]["token_budget"], "temperature": args.temperature,
+                             "seconds": record["seconds"], "steps": record["steps"],
+                             "preemptions": record["config"]["preemptions"]}
     print(json.dumps(result))
     return 0
 

@@ -53,7 +53,10 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--num-pages", type=int, default=None)
     p.add_argument("--max-batch", type=int, default=8, help="most requests in one step")
     p.add_argument("--max-tokens", type=int, default=None, help="most tokens in one step (the budget)")
-    p.add_argument("--chunk", type=int, default=256, help="longest prompt portion in one step")
+    p.add_argument("--chunk", type=int, default=256,
+                   help="a prompt's portion of a step; what the step's budget (--max-tokens) has left when every "
+                        "prompt has its portion extends the portions in order, unless --fixed-chunk is given")
+    p.add_argument("--fixed-chunk", action="store_true", help="no prompt portion is longer than --chunk tokens")
     p.add_argument("--set", dest="overrides", action="append", default=[], metavar="FIELD=VALUE",
                    help="set a field of the model's configuration that is an option of the engine rather than a key of "
                         "config.json (for Qwen3: rope_pairing=half, the channels a rotation pairs); may be repeated")
@@ -119,7 +122,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     overrides = dict(parse_overrides(args.overrides), **args.architecture_options)
     config.apply_overrides(overrides, "the command line")
     options = dict(max_batch_size=args.max_batch, chunk_size=args.chunk, page_size=args.page_size,
-                   num_pages=args.num_pages, max_num_batched_tokens=args.max_tokens, seed=args.seed)
+                   num_pages=args.num_pages, max_num_batched_tokens=args.max_tokens, seed=args.seed,
+                   extend_portions=not args.fixed_chunk)
     if args.random_weights:
         init = args.init if args.init == "fan_in" else float(args.init)
         llm = LLM.from_config_random(config, weights_seed=args.seed, init=init, dtype=dtype, device=args.device, **options)

@@ -40,13 +40,13 @@ class ContinuousBatchEngine:
     def __init__(self, model: Any, max_batch_size: int, chunk_size: int, *, page_size: int = 16,
                  num_pages: int = 1024, max_sequences: int = DEFAULT_MAX_SEQUENCES,
                  max_num_batched_tokens: Optional[int] = None, eos_token_ids: Sequence[int] = (),
-                 banned_tokens: Optional[Sequence[int]] = None, seed: int = 0):
+                 banned_tokens: Optional[Sequence[int]] = None, seed: int = 0, extend_portions: bool = True):
         self.model = model
         slots = max(max_sequences, max_batch_size)
         self.runner = ModelRunner(model, page_size=page_size, num_pages=num_pages, max_requests=slots)
         self.scheduler = ContinuousBatchScheduler(
             max_batch_size, max_sequences, chunk_size, max_num_batched_tokens, cache=self.runner.cache,
-            max_positions=model.spec.max_positions)
+            max_positions=model.spec.max_positions, extend_portions=extend_portions)
         self.sampler = Sampler(model.vocab_size, slots, model.device, banned_tokens)
         self.eos_token_ids = list(eos_token_ids)
         self.seed = int(seed)
@@ -62,6 +62,15 @@ class ContinuousBatchEngine:
             if not 0 <= int(tok) < vocab:
                 raise ValueError(f"prompt token id {tok} is outside the vocabulary of {vocab}")
         return self.scheduler.add_request(prompt_tokens, max_new_tokens, sampling)
+
+    def admit_as_computed(self, request_id: int, computed: int) -> None:
+        """For measurements at a given context: the request is admitted at once and its first ``computed`` tokens count
+        as computed, with whatever its pages hold for keys and values
+        (``ContinuousBatchScheduler.admit_as_computed``).  What it generates means nothing."""
+        self.scheduler.admit_as_computed(request_id, computed)
+        request = self.scheduler.get_request(request_id)
+        self.sampler.start_request(self.runner.cache.slot_of(request_id), request.sampling,
+                                   request.prompt_tokens + request.generated_tokens)
 
     # -------------------------------------------------------------------- loop
     def step(self) -> ScheduledBatch:
@@ -208,7 +217,10 @@ class ContinuousBatchEngine:
         if finished:
             self.scheduler.update_after_step(finished, count_step=False)
 
-    def run_until_complete(self, print_progress: bool = False, one_step_ahead: bool = True) -> None:
+    def run_until_complete(self, print_progress: bool = False, one_step_ahead: bool = True,
+                           max_steps: Optional[int] = None) -> int:
+        """Run until every request has finished, or for ``max_steps`` steps (all of them waited for when it returns;
+        what remains goes on with the next call).  Returns the number of steps run."""
         step = 0
         flight: Optional[_InFlight] = None
         try:
@@ -217,12 +229,13 @@ class ContinuousBatchEngine:
                     s = self.scheduler.get_stats()
                     print(f"[pulse_infer_amd] step {step}: {s.num_running} requests running, {s.num_waiting} waiting, "
                           f"{s.num_finished} finished", file=sys.stderr, flush=True)
+                more = max_steps is None or step < max_steps
                 if not one_step_ahead:
-                    if not self.scheduler.has_work() or self.step().empty():
+                    if not more or not self.scheduler.has_work() or self.step().empty():
                         break
                     step += 1
                     continue
-                batch = self.scheduler.schedule_next_batch() if self.scheduler.has_work() else None
+                batch = self.scheduler.schedule_next_batch() if more and self.scheduler.has_work() else None
                 self.last_batch = batch if batch is not None else self.last_batch
                 queued = self._launch(batch, flight) if batch is not None and not batch.empty() else None
                 if flight is not None:
@@ -244,8 +257,9 @@ class ContinuousBatchEngine:
                     pass
         if print_progress:
             s = self.scheduler.get_stats()
-            print(f"[pulse_infer_amd] all {s.total_requests} requests finished after {step} steps", file=sys.stderr,
-                  flush=True)
+            print(f"[pulse_infer_amd] {s.num_finished} of {s.total_requests} requests finished after {step} steps",
+                  file=sys.stderr, flush=True)
+        return step
 
     # ----------------------------------------------------------------- results
     def get_result(self, request_id: int) -> List[int]:
@@ -273,7 +287,7 @@ class LLM:
 
     def __init__(self, model: Any, config: Any = None, *, max_batch_size: int = 8, chunk_size: int = 256,
                  page_size: int = 16, num_pages: Optional[int] = None, max_sequences: int = DEFAULT_MAX_SEQUENCES,
-                 max_num_batched_tokens: Optional[int] = None, seed: int = 0):
+                 max_num_batched_tokens: Optional[int] = None, seed: int = 0, extend_portions: bool = True):
         self.model = model
         self.config = config
         if num_pages is None:
@@ -283,7 +297,8 @@ class LLM:
         eos = list(getattr(config, "eos_token_ids", []) or [])
         self.engine = ContinuousBatchEngine(
             model, max_batch_size, chunk_size, page_size=page_size, num_pages=num_pages, max_sequences=max_sequences,
-            max_num_batched_tokens=max_num_batched_tokens, eos_token_ids=eos, seed=seed)
+            max_num_batched_tokens=max_num_batched_tokens, eos_token_ids=eos, seed=seed,
+            extend_portions=extend_portions)
 
     @classmethod
     def from_pretrained(cls, model_dir: str, dtype: str = "bfloat16", device: str = "cuda:0",

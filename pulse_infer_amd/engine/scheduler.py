@@ -11,7 +11,8 @@ What the reference leaves out is decided here:
   prefilling requests in order of arrival, each at most ``chunk_size`` tokens,
   cut anywhere; if budget is left when every one of them has its portion, the
   portions are extended in the same order (a lone long prompt runs in steps
-  of the whole budget).
+  of the whole budget) unless ``extend_portions`` is off, which keeps every
+  portion at ``chunk_size`` tokens at most, as the reference's are.
 * **pages** — every portion is reserved in the cache before the step; a request
   is admitted only if its first portion fits.  When a running request cannot
   get the page it needs, the most recently admitted running request is
@@ -84,7 +85,13 @@ class Stats:
 class ContinuousBatchScheduler:
     def __init__(self, max_batch_size: int, max_sequences: int, chunk_size: int = 256,
                  max_num_batched_tokens: Optional[int] = None, cache: Optional[CacheManager] = None,
-                 max_positions: Optional[int] = None):
+                 max_positions: Optional[int] = None, extend_portions: bool = True):
+        """``chunk_size`` is what the reference calls so (every prompt gets a portion of that many tokens in every
+        step, continuous_batch_scheduler.hpp:27-147) as long as ``extend_portions`` is off.  With it on (the default)
+        ``chunk_size`` is a portion's share of a step when several prompts want one: what the step's budget
+        (``max_num_batched_tokens``, by default ``max_batch_size`` chunks) still has when every prompt has its share
+        goes to the same portions in order, so a prompt that has a step to itself runs in portions of the whole
+        budget."""
         if max_batch_size <= 0 or max_sequences <= 0 or chunk_size <= 0:
             raise ValueError("max_batch_size, max_sequences and chunk_size must be positive")
         self.max_batch_size = int(max_batch_size)
@@ -96,6 +103,7 @@ class ContinuousBatchScheduler:
             raise ValueError("max_num_batched_tokens must be positive")
         self.cache = cache
         self.max_positions = max_positions
+        self.extend_portions = bool(extend_portions)
         self.next_request_id = 0
         self.waiting: Deque[InferenceRequest] = deque()
         self.running: List[InferenceRequest] = []
@@ -121,6 +129,28 @@ class ContinuousBatchScheduler:
         self.waiting.append(request)
         self.request_map[request.request_id] = request
         return request.request_id
+
+    def admit_as_computed(self, request_id: int, computed: int) -> None:
+        """Admit a waiting request at once and let the first ``computed`` tokens of its stream count as computed: pages
+        are reserved for them and the cursor stands behind them, but no step has run them, so their keys and values are
+        whatever the pages hold.  For measurements at a given context (a decode step does the same work over a cache
+        that only looks computed); never for requests whose output matters."""
+        request = self.request_map[request_id]
+        if request not in self.waiting or request.num_computed_tokens != 0:
+            raise SchedulerError(f"request {request_id} is not waiting at its start")
+        if not 0 < computed < request.total_input_tokens:
+            raise SchedulerError(f"request {request_id}: {computed} tokens cannot count as computed, it has "
+                                 f"{request.total_input_tokens} and must run one at least")
+        if len(self.running) >= self.max_sequences:
+            raise SchedulerError(f"{self.max_sequences} requests are running already")
+        self.waiting.remove(request)
+        if self.cache is not None:
+            self.cache.add_request(request_id)
+            self.cache.reserve(request_id, computed)
+            self.cache.advance(request_id, computed)
+        request.start_running()
+        request.num_computed_tokens = computed
+        self.running.append(request)
 
     # --------------------------------------------------------------- decisions
     def _fits(self, request: InferenceRequest, length: int) -> bool:
@@ -249,7 +279,7 @@ class ContinuousBatchScheduler:
         # 4. what is left of the budget (fewer requests in their prompts than it has room for) extends this step's
         #    prompt portions, in their order: a lone long prompt then runs in steps of the whole budget, whose
         #    matrix products are far more efficient than those of a chunk's rows
-        for i, portion in enumerate(batch.portions):
+        for i, portion in enumerate(batch.portions if self.extend_portions else ()):
             if budget <= 0:
                 break
             if portion.samples:   # it brings all that its request has pending

@@ -183,6 +183,33 @@ def test_budget_that_is_left_extends_the_portions_in_order():
     c2.check()
 
 
+def test_portions_stay_at_the_chunk_size_when_extension_is_off():
+    """``extend_portions=False``: the reference's meaning of the chunk size, no portion longer than it whatever the
+    budget has left; and a request that is admitted as computed goes on from there."""
+    c = _cache(pages=64)
+    s = ContinuousBatchScheduler(4, 4, chunk_size=8, max_num_batched_tokens=40, cache=c, max_positions=256,
+                                 extend_portions=False)
+    a = s.add_request(list(range(30)), 2)
+    b = s.add_request(list(range(5)), 2)
+    sizes = []
+    while s.get_request(a).is_prefill:
+        batch = s.schedule_next_batch()
+        sizes.append([(p.request.request_id, len(p.tokens)) for p in batch.portions])
+        _finish_step(s, batch, finished=[b] if len(sizes) == 1 else [])
+    assert sizes == [[(a, 8), (b, 5)], [(a, 8)], [(a, 8)], [(a, 6)]]
+    d = s.add_request(list(range(21)), 3)
+    with pytest.raises(SchedulerError, match="cannot count as computed"):
+        s.admit_as_computed(d, 21)
+    s.admit_as_computed(d, 20)
+    assert c.computed(d) == 20 and len(c.table(0, d)) == 5 and s.get_request(d).state == RequestState.RUNNING
+    batch = s.schedule_next_batch()
+    assert [(p.request.request_id, p.tokens, p.start, p.samples) for p in batch.portions if p.request.request_id == d] == \
+        [(d, [20], 20, True)]
+    with pytest.raises(SchedulerError, match="not waiting"):
+        s.admit_as_computed(d, 3)
+    c.check()
+
+
 def test_what_can_never_fit_is_refused():
     c = _cache(pages=2)
     s = ContinuousBatchScheduler(2, 2, chunk_size=8, cache=c, max_positions=16)
