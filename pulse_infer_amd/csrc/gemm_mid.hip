@@ -50,8 +50,9 @@ __device__ __forceinline__ bf16x8 zeros8() {
     return z;
 }
 
-// NW wavefronts of 16 weight rows each a workgroup; MT tiles of 16 rows of X; KC k a chunk (steps of 32).
-template <int NW, int MT, int KC, bool SWIGLU>
+// NW wavefronts of 16 weight rows each a workgroup; MT tiles of 16 rows of X; KC k a chunk (steps of 32); RING
+// register sets of weight chunks (a wavefront has RING - 1 chunks of its 16 weight rows in flight).
+template <int NW, int MT, int KC, bool SWIGLU, int RING>
 __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* __restrict__ X, int64_t ldx,
                                                                     const bf16_t* __restrict__ W, int64_t ldw,
                                                                     void* __restrict__ C, int64_t ldc, int M, int N,
@@ -68,7 +69,6 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
     constexpr int PIECES = 16 * MT * ROWP;
     constexpr int XP = (PIECES + THREADS - 1) / THREADS;         // pieces a thread stages
     constexpr int PAIRS = KC / 64;                               // pairs of steps a chunk
-    constexpr int RING = 512 / KC;                               // register sets of weight chunks: loads run RING - 1 ahead
 
     const int tid = threadIdx.x;
     const int wave = tid / PULSE_WAVE;
@@ -238,18 +238,26 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
     }
 }
 
+// Weight loads run three chunks of 128 k (1.5 KB a lane group... 12 KB a wavefront) ahead; workgroups of two wavefronts,
+// which are taken where the weight has few rows and the chip holds barely more wavefronts than compute units, run
+// seven chunks ahead: what is in flight must cover the memory's latency at its full rate (6,144 weight rows at 64 rows
+// of X: 20.8 -> PULSE_MID_DEEP us).
+template <int NW, int KC>
+constexpr int ring_for() { return (NW == 2 && KC == 128) ? 8 : 512 / KC; }
+
 template <int NW, int MT, int KC = 128>
 void launch_mid(const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,
                 int k_len, int splits, int mode, bool swiglu, hipStream_t stream) {
     const dim3 grid((N + 16 * NW - 1) / (16 * NW), splits);
     const dim3 block(NW * PULSE_WAVE);
+    constexpr int RING = ring_for<NW, KC>();
     if constexpr (NW % 2 == 0) {
         if (swiglu) {
-            hipLaunchKernelGGL((gemm_mid_kernel<NW, MT, KC, true>), grid, block, 0, stream, X, ldx, W, ldw, C, ldc, M, N, k_len, mode);
+            hipLaunchKernelGGL((gemm_mid_kernel<NW, MT, KC, true, RING>), grid, block, 0, stream, X, ldx, W, ldw, C, ldc, M, N, k_len, mode);
             return;
         }
     }
-    hipLaunchKernelGGL((gemm_mid_kernel<NW, MT, KC, false>), grid, block, 0, stream, X, ldx, W, ldw, C, ldc, M, N, k_len, mode);
+    hipLaunchKernelGGL((gemm_mid_kernel<NW, MT, KC, false, RING>), grid, block, 0, stream, X, ldx, W, ldw, C, ldc, M, N, k_len, mode);
 }
 
 template <int NW>

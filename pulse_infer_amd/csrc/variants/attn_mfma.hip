@@ -72,7 +72,9 @@ struct MfmaArgs {
     const bf16_t* vc;
     const int* positions;
     const int* block_table;
-    const int* items;  // [n_items, 4]: first token row, number of tokens, row of the block table, 0
+    const int* items;  // [n_items, 4]: first token row, number of tokens, row of the block table, 0; or null: item i
+                       // is token i alone with row i of the block table (a step of decoded tokens in the order of
+                       // its requests), which saves every workgroup a trip to memory before its first load of keys
     int bt_width;
     int n_items;
     int nq, nkv, group;
@@ -254,9 +256,10 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
     // Everything the first loads of keys need comes with the item (the block table's row too), so that the chain of
     // dependent trips to memory before a workgroup streams is item -> block table -> keys.  The positions (which only
     // decide masks and the end of the walk) and q travel at the same time.
-    const int row0 = a.items[4 * item];
-    const int ntok = a.items[4 * item + 1];
-    const int* bt = a.block_table + static_cast<int64_t>(a.items[4 * item + 2]) * a.bt_width;
+    const bool listed = a.items != nullptr;
+    const int row0 = listed ? a.items[4 * item] : item;
+    const int ntok = listed ? a.items[4 * item + 1] : 1;
+    const int* bt = a.block_table + static_cast<int64_t>(listed ? a.items[4 * item + 2] : item) * a.bt_width;
     const int hi = a.positions[row0 + ntok - 1];    // last key any column of the item may see
     const int split_size = a.plan ? a.plan[1 + a.n_items * a.n_splits + item]
                            : (a.live_context && a.n_splits > 1)
@@ -523,8 +526,14 @@ __global__ __launch_bounds__(WAVES* PULSE_WAVE) PULSE_ATTN_WAVES_PER_EU void att
         BlockRegs xa, xb;
         const bool early = a.window == 0;
         int b = split_begin / BLOCK_KEYS + wave;
-        if (early && b <= (split_begin + split_size - 1) / BLOCK_KEYS) load_block(b, load_pages(b), xa);
-        load_q();   // behind the keys' pages in the queue: results come back in the order asked for
+        // Results come back in the order asked for.  Plain: the keys first, q behind them (it is needed only when
+        // the first keys are there).  FUSED: q, the token's raw key and what their preparation needs go out between
+        // the first block's pages and its keys, which wait for the pages anyway: they arrive a trip before the keys,
+        // and the preparation runs while the keys are on their way instead of after they have come.
+        const BlockPages p0 = load_pages(b);
+        if (FUSED) load_q();
+        if (early && b <= (split_begin + split_size - 1) / BLOCK_KEYS) load_block(b, p0, xa);
+        if (!FUSED) load_q();
         if (split_begin > hi) return;                   // nothing here; the merge does not read this split
         split_end = min(split_begin + split_size, hi + 1);
         const int first_block = max(split_begin, lo_item) / BLOCK_KEYS;
@@ -1329,7 +1338,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_mfma_reduce_kernel(const 
     // pairs of every split and the first partial outputs.  What of that a row does not use is read and dropped.
     const int item = blockIdx.x / per;
     const int tok = blockIdx.x % per;
-    const int row0 = items[4 * item], ntok = items[4 * item + 1];
+    const int row0 = items ? items[4 * item] : item, ntok = items ? items[4 * item + 1] : 1;   // (null: item i is token i)
     const int split_size = plan ? plan[1 + n_items * n_splits + item]
                            : live_context ? live_split_size(*live_context, n_splits, static_split_size) : static_split_size;
     if (tok >= ntok) return;   // only the rows of this launch's items have partial results
@@ -1447,7 +1456,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void attn_plan_kernel(const int* __re
     };
     int longest = 1;
     for (int i = tid; i < n_items; i += PLAN_THREADS) {
-        const int c = positions[items[4 * i] + items[4 * i + 1] - 1] + 1;
+        const int c = positions[items ? items[4 * i] + items[4 * i + 1] - 1 : i] + 1;
         s_ctx[i] = c;
         longest = max(longest, c);
     }
@@ -1561,7 +1570,8 @@ int launch_attn_mfma(const void* q, int64_t q_stride, void* out, int64_t o_strid
                   "attn_mfma: scratch is missing or not 16-byte aligned");
     PULSE_REQUIRE(n_splits <= MAX_SPLITS, "attn_mfma: at most %d splits, got %d", MAX_SPLITS, n_splits);
     PULSE_REQUIRE(n_splits < 65536 && static_cast<int64_t>(n_items) * nkv * ((nq / nkv + 15) / 16) * n_splits < (int64_t{1} << 31), "attn_mfma: grid too large");
-    PULSE_REQUIRE(q && out && kcache && vcache && positions && block_table && items, "attn_mfma: null pointer");
+    PULSE_REQUIRE(q && out && kcache && vcache && positions && block_table, "attn_mfma: null pointer");
+    PULSE_REQUIRE(items || (prep && n_items == tokens), "attn_mfma: only decoded tokens, one an item, can do without a list of items");
     if (tokens == 0 || n_items == 0) return 0;
     const int group = nq / nkv;
     int gp = 1;
@@ -1630,7 +1640,7 @@ extern "C" int pulse_attn_plan_max_pairs() { return PLAN_MAX_PAIRS; }
 
 extern "C" int pulse_attn_plan(const int* items, const int* positions, int n_items, int n_splits, int slots,
                                int first_wave, int min_keys, int* plan, hipStream_t stream) {
-    PULSE_REQUIRE(items && positions && plan, "attn_plan: null pointer");
+    PULSE_REQUIRE(positions && plan, "attn_plan: null pointer");   // (items may be null: item i is token i)
     PULSE_REQUIRE(n_items >= 1 && n_splits >= 1 && static_cast<int64_t>(n_items) * n_splits <= PLAN_MAX_PAIRS,
                   "attn_plan: %d items in up to %d splits are more than %d pairs", n_items, n_splits, PLAN_MAX_PAIRS);
     PULSE_REQUIRE(slots >= 1 && first_wave >= 1 && min_keys >= 1, "attn_plan: slots, first_wave and min_keys must be positive");
@@ -1653,7 +1663,7 @@ extern "C" int pulse_attn_decode_takes(int rotary_dim, int pairing) {
 // bfloat16 [D], or null) and rotation (cos_t, sin_t float32 [tokens, rotary_dim / 2], or null) of q and, with new_key,
 // of the token's key happen inside; with new_key the key and the value are also written to the token's page (kcache
 // and vcache are written then).  Without new_key the pages already hold the token (a run that reads another run's
-// cache).  The rest as pulse_attn_mfma.
+// cache).  items may be null: item i is then token i with row i of the block table.  The rest as pulse_attn_mfma.
 extern "C" int pulse_attn_decode(const void* qkv, int64_t qkv_stride, void* out, int64_t o_stride, void* kcache,
                                  void* vcache, const int* positions, const int* block_table, int bt_width,
                                  const int* items, int n_items, int tokens, int nq, int nkv, int page_size,

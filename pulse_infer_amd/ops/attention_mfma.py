@@ -170,7 +170,7 @@ def plan_fits(n_items: int, n_splits: int) -> bool:
     return 1 <= n_items and n_items * n_splits <= 1024     # PLAN_MAX_PAIRS of attn_mfma.hip
 
 
-def attn_plan(items: torch.Tensor, positions: torch.Tensor, n_splits: int, slots: int, first_wave: int,
+def attn_plan(items: Optional[torch.Tensor], positions: torch.Tensor, n_splits: int, slots: int, first_wave: int,
               plan: torch.Tensor, d: int, min_keys: int = PLAN_MIN_KEYS) -> None:
     """The plan of a step whose contexts differ much (on the device, from ``positions`` as they are now): every
     item's keys are cut into min(n_splits, ceil(context / T)) even splits, T the smallest length with at most
@@ -178,9 +178,12 @@ def attn_plan(items: torch.Tensor, positions: torch.Tensor, n_splits: int, slots
     ``plan``: int32 [plan_ints(items, n_splits)], to be passed to ``attn_mfma`` / ``attn_decode`` with the same items,
     positions and n_splits."""
     _gpu("attn_plan", items, positions, plan)
-    n_items = items.numel() // ITEM_INTS
-    _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() % ITEM_INTS == 0,
-          "attn_plan: items must be int32 quadruples")
+    if items is None:        # every token an item of its own, in order (decoded tokens)
+        n_items = positions.numel()
+    else:
+        n_items = items.numel() // ITEM_INTS
+        _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() % ITEM_INTS == 0,
+              "attn_plan: items must be int32 quadruples")
     _need(positions.dtype == torch.int32 and positions.is_contiguous(), "attn_plan: positions must be contiguous int32")
     _need(plan_fits(n_items, n_splits), f"attn_plan: {n_items} items in up to {n_splits} splits do not fit a plan")
     _planned(plan, n_items, n_splits)
@@ -301,7 +304,8 @@ def decode_takes(d: int, rotary_dim: int, pairing: int) -> bool:
 
 
 def attn_decode(qkv: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int, kcache: torch.Tensor,
-                vcache: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor, items: torch.Tensor,
+                vcache: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
+                items: Optional[torch.Tensor],
                 scale: float, window: int, split_size: int, n_splits: int, max_context: int,
                 part_o: Optional[torch.Tensor], part_ml: Optional[torch.Tensor], q_w: Optional[torch.Tensor],
                 k_w: Optional[torch.Tensor], eps: float, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
@@ -309,12 +313,14 @@ def attn_decode(qkv: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int,
                 plan: Optional[torch.Tensor] = None) -> None:
     """Attention for decoded tokens from the raw projection output ``qkv`` [tokens, (nq + 2 nkv) d]: per-head norm
     and rotation of q and of the token's own key happen inside the kernel; with ``new_key`` key and value are also
-    written to the token's page.  Every item must hold one token.  ``live_context``, ``plan``: as for ``attn_mfma``."""
+    written to the token's page.  Every item must hold one token; ``items`` None says that item i is token i with row
+    i of the block table (a step of decoded tokens in the order of its requests), which spares every workgroup the
+    trip to memory for its item.  ``live_context``, ``plan``: as for ``attn_mfma``."""
     _gpu("attn_decode", qkv, out, kcache, vcache, positions, block_table, items, part_o, part_ml, q_w, k_w, cos, sin,
          live_context, plan)
     _live(live_context)
-    _planned(plan, items.numel() // ITEM_INTS, n_splits)
     tokens = qkv.shape[0]
+    _planned(plan, tokens, n_splits)
     _need(qkv.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and qkv.stride(1) == 1 and out.stride(1) == 1,
           "attn_decode: qkv and out must be bfloat16 matrices with contiguous rows")
     _need(qkv.shape[1] >= (nq + (2 * nkv if new_key else 0)) * d and out.shape[1] >= nq * d and out.shape[0] == tokens,
@@ -325,8 +331,10 @@ def attn_decode(qkv: torch.Tensor, out: torch.Tensor, nq: int, nkv: int, d: int,
     _int_vec("attn_decode: positions", positions, tokens)
     _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.is_contiguous(),
           "attn_decode: block_table must be contiguous int32 [entries, width]")
-    _need(items.dtype == torch.int32 and items.is_contiguous() and items.numel() == ITEM_INTS * tokens,
+    _need(items is None or (items.dtype == torch.int32 and items.is_contiguous() and items.numel() == ITEM_INTS * tokens),
           "attn_decode: one int32 quadruple for every token")
+    _need(items is not None or block_table.shape[0] >= tokens, "attn_decode: without items every token needs its row "
+          "of the block table")
     for name, w in (("q_w", q_w), ("k_w", k_w)):
         _need(w is None or (w.dtype == torch.bfloat16 and w.numel() == d and w.is_contiguous()),
               f"attn_decode: {name} must hold {d} bfloat16 values")

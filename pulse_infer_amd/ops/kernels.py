@@ -248,6 +248,66 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool =
          _i64(ldcopy), _ptr(copy_scale), _stream(), label=f"N={n} K={k}")
 
 
+ROWS_MAX_ROWS = 64
+ROWS_CHUNK = 256
+
+
+def gemm_rows_takes(m: int, n: int, k: int) -> bool:
+    """Whether ``gemm_rows`` takes a shape (as pulse_gemm_rows_takes)."""
+    return 1 <= m <= ROWS_MAX_ROWS and n > 0 and n % 16 == 0 and k > 0 and k % ROWS_CHUNK == 0
+
+
+def gemm_rows(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool = False,
+              sumsq_out: Optional[torch.Tensor] = None, row_scale: Optional[tuple] = None,
+              copy_out: Optional[torch.Tensor] = None, copy_scale: Optional[torch.Tensor] = None, slabs: int = 0) -> None:
+    """out = a @ w^T for up to 64 rows of bfloat16 and a weight of few rows: a workgroup owns 16 weight rows and all
+    of K, its four wavefronts share K out among themselves (the regime of 17 to 64 rows for the projections around
+    attention and the feed-forward's way back).
+
+    ``out`` bfloat16 [M, N] is stored; with ``add`` the product is added to ``out`` float32 [M, N].  The fusions are
+    those of ``gemm_skinny``: ``row_scale = (sumsq, eps)`` multiplies row m of the product by
+    1 / sqrt(sum(sumsq[m]) / K + eps) first; with ``add``, ``sumsq_out`` [M, N / 16] takes the sums of squares of the
+    updated rows, 16 columns a part, and ``copy_out`` [M, N] bfloat16 the updated rows once more, every column
+    multiplied by its ``copy_scale`` (bfloat16 [N]; None: as it is)."""
+    scale_sumsq, scale_eps = row_scale if row_scale is not None else (None, 0.0)
+    _gpu("gemm_rows", a, w, out, sumsq_out, copy_out, scale_sumsq, copy_scale)
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and w.dim() == 2
+          and a.stride(1) == 1 and w.stride(1) == 1, "gemm_rows: a and w must be bfloat16 matrices with contiguous rows")
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k, f"gemm_rows: inner sizes differ ({k} and {w.shape[1]})")
+    _need(gemm_rows_takes(m, n, k), f"gemm_rows: M={m} N={n} K={k} is not a shape it takes")
+    _need(tuple(out.shape) == (m, n) and out.stride(1) == 1, f"gemm_rows: out must be [{m}, {n}]")
+    if add:
+        _need(out.dtype == torch.float32, "gemm_rows: adding needs a float32 target")
+        mode = 2
+    else:
+        _need(out.dtype == torch.bfloat16 and sumsq_out is None and copy_out is None,
+              "gemm_rows: a stored result is bfloat16; sums of squares and the copy come with add")
+        mode = 0
+    if sumsq_out is not None:
+        _need(sumsq_out.dtype == torch.float32 and sumsq_out.is_contiguous() and sumsq_out.dim() == 2
+              and sumsq_out.shape[0] >= m and sumsq_out.shape[1] == n // 16,
+              "gemm_rows: sumsq_out must be a contiguous float32 [M, N / 16]")
+    if copy_out is not None:
+        _need(copy_out.dtype == torch.bfloat16 and tuple(copy_out.shape) == (m, n) and copy_out.stride(1) == 1,
+              f"gemm_rows: copy_out must be bfloat16 [{m}, {n}]")
+    ldcopy = 0 if copy_out is None else (copy_out.stride(0) if m > 1 else n)
+    _need(copy_scale is None or (copy_out is not None and copy_scale.dtype == torch.bfloat16 and copy_scale.numel() == n
+                                 and copy_scale.is_contiguous()),
+          f"gemm_rows: copy_scale must hold {n} bfloat16 values and comes with copy_out")
+    scale_parts = 0
+    if scale_sumsq is not None:
+        _need(scale_sumsq.dtype == torch.float32 and scale_sumsq.dim() == 2 and scale_sumsq.shape[0] >= m
+              and scale_sumsq.is_contiguous() and scale_sumsq.shape[1] > 0 and scale_sumsq.data_ptr() % 16 == 0,
+              "gemm_rows: the row sums of squares must be a contiguous, 16-byte aligned float32 [M, parts]")
+        scale_parts = scale_sumsq.shape[1]
+    call("pulse_gemm_rows", _ptr(a), _i64(a.stride(0) if m > 1 else k), _ptr(w), _i64(w.stride(0) if n > 1 else k),
+         _ptr(out), _i64(out.stride(0) if m > 1 else n), _i32(m), _i32(n), _i32(k), _i32(mode), _ptr(scale_sumsq),
+         _i32(scale_parts), _f32(scale_eps), _ptr(sumsq_out), _ptr(copy_out), _i64(ldcopy), _ptr(copy_scale),
+         _i32(slabs), _stream(), label=f"N={n} K={k}")
+
+
 MID_MAX_ROWS = 192
 
 

@@ -191,7 +191,8 @@ class PagedAttention(Part):
                     if pkey not in ctx.extras:
                         made = ctx.workspace.buffer(f"attention.plan:{n_splits}:{slots}:{first}",
                                                     attention_mfma.plan_ints(n_items, n_splits), 1, torch.int32)
-                        attention_mfma.attn_plan(short_items, ctx.positions, n_splits, slots, first, made, self.d)
+                        attention_mfma.attn_plan(short_items if raw is None else None, ctx.positions, n_splits, slots,
+                                                 first, made, self.d)
                         ctx.extras[pkey] = made
                     plan = ctx.extras[pkey]
             part_o = part_ml = None
@@ -201,8 +202,9 @@ class PagedAttention(Part):
                 part_ml = ctx.workspace.buffer("attention.part_ml", rows, 2, torch.float32)
             if raw is not None:
                 tables, write = raw
+                # (no list of items: the step's tokens are its requests' in order, each with its row of the table)
                 attention_mfma.attn_decode(
-                    q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions, table, short_items,
+                    q, out, self.nq, self.nkv, self.d, cache.keys, cache.values, ctx.positions, table, None,
                     self.scale, window, split_size, n_splits, max_context, part_o, part_ml, self.q_w, self.k_w,
                     self.eps, tables.cos if tables is not None else None, tables.sin if tables is not None else None,
                     tables.rotary_dim if tables is not None else 0, tables.pairing if tables is not None else 0,

@@ -66,6 +66,12 @@ class Linear:
                 # are enough of them (measured: logits of a 152K vocabulary 212 to 237 us against the library's 276 to
                 # 281; 6,144 rows of qkv 17 to 21 us against 15 to 18, which a step without a library call, recorded
                 # and replayed as a whole, makes up several times over).
+                if self.takes_shared_k(x, w, out):
+                    # few weight rows (qkv): a workgroup owns two 16-row slabs and all of K, which its wavefronts
+                    # share out among themselves (6,144 weight rows of 4,096: 14.1 / 15.0 / 18.7 us at 24 / 32 / 64
+                    # rows against 17.2 / 17.1 / 22.2 with a wavefront a slab; the library 14.7 / 15.1 / 17.8)
+                    kernels.gemm_rows(x, w, out, slabs=2)
+                    return out
                 waves = 10 if w.shape[0] >= 64 * compute_units() else 2
                 kernels.gemm_mid(x, w, out.view(1, *out.shape) if out.dtype == torch.float32 else out, waves=waves)
                 return out
@@ -183,6 +189,12 @@ class Linear:
         if out.dtype == torch.float32:
             return out.is_contiguous() and out.data_ptr() % 16 == 0 and w.shape[0] % 4 == 0
         return out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.stride(0) % 4 == 0 and out.data_ptr() % 16 == 0
+
+    def takes_shared_k(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
+        """Whether a bfloat16 product of 17 to 64 rows runs with the inner dimension shared out inside a workgroup:
+        weights of so few rows that a wavefront a slab leaves most of the chip's wavefront slots empty."""
+        return (out.dtype == torch.bfloat16 and w.shape[0] <= 32 * compute_units()
+                and kernels.gemm_rows_takes(x.shape[0], w.shape[0], w.shape[1]))
 
     def takes_mid(self, x: torch.Tensor) -> bool:
         return (self.library and x.dtype == torch.bfloat16 and self.MID_ROWS[0] <= x.shape[0] <= self.MID_ROWS[1]

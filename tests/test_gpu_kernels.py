@@ -890,7 +890,8 @@ def test_attn_mfma_refuses_other_sizes(k):
 ])
 @pytest.mark.parametrize("split", [None, 32, 128, "bucket", "planned", "planned_short"])
 @pytest.mark.parametrize("new_key", [True, False])
-def test_attn_decode_from_raw(k, case, split, new_key):
+@pytest.mark.parametrize("listed", [True, False])
+def test_attn_decode_from_raw(k, case, split, new_key, listed):
     """Decoded tokens straight from the raw projection output: per-head norm, rotation, the token's own key and
     value (used from registers, written to the page) inside the attention kernel, against the plain formulas and
     against what the separate preparation kernel writes.  With new_key False the pages already hold the token.
@@ -898,7 +899,8 @@ def test_attn_decode_from_raw(k, case, split, new_key):
     longest context there is: the split that holds a token's position, whose workgroup writes its key, moves with it.
     "planned": the same launch with a plan made on the device from the positions (every item its own split size, the
     workgroups in the plan's order, items of one split finished without the merge); "planned_short": splits down to a
-    block of keys, so that every item is cut as far as the launch allows."""
+    block of keys, so that every item is cut as far as the launch allows.  ``listed`` False: no list of items is given,
+    item i is token i with row i of the block table."""
     from pulse_infer_amd.ops import attention_mfma as M
     nq, nkv, d, rot, bs, window, lens = (case[x] for x in ("nq", "nkv", "d", "rot", "bs", "window", "lens"))
     pairing = 0 if case["pairing"] == "interleaved" else 1
@@ -968,14 +970,15 @@ def test_attn_decode_from_raw(k, case, split, new_key):
     if split in ("planned", "planned_short"):
         plan = torch.full((M.plan_ints(n, n_splits),), -77, dtype=torch.int32, device=DEV)
         slots = 2 * n if split == "planned" else 1000
-        M.attn_plan(items, pos_t, n_splits, slots, 2, plan, d, min_keys=64 if split == "planned" else 32)
+        M.attn_plan(items if listed else None, pos_t, n_splits, slots, 2, plan, d, min_keys=64 if split == "planned" else 32)
         sizes = plan[1 + n * n_splits:].tolist()
         assert all(sz % 32 == 0 and sz * n_splits >= c for sz, c in zip(sizes, lens))
         if split == "planned_short":
             assert sizes == [max(32, ((c + n_splits - 1) // n_splits + 31) // 32 * 32) for c in lens]
     raw = qkv.clone()
-    M.attn_decode(qkv, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), items, scale, window, split_size, n_splits,
-                  max_ctx, part_o, part_ml, qw, kw, eps, cos, sin, rot, pairing, new_key, live_context=live, plan=plan)
+    M.attn_decode(qkv, out, nq, nkv, d, kc, vc, pos_t, table.to(DEV), items if listed else None, scale, window,
+                  split_size, n_splits, max_ctx, part_o, part_ml, qw, kw, eps, cos, sin, rot, pairing, new_key,
+                  live_context=live, plan=plan)
     assert torch.equal(qkv, raw)                   # the projection output stays raw
     got = out.cpu().to(F64).reshape(n, nq, d)
     for t, p in enumerate(positions):
@@ -1207,6 +1210,73 @@ def test_gemm_mid_swiglu(k, m, inter, kk):
         out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
         k.gemm_mid(a, mixed, out, swiglu=True, waves=waves)
         assert torch.allclose(out.cpu().to(F64), want, atol=1e-2, rtol=1e-2), waves
+
+
+@pytest.mark.parametrize("m", [1, 17, 33, 48, 64])
+@pytest.mark.parametrize("n,kk", [(16, 256), (80, 512), (528, 2304), (6144, 4096)])
+def test_gemm_rows(k, m, n, kk):
+    """The product for 17 to 64 rows of a weight with few rows (a workgroup owns whole slabs and all of K, its
+    wavefronts share K out and meet in LDS), at every number of slabs a workgroup, against float64: stored as
+    bfloat16; added into float32 with the new rows' sums of squares (16 columns a part) and the rounded, scaled copy;
+    and with its rows scaled by 1 / sqrt(mean + eps) from the parts of their sums of squares.  A wavefront that took
+    another's share of K, a chunk of X staged to the wrong place or partial sums met in another order would show."""
+    a, aref = as_stored(rnd(m, kk, seed=190), torch.bfloat16)
+    w, wref = as_stored(rnd(n, kk, seed=191, scale=kk ** -0.5), torch.bfloat16)
+    want = aref @ wref.T
+    first = None
+    for slabs in (0, 1, 2, 4):
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+        k.gemm_rows(a, w, out, slabs=slabs)
+        assert torch.allclose(out.cpu().to(F64), want, atol=2e-2, rtol=1e-2), slabs
+        first = out if first is None else first
+        assert torch.equal(out, first)                      # the sums do not depend on the workgroup's shape
+    # rows scaled behind the product: the parts of the rows' sums of squares in, 1 / sqrt(mean + eps) times the row out
+    eps = 1e-5
+    for parts in (1, 6, 64):
+        sumsq = (torch.rand(m + 2, parts, generator=torch.Generator().manual_seed(parts)) * kk / parts).to(DEV)
+        rstd = 1.0 / torch.sqrt(sumsq.cpu().to(F64)[:m].sum(dim=1) / kk + eps)
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+        k.gemm_rows(a, w, out, row_scale=(sumsq, eps))
+        assert torch.allclose(out.cpu().to(F64), want * rstd[:, None], atol=2e-2, rtol=1e-2), parts
+    # added into float32, with what the next product needs to do without a norm kernel
+    base = rnd(m, n, seed=192).to(DEV)
+    scale, sref = as_stored(1 + 0.1 * rnd(n, seed=193), torch.bfloat16)
+    for slabs in (1, 2, 4):
+        res = base.clone()
+        sums = torch.full((m + 1, n // 16), float("nan"), device=DEV)
+        copy = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+        k.gemm_rows(a, w, res, add=True, sumsq_out=sums, copy_out=copy, copy_scale=scale, slabs=slabs)
+        new = base.cpu().to(F64) + want
+        got = res.cpu().to(F64)
+        assert torch.allclose(got, new, atol=1e-3, rtol=1e-5)
+        assert torch.allclose(sums[:m].cpu().to(F64), (got ** 2).view(m, n // 16, 16).sum(dim=2), rtol=1e-5, atol=1e-6)
+        assert bool(torch.isnan(sums[m]).all())                                     # nothing beyond the rows
+        assert torch.equal(copy.cpu(), (res.cpu() * scale.cpu().float()).to(torch.bfloat16))   # one rounding of the float32 product
+    plain = base.clone()
+    k.gemm_rows(a, w, plain, add=True)
+    assert torch.equal(plain, res)
+    if m > 1:                                                # strided rows (views into wider buffers)
+        wide = torch.zeros(m, kk + 24, dtype=torch.bfloat16, device=DEV)
+        wide[:, :kk] = a
+        out = torch.zeros(m, n + 8, dtype=torch.bfloat16, device=DEV)
+        k.gemm_rows(wide[:, :kk], w, out[:, :n])
+        assert torch.equal(out[:, :n], first) and bool((out[:, n:] == 0).all())
+
+
+def test_gemm_rows_refuses(k):
+    from pulse_infer_amd.ops import KernelError
+    a = torch.zeros(65, 256, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(64, 256, dtype=torch.bfloat16, device=DEV)
+    assert k.gemm_rows_takes(64, 64, 256) and not k.gemm_rows_takes(65, 64, 256)
+    assert not k.gemm_rows_takes(8, 72, 256) and not k.gemm_rows_takes(8, 64, 384)
+    with pytest.raises(KernelError, match="not a shape"):
+        k.gemm_rows(a, w, torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(KernelError, match="float32 target"):
+        k.gemm_rows(a[:8], w, torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV), add=True)
+    with pytest.raises(KernelError, match="come with add"):
+        k.gemm_rows(a[:8], w, torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV), sumsq_out=torch.zeros(8, 4, device=DEV))
+    with pytest.raises(KernelError, match="slabs"):
+        k.gemm_rows(a[:8], w, torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV), slabs=3)
 
 
 def test_gemm_mid_refuses(k):
