@@ -62,6 +62,8 @@ def build_parser() -> argparse.ArgumentParser:
                         "config.json (for Qwen3: rope_pairing=half, the channels a rotation pairs); may be repeated")
     p.add_argument("--strict", action="store_true", help="a tensor that no part of the model asks for is an error")
     p.add_argument("--stats", action="store_true")
+    p.add_argument("--log-level", default=None, help="trace, debug, info, warn, error, critical or off "
+                                                     "(default: $PULSE_LOG_LEVEL, else info); messages go to standard error")
     return p
 
 
@@ -107,6 +109,9 @@ def parse_overrides(items: List[str]) -> dict:
 def main(argv: Optional[List[str]] = None) -> int:
     args = parse_args(argv)
     model_dir = args.model_path
+    if args.log_level:
+        from . import log
+        log.set_level(args.log_level)
     dtype = {"bf16": "bfloat16", "f32": "float32"}.get(args.dtype, args.dtype)
 
     import torch

@@ -93,7 +93,8 @@ def existing_library() -> Optional[str]:
 
 
 def _log(msg: str) -> None:
-    print(f"[pulse_infer_amd] {msg}", file=sys.stderr, flush=True)
+    from .. import log
+    log.info(msg)
 
 
 def build(force: bool = False, verbose: bool = True) -> str:

@@ -8,12 +8,12 @@ text: ``add_request``, ``run_until_complete``, ``get_result``, ``get_request``,
 """
 from __future__ import annotations
 
-import sys
 import time
 from typing import Any, Dict, List, Optional, Sequence
 
 import torch
 
+from .. import log
 from ..models.factory import build_model, load_model
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
@@ -225,10 +225,11 @@ class ContinuousBatchEngine:
         flight: Optional[_InFlight] = None
         try:
             while True:
-                if print_progress and step % 10 == 0 and self.scheduler.has_work():
+                if step % 10 == 0 and self.scheduler.has_work() and (print_progress or log.enabled("debug")):
                     s = self.scheduler.get_stats()
-                    print(f"[pulse_infer_amd] step {step}: {s.num_running} requests running, {s.num_waiting} waiting, "
-                          f"{s.num_finished} finished", file=sys.stderr, flush=True)
+                    (log.info if print_progress else log.debug)(
+                        f"step {step}: {s.num_running} requests running, {s.num_waiting} waiting, "
+                        f"{s.num_finished} finished")
                 more = max_steps is None or step < max_steps
                 if not one_step_ahead:
                     if not more or not self.scheduler.has_work() or self.step().empty():
@@ -255,10 +256,12 @@ class ContinuousBatchEngine:
                     self._settle(flight)
                 except Exception:      # (the device may be what failed; the error under way says more than this one)
                     pass
-        if print_progress:
+        if print_progress or log.enabled("debug"):
             s = self.scheduler.get_stats()
-            print(f"[pulse_infer_amd] {s.num_finished} of {s.total_requests} requests finished after {step} steps",
-                  file=sys.stderr, flush=True)
+            (log.info if print_progress else log.debug)(
+                f"{s.num_finished} of {s.total_requests} requests finished after {step} steps "
+                f"({s.num_preemptions} preemptions, {self.runner.graph_records} steps recorded, "
+                f"{self.runner.graph_replays} replayed)")
         return step
 
     # ----------------------------------------------------------------- results

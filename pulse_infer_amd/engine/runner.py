@@ -20,6 +20,7 @@ from typing import Any, Hashable, List, Optional, Sequence
 import numpy as np
 import torch
 
+from .. import log
 from ..cache.manager import CacheManager
 from ..models.causal_lm import CausalLM
 from ..parts.base import EntryMeta, StepContext, contexts_uneven
@@ -318,6 +319,8 @@ class ModelRunner:
                 return logits
             self._graphs[key] = rec
             self.graph_records += 1
+            log.debug(f"recorded the step of {key[0]} tokens for contexts up to {key[1]}"
+                      f"{' (uneven)' if key[2] else ''}: {self.graph_records} recordings")
             if len(self._graphs) > self.GRAPH_LIMIT:   # oldest recording out: contexts move on to higher buckets
                 self._graphs.pop(next(iter(self._graphs)))
             return logits

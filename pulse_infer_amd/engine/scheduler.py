@@ -32,6 +32,7 @@ from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, List, Optional, Sequence
 
+from .. import log
 from ..cache.manager import CacheManager
 from ..sampling.params import SamplingParams
 from .request import InferenceRequest, RequestState
@@ -176,6 +177,8 @@ class ContinuousBatchScheduler:
         return lo
 
     def _preempt(self, victim: InferenceRequest, batch: ScheduledBatch) -> None:
+        log.debug(f"request {victim.request_id} gives its pages back after {victim.num_computed_tokens} tokens "
+                  f"(preemption {self.num_preemptions + 1})")
         self.running.remove(victim)
         if self.cache is not None and self.cache.has_request(victim.request_id):
             self.cache.free_request(victim.request_id)
