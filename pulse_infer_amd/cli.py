@@ -62,6 +62,10 @@ def build_parser() -> argparse.ArgumentParser:
                         "config.json (for Qwen3: rope_pairing=half, the channels a rotation pairs); may be repeated")
     p.add_argument("--strict", action="store_true", help="a tensor that no part of the model asks for is an error")
     p.add_argument("--stats", action="store_true")
+    p.add_argument("--own-products", choices=["none", "swiglu", "all"], default=None,
+                   help="which bfloat16 products of 256 and more rows run as this package's tiled product instead of the "
+                        "vendor library's: gate and up with SwiGLU inside, all of them, or none "
+                        "(default: $PULSE_OWN_PRODUCTS, else none)")
     p.add_argument("--log-level", default=None, help="trace, debug, info, warn, error, critical or off "
                                                      "(default: $PULSE_LOG_LEVEL, else info); messages go to standard error")
     return p
@@ -112,6 +116,9 @@ def main(argv: Optional[List[str]] = None) -> int:
     if args.log_level:
         from . import log
         log.set_level(args.log_level)
+    if args.own_products:
+        from .parts import linear
+        linear.OWN_MANY_ROWS = args.own_products
     dtype = {"bf16": "bfloat16", "f32": "float32"}.get(args.dtype, args.dtype)
 
     import torch

@@ -238,12 +238,11 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_mid_kernel(const bf16_t* 
     }
 }
 
-// Weight loads run three chunks of 128 k (1.5 KB a lane group... 12 KB a wavefront) ahead; workgroups of two wavefronts,
-// which are taken where the weight has few rows and the chip holds barely more wavefronts than compute units, run
-// seven chunks ahead: what is in flight must cover the memory's latency at its full rate (6,144 weight rows at 64 rows
-// of X: 20.8 -> PULSE_MID_DEEP us).
+// Weight loads run three chunks of 128 k ahead (512 / KC slots of the ring). Seven chunks ahead for workgroups of two
+// wavefronts, which are taken where the weight has few rows, was measured and changed nothing (6,144 weight rows at
+// 64 rows of X: 20.8 us with either depth), so every shape keeps the shallow ring and its registers.
 template <int NW, int KC>
-constexpr int ring_for() { return (NW == 2 && KC == 128) ? 8 : 512 / KC; }
+constexpr int ring_for() { return 512 / KC; }
 
 template <int NW, int MT, int KC = 128>
 void launch_mid(const bf16_t* X, int64_t ldx, const bf16_t* W, int64_t ldw, void* C, int64_t ldc, int M, int N,

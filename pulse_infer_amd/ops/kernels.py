@@ -308,6 +308,50 @@ def gemm_rows(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, add: bool = F
          _i32(slabs), _stream(), label=f"N={n} K={k}")
 
 
+TILE_K = 64      # k a stage of the many-rows product
+TILE_ROWS = 256  # rows of X and of W an output tile
+
+
+def gemm_tile_takes(m: int, n: int, k: int, swiglu: bool = False, splits: int = 1, float32: bool = False) -> bool:
+    """Whether ``gemm_tile`` takes a shape (as pulse_gemm_tile_takes)."""
+    if m <= 0 or n <= 0 or k <= 0 or splits < 1 or (splits > 1 and not float32) or (swiglu and float32):
+        return False
+    step = 32 if swiglu else (4 if float32 else 8)
+    return k % (TILE_K * splits) == 0 and n % step == 0
+
+
+def gemm_tile(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, swiglu: bool = False) -> None:
+    """a @ w^T for many rows of bfloat16 (prompt portions): output tiles of 256 x 256 on the matrix cores, float32
+    accumulation, one rounding.
+
+    ``out`` bfloat16 [M, N]: the product; with ``swiglu`` the weight holds gate and up rows in alternating slabs of 16
+    and out [M, N / 2] is silu(gate) * up.  ``out`` float32 [splits, M, N] (or [M, N]): the partial products of equal
+    shares of K, which the consumer adds up in order."""
+    _gpu("gemm_tile", a, w, out)
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and w.dim() == 2
+          and a.stride(1) == 1 and w.stride(1) == 1, "gemm_tile: a and w must be bfloat16 matrices with contiguous rows")
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k, f"gemm_tile: inner sizes differ ({k} and {w.shape[1]})")
+    if out.dtype == torch.float32:
+        parts = out if out.dim() == 3 else out.view(1, *out.shape)
+        splits = parts.shape[0]
+        _need(not swiglu and tuple(parts.shape[1:]) == (m, n) and parts.stride(2) == 1,
+              f"gemm_tile: float32 results go to [shares, {m}, {n}] with contiguous rows")
+        _need(gemm_tile_takes(m, n, k, splits=splits, float32=True),
+              f"gemm_tile: M={m} N={n} K={k} in {splits} shares is not a shape it takes")
+        mode, ldc, part_stride = 2, (parts.stride(1) if m > 1 else n), (parts.stride(0) if splits > 1 else 0)
+    else:
+        cols = n // 2 if swiglu else n
+        _need(gemm_tile_takes(m, n, k, swiglu=swiglu), f"gemm_tile: M={m} N={n} K={k} is not a shape it takes")
+        _need(out.dtype == torch.bfloat16 and out.dim() == 2 and tuple(out.shape) == (m, cols) and out.stride(1) == 1,
+              f"gemm_tile: out must be bfloat16 [{m}, {cols}]")
+        mode, ldc, part_stride, splits = (1 if swiglu else 0), (out.stride(0) if m > 1 else cols), 0, 1
+    call("pulse_gemm_tile", _ptr(a), _i64(a.stride(0) if m > 1 else k), _ptr(w), _i64(w.stride(0) if n > 1 else k),
+         _ptr(out), _i64(ldc), _i32(m), _i32(n), _i32(k), _i32(mode), _i32(splits), _i64(part_stride), _stream(),
+         label=f"N={n} K={k}")
+
+
 MID_MAX_ROWS = 192
 
 

@@ -6,12 +6,16 @@ Three products stand behind it:
   matrix-core kernel, which can also add into the float32 residual or apply SwiGLU;
 * many rows of bfloat16: the vendor library's product (torch.matmul / torch.mm,
   i.e. hipBLASLt/rocBLAS, float32 accumulation, bfloat16 or float32 output), as
-  the reference uses cuBLAS (src/ops/kernels/cuda/matmul_kernel.cu:132-154);
+  the reference uses cuBLAS (src/ops/kernels/cuda/matmul_kernel.cu:132-154), or this
+  package's product in output tiles of 256 x 256, which can apply SwiGLU on the way
+  out or leave float32 results of shares of the inner dimension (``OWN_MANY_ROWS``
+  says which products go there);
 * the float32 run, and any weight kept in 32-bit: this package's own
   fused-multiply-add kernel, with no reduced-precision mode anywhere.
 """
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -20,6 +24,17 @@ from ..ops import kernels, timing
 from ..ops.device import compute_units
 from .base import LazyNorm, RowStats, Workspace
 
+
+# Which products of many rows (256 and more) run as this package's tiled product instead of the library's: "none";
+# "swiglu": gate and up with SwiGLU inside, which saves the pass over twice the feed-forward's width; "all": every
+# product of bfloat16 (a step then makes no library call).  PULSE_OWN_PRODUCTS sets it.  Measured through the
+# serving loop: a prompt of 2,048 tokens of the 8B shape 73.9K tokens/s with "none", 72.9K with "swiglu", 71.6K with
+# "all" (alone and with the chip warm, gate+up with SwiGLU inside takes 310 us against the library's 328 + 30 for
+# the pass; between the other kernels of a step the library's product takes 278); serving of the 8B shape 4,334 /
+# 4,313 / 4,248 tokens/s, of the 14B shape 2,637 / 2,723 / 2,632.  So the library stays the default.
+OWN_MANY_ROWS = os.environ.get("PULSE_OWN_PRODUCTS", "none")
+if OWN_MANY_ROWS not in ("none", "swiglu", "all"):
+    raise ValueError(f"PULSE_OWN_PRODUCTS must be none, swiglu or all, not '{OWN_MANY_ROWS}'")
 
 library_calls = 0   # products that went to the vendor library so far (a step that made none can be recorded as a graph)
 
@@ -50,7 +65,9 @@ class Linear:
             kernels.gemm_skinny(x.x, w, out, swiglu=swiglu, row_scale=(x.sumsq, x.eps))
             return out
         if swiglu:
-            if x.shape[0] > kernels.SKINNY_FAST_ROWS:
+            if x.shape[0] > self.MID_ROWS[1]:
+                kernels.gemm_tile(x, w, out, swiglu=True)
+            elif x.shape[0] > kernels.SKINNY_FAST_ROWS:
                 kernels.gemm_mid(x, w, out, swiglu=True, waves=self.swiglu_waves_for(x.shape[0]) or 4)
             else:
                 kernels.gemm_skinny(x, w, out, swiglu=True)
@@ -74,6 +91,10 @@ class Linear:
                     return out
                 waves = 10 if w.shape[0] >= 64 * compute_units() else 2
                 kernels.gemm_mid(x, w, out.view(1, *out.shape) if out.dtype == torch.float32 else out, waves=waves)
+                return out
+            if own and out.dtype == torch.bfloat16 and self.takes_tiles(x, w) and out.stride(1) == 1 \
+                    and out.stride(0) % 8 == 0 and out.data_ptr() % 16 == 0:
+                kernels.gemm_tile(x, w, out)
                 return out
             global library_calls
             library_calls += 1
@@ -109,6 +130,13 @@ class Linear:
             parts = workspace.buffer(f"linear.parts.{self.out_features}.{self.in_features}", splits * rows,
                                      self.out_features, torch.float32).view(splits, rows, self.out_features)
             kernels.gemm_mid(x, self.weight, parts, splits=splits, waves=waves)
+            return parts
+        splits = self.tile_shares_for(x) if workspace is not None else 0
+        if splits:
+            rows = x.shape[0]
+            parts = workspace.buffer(f"linear.parts.{self.out_features}.{self.in_features}", splits * rows,
+                                     self.out_features, torch.float32).view(splits, rows, self.out_features)
+            kernels.gemm_tile(x, self.weight, parts)
             return parts
         splits = self.library_shares_for(x) if workspace is not None else 0
         if splits:
@@ -189,6 +217,29 @@ class Linear:
         if out.dtype == torch.float32:
             return out.is_contiguous() and out.data_ptr() % 16 == 0 and w.shape[0] % 4 == 0
         return out.dtype == torch.bfloat16 and out.stride(1) == 1 and out.stride(0) % 4 == 0 and out.data_ptr() % 16 == 0
+
+    TILE_MIN_ROWS = 256          # from here on the tiled product for many rows is a candidate
+
+    def takes_tiles(self, x: torch.Tensor, w: Optional[torch.Tensor] = None, swiglu: bool = False) -> bool:
+        """Whether a product of this many rows runs as this package's tiled product (``OWN_MANY_ROWS`` allowing)."""
+        w = self.weight if w is None else w
+        if OWN_MANY_ROWS == "none" or (OWN_MANY_ROWS == "swiglu" and not swiglu):
+            return False
+        return (self.library and x.dtype == torch.bfloat16 and x.shape[0] >= self.TILE_MIN_ROWS and self.operands_ok(x)
+                and kernels.gemm_tile_takes(x.shape[0], w.shape[0], w.shape[1], swiglu=swiglu))
+
+    def tile_shares_for(self, x: torch.Tensor) -> int:
+        """Into how many shares of the inner dimension the tiled product of many rows is cut when it adds into the
+        residual (float32 results that the next norm adds up); 0: not this product.  As many shares as bring the
+        tiles to the number of compute units, at most 8."""
+        if OWN_MANY_ROWS != "all" or not self.takes_tiles(x) or self.out_features % 4:
+            return 0
+        tile = kernels.TILE_ROWS
+        tiles = ((x.shape[0] + tile - 1) // tile) * ((self.out_features + tile - 1) // tile)
+        splits = max(1, min(8, compute_units() // tiles))
+        while splits > 1 and self.in_features % (splits * kernels.TILE_K):
+            splits -= 1
+        return splits
 
     def takes_shared_k(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
         """Whether a bfloat16 product of 17 to 64 rows runs with the inner dimension shared out inside a workgroup:

@@ -67,6 +67,8 @@ class GatedMLP(Part):
         elif (self.slab and self.gate_up.takes_mid(x) and (2 * self.inter) % 32 == 0
               and kernels.gemm_mid_takes(tokens, 2 * self.inter, self.hidden)):
             self.gate_up.forward(x, z, swiglu=True)   # 17 to 64 rows: X shared through LDS, SwiGLU in the epilogue
+        elif self.slab and self.gate_up.takes_tiles(x, swiglu=True):
+            self.gate_up.forward(x, z, swiglu=True)   # many rows: output tiles on the matrix cores, SwiGLU on the way out
         else:
             gu = ws.buffer("mlp.gate_up", tokens, 2 * self.inter, self.act_dtype)
             self.gate_up.forward(x, gu, own=False)   # (the shapes that come here at 17 to 64 rows are those the library wins)

@@ -1279,6 +1279,109 @@ def test_gemm_rows_refuses(k):
         k.gemm_rows(a[:8], w, torch.zeros(8, 64, dtype=torch.bfloat16, device=DEV), slabs=3)
 
 
+@pytest.mark.parametrize("m,n,kk", [(1, 32, 64), (256, 256, 64), (300, 520, 192), (257, 1056, 4160), (2048, 2304, 512),
+                                    (2500, 264, 128)])
+def test_gemm_tile(k, m, n, kk):
+    """The product for many rows (output tiles of 256 x 256, four wavefronts, K in steps of 64 through two LDS stages
+    filled straight from memory) against float64: bfloat16 results, float32 results of 1, 2 and 4 shares of K, rows
+    that are views into wider buffers; tiles that hang over both edges, a single step of K and one more than the
+    stages, panels of eight and of fewer tiles.  A piece of a row copied to another place than the operand reads look
+    for it in, a quarter of the tile or a k group swapped, a stage read before its copies had landed or overwritten
+    before its last read: all of them change results by their own size."""
+    a, aref = as_stored(rnd(m, kk, seed=201), torch.bfloat16)
+    w, wref = as_stored(rnd(n, kk, seed=202, scale=kk ** -0.5), torch.bfloat16)
+    want = aref @ wref.T
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    k.gemm_tile(a, w, out)
+    assert torch.allclose(out.cpu().to(F64), want, atol=2e-2, rtol=1e-2)
+    again = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    k.gemm_tile(a, w, again)
+    assert torch.equal(out, again)
+    for splits in (1, 2, 4):
+        if kk % (64 * splits):
+            continue
+        parts = torch.full((splits, m + 1, n), float("nan"), device=DEV)[:, :m]
+        k.gemm_tile(a, w, parts)
+        total = parts.cpu().to(F64).sum(dim=0)
+        assert torch.allclose(total, want, atol=1e-4, rtol=1e-5), splits
+        if splits == 1:
+            assert torch.equal(parts[0].to(torch.bfloat16), out)      # the same sums, rounded once
+            flat = torch.full((m, n), float("nan"), device=DEV)
+            k.gemm_tile(a, w, flat)
+            assert torch.equal(flat, parts[0])
+    wide = torch.zeros(m, kk + 24, dtype=torch.bfloat16, device=DEV)
+    wide[:, :kk] = a
+    padded = torch.zeros(m, n + 8, dtype=torch.bfloat16, device=DEV)
+    k.gemm_tile(wide[:, :kk], w, padded[:, :n])
+    assert torch.equal(padded[:, :n], out) and bool((padded[:, n:] == 0).all())
+
+
+@pytest.mark.parametrize("m,inter,kk", [(256, 128, 64), (700, 1008, 256), (1030, 2064, 1088)])
+def test_gemm_tile_swiglu(k, m, inter, kk):
+    """SwiGLU on the way out of the many-rows product, gate and up rows in alternating slabs of 16 (a tile's last
+    pair of slabs included), against float64 and against the product followed by the SwiGLU kernel."""
+    a, aref = as_stored(rnd(m, kk, seed=203), torch.bfloat16)
+    gate, gref = as_stored(rnd(inter, kk, seed=204, scale=kk ** -0.5), torch.bfloat16)
+    up, uref = as_stored(rnd(inter, kk, seed=205, scale=kk ** -0.5), torch.bfloat16)
+    mixed = torch.stack([gate.view(-1, 16, kk), up.view(-1, 16, kk)], dim=1).reshape(2 * inter, kk).contiguous()
+    want = P.silu(aref @ gref.T) * (aref @ uref.T)
+    out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+    k.gemm_tile(a, mixed, out, swiglu=True)
+    assert torch.allclose(out.cpu().to(F64), want, atol=1e-2, rtol=1e-2)
+    gu = torch.empty(m, 2 * inter, dtype=torch.bfloat16, device=DEV)
+    k.gemm_tile(a, mixed, gu)
+    z = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    k.swiglu(gu, z, slab=16)                                  # (this one rounds gate and up before it multiplies)
+    assert torch.allclose(out.float(), z.float(), atol=1e-2, rtol=2e-2)
+
+
+def test_gemm_tile_at_the_benchmark_shape(k):
+    """gate and up of the benchmark's layer for a prompt of 2,048 tokens (768 tiles, three for every compute unit,
+    64 steps of K each): SwiGLU inside against the float32 product of the same rounded operands followed by the
+    formula, the bfloat16 product against the library's, and o's shape in two shares of K."""
+    m, inter, kk = 2048, 12288, 4096
+    a = rnd(m, kk, seed=206).to(torch.bfloat16).to(DEV)
+    mixed = rnd(2 * inter, kk, seed=207, scale=kk ** -0.5).to(torch.bfloat16).to(DEV)
+    ref = a.float() @ mixed.float().T                          # float32 on the device (no reduced-precision mode)
+    slabs = ref.view(m, inter // 16, 2, 16)
+    want = (torch.nn.functional.silu(slabs[:, :, 0]) * slabs[:, :, 1]).reshape(m, inter)
+    out = torch.full((m, inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+    k.gemm_tile(a, mixed, out, swiglu=True)
+    assert torch.allclose(out.float(), want, atol=1e-2, rtol=1e-2)
+    plain = torch.full((m, 2 * inter), float("nan"), dtype=torch.bfloat16, device=DEV)
+    k.gemm_tile(a, mixed, plain)
+    assert torch.allclose(plain.float(), ref, atol=2e-2, rtol=1e-2)
+    library = torch.matmul(a, mixed.t())
+    assert torch.allclose(plain.float(), library.float(), atol=2e-2, rtol=2e-2)
+    del ref, slabs, want, out, plain, library
+    w_o = mixed[:4096]
+    parts = torch.full((2, m, 4096), float("nan"), device=DEV)
+    k.gemm_tile(a, w_o, parts)
+    assert torch.allclose(parts.sum(dim=0), a.float() @ w_o.float().T, atol=1e-3, rtol=1e-4)
+    half = kk // 2
+    assert torch.allclose(parts[1], a[:, half:].float() @ w_o[:, half:].float().T, atol=1e-3, rtol=1e-4)
+
+
+def test_gemm_tile_refuses(k):
+    from pulse_infer_amd.ops import KernelError
+    a = torch.zeros(300, 192, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(64, 192, dtype=torch.bfloat16, device=DEV)
+    assert k.gemm_tile_takes(300, 64, 192) and not k.gemm_tile_takes(300, 64, 96) and not k.gemm_tile_takes(300, 60, 192)
+    assert k.gemm_tile_takes(300, 64, 192, swiglu=True) and not k.gemm_tile_takes(300, 48, 192, swiglu=True)
+    assert k.gemm_tile_takes(300, 60, 192, splits=3, float32=True) and not k.gemm_tile_takes(300, 64, 192, splits=2, float32=True)
+    assert not k.gemm_tile_takes(300, 64, 192, splits=3)
+    with pytest.raises(KernelError, match="not a shape"):
+        k.gemm_tile(a[:, :96].contiguous(), w[:, :96].contiguous(), torch.zeros(300, 64, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(KernelError, match="not a shape"):
+        k.gemm_tile(a, w, torch.zeros(2, 300, 64, device=DEV))
+    with pytest.raises(KernelError, match=r"out must be bfloat16 \[300, 32\]"):
+        k.gemm_tile(a, w, torch.zeros(300, 64, dtype=torch.bfloat16, device=DEV), swiglu=True)
+    with pytest.raises(KernelError, match="inner sizes"):
+        k.gemm_tile(a, w[:, :128].contiguous(), torch.zeros(300, 64, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(KernelError, match="float32 results go to"):
+        k.gemm_tile(a, w, torch.zeros(3, 300, 32, device=DEV))
+
+
 def test_gemm_mid_refuses(k):
     from pulse_infer_amd.ops import KernelError
     a = torch.zeros(193, 256, dtype=torch.bfloat16, device=DEV)

@@ -225,6 +225,33 @@ def test_benchmark_layer_sizes(layer_shape, dtype):
     torch.cuda.empty_cache()
 
 
+@pytest.mark.parametrize("policy", ["swiglu", "all"])
+def test_benchmark_layer_sizes_with_this_packages_products_for_many_rows(layer_shape, policy, monkeypatch):
+    """A prompt of 600 tokens at the benchmark's layer sizes, whole and in portions of 300, 260 and 40 tokens, with the
+    products of 256 and more rows in this package's tiled product (gate and up with SwiGLU inside; or all of them, o
+    and down in shares of the inner dimension) against the plain implementation and against the library's products."""
+    from pulse_infer_amd.engine.runner import ModelRunner
+    from pulse_infer_amd.models.factory import load_model
+    from pulse_infer_amd.parts import linear
+
+    folder, _, _, plain = layer_shape
+    ids = token_ids(LAYER_SHAPE["vocab_size"], 600, seed=44)
+    want = plain.logits(ids)
+    _, model = load_model(folder, mode="bfloat16")
+    runner = ModelRunner(model, page_size=16, num_pages=40, max_requests=2)
+    library = run_alone(runner, ids, [len(ids)])
+    monkeypatch.setattr(linear, "OWN_MANY_ROWS", policy)
+    whole = run_alone(runner, ids, [len(ids)])
+    close(whole, want, "bfloat16", f"own products ({policy}), whole")
+    close(whole, library, "bfloat16", f"own products ({policy}) against the library's", SPLIT_TOL)
+    assert not torch.equal(whole, library)                 # (another kernel did run)
+    portions = run_alone(runner, ids, [300, 260, 40])
+    close(portions, want, "bfloat16", f"own products ({policy}), portions")
+    close(portions, whole, "bfloat16", f"own products ({policy}), portions against whole", SPLIT_TOL)
+    del runner, model
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_benchmark_layer_sizes_mixed_with_page_reuse(layer_shape, dtype):
     """Up to four live requests at the benchmark model's layer sizes over a pool of 256 tokens: steps that hold a

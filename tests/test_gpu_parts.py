@@ -114,6 +114,40 @@ def test_feed_forward_part(gpu, mode):
         FEED_FORWARDS.get("gated_mlp")({"hidden_size": hidden, "intermediate_size": inter, "activation": "relu"}, "m", build)
 
 
+@pytest.mark.parametrize("policy", ["none", "swiglu", "all"])
+@pytest.mark.parametrize("rows", [300, 700])
+def test_feed_forward_part_at_many_rows_under_each_choice_of_products(gpu, rows, policy, monkeypatch):
+    """A prompt portion of some hundred rows through the feed-forward with the library's products, with gate and up
+    in this package's tiled product (SwiGLU inside), and with every product in it (the way back in shares of the
+    inner dimension, float32 results that are added to the residual in order): all against float64, and the last
+    one without a library call."""
+    from pulse_infer_amd.ops import kernels
+    from pulse_infer_amd.parts import linear
+    from pulse_infer_amd.parts.base import FEED_FORWARDS
+    monkeypatch.setattr(linear, "OWN_MANY_ROWS", policy)
+    hidden, inter = 192, 448
+    ws = {"m.gate_proj.weight": rnd(inter, hidden, seed=3, scale=hidden ** -0.5),
+          "m.up_proj.weight": rnd(inter, hidden, seed=4, scale=hidden ** -0.5),
+          "m.down_proj.weight": rnd(hidden, inter, seed=5, scale=inter ** -0.5)}
+    build = build_ctx(ws, "bfloat16")
+    mlp = FEED_FORWARDS.get("gated_mlp")({"hidden_size": hidden, "intermediate_size": inter, "activation": "silu"}, "m", build)
+    x = rnd(rows, hidden, seed=6).to(build.act_dtype).to(DEV)
+    ctx = step_ctx(build, list(range(rows)), [0] * rows, [[0]])
+    assert mlp.gate_up.takes_tiles(x, swiglu=True) == (policy != "none")
+    assert mlp.down.takes_tiles(torch.empty(rows, inter, dtype=torch.bfloat16, device=DEV)) == (policy == "all")
+    before = linear.library_calls
+    h0 = rnd(rows, hidden, seed=7).float().to(DEV)
+    h = h0.clone()
+    update = mlp.forward(x, ctx, residual=h)
+    assert linear.library_calls - before == {"none": 2, "swiglu": 1, "all": 0}[policy]
+    w64 = [ws[f"m.{n}_proj.weight"].to(torch.bfloat16).to(F64) for n in ("gate", "up", "down")]
+    want = P.gated_mlp(x.cpu().to(F64), *w64)
+    if policy == "all":
+        assert update.dim() == 3 and update.dtype == torch.float32       # shares of the inner dimension
+    kernels.residual_add(h, update)
+    assert torch.allclose(h.cpu().to(F64) - h0.cpu().to(F64), want, **TOL["bfloat16"])
+
+
 @pytest.mark.parametrize("rows", [1, 7, 16, 20])
 def test_a_norm_is_finished_behind_the_product_that_consumes_it(gpu, rows):
     """The protocol that takes the norm kernels out of a decoding step, on real parts of a width the fused products
