@@ -64,10 +64,10 @@ struct TileArgs {
 // (eight in a row, or sixteen) then lie in different 16-byte places of what LDS serves at once.
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
-// 16 bytes a lane from memory straight into LDS: lane i's piece lands at lds_base + 16 i (a wavefront-wide address).
-// The compiler knows nothing of these copies, so the waits for them are written out below.
-__device__ __forceinline__ void load_to_lds(const void* from, uint32_t lds_base) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_base), "v"(from) : "memory", "m0");
+// 16 bytes a lane from memory straight into LDS: lane i's piece, `offset` bytes behind `base`, lands at lds_base + 16 i
+// (a wavefront-wide address).  The compiler knows nothing of these copies, so the waits for them are written out below.
+__device__ __forceinline__ void load_to_lds(const void* base, uint32_t offset, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_base), "v"(offset), "s"(base) : "memory", "m0");
 }
 
 template <int MODE>
@@ -99,20 +99,21 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_tile_kernel(TileArgs a) {
 
     // Copy: chunk q of a tile is its rows 8 q .. 8 q + 7; lane i brings the piece that belongs at place i % 8 of row
     // i / 8.  Rows past the operand's end are its last row again (their results are not written).
-    const bf16_t* w_from[PER];
-    const bf16_t* x_from[PER];
+    // The address is a base in scalar registers, which moves along K, and a lane's byte offset from it, which does not.
+    const bf16_t* w_base = a.W + static_cast<int64_t>(n0) * a.ldw + static_cast<int64_t>(split) * a.K;
+    const bf16_t* x_base = a.X + static_cast<int64_t>(m0) * a.ldx + static_cast<int64_t>(split) * a.K;
+    uint32_t w_from[PER], x_from[PER];
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
         const int row = (wave * PER + j) * 8 + lane / 8;
         const int c = (lane % 8) ^ swz(row);
-        const int64_t k0 = static_cast<int64_t>(split) * a.K + c * 8;
-        w_from[j] = a.W + static_cast<int64_t>(min(n0 + row, a.N - 1)) * a.ldw + k0;
-        x_from[j] = a.X + static_cast<int64_t>(min(m0 + row, a.M - 1)) * a.ldx + k0;
+        w_from[j] = static_cast<uint32_t>((static_cast<int64_t>(min(n0 + row, a.N - 1) - n0) * a.ldw + c * 8) * 2);
+        x_from[j] = static_cast<uint32_t>((static_cast<int64_t>(min(m0 + row, a.M - 1) - m0) * a.ldx + c * 8) * 2);
     }
     auto load_one = [&](int k, int stage, int j) {   // j: first the wavefront's chunks of W, then of X
         const uint32_t to = lds0 + stage * STAGE_BYTES + wave * PER * 1024;
-        if (j < PER) load_to_lds(w_from[j] + k, to + j * 1024);
-        else load_to_lds(x_from[j - PER] + k, to + OPERAND_BYTES + (j - PER) * 1024);
+        if (j < PER) load_to_lds(w_base + k, w_from[j], to + j * 1024);
+        else load_to_lds(x_base + k, x_from[j - PER], to + OPERAND_BYTES + (j - PER) * 1024);
     };
 
     // Operand reads: lane l holds row l % 32 and the k group l / 32 (8 values) of a 32 x 16 piece.
@@ -141,22 +142,25 @@ __global__ __launch_bounds__(NW* PULSE_WAVE) void gemm_tile_kernel(TileArgs a) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[f][g][i] = 0.f;
 
-    // A quarter of a step: the products of one k group from one set of operand registers, in pairs; behind every
-    // pair one copy instruction (where the quarter has copies) and its share of the next k group's operand reads
-    // into the other set.  Nothing moves across the fences.
+    // A quarter of a step: the products of one k group from one set of operand registers, in pairs; between the two
+    // of a pair one copy instruction (where the quarter has copies), behind the pair its share of the next k group's
+    // operand reads into the other set.  Nothing moves across the fences.
     static_assert(PER <= PAIRS, "a copy instruction a pair of products");
     auto quarter = [&](int use, int rd_stage, int rd_kk, int ld_k, int ld_stage, int ld_first) {
 #pragma unroll
         for (int p = 0; p < PAIRS; ++p) {
-#pragma unroll
-            for (int i = 2 * p; i < 2 * p + 2; ++i)
+            auto product = [&](int i) {
                 acc[i / TM][i % TM] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[use][i / TM], xf[use][i % TM],
                                                                               acc[i / TM][i % TM], 0, 0, 0);
+            };
+            product(2 * p);
             __builtin_amdgcn_sched_barrier(0);
             if (ld_first >= 0 && p < PER) {
                 load_one(ld_k, ld_stage, ld_first + p);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            product(2 * p + 1);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int r = (p * NR + PAIRS - 1) / PAIRS; r < ((p + 1) * NR + PAIRS - 1) / PAIRS; ++r)
                 read_one(rd_stage, rd_kk, use ^ 1, r);
@@ -302,8 +306,9 @@ extern "C" int pulse_gemm_tile(const void* X, int64_t ldx, const void* W, int64_
                   "be a multiple of 64 a share, the weight rows a multiple of 8 (32 with SwiGLU, 4 for float32 results), "
                   "shares need float32 results", M, N, K, mode, splits);
     PULSE_REQUIRE(X && W && C && aligned16(X) && aligned16(W) && aligned16(C), "gemm_tile: operands must be aligned to 16 bytes");
-    PULSE_REQUIRE(ldx >= K && ldw >= K && ldx % 8 == 0 && ldw % 8 == 0, "gemm_tile: rows of X and W must be K long at "
-                  "least and start at multiples of 16 bytes (strides %lld, %lld)", (long long)ldx, (long long)ldw);
+    PULSE_REQUIRE(ldx >= K && ldw >= K && ldx % 8 == 0 && ldw % 8 == 0 && ldx < (1 << 22) && ldw < (1 << 22),
+                  "gemm_tile: rows of X and W must be K long at least, start at multiples of 16 bytes and lie less than "
+                  "4M elements apart (strides %lld, %lld)", (long long)ldx, (long long)ldw);
     const int out_cols = mode == OUT_SWIGLU ? N / 2 : N;
     PULSE_REQUIRE(ldc >= out_cols && ldc % (mode == OUT_F32 ? 4 : 8) == 0, "gemm_tile: rows of the result must be %d long at "
                   "least and start at multiples of 16 bytes (stride %lld)", out_cols, (long long)ldc);
