@@ -31,7 +31,8 @@ from .base import LazyNorm, RowStats, Workspace
 # serving loop: a prompt of 2,048 tokens of the 8B shape 73.9K tokens/s with "none", 72.9K with "swiglu", 71.6K with
 # "all" (alone and with the chip warm, gate+up with SwiGLU inside takes 310 us against the library's 328 + 30 for
 # the pass; between the other kernels of a step the library's product takes 278); serving of the 8B shape 4,334 /
-# 4,313 / 4,248 tokens/s, of the 14B shape 2,637 / 2,723 / 2,632.  So the library stays the default.
+# 4,313 / 4,248 tokens/s, of the 14B shape 2,695 / 2,688 (means of two runs each, "none" and "swiglu"), of the 32B shape
+# 1,258 / 1,264.  So the library stays the default.
 OWN_MANY_ROWS = os.environ.get("PULSE_OWN_PRODUCTS", "none")
 if OWN_MANY_ROWS not in ("none", "swiglu", "all"):
     raise ValueError(f"PULSE_OWN_PRODUCTS must be none, swiglu or all, not '{OWN_MANY_ROWS}'")
