@@ -239,6 +239,7 @@ def test_benchmark_layer_sizes_with_this_packages_products_for_many_rows(layer_s
     want = plain.logits(ids)
     _, model = load_model(folder, mode="bfloat16")
     runner = ModelRunner(model, page_size=16, num_pages=40, max_requests=2)
+    monkeypatch.setattr(linear, "OWN_MANY_ROWS", "none")      # (whatever PULSE_OWN_PRODUCTS says)
     library = run_alone(runner, ids, [len(ids)])
     monkeypatch.setattr(linear, "OWN_MANY_ROWS", policy)
     whole = run_alone(runner, ids, [len(ids)])

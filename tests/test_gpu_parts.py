@@ -66,13 +66,15 @@ def test_norm_part(gpu, mode):
 
 
 @pytest.mark.parametrize("rows,n,splits", [(300, 768, 4), (700, 768, 4), (1800, 2048, 2)])
-def test_linear_adds_into_the_residual_through_shares_of_the_library_product(gpu, rows, n, splits):
+def test_linear_adds_into_the_residual_through_shares_of_the_library_product(gpu, rows, n, splits, monkeypatch):
     """Many rows, a wide inner dimension and few output tiles: ``Linear.add_into`` runs the library's product as a
     batch over shares of the inner dimension and hands back their float32 results, which the norm's kernel (and the
     plain addition) add to the residual in order."""
     from pulse_infer_amd.ops import kernels
     from pulse_infer_amd.parts.base import Workspace
+    from pulse_infer_amd.parts import linear
     from pulse_infer_amd.parts.linear import Linear
+    monkeypatch.setattr(linear, "OWN_MANY_ROWS", "none")      # (whatever PULSE_OWN_PRODUCTS says)
     k = 8192
     w = rnd(n, k, seed=3, scale=k ** -0.5).to(DEV)
     x = rnd(rows, k, seed=4).to(DEV)
